@@ -1,0 +1,125 @@
+/*
+ * ldist -- L_p / L_inf distance-neuron operators for AMD MI355X (gfx950).
+ *
+ * C ABI of libldist_hip.so.  Plain pointers and sizes only: every pointer is a
+ * DEVICE pointer to float32 / int32 data on the current HIP device, `stream`
+ * is a hipStream_t passed as void* (NULL = the default stream).  All calls are
+ * asynchronous with respect to the host: they enqueue kernels on `stream` and
+ * return.  The library allocates nothing, keeps no state between calls and
+ * never frees or retains the caller's buffers, like the reference launchers
+ * (model/norm_dist.py:10-15,34,37,42,45,63-64 allocate everything in Python).
+ *
+ * Each of the seven core entry points replaces one `*_cuda` launcher declared
+ * in the reference's binding (model/norm_dist.cpp:7-20) and keeps its argument
+ * order; `stream` is appended.  As there, CO and CI are totals over all groups.
+ *
+ * Tensor layout, all contiguous (model/inf_dist_cuda.cu:29-33,65-66):
+ *   input   (B, CI, HW)   element ((b*G + g)*K  + k )*HW + hw,   K  = CI/G
+ *   weight  (CO, K)       element  (g*NG + n)*K + k,             NG = CO/G
+ *   output  (B, CO, HW)   element ((b*G + g)*NG + n )*HW + hw    (also pos, grad_output)
+ *
+ * Return value: LDIST_OK, or a negative LDIST_E* code.  Nothing is launched
+ * when an argument check fails.  No C++ exception crosses this boundary.
+ */
+#ifndef LDIST_H
+#define LDIST_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LDIST_VERSION 100 /* major*10000 + minor*100 + patch */
+
+enum {
+    LDIST_OK = 0,
+    LDIST_EINVAL = -1,  /* null pointer, non-positive size, CI % G or CO % G non-zero, p <= 1 or NaN */
+    LDIST_ERANGE = -2,  /* a tensor has 2^31 or more elements (kernels index with 32 bits) */
+    LDIST_ELAUNCH = -3, /* the HIP runtime reported an error at launch (see ldist_last_hip_error) */
+    LDIST_EDEVICE = -4  /* the current device is not a gfx950 the library was built for */
+};
+
+typedef void* ldist_stream_t; /* hipStream_t */
+
+int ldist_version(void);
+const char* ldist_strerror(int code);
+/* hipError_t of the last failed launch made by the calling thread (0 if none). */
+int ldist_last_hip_error(void);
+
+/* Testing and tuning knob, no counterpart in the reference: forces the workgroup
+ * tiling of the three forward kernels.  -1 = choose by shape (default), 0 = 128x80
+ * tile with two k-groups, 1 = 128x64, 2 = 256x32.  Process-wide; not thread safe. */
+int ldist_set_tile_override(int choice);
+
+/* L_inf forward.  Replaces inf_dist_forward_cuda (model/norm_dist.cpp:13-14,
+ * model/inf_dist_cuda.cu:173-180).
+ *   output[m,n] = max_k |x[m,k] - w[n,k]|
+ *   pos[m,n]    = k*, the LOWEST k attaining the maximum, with bit 31 set when
+ *                 x[m,k*] - w[n,k*] < 0; 0 when the maximum is 0.
+ * A NaN difference never wins.  Values and indices are bit-exact with the
+ * reference rule "scan k ascending, update on strict >" (inf_dist_cuda.cu:36-43). */
+int ldist_inf_dist_forward(const float* input, const float* weight, int B, int CO, int CI, int G, int HW,
+                           float* output, int32_t* pos, ldist_stream_t stream);
+
+/* Interval-bound forward.  Replaces inf_dist_bound_forward_cuda
+ * (model/norm_dist.cpp:15-16, model/inf_dist_cuda.cu:181-188).
+ *   output_upper = max_k max(|l-w|, |u-w|)
+ *   output_lower = max_k min(|l-w|, |u-w|) over the k where not (l-w < 0 < u-w), else 0 */
+int ldist_inf_dist_bound_forward(const float* input_lower, const float* input_upper, const float* weight, int B,
+                                 int CO, int CI, int G, int HW, float* output_lower, float* output_upper,
+                                 ldist_stream_t stream);
+
+/* L_inf backward w.r.t. input.  Replaces inf_dist_backward_input_cuda
+ * (model/norm_dist.cpp:17-18, model/inf_dist_cuda.cu:189-196).
+ *   grad_input[b, g*K + idx, hw] += (pos >= 0 ? g : -g),  idx = pos & 0x7fffffff
+ * grad_input must hold zeros (or the values to accumulate onto) on entry,
+ * as the reference requires (model/norm_dist.py:34). */
+int ldist_inf_dist_backward_input(const float* grad_output, const int32_t* pos, int B, int CO, int CI, int G, int HW,
+                                  float* grad_input, ldist_stream_t stream);
+
+/* L_inf backward w.r.t. weight.  Replaces inf_dist_backward_weight_cuda
+ * (model/norm_dist.cpp:19-20, model/inf_dist_cuda.cu:197-204).
+ *   grad_weight[g*NG + n, idx] += (pos < 0 ? g : -g), summed over b and hw
+ * grad_weight must hold zeros (or the values to accumulate onto) on entry (model/norm_dist.py:37). */
+int ldist_inf_dist_backward_weight(const float* grad_output, const int32_t* pos, int B, int CO, int CI, int G, int HW,
+                                   float* grad_weight, ldist_stream_t stream);
+
+/* p-norm forward, p > 1.  Replaces norm_dist_forward_cuda
+ * (model/norm_dist.cpp:7-8, model/norm_dist_cuda.cu:427-437).
+ *   output = m * (1e-10*(1e-10/m)^p + sum_k (|x-w|/m)^p)^(1/p),  m = max(1e-10, max_k |x-w|)
+ * i.e. (sum |x-w|^p)^(1/p) evaluated with the reference's max-normalised
+ * stabilisation and seeds (norm_dist_cuda.cu:232-233,253-264,289). */
+int ldist_norm_dist_forward(const float* input, const float* weight, int B, int CO, int CI, int G, int HW,
+                            float* output, float p, ldist_stream_t stream);
+
+/* p-norm backward w.r.t. input.  Replaces norm_dist_backward_input_cuda
+ * (model/norm_dist.cpp:9-10, model/norm_dist_cuda.cu:438-448).
+ *   grad_input[m,k] = sum_n g[m,n] * (|x-w| / output[m,n])^(p-1) * (x-w > 0 ? 1 : -1)
+ * Every element of grad_input is written; it may be uninitialised on entry (model/norm_dist.py:42). */
+int ldist_norm_dist_backward_input(const float* grad_output, const float* input, const float* weight,
+                                   const float* output, int B, int CO, int CI, int G, int HW, float* grad_input,
+                                   float p, ldist_stream_t stream);
+
+/* p-norm backward w.r.t. weight.  Replaces norm_dist_backward_weight_cuda
+ * (model/norm_dist.cpp:11-12, model/norm_dist_cuda.cu:449-459).
+ *   grad_weight[n,k] += sum_{b,hw} g * (|w-x| / output)^(p-1) * (w-x > 0 ? 1 : -1)
+ * grad_weight must hold zeros (or the values to accumulate onto) on entry (model/norm_dist.py:45). */
+int ldist_norm_dist_backward_weight(const float* grad_output, const float* input, const float* weight,
+                                    const float* output, int B, int CO, int CI, int G, int HW, float* grad_weight,
+                                    float p, ldist_stream_t stream);
+
+/* The two scatter backward passes again, but writing EVERY element of the
+ * gradient (zeros where nothing lands) so the caller can pass uninitialised
+ * memory and skip its own zero fill.  No counterpart in the reference, which
+ * needs torch.zeros_like first (model/norm_dist.py:34,37); results are equal
+ * to zero-fill followed by the accumulate entry points above. */
+int ldist_inf_dist_backward_input_overwrite(const float* grad_output, const int32_t* pos, int B, int CO, int CI,
+                                            int G, int HW, float* grad_input, ldist_stream_t stream);
+int ldist_inf_dist_backward_weight_overwrite(const float* grad_output, const int32_t* pos, int B, int CO, int CI,
+                                             int G, int HW, float* grad_weight, ldist_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LDIST_H */

@@ -1,0 +1,148 @@
+// Stage pipeline and output addressing shared by the three forward kernels
+// (L_inf with argmax, interval bound, p-norm).
+#pragma once
+#include "kernels.hpp"
+#include "tile.hpp"
+
+namespace ldist {
+
+// Global -> register -> LDS staging of one pipeline stage: NX input panels
+// (x, or lower and upper) followed by the weight panel.
+template <class GEO, bool CONV, int VEC, int NX>
+struct Stager {
+    static constexpr int STAGE = NX * GEO::XS + GEO::WS;  // floats per stage
+    // Two LDS buffers (one barrier per stage) when that still lets a CU hold two waves
+    // per SIMD, i.e. one 512-lane or two 256-lane workgroups in 160 KB; else one buffer.
+    static constexpr int NBUF = (2 * STAGE * 4 * (GEO::KS == 1 ? 2 : 1) <= 160 * 1024) ? 2 : 1;
+    static constexpr size_t LDS_BYTES = (size_t)NBUF * STAGE * sizeof(float);
+    using WLoad = RowsK<GEO::BN, GEO::SN, GEO::NT, GEO::KK, VEC>;
+    using XLoadK = RowsK<GEO::BM, GEO::SM, GEO::NT, GEO::KK, VEC>;
+    using XLoadM = RowsM<GEO::BM, GEO::SM, GEO::NT, GEO::KK, VEC>;
+    WLoad wl;
+    XLoadK xlk[NX];
+    XLoadM xlm[NX];
+    int off_m[XLoadM::N];
+    const float* wbase;
+    const float* in[NX];
+    int K, ld_x, rows_x, rows_w, kstride, tid;
+
+    __device__ __forceinline__ void init(const float* const (&input)[NX], const float* weight, const Dims& d, int m0,
+                                         int n0, int g, int tid_) {
+        tid = tid_;
+        K = d.K;
+        wbase = weight + ((size_t)g * d.NG + n0) * K;
+        rows_w = d.NG - n0;
+        rows_x = d.M - m0;
+        kstride = d.HW;
+        ld_x = d.G * K;
+#pragma unroll
+        for (int q = 0; q < NX; q++)
+            in[q] = CONV ? input[q] : input[q] + ((size_t)m0 * d.G + g) * K;  // fc: row m is image b
+        if constexpr (CONV) XLoadM::offsets(off_m, m0, d.M, d.HW, d.G, g, K, tid);
+    }
+    __device__ __forceinline__ void load(int k0) {
+        wl.load(wbase, K, rows_w, k0, K, tid);
+#pragma unroll
+        for (int q = 0; q < NX; q++) {
+            if constexpr (CONV) xlm[q].load(in[q], off_m, kstride, k0, K, tid);
+            else xlk[q].load(in[q], ld_x, rows_x, k0, K, tid);
+        }
+    }
+    // For the interval kernel (NX == 2: lower, upper): true when some value this lane
+    // just loaded breaks lower <= upper, or is NaN or infinite (weights included).
+    __device__ __forceinline__ bool interval_is_irregular() const {
+        static_assert(NX <= 2, "");
+        bool bad = false;
+        if constexpr (NX == 2) {
+            constexpr float INF = __builtin_inff();
+            if constexpr (CONV) {
+#pragma unroll
+                for (int i = 0; i < XLoadM::N; i++)
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) {
+                        const float l = xlm[0].v[i][e], u = xlm[1].v[i][e];
+                        bad |= !(l <= u && __builtin_fabsf(l) < INF && __builtin_fabsf(u) < INF);
+                    }
+            } else {
+#pragma unroll
+                for (int i = 0; i < XLoadK::N; i++)
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) {
+                        const float l = xlk[0].v[i][e], u = xlk[1].v[i][e];
+                        bad |= !(l <= u && __builtin_fabsf(l) < INF && __builtin_fabsf(u) < INF);
+                    }
+            }
+#pragma unroll
+            for (int i = 0; i < WLoad::N; i++)
+#pragma unroll
+                for (int e = 0; e < VEC; e++) bad |= !(__builtin_fabsf(wl.v[i][e]) < INF);
+        }
+        return bad;
+    }
+    __device__ __forceinline__ void store(float* stage) const {
+#pragma unroll
+        for (int q = 0; q < NX; q++) {
+            if constexpr (CONV) xlm[q].store(stage + q * GEO::XS, tid);
+            else xlk[q].store(stage + q * GEO::XS, tid);
+        }
+        wl.store(stage + NX * GEO::XS, tid);
+    }
+};
+
+// Element offsets of row m of the input (k = 0) and of the output (n = 0), and
+// the element strides of k and n, for either layout.
+template <bool CONV>
+struct RowAddr {
+    size_t x, o;
+    int xk, on;
+    __device__ __forceinline__ RowAddr(const Dims& d, int m, int g) {
+        if constexpr (CONV) {
+            const int b = m / d.HW, hw = m % d.HW;
+            x = ((size_t)(b * d.G + g) * d.K) * d.HW + hw;
+            o = ((size_t)(b * d.G + g) * d.NG) * d.HW + hw;
+            xk = d.HW;
+            on = d.HW;
+        } else {
+            x = ((size_t)m * d.G + g) * d.K;
+            o = ((size_t)m * d.G + g) * d.NG;
+            xk = 1;
+            on = 1;
+        }
+    }
+};
+
+inline Dims make_dims(const Problem& pr) { return Dims{pr.B, pr.G, pr.K, pr.NG, pr.HW, pr.B * pr.HW, 0, 0}; }
+
+inline bool can_vec4(const Problem& pr, const void* a, const void* b, const void* c = nullptr) {
+    return pr.K % 4 == 0 && (pr.HW == 1 || pr.HW % 4 == 0) && aligned16(a) && aligned16(b) && aligned16(c);
+}
+
+// Launches KERNEL<GEO, CONV, VEC>::run for the layout and vector width of the
+// problem.  KERNEL is a class template wrapping the __global__ function so that
+// one dispatcher serves all forward kernels.
+template <template <class, bool, int> class KERNEL, class GEO, class... Args>
+hipError_t launch_forward(const Problem& pr, bool vec4, hipStream_t stream, Args... args) {
+    Dims d = make_dims(pr);
+    d.tiles_m = (d.M + GEO::BM - 1) / GEO::BM;
+    d.tiles_n = (d.NG + GEO::BN - 1) / GEO::BN;
+    const unsigned grid = (unsigned)d.tiles_m * d.tiles_n * d.G;
+    if (pr.HW == 1)
+        return vec4 ? KERNEL<GEO, false, 4>::launch(grid, d, pr.device, stream, args...)
+                    : KERNEL<GEO, false, 1>::launch(grid, d, pr.device, stream, args...);
+    return vec4 ? KERNEL<GEO, true, 4>::launch(grid, d, pr.device, stream, args...)
+                : KERNEL<GEO, true, 1>::launch(grid, d, pr.device, stream, args...);
+}
+
+template <template <class, bool, int> class KERNEL, class... Args>
+hipError_t dispatch_forward(const Problem& pr, bool vec4, hipStream_t stream, Args... args) {
+    switch (choose_tile(pr.B * pr.HW, pr.NG, pr.G, pr.num_cu)) {
+        case TileChoice::M128N80K2:
+            return launch_forward<KERNEL, Geo<128, 80, 8, 5, 2>>(pr, vec4, stream, args...);
+        case TileChoice::M256N32K1:
+            return launch_forward<KERNEL, Geo<256, 32, 8, 4, 1>>(pr, vec4, stream, args...);
+        default:
+            return launch_forward<KERNEL, Geo<128, 64, 8, 4, 1>>(pr, vec4, stream, args...);
+    }
+}
+
+}  // namespace ldist

@@ -1,0 +1,208 @@
+// L_inf distance backward: the gradient of out[m,n] = |x[m,k*] - w[n,k*]| flows to
+// exactly one input and one weight element, the argmax k* recorded in pos
+// (bit 31 = sign of x - w).  Semantics follow the reference kernels
+// model/inf_dist_cuda.cu:143-171:
+//   grad_input [b, g*K + idx, hw] += (pos >= 0 ? g : -g)
+//   grad_weight[g*NG + n, idx]    += (pos <  0 ? g : -g)
+// The reference issues one global atomic per (m,n).  Here every workgroup owns a
+// slab of the gradient, gathers its contributions in LDS bins (ds_add_f32) and
+// writes the slab out with coalesced stores, so the pass is bounded by streaming
+// grad_output/pos in and the gradient out.  In "overwrite" mode the slab is
+// stored whole (zeros included), which replaces the caller's zero fill.
+#include "kernels.hpp"
+
+namespace ldist {
+
+struct BwdDims {
+    int B, G, K, NG, HW;
+};
+
+// ---- grad_input ------------------------------------------------------------
+// Workgroup = (image b, group g, TH consecutive hw, KC consecutive k).
+// bins[kc][th]; element (k, hw) of the slab lives at ((b*G+g)*K + k)*HW + hw.
+template <bool OVERWRITE>
+__global__ void __launch_bounds__(256)
+inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* __restrict__ pos,
+                          float* __restrict__ grad_input, BwdDims d, int th_log2, int KC, int hw_tiles) {
+    extern __shared__ float bins[];
+    const int TH = 1 << th_log2;
+    const int tile = blockIdx.x % hw_tiles;
+    const int bg = blockIdx.x / hw_tiles;  // b*G + g
+    const int hw0 = tile * TH;
+    const int k0 = blockIdx.y * KC;
+    const int kc = min(KC, d.K - k0);
+    const int nb = kc * TH;
+    for (int e = threadIdx.x; e < nb; e += 256) bins[e] = 0.f;
+    __syncthreads();
+
+    const size_t obase = (size_t)bg * d.NG * d.HW;
+    const int total = d.NG * TH;
+    for (int e = threadIdx.x; e < total; e += 256) {
+        const int n = e >> th_log2, j = e & (TH - 1);
+        const int hw = hw0 + j;
+        if (hw < d.HW) {
+            const size_t o = obase + (size_t)n * d.HW + hw;
+            const int p = pos[o];
+            const int idx = (p & 0x7fffffff) - k0;
+            if (idx >= 0 && idx < kc) {
+                const float gv = grad_output[o];
+                atomicAdd(&bins[(idx << th_log2) + j], p >= 0 ? gv : -gv);
+            }
+        }
+    }
+    __syncthreads();
+
+    const size_t xbase = ((size_t)bg * d.K + k0) * d.HW;
+    for (int e = threadIdx.x; e < nb; e += 256) {
+        const int k = e >> th_log2, j = e & (TH - 1);
+        const int hw = hw0 + j;
+        if (hw < d.HW) {
+            float* dst = grad_input + xbase + (size_t)k * d.HW + hw;
+            const float v = bins[e];
+            if (OVERWRITE) *dst = v;
+            else if (v != 0.f) *dst += v;
+        }
+    }
+}
+
+// ---- grad_weight -----------------------------------------------------------
+// Workgroup = (group g, NB consecutive outputs n, KC consecutive k, a slice of
+// the images b).  For one image the NB rows of grad_output/pos are one
+// contiguous run of NB*HW elements.  bins[nb][kc].
+// When the images are split over several workgroups (SPLIT) the bins are added
+// to grad_weight with global atomics, otherwise the workgroup is the only
+// writer of its slab.
+template <bool OVERWRITE, bool SPLIT>
+__global__ void __launch_bounds__(256)
+inf_backward_weight_kernel(const float* __restrict__ grad_output, const int32_t* __restrict__ pos,
+                           float* __restrict__ grad_weight, BwdDims d, int NB, int KC, int n_blocks, int b_per_wg) {
+    extern __shared__ float bins[];
+    const int nblk = blockIdx.x % n_blocks;
+    const int g = blockIdx.x / n_blocks;
+    const int n0 = nblk * NB;
+    const int nb = min(NB, d.NG - n0);
+    const int k0 = blockIdx.y * KC;
+    const int kc = min(KC, d.K - k0);
+    const int b0 = blockIdx.z * b_per_wg;
+    const int b1 = min(d.B, b0 + b_per_wg);
+    for (int e = threadIdx.x; e < nb * kc; e += 256) bins[e] = 0.f;
+    __syncthreads();
+
+    const int run = nb * d.HW;  // contiguous elements per image
+    const size_t img_stride = (size_t)d.G * d.NG * d.HW;
+    const size_t first = ((size_t)g * d.NG + n0) * d.HW;
+    if (d.HW == 1) {
+        // several images per pass: element i -> (image i / nb, output i % nb)
+        const int total = (b1 - b0) * nb;
+        for (int i = threadIdx.x; i < total; i += 256) {
+            const int bb = i / nb, nn = i - bb * nb;
+            const size_t o = (size_t)(b0 + bb) * img_stride + first + nn;
+            const int p = pos[o];
+            const int idx = (p & 0x7fffffff) - k0;
+            if (idx >= 0 && idx < kc) {
+                const float gv = grad_output[o];
+                atomicAdd(&bins[nn * kc + idx], p < 0 ? gv : -gv);
+            }
+        }
+    } else {
+        for (int b = b0; b < b1; b++) {
+            const size_t base = (size_t)b * img_stride + first;
+            for (int e = threadIdx.x; e < run; e += 256) {
+                const int nn = e / d.HW;
+                const int p = pos[base + e];
+                const int idx = (p & 0x7fffffff) - k0;
+                if (idx >= 0 && idx < kc) {
+                    const float gv = grad_output[base + e];
+                    atomicAdd(&bins[nn * kc + idx], p < 0 ? gv : -gv);
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    for (int e = threadIdx.x; e < nb * kc; e += 256) {
+        const int nn = e / kc, k = e - nn * kc;
+        float* dst = grad_weight + ((size_t)g * d.NG + n0 + nn) * d.K + k0 + k;
+        const float v = bins[e];
+        if (SPLIT) {
+            if (v != 0.f) atomicAdd(dst, v);
+        } else if (OVERWRITE) {
+            *dst = v;
+        } else if (v != 0.f) {
+            *dst += v;
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256) fill_zero_kernel(float* __restrict__ p, size_t n) {
+    const size_t stride = (size_t)gridDim.x * 256 * 4;
+    for (size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4; i < n; i += stride) {
+        if (i + 4 <= n && (reinterpret_cast<uintptr_t>(p + i) & 15u) == 0) {
+            *reinterpret_cast<float4*>(p + i) = make_float4(0.f, 0.f, 0.f, 0.f);
+        } else {
+            for (size_t j = i; j < n && j < i + 4; j++) p[j] = 0.f;
+        }
+    }
+}
+
+static constexpr int kBinFloats = 16384;  // 64 KB of LDS bins per workgroup
+
+hipError_t inf_backward_input(const float* grad_output, const int32_t* pos, float* grad_input, const Problem& pr,
+                              bool overwrite, hipStream_t stream) {
+    const BwdDims d{pr.B, pr.G, pr.K, pr.NG, pr.HW};
+    // widest hw tile (power of two, at most 64) whose bins still cover all K channels in one pass
+    int th_log2 = 0;
+    while ((2 << th_log2) <= pr.HW && (2 << th_log2) <= 64 && (size_t)(2 << th_log2) * pr.K <= kBinFloats) th_log2++;
+    const int TH = 1 << th_log2;
+    const int KC = min(pr.K, kBinFloats / TH);
+    const int hw_tiles = (pr.HW + TH - 1) / TH;
+    const dim3 grid((unsigned)pr.B * pr.G * hw_tiles, (unsigned)((pr.K + KC - 1) / KC));
+    const size_t lds = (size_t)KC * TH * sizeof(float);
+    if (overwrite)
+        hipLaunchKernelGGL(inf_backward_input_kernel<true>, grid, dim3(256), lds, stream, grad_output, pos,
+                           grad_input, d, th_log2, KC, hw_tiles);
+    else
+        hipLaunchKernelGGL(inf_backward_input_kernel<false>, grid, dim3(256), lds, stream, grad_output, pos,
+                           grad_input, d, th_log2, KC, hw_tiles);
+    return hipGetLastError();
+}
+
+hipError_t inf_backward_weight(const float* grad_output, const int32_t* pos, float* grad_weight, const Problem& pr,
+                               bool overwrite, hipStream_t stream) {
+    const BwdDims d{pr.B, pr.G, pr.K, pr.NG, pr.HW};
+    const int NB = min(pr.NG, 8);
+    const int KC = min(pr.K, kBinFloats / NB);
+    const int n_blocks = (pr.NG + NB - 1) / NB;
+    const int k_ranges = (pr.K + KC - 1) / KC;
+    const long slabs = (long)pr.G * n_blocks * k_ranges;
+    // split the images over workgroups only when the slabs alone cannot fill the device
+    int splits = 1;
+    if (slabs < 2L * pr.num_cu) {
+        const long rows = (long)pr.B * pr.HW;
+        const long by_work = max(1L, rows * NB / 16384);  // keep at least 16K contributions per workgroup
+        splits = (int)min((long)pr.B, min(by_work, (4L * pr.num_cu + slabs - 1) / slabs));
+        if (splits > 65535) splits = 65535;
+    }
+    const int b_per_wg = (pr.B + splits - 1) / splits;
+    splits = (pr.B + b_per_wg - 1) / b_per_wg;
+    const dim3 grid((unsigned)(pr.G * n_blocks), (unsigned)k_ranges, (unsigned)splits);
+    const size_t lds = (size_t)NB * KC * sizeof(float);
+    if (splits > 1) {
+        if (overwrite) {
+            const size_t n = (size_t)pr.G * pr.NG * pr.K;
+            const unsigned blocks = (unsigned)min((size_t)4096, (n + 1023) / 1024);
+            hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, stream, grad_weight, n);
+        }
+        hipLaunchKernelGGL((inf_backward_weight_kernel<false, true>), grid, dim3(256), lds, stream, grad_output, pos,
+                           grad_weight, d, NB, KC, n_blocks, b_per_wg);
+    } else if (overwrite) {
+        hipLaunchKernelGGL((inf_backward_weight_kernel<true, false>), grid, dim3(256), lds, stream, grad_output, pos,
+                           grad_weight, d, NB, KC, n_blocks, b_per_wg);
+    } else {
+        hipLaunchKernelGGL((inf_backward_weight_kernel<false, false>), grid, dim3(256), lds, stream, grad_output,
+                           pos, grad_weight, d, NB, KC, n_blocks, b_per_wg);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace ldist

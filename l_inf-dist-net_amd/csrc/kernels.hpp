@@ -1,0 +1,72 @@
+// Internal interface between the C ABI (ldist_api.hip) and the kernel files.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ldist {
+
+struct Problem {
+    int B, G, K, NG, HW;  // K = CI/G, NG = CO/G
+    int num_cu;           // compute units of the current device
+    int device;
+};
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+enum class TileChoice { M128N80K2, M128N64K1, M256N32K1 };
+
+// Picks the workgroup tiling that leaves the fewest padded (m,n) cells per CU.
+// M128N80K2 (512 lanes, two k-groups) fills a CU with one workgroup and divides
+// 512 x 5120 into exactly 256 tiles; M128N64K1 is the general shape;
+// M256N32K1 serves grouped layers with few outputs per group.
+// -1 = choose by shape; 0, 1, 2 force M128N80K2, M128N64K1, M256N32K1 (tests and tuning).
+extern int g_tile_override;
+
+inline TileChoice choose_tile(int M, int NG, int G, int num_cu) {
+    if (g_tile_override >= 0 && g_tile_override <= 2) return static_cast<TileChoice>(g_tile_override);
+    struct Cand { TileChoice c; int bm, bn; bool two_groups; };
+    const Cand cands[3] = {{TileChoice::M128N80K2, 128, 80, true},
+                           {TileChoice::M128N64K1, 128, 64, false},
+                           {TileChoice::M256N32K1, 256, 32, false}};
+    double best = 1e300;
+    TileChoice pick = TileChoice::M128N64K1;
+    for (const Cand& c : cands) {
+        const long tiles = (long)((M + c.bm - 1) / c.bm) * ((NG + c.bn - 1) / c.bn) * G;
+        const long rounds = (tiles + num_cu - 1) / num_cu;
+        double cost = (double)rounds * c.bm * c.bn;
+        // a lone single-group workgroup leaves one wave per SIMD: latency shows
+        if (!c.two_groups && tiles < 2L * num_cu) cost *= 1.25;
+        if (cost < best) { best = cost; pick = c.c; }
+    }
+    return pick;
+}
+
+// Sets the dynamic-LDS limit of a kernel once per device.
+template <class Kern>
+inline hipError_t allow_lds(Kern kern, size_t bytes, int device) {
+    static bool done[64] = {};
+    if (device >= 0 && device < 64 && done[device]) return hipSuccess;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e == hipSuccess && device >= 0 && device < 64) done[device] = true;
+    return e;
+}
+
+hipError_t inf_forward(const float* input, const float* weight, float* output, int32_t* pos, const Problem& pr,
+                       hipStream_t stream);
+hipError_t bound_forward(const float* lower, const float* upper, const float* weight, float* out_lower,
+                         float* out_upper, const Problem& pr, hipStream_t stream);
+hipError_t inf_backward_input(const float* grad_output, const int32_t* pos, float* grad_input, const Problem& pr,
+                              bool overwrite, hipStream_t stream);
+hipError_t inf_backward_weight(const float* grad_output, const int32_t* pos, float* grad_weight, const Problem& pr,
+                               bool overwrite, hipStream_t stream);
+hipError_t norm_forward(const float* input, const float* weight, float* output, float p, const Problem& pr,
+                        hipStream_t stream);
+hipError_t norm_backward_input(const float* grad_output, const float* input, const float* weight,
+                               const float* output, float* grad_input, float p, const Problem& pr,
+                               hipStream_t stream);
+hipError_t norm_backward_weight(const float* grad_output, const float* input, const float* weight,
+                                const float* output, float* grad_weight, float p, const Problem& pr,
+                                hipStream_t stream);
+
+}  // namespace ldist

@@ -1,0 +1,172 @@
+// C ABI of libldist_hip.so (declared in include/ldist.h): argument checks, device
+// lookup and error mapping around the kernel launchers.  Nothing here allocates
+// device memory or synchronises; every call only enqueues work on `stream`.
+#include "../../include/ldist.h"
+
+#include <cmath>
+#include <string>
+
+#include "kernels.hpp"
+
+namespace ldist {
+int g_tile_override = -1;
+}
+
+namespace {
+
+thread_local int g_last_hip_error = 0;
+
+struct DeviceInfo {
+    int num_cu = 0;
+    bool is_gfx950 = false;
+    bool known = false;
+};
+
+// Compute-unit count and architecture of the current device (looked up once per device).
+int current_device(ldist::Problem& pr) {
+    static DeviceInfo info[64];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { g_last_hip_error = (int)e; return LDIST_ELAUNCH; }
+    DeviceInfo local;
+    DeviceInfo& di = (dev >= 0 && dev < 64) ? info[dev] : local;
+    if (!di.known) {
+        hipDeviceProp_t prop;
+        e = hipGetDeviceProperties(&prop, dev);
+        if (e != hipSuccess) { g_last_hip_error = (int)e; return LDIST_ELAUNCH; }
+        di.num_cu = prop.multiProcessorCount;
+        di.is_gfx950 = std::string(prop.gcnArchName).rfind("gfx950", 0) == 0;
+        di.known = true;
+    }
+    if (!di.is_gfx950) return LDIST_EDEVICE;
+    pr.num_cu = di.num_cu > 0 ? di.num_cu : 256;
+    pr.device = dev;
+    return LDIST_OK;
+}
+
+int check_dims(int B, int CO, int CI, int G, int HW, ldist::Problem& pr) {
+    if (B <= 0 || CO <= 0 || CI <= 0 || G <= 0 || HW <= 0) return LDIST_EINVAL;
+    if (CI % G != 0 || CO % G != 0) return LDIST_EINVAL;
+    const long long lim = 1LL << 31;
+    const long long rows = (long long)B * HW;
+    if (rows >= lim || rows * CI >= lim || rows * CO >= lim || (long long)CO * (CI / G) >= lim) return LDIST_ERANGE;
+    pr.B = B; pr.G = G; pr.K = CI / G; pr.NG = CO / G; pr.HW = HW;
+    return current_device(pr);
+}
+
+int finish(hipError_t e) {
+    if (e == hipSuccess) return LDIST_OK;
+    g_last_hip_error = (int)e;
+    return LDIST_ELAUNCH;
+}
+
+bool valid_p(float p) { return p > 1.0f && std::isfinite(p); }
+
+}  // namespace
+
+extern "C" {
+
+int ldist_version(void) { return LDIST_VERSION; }
+
+const char* ldist_strerror(int code) {
+    switch (code) {
+        case LDIST_OK: return "ok";
+        case LDIST_EINVAL: return "invalid argument (null pointer, non-positive size, CI % G or CO % G != 0, or p not > 1)";
+        case LDIST_ERANGE: return "tensor too large (2^31 or more elements)";
+        case LDIST_ELAUNCH: return "HIP runtime error at launch";
+        case LDIST_EDEVICE: return "current device is not gfx950";
+        default: return "unknown error";
+    }
+}
+
+int ldist_last_hip_error(void) { return g_last_hip_error; }
+
+int ldist_set_tile_override(int choice) {
+    if (choice < -1 || choice > 2) return LDIST_EINVAL;
+    ldist::g_tile_override = choice;
+    return LDIST_OK;
+}
+
+int ldist_inf_dist_forward(const float* input, const float* weight, int B, int CO, int CI, int G, int HW,
+                           float* output, int32_t* pos, ldist_stream_t stream) {
+    if (!input || !weight || !output || !pos) return LDIST_EINVAL;
+    ldist::Problem pr{};
+    if (int rc = check_dims(B, CO, CI, G, HW, pr)) return rc;
+    return finish(ldist::inf_forward(input, weight, output, pos, pr, (hipStream_t)stream));
+}
+
+int ldist_inf_dist_bound_forward(const float* input_lower, const float* input_upper, const float* weight, int B,
+                                 int CO, int CI, int G, int HW, float* output_lower, float* output_upper,
+                                 ldist_stream_t stream) {
+    if (!input_lower || !input_upper || !weight || !output_lower || !output_upper) return LDIST_EINVAL;
+    ldist::Problem pr{};
+    if (int rc = check_dims(B, CO, CI, G, HW, pr)) return rc;
+    return finish(ldist::bound_forward(input_lower, input_upper, weight, output_lower, output_upper, pr,
+                                       (hipStream_t)stream));
+}
+
+static int inf_backward_input_impl(const float* grad_output, const int32_t* pos, int B, int CO, int CI, int G,
+                                   int HW, float* grad_input, bool overwrite, ldist_stream_t stream) {
+    if (!grad_output || !pos || !grad_input) return LDIST_EINVAL;
+    ldist::Problem pr{};
+    if (int rc = check_dims(B, CO, CI, G, HW, pr)) return rc;
+    return finish(ldist::inf_backward_input(grad_output, pos, grad_input, pr, overwrite, (hipStream_t)stream));
+}
+
+static int inf_backward_weight_impl(const float* grad_output, const int32_t* pos, int B, int CO, int CI, int G,
+                                    int HW, float* grad_weight, bool overwrite, ldist_stream_t stream) {
+    if (!grad_output || !pos || !grad_weight) return LDIST_EINVAL;
+    ldist::Problem pr{};
+    if (int rc = check_dims(B, CO, CI, G, HW, pr)) return rc;
+    return finish(ldist::inf_backward_weight(grad_output, pos, grad_weight, pr, overwrite, (hipStream_t)stream));
+}
+
+int ldist_inf_dist_backward_input(const float* grad_output, const int32_t* pos, int B, int CO, int CI, int G, int HW,
+                                  float* grad_input, ldist_stream_t stream) {
+    return inf_backward_input_impl(grad_output, pos, B, CO, CI, G, HW, grad_input, false, stream);
+}
+
+int ldist_inf_dist_backward_weight(const float* grad_output, const int32_t* pos, int B, int CO, int CI, int G, int HW,
+                                   float* grad_weight, ldist_stream_t stream) {
+    return inf_backward_weight_impl(grad_output, pos, B, CO, CI, G, HW, grad_weight, false, stream);
+}
+
+int ldist_inf_dist_backward_input_overwrite(const float* grad_output, const int32_t* pos, int B, int CO, int CI,
+                                            int G, int HW, float* grad_input, ldist_stream_t stream) {
+    return inf_backward_input_impl(grad_output, pos, B, CO, CI, G, HW, grad_input, true, stream);
+}
+
+int ldist_inf_dist_backward_weight_overwrite(const float* grad_output, const int32_t* pos, int B, int CO, int CI,
+                                             int G, int HW, float* grad_weight, ldist_stream_t stream) {
+    return inf_backward_weight_impl(grad_output, pos, B, CO, CI, G, HW, grad_weight, true, stream);
+}
+
+int ldist_norm_dist_forward(const float* input, const float* weight, int B, int CO, int CI, int G, int HW,
+                            float* output, float p, ldist_stream_t stream) {
+    if (!input || !weight || !output || !valid_p(p)) return LDIST_EINVAL;
+    ldist::Problem pr{};
+    if (int rc = check_dims(B, CO, CI, G, HW, pr)) return rc;
+    return finish(ldist::norm_forward(input, weight, output, p, pr, (hipStream_t)stream));
+}
+
+int ldist_norm_dist_backward_input(const float* grad_output, const float* input, const float* weight,
+                                   const float* output, int B, int CO, int CI, int G, int HW, float* grad_input,
+                                   float p, ldist_stream_t stream) {
+    if (!grad_output || !input || !weight || !output || !grad_input || !valid_p(p)) return LDIST_EINVAL;
+    ldist::Problem pr{};
+    if (int rc = check_dims(B, CO, CI, G, HW, pr)) return rc;
+    return finish(ldist::norm_backward_input(grad_output, input, weight, output, grad_input, p, pr,
+                                             (hipStream_t)stream));
+}
+
+int ldist_norm_dist_backward_weight(const float* grad_output, const float* input, const float* weight,
+                                    const float* output, int B, int CO, int CI, int G, int HW, float* grad_weight,
+                                    float p, ldist_stream_t stream) {
+    if (!grad_output || !input || !weight || !output || !grad_weight || !valid_p(p)) return LDIST_EINVAL;
+    ldist::Problem pr{};
+    if (int rc = check_dims(B, CO, CI, G, HW, pr)) return rc;
+    return finish(ldist::norm_backward_weight(grad_output, input, weight, output, grad_weight, p, pr,
+                                              (hipStream_t)stream));
+}
+
+}  // extern "C"

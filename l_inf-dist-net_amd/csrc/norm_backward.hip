@@ -1,0 +1,198 @@
+// p-norm distance backward, p > 1 (reference model/norm_dist_cuda.cu:294-425):
+//   grad_input [m,k]  = sum_n g[m,n] * (|x-w| / out[m,n])^(p-1) * sign(x-w)     (:294-297, every element written)
+//   grad_weight[n,k] += sum_m g[m,n] * (|w-x| / out[m,n])^(p-1) * sign(w-x)     (:363-366, added to the buffer)
+// Both are the same reduction with the roles of x and w exchanged:
+//   P[a,k] = sum_r c[a,r] * (|Q[a,k] - O[r,k]| * rinv[a,r])^(p-1) * sign(Q - O)
+// grad_input: a = m, r = n, Q = x, O = w;  grad_weight: a = n, r = m, Q = w, O = x.
+// A workgroup owns a 64 x 64 tile of P; each lane keeps a 4 x 4 patch of Q and of
+// the sums in registers and walks r in stages of 32 whose O, c and rinv panels sit
+// in LDS.  The work is bound by the transcendental unit (one v_log_f32 and one
+// v_exp_f32 per term; p-1 = 1, 2, 3, 7 use multiplies only), so the loads are
+// plain coalesced 32-bit accesses.
+#include "kernels.hpp"
+#include "pow.hpp"
+
+namespace ldist {
+
+struct NbDims {
+    int B, G, K, NG, HW, M;
+};
+
+constexpr int BA = 64, BKO = 64, RB = 32, LDP = 65;  // tile, stage depth, padded LDS row
+
+// WEIGHT = false: grad_input.  WEIGHT = true: grad_weight.
+template <bool WEIGHT, bool CONV>
+struct Views {
+    const float* x; const float* w; const float* out; const float* go;
+    NbDims d; int g;
+    // rows of P: a in [0, A); reduction: r in [0, R)
+    __device__ __forceinline__ int A() const { return WEIGHT ? d.NG : d.M; }
+    // address of x[m][k], w[n][k], and of the (m,n) element of out / grad_output
+    __device__ __forceinline__ size_t x_at(int m, int k) const {
+        if (CONV) { const int b = m / d.HW, hw = m - b * d.HW; return ((size_t)(b * d.G + g) * d.K + k) * d.HW + hw; }
+        return ((size_t)m * d.G + g) * d.K + k;
+    }
+    __device__ __forceinline__ size_t w_at(int n, int k) const { return ((size_t)g * d.NG + n) * d.K + k; }
+    __device__ __forceinline__ size_t o_at(int m, int n) const {
+        if (CONV) { const int b = m / d.HW, hw = m - b * d.HW; return ((size_t)(b * d.G + g) * d.NG + n) * d.HW + hw; }
+        return ((size_t)m * d.G + g) * d.NG + n;
+    }
+};
+
+template <bool WEIGHT, bool CONV, bool SPLIT>
+__global__ void __launch_bounds__(256)
+norm_backward_kernel(const float* __restrict__ grad_output, const float* __restrict__ input,
+                     const float* __restrict__ weight, const float* __restrict__ output, float* __restrict__ grad,
+                     float p, NbDims d, int tiles_a, int tiles_k, int r_per_wg) {
+    __shared__ float Os[RB * LDP];  // O[r][k]
+    __shared__ float Cs[RB * LDP];  // c[r][a]     = grad_output
+    __shared__ float Rs[RB * LDP];  // rinv[r][a]  = 1 / output
+    const int tid = threadIdx.x;
+    const int ta = blockIdx.x % tiles_a;
+    const int rest = blockIdx.x / tiles_a;
+    const int tk = rest % tiles_k;
+    const int g = rest / tiles_k;
+    const int a0 = ta * BA, k0 = tk * BKO;
+    const Views<WEIGHT, CONV> v{input, weight, output, grad_output, d, g};
+    const int A = v.A();
+    const int R = WEIGHT ? d.M : d.NG;
+    const int r_begin = blockIdx.y * r_per_wg;
+    const int r_end = min(R, r_begin + r_per_wg);
+    const int tx = tid & 15, ty = tid >> 4;  // lane's patch: rows a0 + ty*4.., columns k0 + tx*4..
+    const float e = p - 1.0f;
+    const int ie = small_int_power(e);
+
+    float q[4][4], acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int a = a0 + ty * 4 + i, k = k0 + tx * 4 + j;
+            acc[i][j] = 0.f;
+            q[i][j] = (a < A && k < d.K) ? (WEIGHT ? weight[v.w_at(a, k)] : input[v.x_at(a, k)]) : 0.f;
+        }
+
+    // In memory the k axis is contiguous for w (always) and for x when HW == 1;
+    // the a/r axes of out and grad_output are contiguous along n when HW == 1 and
+    // along m (= hw) otherwise.  Lanes follow the contiguous axis of each panel.
+    constexpr bool O_K_CONTIG = !(WEIGHT && CONV);         // O = w, or x in the fc layout
+    constexpr bool C_A_CONTIG = WEIGHT ? !CONV : CONV;     // is `a` the contiguous axis of out/grad_output
+    for (int r0 = r_begin; r0 < r_end; r0 += RB) {
+        __syncthreads();
+#pragma unroll
+        for (int it = 0; it < RB * 64 / 256; it++) {
+            const int id = tid + it * 256;
+            {
+                const int rr = O_K_CONTIG ? id >> 6 : id & (RB - 1);
+                const int cc = O_K_CONTIG ? id & 63 : id >> 5;
+                const int r = r0 + rr, k = k0 + cc;
+                float val = 0.f;
+                if (r < r_end && k < d.K) val = WEIGHT ? input[v.x_at(r, k)] : weight[v.w_at(r, k)];
+                Os[rr * LDP + cc] = val;
+            }
+            {
+                const int rr = C_A_CONTIG ? id >> 6 : id & (RB - 1);
+                const int cc = C_A_CONTIG ? id & 63 : id >> 5;
+                const int r = r0 + rr, a = a0 + cc;
+                float c = 0.f, ri = 0.f;
+                if (r < r_end && a < A) {
+                    const size_t o = WEIGHT ? v.o_at(r, a) : v.o_at(a, r);
+                    c = grad_output[o];
+                    ri = __builtin_amdgcn_rcpf(output[o]);
+                }
+                Cs[rr * LDP + cc] = c;
+                Rs[rr * LDP + cc] = ri;
+            }
+        }
+        __syncthreads();
+        auto reduce = [&](auto power) {
+#pragma unroll 2
+            for (int rr = 0; rr < RB; rr++) {
+                float o[4], c[4], ri[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) o[j] = Os[rr * LDP + tx * 4 + j];
+#pragma unroll
+                for (int i = 0; i < 4; i++) { c[i] = Cs[rr * LDP + ty * 4 + i]; ri[i] = Rs[rr * LDP + ty * 4 + i]; }
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const float t = q[i][j] - o[j];
+                        const float pw = power(__builtin_fabsf(t) * ri[i]);
+                        // sign(t) * pw; at t == 0 the power is 0 and the sign is irrelevant
+                        acc[i][j] += c[i] * __builtin_copysignf(pw, t);
+                    }
+            }
+        };
+        switch (ie) {
+            case 1: reduce([](float u) { return u; }); break;
+            case 2: reduce([](float u) { return pow_int<2>(u); }); break;
+            case 3: reduce([](float u) { return pow_int<3>(u); }); break;
+            case 7: reduce([](float u) { return pow_int<7>(u); }); break;
+            default: reduce([e](float u) { return pow_pos(u, e); }); break;
+        }
+    }
+
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int a = a0 + ty * 4 + i, k = k0 + tx * 4 + j;
+            if (a < A && k < d.K) {
+                if (WEIGHT) {
+                    float* dst = grad + v.w_at(a, k);
+                    if (SPLIT) atomicAdd(dst, acc[i][j]);
+                    else *dst += acc[i][j];
+                } else {
+                    grad[v.x_at(a, k)] = acc[i][j];
+                }
+            }
+        }
+}
+
+template <bool WEIGHT>
+static hipError_t launch_norm_backward(const float* grad_output, const float* input, const float* weight,
+                                       const float* output, float* grad, float p, const Problem& pr,
+                                       hipStream_t stream) {
+    const NbDims d{pr.B, pr.G, pr.K, pr.NG, pr.HW, pr.B * pr.HW};
+    const int A = WEIGHT ? d.NG : d.M;
+    const int R = WEIGHT ? d.M : d.NG;
+    const int tiles_a = (A + BA - 1) / BA, tiles_k = (d.K + BKO - 1) / BKO;
+    const long tiles = (long)tiles_a * tiles_k * d.G;
+    int splits = 1;
+    if (WEIGHT && tiles < 2L * pr.num_cu) {  // few output tiles, long reduction over the rows: share it out
+        const long want = (4L * pr.num_cu + tiles - 1) / tiles;
+        const long most = max(1L, (long)R / (4 * RB));
+        splits = (int)min(want, most);
+    }
+    int r_per_wg = (R + splits - 1) / splits;
+    r_per_wg = (r_per_wg + RB - 1) / RB * RB;
+    splits = (R + r_per_wg - 1) / r_per_wg;
+    const dim3 grid((unsigned)tiles, (unsigned)splits);
+    const bool conv = pr.HW != 1;
+#define LDIST_LAUNCH(W, C, S)                                                                                      \
+    hipLaunchKernelGGL((norm_backward_kernel<W, C, S>), grid, dim3(256), 0, stream, grad_output, input, weight,    \
+                       output, grad, p, d, tiles_a, tiles_k, r_per_wg)
+    if (WEIGHT) {
+        if (splits > 1) { if (conv) LDIST_LAUNCH(WEIGHT, true, true); else LDIST_LAUNCH(WEIGHT, false, true); }
+        else { if (conv) LDIST_LAUNCH(WEIGHT, true, false); else LDIST_LAUNCH(WEIGHT, false, false); }
+    } else {
+        if (conv) LDIST_LAUNCH(WEIGHT, true, false); else LDIST_LAUNCH(WEIGHT, false, false);
+    }
+#undef LDIST_LAUNCH
+    return hipGetLastError();
+}
+
+hipError_t norm_backward_input(const float* grad_output, const float* input, const float* weight,
+                               const float* output, float* grad_input, float p, const Problem& pr,
+                               hipStream_t stream) {
+    return launch_norm_backward<false>(grad_output, input, weight, output, grad_input, p, pr, stream);
+}
+
+hipError_t norm_backward_weight(const float* grad_output, const float* input, const float* weight,
+                                const float* output, float* grad_weight, float p, const Problem& pr,
+                                hipStream_t stream) {
+    return launch_norm_backward<true>(grad_output, input, weight, output, grad_weight, p, pr, stream);
+}
+
+}  // namespace ldist

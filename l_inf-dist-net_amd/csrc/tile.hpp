@@ -1,0 +1,274 @@
+// Shared building blocks of the "tropical GEMM" forward kernels (gfx950, wave64).
+//
+// A workgroup owns a BM x BN tile of the (row m, output n) plane of one group
+// and walks the reduction axis k in stages of KS*32 values.  The x and w panels
+// of a stage sit in LDS as P[kk][m] (k-major, m contiguous) so that a lane reads
+// the TM row values / TN column values it needs for one k with 128-bit LDS
+// loads, and every value fetched from LDS is reused TN (resp. TM) times from
+// registers.  The KS "k-groups" of a workgroup (each (BM/TM)*(BN/TN) lanes)
+// share the panels and take alternate 32-wide chunks of k; their partial
+// results are merged through LDS at the end.  This keeps two waves per SIMD
+// busy on shapes whose m x n plane alone is too small to fill 256 CUs.
+//
+// Tensor layout (reference model/inf_dist_cuda.cu:29-33,65-66):
+//   input (B, CI, HW): ((b*G + g)*K + k)*HW + hw     weight (CO, K): (g*NG + n)*K + k
+//   output (B, CO, HW): ((b*G + g)*NG + n)*HW + hw
+// "fc" kernels are the HW == 1 case (k contiguous in x), "conv" kernels the
+// HW > 1 case (the row index hw is contiguous in x and in the output).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace ldist {
+
+constexpr int kChunk = 32;  // k values between two "did the maximum move" checks
+
+struct Dims {
+    int B, G, K, NG, HW;  // K = CI/G, NG = CO/G
+    int M;                // B*HW rows
+    int tiles_m, tiles_n;
+};
+
+// XOR applied to the m (or n) coordinate of LDS row kk.  It permutes aligned
+// groups of four floats inside aligned blocks of 32, so 128-bit accesses stay
+// contiguous, panel rows need no padding, and the transposing 32-bit stores of
+// the fc loader (16 lanes along k, 4 along m) hit 32 distinct banks.
+__device__ __forceinline__ constexpr int swz(int kk) { return ((kk >> 2) & 7) << 2; }
+
+template <int BM_, int BN_, int TM_, int TN_, int KS_>
+struct Geo {
+    static constexpr int BM = BM_, BN = BN_, TM = TM_, TN = TN_, KS = KS_;
+    static constexpr int KK = KS * kChunk;       // k values per stage
+    static constexpr int TX = BN / TN;           // lanes along n
+    static constexpr int TY = BM / TM;           // lanes along m
+    static constexpr int NGRP = TX * TY;         // lanes per k-group
+    static constexpr int NT = NGRP * KS;         // workgroup size
+    static constexpr int SM = (BM + 31) / 32 * 32;  // LDS row lengths
+    static constexpr int SN = (BN + 31) / 32 * 32;
+    static constexpr int XS = KK * SM;           // floats of one x panel
+    static constexpr int WS = KK * SN;
+    static_assert(TM == 4 || TM == 8, "TM");
+    static_assert(TN == 4 || TN == 5 || TN == 8, "TN");
+    static_assert(BM % TM == 0 && BN % TN == 0, "tile");
+    static_assert(NT % 64 == 0, "whole waves");
+
+    // Tile-local row of the i-th value a lane owns.  Eight values are two runs
+    // of four, BM/2 apart, so that neighbouring lanes read neighbouring 16 bytes.
+    __device__ static constexpr int row(int ty, int i) {
+        return TM == 8 ? (i < 4 ? ty * 4 + i : BM / 2 + ty * 4 + (i - 4)) : ty * 4 + i;
+    }
+    __device__ static constexpr int col(int tx, int j) {
+        return TN == 8 ? (j < 4 ? tx * 4 + j : BN / 2 + tx * 4 + (j - 4))
+             : TN == 5 ? (j < 4 ? tx * 4 + j : TX * 4 + tx)
+                       : tx * 4 + j;
+    }
+};
+
+// LDS address of the first value a lane reads in row kk (kk a multiple of 4: the
+// swizzle is constant over an aligned run of four rows, so rows kk+1..kk+3 are
+// plain row strides away).  BM/2 and BN/2 are multiples of 32, which the XOR
+// never touches, so the second run of four sits at a fixed distance as well.
+template <class GEO>
+struct LanePtr {
+    const float* x;   // x panel, row kk, this lane's first run of four rows
+    const float* w;   // w panel, row kk, this lane's first run of four columns
+    const float* w5;  // w panel, row kk, the lane's fifth column (TN == 5 only)
+    __device__ __forceinline__ void set(const float* xp, const float* wp, int kk, int tx, int ty) {
+        const int s = swz(kk);
+        x = xp + kk * GEO::SM + ((ty * 4) ^ s);
+        w = wp + kk * GEO::SN + ((tx * 4) ^ s);
+        if constexpr (GEO::TN == 5) w5 = wp + kk * GEO::SN + ((GEO::TX * 4 + tx) ^ s);
+    }
+};
+
+template <class GEO>
+__device__ __forceinline__ void read_x(const float* __restrict__ p, int r, float (&xf)[GEO::TM]) {
+    float4 a = *reinterpret_cast<const float4*>(p + r * GEO::SM);
+    xf[0] = a.x; xf[1] = a.y; xf[2] = a.z; xf[3] = a.w;
+    if constexpr (GEO::TM == 8) {
+        float4 b = *reinterpret_cast<const float4*>(p + r * GEO::SM + GEO::BM / 2);
+        xf[4] = b.x; xf[5] = b.y; xf[6] = b.z; xf[7] = b.w;
+    }
+}
+
+template <class GEO>
+__device__ __forceinline__ void read_w(const LanePtr<GEO>& lp, int r, float (&wf)[GEO::TN]) {
+    float4 a = *reinterpret_cast<const float4*>(lp.w + r * GEO::SN);
+    wf[0] = a.x; wf[1] = a.y; wf[2] = a.z; wf[3] = a.w;
+    if constexpr (GEO::TN == 8) {
+        float4 b = *reinterpret_cast<const float4*>(lp.w + r * GEO::SN + GEO::BN / 2);
+        wf[4] = b.x; wf[5] = b.y; wf[6] = b.z; wf[7] = b.w;
+    }
+    if constexpr (GEO::TN == 5) wf[4] = lp.w5[r * GEO::SN];
+}
+
+// Operand registers of KP consecutive k rows (1 or 2): NX x-like panels (1, or 2
+// for the lower/upper interval ends) and the w panel.
+template <class GEO, int NX, int KP>
+struct Frag {
+    float x[NX][KP][GEO::TM];
+    float w[KP][GEO::TN];
+    // rows r .. r+KP-1 relative to lp's row; xstride = floats between the x panels
+    __device__ __forceinline__ void read(const LanePtr<GEO>& lp, int r, int xstride) {
+#pragma unroll
+        for (int q = 0; q < NX; q++)
+#pragma unroll
+            for (int e = 0; e < KP; e++) read_x<GEO>(lp.x + q * xstride, r + e, x[q][e]);
+#pragma unroll
+        for (int e = 0; e < KP; e++) read_w<GEO>(lp, r + e, w[e]);
+    }
+};
+
+// Walks one 32-row chunk of the panels and calls f(frag) once per KP k rows.
+// 2*KP rows per trip, as two fragments: the operands of the next fragment are
+// fetched from LDS while the current one is being reduced.  The loop is kept
+// rolled on purpose: unrolled, the compiler hoists every LDS read of the chunk
+// above the arithmetic and spills the accumulators.
+template <class GEO, int NX, int KP, class F>
+__device__ __forceinline__ void sweep_chunk(const float* xp, const float* wp, int tx, int ty, F&& f) {
+    static_assert(KP == 1 || KP == 2, "a trip must stay inside one aligned run of four rows");
+    constexpr int XSTRIDE = GEO::XS;
+    Frag<GEO, NX, KP> a, b;
+    LanePtr<GEO> cur, nxt;
+    cur.set(xp, wp, 0, tx, ty);
+    a.read(cur, 0, XSTRIDE);
+#pragma unroll 1
+    for (int kk = 0; kk < kChunk; kk += 2 * KP) {
+        b.read(cur, KP, XSTRIDE);
+        f(a);
+        nxt.set(xp, wp, (kk + 2 * KP) & (kChunk - 1), tx, ty);  // the last trip re-reads row 0; harmless
+        a.read(nxt, 0, XSTRIDE);
+        f(b);
+        cur = nxt;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Stage loaders: global -> registers (issued early) -> LDS (after the compute).
+// RowsK<ROWS, LD, NT, KK, VEC> covers a panel whose rows are k-contiguous in
+// memory (weight always; input when HW == 1).  Lanes run along k first, so a
+// wave reads whole 64..256-byte row segments; the store transposes into P[kk][r].
+// Values outside the matrix (r >= rows_valid, k >= K) are loaded as 0, which is
+// neutral for every reduction here (|0 - 0| never raises a maximum or a sum).
+// ---------------------------------------------------------------------------
+template <int ROWS, int LD, int NT, int KK, int VEC>
+struct RowsK {
+    static constexpr int PER_ROW = KK / VEC;               // vectors per panel row
+    static constexpr int TOTAL = ROWS * PER_ROW;
+    static constexpr int N = (TOTAL + NT - 1) / NT;        // vectors per lane
+    float v[N][VEC];
+
+    // base: pointer to (row 0 of the tile, k = 0); ld: elements between rows.
+    __device__ __forceinline__ void load(const float* __restrict__ base, int ld, int rows_valid, int k0, int K,
+                                         int tid) {
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const int id = tid + i * NT;
+            const int r = id / PER_ROW, kq = id % PER_ROW;
+            const int k = k0 + kq * VEC;
+            const bool ok = (TOTAL % NT == 0 || id < TOTAL) && r < rows_valid;
+            const float* p = base + (size_t)r * ld + k;
+            if constexpr (VEC == 4) {
+                float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (ok && k < K) t = *reinterpret_cast<const float4*>(p);  // K % 4 == 0 on this path
+                v[i][0] = t.x; v[i][1] = t.y; v[i][2] = t.z; v[i][3] = t.w;
+            } else {
+                v[i][0] = (ok && k < K) ? *p : 0.f;
+            }
+        }
+    }
+    __device__ __forceinline__ void store(float* __restrict__ panel, int tid) const {
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const int id = tid + i * NT;
+            if (TOTAL % NT != 0 && id >= TOTAL) continue;
+            const int r = id / PER_ROW, kq = id % PER_ROW;
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                const int kk = kq * VEC + e;
+                panel[kk * LD + (r ^ swz(kk))] = v[i][e];
+            }
+        }
+    }
+};
+
+// RowsM covers the input panel of the conv layout: for a fixed k the rows
+// m = b*HW + hw are contiguous in memory (within one b), so lanes run along m
+// and the LDS store needs no transpose.  VEC == 4 requires HW % 4 == 0, which
+// keeps every aligned run of four rows inside one image b.
+template <int ROWS, int LD, int NT, int KK, int VEC>
+struct RowsM {
+    static constexpr int PER_K = ROWS / VEC;
+    static constexpr int TOTAL = KK * PER_K;
+    static constexpr int N = (TOTAL + NT - 1) / NT;
+    static_assert(NT % PER_K == 0 || PER_K % NT == 0, "lane keeps its rows across iterations");
+    float v[N][VEC];
+
+    // off_m: element offset of (row, k = group's first channel) for this lane's
+    // first row, or -1 if that row is outside the matrix; kstride = HW.
+    __device__ __forceinline__ void load(const float* __restrict__ input, const int (&off_m)[N], int kstride, int k0,
+                                         int K, int tid) {
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const int id = tid + i * NT;
+            const int kk = id / PER_K;
+            const int k = k0 + kk;
+            const bool ok = (TOTAL % NT == 0 || id < TOTAL) && off_m[i] >= 0 && k < K;
+            const float* p = input + (size_t)off_m[i] + (size_t)k * kstride;
+            if constexpr (VEC == 4) {
+                float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (ok) t = *reinterpret_cast<const float4*>(p);
+                v[i][0] = t.x; v[i][1] = t.y; v[i][2] = t.z; v[i][3] = t.w;
+            } else {
+                v[i][0] = ok ? *p : 0.f;
+            }
+        }
+    }
+    __device__ __forceinline__ void store(float* __restrict__ panel, int tid) const {
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const int id = tid + i * NT;
+            if (TOTAL % NT != 0 && id >= TOTAL) continue;
+            const int kk = id / PER_K, mq = id % PER_K;
+            if constexpr (VEC == 4) {
+                *reinterpret_cast<float4*>(panel + kk * LD + ((mq * 4) ^ swz(kk))) =
+                    make_float4(v[i][0], v[i][1], v[i][2], v[i][3]);
+            } else {
+                panel[kk * LD + (mq ^ swz(kk))] = v[i][0];
+            }
+        }
+    }
+    // Fills off_m for this lane: rows of the tile start at global row m0.
+    __device__ __forceinline__ static void offsets(int (&off_m)[N], int m0, int M, int HW, int G, int g, int K,
+                                                   int tid) {
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const int id = tid + i * NT;
+            const int mq = id % PER_K;
+            const int m = m0 + mq * VEC;
+            if (m < M) {
+                const int b = m / HW, hw = m % HW;
+                off_m[i] = ((b * G + g) * K) * HW + hw;
+            } else {
+                off_m[i] = -1;
+            }
+        }
+    }
+};
+
+// Maps the linear workgroup id to (tile_m, tile_n, group).  Consecutive ids go
+// to different XCDs (8 per device, each with its own L2); the remap hands every
+// XCD one contiguous run of tiles, m fastest, so the workgroups that share an
+// L2 also share their w strip (and, across runs, their x strips).
+__device__ __forceinline__ void tile_of_block(const Dims& d, int& tm, int& tn, int& g) {
+    const int total = gridDim.x;
+    int id = blockIdx.x;
+    constexpr int XCD = 8;
+    if (total % XCD == 0) id = (id % XCD) * (total / XCD) + id / XCD;
+    tm = id % d.tiles_m;
+    const int r = id / d.tiles_m;
+    tn = r % d.tiles_n;
+    g = r / d.tiles_n;
+}
+
+}  // namespace ldist

@@ -1,0 +1,162 @@
+"""Drop-in for the reference's native module ``norm_dist_cpp``.
+
+The seven functions keep the names, positional order and in-place contract of
+the reference binding (model/norm_dist.cpp:22-100): they take torch tensors,
+write into caller-allocated tensors and return None.  Each one checks its
+arguments like the reference (device, contiguity; a failed check raises
+RuntimeError) plus the shape relations the reference leaves unchecked, then
+calls the matching C-ABI entry point of libldist_hip.so on the current HIP
+stream of the tensors' device.
+"""
+import torch
+
+from . import _lib
+
+
+def _check_input(t, name, dtype=torch.float32):
+    # reference CHECK_INPUT: is_cuda and is_contiguous (model/norm_dist.cpp:3-5);
+    # the dtype test is what data_ptr<float>() enforces there
+    if not isinstance(t, torch.Tensor):
+        raise RuntimeError(f"{name} must be a tensor")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+    if t.dtype != dtype:
+        raise RuntimeError(f"{name} must have dtype {dtype}, got {t.dtype}")
+
+
+def _same_device(*ts):
+    dev = ts[0].device
+    for t in ts[1:]:
+        if t.device != dev:
+            raise RuntimeError("all tensors must be on the same device")
+    return dev
+
+
+def _expect(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _call(name, device, *args):
+    with torch.cuda.device(device):
+        stream = torch.cuda.current_stream(device).cuda_stream
+        rc = getattr(_lib.lib(), name)(*args, stream)
+    _lib.check(rc, name)
+
+
+def _p(t):
+    return t.data_ptr()
+
+
+def norm_dist_forward(input, weight, output, G, p):
+    """model/norm_dist.cpp:22-28."""
+    for t, n in ((input, "input"), (weight, "weight"), (output, "output")):
+        _check_input(t, n)
+    dev = _same_device(input, weight, output)
+    B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
+    _expect(input.dim() == 3 and output.dim() == 3 and weight.dim() == 2, "input/output must be 3-D, weight 2-D")
+    _expect(weight.size(0) == CO and weight.size(1) * G == CI, "weight must be (CO, CI/G)")
+    _expect(output.size(0) == B and output.size(2) == HW, "output must be (B, CO, HW)")
+    _call("ldist_norm_dist_forward", dev, _p(input), _p(weight), B, CO, CI, G, HW, _p(output), float(p))
+
+
+def norm_dist_backward_input(grad_output, input, weight, output, grad_input, G, p):
+    """model/norm_dist.cpp:30-40."""
+    for t, n in ((grad_output, "grad_output"), (input, "input"), (weight, "weight"), (output, "output"),
+                 (grad_input, "grad_input")):
+        _check_input(t, n)
+    dev = _same_device(grad_output, input, weight, output, grad_input)
+    B, CO, CI, HW = grad_output.size(0), output.size(1), input.size(1), input.size(2)
+    _expect(weight.size(0) == CO and weight.size(1) * G == CI, "weight must be (CO, CI/G)")
+    _expect(tuple(output.shape) == (B, CO, HW) and tuple(grad_output.shape) == (B, CO, HW),
+            "output and grad_output must be (B, CO, HW)")
+    _expect(tuple(grad_input.shape) == tuple(input.shape) and input.size(0) == B, "grad_input must match input")
+    _call("ldist_norm_dist_backward_input", dev, _p(grad_output), _p(input), _p(weight), _p(output), B, CO, CI, G, HW,
+          _p(grad_input), float(p))
+
+
+def norm_dist_backward_weight(grad_output, input, weight, output, grad_weight, G, p):
+    """model/norm_dist.cpp:42-52.  grad_weight is accumulated onto (the caller zero-fills it)."""
+    for t, n in ((grad_output, "grad_output"), (input, "input"), (weight, "weight"), (output, "output"),
+                 (grad_weight, "grad_weight")):
+        _check_input(t, n)
+    dev = _same_device(grad_output, input, weight, output, grad_weight)
+    B, CO, CI, HW = grad_output.size(0), output.size(1), input.size(1), input.size(2)
+    _expect(weight.size(0) == CO and weight.size(1) * G == CI, "weight must be (CO, CI/G)")
+    _expect(tuple(output.shape) == (B, CO, HW) and tuple(grad_output.shape) == (B, CO, HW),
+            "output and grad_output must be (B, CO, HW)")
+    _expect(tuple(grad_weight.shape) == tuple(weight.shape) and input.size(0) == B, "grad_weight must match weight")
+    _call("ldist_norm_dist_backward_weight", dev, _p(grad_output), _p(input), _p(weight), _p(output), B, CO, CI, G,
+          HW, _p(grad_weight), float(p))
+
+
+def inf_dist_forward(input, weight, output, pos, G):
+    """model/norm_dist.cpp:54-62."""
+    for t, n in ((input, "input"), (weight, "weight"), (output, "output")):
+        _check_input(t, n)
+    _check_input(pos, "pos", torch.int32)
+    dev = _same_device(input, weight, output, pos)
+    B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
+    _expect(input.dim() == 3 and weight.dim() == 2, "input must be 3-D, weight 2-D")
+    _expect(weight.size(0) == CO and weight.size(1) * G == CI, "weight must be (CO, CI/G)")
+    _expect(tuple(output.shape) == (B, CO, HW) and tuple(pos.shape) == (B, CO, HW), "output and pos must be (B, CO, HW)")
+    _call("ldist_inf_dist_forward", dev, _p(input), _p(weight), B, CO, CI, G, HW, _p(output), _p(pos))
+
+
+def inf_dist_bound_forward(input_lower, input_upper, weight, output_lower, output_upper, G):
+    """model/norm_dist.cpp:64-74."""
+    for t, n in ((input_lower, "input_lower"), (input_upper, "input_upper"), (weight, "weight"),
+                 (output_lower, "output_lower"), (output_upper, "output_upper")):
+        _check_input(t, n)
+    dev = _same_device(input_lower, input_upper, weight, output_lower, output_upper)
+    B, CO, CI, HW = input_lower.size(0), output_lower.size(1), input_lower.size(1), input_lower.size(2)
+    _expect(tuple(input_upper.shape) == tuple(input_lower.shape), "input_upper must match input_lower")
+    _expect(weight.size(0) == CO and weight.size(1) * G == CI, "weight must be (CO, CI/G)")
+    _expect(tuple(output_lower.shape) == (B, CO, HW) and tuple(output_upper.shape) == (B, CO, HW),
+            "outputs must be (B, CO, HW)")
+    _call("ldist_inf_dist_bound_forward", dev, _p(input_lower), _p(input_upper), _p(weight), B, CO, CI, G, HW,
+          _p(output_lower), _p(output_upper))
+
+
+def _inf_backward_input(name, grad_output, pos, grad_input, G):
+    _check_input(grad_output, "grad_output")
+    _check_input(pos, "pos", torch.int32)
+    _check_input(grad_input, "grad_input")
+    dev = _same_device(grad_output, pos, grad_input)
+    B, CO, CI, HW = grad_output.size(0), grad_output.size(1), grad_input.size(1), grad_input.size(2)
+    _expect(tuple(pos.shape) == tuple(grad_output.shape), "pos must match grad_output")
+    _expect(grad_input.size(0) == B and grad_output.size(2) == HW, "grad_input must be (B, CI, HW)")
+    _call(name, dev, _p(grad_output), _p(pos), B, CO, CI, G, HW, _p(grad_input))
+
+
+def _inf_backward_weight(name, grad_output, pos, grad_weight, G):
+    _check_input(grad_output, "grad_output")
+    _check_input(pos, "pos", torch.int32)
+    _check_input(grad_weight, "grad_weight")
+    dev = _same_device(grad_output, pos, grad_weight)
+    B, CO, CI, HW = grad_output.size(0), grad_output.size(1), grad_weight.size(1) * G, grad_output.size(2)
+    _expect(tuple(pos.shape) == tuple(grad_output.shape), "pos must match grad_output")
+    _expect(grad_weight.size(0) == CO, "grad_weight must be (CO, CI/G)")
+    _call(name, dev, _p(grad_output), _p(pos), B, CO, CI, G, HW, _p(grad_weight))
+
+
+def inf_dist_backward_input(grad_output, pos, grad_input, G):
+    """model/norm_dist.cpp:76-82.  Accumulates onto grad_input (the caller zero-fills it)."""
+    _inf_backward_input("ldist_inf_dist_backward_input", grad_output, pos, grad_input, G)
+
+
+def inf_dist_backward_weight(grad_output, pos, grad_weight, G):
+    """model/norm_dist.cpp:84-90.  Accumulates onto grad_weight (the caller zero-fills it)."""
+    _inf_backward_weight("ldist_inf_dist_backward_weight", grad_output, pos, grad_weight, G)
+
+
+# No counterpart in the reference: same results as zero-fill + the two functions above,
+# but every element of the gradient is written, so the buffer may be torch.empty.
+def inf_dist_backward_input_overwrite(grad_output, pos, grad_input, G):
+    _inf_backward_input("ldist_inf_dist_backward_input_overwrite", grad_output, pos, grad_input, G)
+
+
+def inf_dist_backward_weight_overwrite(grad_output, pos, grad_weight, G):
+    _inf_backward_weight("ldist_inf_dist_backward_weight_overwrite", grad_output, pos, grad_weight, G)

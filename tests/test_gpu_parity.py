@@ -1,0 +1,203 @@
+"""GPU parity: the HIP kernels, called through the C ABI, against the CPU oracle on the same seeded inputs.
+
+Bars: L_inf forward values and indices and the interval bounds are bit-exact
+(torch.equal); scatter gradients and everything p-norm are within rel 1e-5 /
+abs 1e-6 of the oracle's double-precision result.
+"""
+import pytest
+import torch
+
+import oracle
+from helpers import SIGN, gen, make_inputs
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-5, 1e-6
+
+# B, CO, CI, G, HW   -- fc and conv layouts, ragged sizes, groups, vector and scalar load paths
+SHAPES = [
+    (5, 7, 3, 1, 1),          # tiny, few outputs (one-wave-per-row kernel)
+    (33, 100, 77, 1, 1),      # K % 4 != 0: scalar loads, ragged M / N / K
+    (130, 70, 260, 1, 1),     # vector loads, M and N tails, K tail inside a chunk
+    (64, 96, 96, 3, 1),       # groups, K = 32 exactly one chunk
+    (64, 48, 96, 3, 1),       # groups with 16 outputs each
+    (256, 160, 784, 1, 1),    # MNIST-sized K, two N tiles of 80
+    (512, 10, 640, 1, 1),     # classification head
+    (2, 8, 12, 1, 16),        # conv layout, HW % 4 == 0
+    (3, 6, 9, 3, 5),          # conv layout, scalar loads, groups
+    (2, 64, 64, 2, 64),       # conv layout, 32 outputs per group
+    (4, 128, 1152, 4, 100),   # the unfolded 3x3 conv layer shape at a small image
+    (1, 40, 2000, 1, 36),     # conv layout, long K
+]
+TILES = [-1, 0, 1, 2]
+
+
+@pytest.fixture(autouse=True)
+def _reset_tile():
+    from gpu_common import set_tile
+    yield
+    set_tile(-1)
+
+
+@pytest.mark.parametrize("tile", TILES)
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("quant", [None, 8])
+def test_inf_forward_bit_exact(shape, tile, quant):
+    from gpu_common import gpu_inf_forward, say, set_tile
+    B, CO, CI, G, HW = shape
+    say("inf_forward", shape, "tile", tile, "quant", quant)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=sum(shape), quantize=quant)
+    set_tile(tile)
+    out, pos = gpu_inf_forward(x, w, G)
+    eo, ep = oracle.inf_dist_forward(x, w, G)
+    assert torch.equal(out, eo)
+    assert torch.equal(pos, ep)
+
+
+def test_inf_forward_known_answers_and_specials():
+    from gpu_common import gpu_inf_forward
+    nan, inf = float("nan"), float("inf")
+    x = torch.tensor([[0.0, 2.0, 0.0], [2.0, 0.0, 0.0], [1.0, 1.0, 1.0], [nan, 1.0, 0.5], [nan, nan, nan],
+                      [0.0, inf, 2.0], [0.0, -inf, inf]]).reshape(7, 3, 1)
+    w = torch.tensor([[1.0, 1.0, 1.0], [0.0, 0.0, 0.0]])
+    out, pos = gpu_inf_forward(x, w, 1)
+    eo, ep = oracle.inf_dist_forward(x, w, 1, literal=True)
+    assert torch.equal(out, eo) and torch.equal(pos, ep)
+    assert pos[0, 0, 0].item() == (0 | SIGN) and pos[1, 0, 0].item() == 0 and pos[2, 0, 0].item() == 0
+
+
+@pytest.mark.parametrize("tile", TILES)
+@pytest.mark.parametrize("shape", SHAPES)
+def test_bound_forward_bit_exact(shape, tile):
+    from gpu_common import gpu_bound_forward, say, set_tile
+    B, CO, CI, G, HW = shape
+    say("bound_forward", shape, "tile", tile)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=1 + sum(shape))
+    lo, up = (x - 8 / 255).clamp(0, 1).contiguous(), (x + 8 / 255).clamp(0, 1).contiguous()
+    set_tile(tile)
+    ol, ou = gpu_bound_forward(lo, up, w, G)
+    el, eu = oracle.inf_dist_bound_forward(lo, up, w, G)
+    assert torch.equal(ol, el) and torch.equal(ou, eu)
+    # degenerate box reproduces the value forward bit for bit
+    ol, ou = gpu_bound_forward(x, x, w, G)
+    ev, _ = oracle.inf_dist_forward(x, w, G)
+    assert torch.equal(ol, ev) and torch.equal(ou, ev)
+
+
+@pytest.mark.parametrize("shape", [(33, 100, 77, 1, 1), (130, 70, 260, 1, 1), (2, 64, 64, 2, 64)])
+def test_bound_forward_irregular_boxes_match_reference_predicate(shape):
+    # lower > upper, NaN and infinities: the kernel must fall back to the literal predicate
+    from gpu_common import gpu_bound_forward
+    B, CO, CI, G, HW = shape
+    x, w = make_inputs(B, CO, CI, G, HW, seed=9)
+    g = gen(4)
+    lo = (x - 0.1).contiguous()
+    up = (x + 0.1).contiguous()
+    flip = torch.rand(x.shape, generator=g) < 0.05
+    lo2 = torch.where(flip, up, lo).contiguous()
+    up2 = torch.where(flip, lo, up).contiguous()
+    lo2[0, 0, 0] = float("nan")
+    up2[-1, -1, -1] = float("inf")
+    w2 = w.clone()
+    w2[0, 0] = float("-inf")
+    for (a, b, ww) in ((lo2, up2, w), (lo, up, w2)):
+        ol, ou = gpu_bound_forward(a, b, ww, G)
+        el, eu = oracle.inf_dist_bound_forward(a, b, ww, G)
+        assert torch.equal(torch.nan_to_num(ol, nan=-1.0), torch.nan_to_num(el, nan=-1.0))
+        assert torch.equal(torch.nan_to_num(ou, nan=-1.0), torch.nan_to_num(eu, nan=-1.0))
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("overwrite", [False, True])
+def test_inf_backward(shape, overwrite):
+    from gpu_common import DEV, cpp, say
+    B, CO, CI, G, HW = shape
+    say("inf_backward", shape, "overwrite", overwrite)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=2 + sum(shape), quantize=16)
+    _, pos = oracle.inf_dist_forward(x, w, G)
+    go = torch.randn(B, CO, HW, generator=gen(5))
+    ex = oracle.inf_dist_backward_input(go, pos, CI, G)
+    ew = oracle.inf_dist_backward_weight(go, pos, CI, G)
+    if overwrite:
+        gx = torch.full((B, CI, HW), float("nan"), device=DEV)
+        gw = torch.full((CO, CI // G), float("nan"), device=DEV)
+        cpp.inf_dist_backward_input_overwrite(go.to(DEV), pos.to(DEV), gx, G)
+        cpp.inf_dist_backward_weight_overwrite(go.to(DEV), pos.to(DEV), gw, G)
+    else:
+        gx = torch.full((B, CI, HW), 0.5, device=DEV)
+        gw = torch.full((CO, CI // G), -0.25, device=DEV)
+        cpp.inf_dist_backward_input(go.to(DEV), pos.to(DEV), gx, G)
+        cpp.inf_dist_backward_weight(go.to(DEV), pos.to(DEV), gw, G)
+        ex, ew = ex + 0.5, ew - 0.25
+    torch.cuda.synchronize()
+    torch.testing.assert_close(gx.cpu(), ex, rtol=RTOL, atol=ATOL)
+    torch.testing.assert_close(gw.cpu(), ew, rtol=RTOL, atol=ATOL)
+
+
+PNORM_SHAPES = [s for s in SHAPES if s[1] * s[2] * s[0] * s[4] <= 40_000_000]
+
+
+@pytest.mark.parametrize("tile", [-1, 0, 2])
+@pytest.mark.parametrize("shape", PNORM_SHAPES)
+@pytest.mark.parametrize("p", [8.0, 2.0, 3.5, 37.0, 1000.0])
+def test_norm_forward(shape, tile, p):
+    from gpu_common import gpu_norm_forward, say, set_tile
+    B, CO, CI, G, HW = shape
+    say("norm_forward", shape, "tile", tile, "p", p)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=3 + sum(shape))
+    set_tile(tile)
+    out = gpu_norm_forward(x, w, G, p)
+    torch.testing.assert_close(out, oracle.norm_dist_forward(x, w, G, p), rtol=RTOL, atol=ATOL)
+
+
+def test_norm_forward_scale_robust_and_seeded():
+    from gpu_common import gpu_norm_forward
+    x, w = make_inputs(40, 50, 132, 1, 1, seed=4)
+    for scale in (1e-6, 1.0, 1e6, 1e18):
+        xs, ws = (x * scale).contiguous(), (w * scale).contiguous()
+        out = gpu_norm_forward(xs, ws, 1, 8.0)
+        torch.testing.assert_close(out, oracle.norm_dist_forward(xs, ws, 1, 8.0), rtol=RTOL, atol=0)
+    same = torch.full((3, 8, 1), 0.25)
+    out = gpu_norm_forward(same, torch.full((17, 8), 0.25), 1, 8.0)
+    torch.testing.assert_close(out, oracle.norm_dist_forward(same, torch.full((17, 8), 0.25), 1, 8.0), rtol=1e-4,
+                               atol=0)
+
+
+@pytest.mark.parametrize("shape", PNORM_SHAPES)
+@pytest.mark.parametrize("p", [8.0, 2.0, 3.0, 4.0, 5.5, 100.0])
+def test_norm_backward(shape, p):
+    from gpu_common import DEV, cpp, say
+    B, CO, CI, G, HW = shape
+    say("norm_backward", shape, "p", p)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=6 + sum(shape))
+    go = torch.randn(B, CO, HW, generator=gen(7))
+    out = oracle.norm_dist_forward(x, w, G, p)
+    ex = oracle.norm_dist_backward_input(go, x, w, out, G, p)
+    ew = oracle.norm_dist_backward_weight(go, x, w, out, G, p)
+    gx = torch.full((B, CI, HW), float("nan"), device=DEV)
+    gw = torch.full((CO, CI // G), 0.125, device=DEV)
+    args = (go.to(DEV), x.to(DEV), w.to(DEV), out.to(DEV))
+    cpp.norm_dist_backward_input(*args, gx, G, p)
+    cpp.norm_dist_backward_weight(*args, gw, G, p)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(gx.cpu(), ex, rtol=RTOL, atol=ATOL)
+    torch.testing.assert_close(gw.cpu(), ew + 0.125, rtol=RTOL, atol=ATOL)
+
+
+def test_error_codes_and_checks():
+    from gpu_common import DEV, cpp, pkg
+    lib = pkg._lib.lib()
+    x = torch.zeros(2, 6, 1, device=DEV)
+    w = torch.zeros(4, 6, device=DEV)
+    out = torch.empty(2, 4, 1, device=DEV)
+    pos = torch.empty(2, 4, 1, device=DEV, dtype=torch.int32)
+    assert lib.ldist_inf_dist_forward(None, w.data_ptr(), 2, 4, 6, 1, 1, out.data_ptr(), pos.data_ptr(), None) == -1
+    assert lib.ldist_inf_dist_forward(x.data_ptr(), w.data_ptr(), 2, 4, 6, 4, 1, out.data_ptr(), pos.data_ptr(),
+                                      None) == -1  # CI % G
+    assert lib.ldist_norm_dist_forward(x.data_ptr(), w.data_ptr(), 2, 4, 6, 1, 1, out.data_ptr(), 1.0, None) == -1
+    with pytest.raises(RuntimeError):
+        cpp.inf_dist_forward(x.cpu(), w, out, pos, 1)
+    with pytest.raises(RuntimeError):
+        cpp.inf_dist_forward(x.expand(2, 6, 2)[:, :, :1], w, out, pos, 1)  # not contiguous
+    with pytest.raises(RuntimeError):
+        cpp.norm_dist_forward(x, w, out, 1, 0.5)
