@@ -13,6 +13,41 @@
 
 namespace ldist {
 
+// Lowest k in [0, len) with |x[k] - w[k]| == best, as kb + k with bit 31 carrying the
+// sign of the difference; 0 if none.  All 32 operand pairs are fetched before the
+// first comparison so the loads overlap.  XVEC: both rows are contiguous, 16-byte
+// aligned and len is a multiple of 4.
+template <bool XVEC>
+__device__ __forceinline__ int locate_in_chunk(const float* __restrict__ xr, int xk, const float* __restrict__ wr,
+                                               int len, float best, int kb) {
+    float xv[kChunk], wv[kChunk];
+    if constexpr (XVEC) {
+#pragma unroll
+        for (int q = 0; q < kChunk / 4; q++) {
+            float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+            if (q * 4 < len) {
+                a = reinterpret_cast<const float4*>(xr)[q];
+                b = reinterpret_cast<const float4*>(wr)[q];
+            }
+            xv[q * 4] = a.x; xv[q * 4 + 1] = a.y; xv[q * 4 + 2] = a.z; xv[q * 4 + 3] = a.w;
+            wv[q * 4] = b.x; wv[q * 4 + 1] = b.y; wv[q * 4 + 2] = b.z; wv[q * 4 + 3] = b.w;
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < kChunk; k++) {
+            xv[k] = k < len ? xr[(size_t)k * xk] : 0.f;
+            wv[k] = k < len ? wr[k] : 0.f;
+        }
+    }
+    int p = 0;
+#pragma unroll
+    for (int k = kChunk - 1; k >= 0; k--) {  // descending: the lowest match is written last
+        const float df = xv[k] - wv[k];
+        if (__builtin_fabsf(df) == best) p = (kb + k) | (__float_as_int(df) & 0x80000000);
+    }
+    return p;
+}
+
 template <class GEO, bool CONV, int VEC>
 __global__ void __launch_bounds__(GEO::NT, 2)
 inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ weight, float* __restrict__ output,
@@ -21,7 +56,7 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
     constexpr int NGRP = GEO::NGRP;
     using Stage = Stager<GEO, CONV, VEC, 1>;
     constexpr int STAGE = Stage::STAGE, NBUF = Stage::NBUF;
-    static_assert(2 * (KS - 1) * TM * TN * NGRP <= NBUF * STAGE, "merge area fits in the panels");
+    static_assert(KS == 1 || 2 * TM * TN * NGRP <= NBUF * STAGE, "merge area fits in the panels");
     extern __shared__ __align__(16) float lds[];
 
     int tm, tn, g;
@@ -78,38 +113,43 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
         __syncthreads();
     }
 
-    // Merge the k-groups: the larger value wins, equal values keep the lower chunk.
-    if constexpr (KS > 1) {
-        float* mv = lds;  // [KS-1][TM*TN][NGRP] values, then as many chunk ids
-        int* mi = reinterpret_cast<int*>(lds) + (KS - 1) * TM * TN * NGRP;
-        if (grp > 0) {
+    // Merge the two k-groups.  Each group finishes half of the lane's rows, so it needs the
+    // other group's candidates for that half only: the larger value wins, equal values keep
+    // the lower chunk.
+    static_assert(KS == 1 || KS == 2, "the merge below pairs two k-groups");
+    constexpr int TMH = TM / KS;          // rows finished by each group
+    if constexpr (KS == 2) {
+        float* mv = lds;  // [2 groups][TMH*TN][NGRP] values, then as many chunk ids
+        int* mi = reinterpret_cast<int*>(lds) + 2 * TMH * TN * NGRP;
 #pragma unroll
-            for (int i = 0; i < TM; i++)
+        for (int i = 0; i < TM; i++) {
+            const bool mine = (i / TMH) == grp;
+            if (mine) continue;  // rows of the other group: hand my candidates over
 #pragma unroll
-                for (int j = 0; j < TN; j++) {
-                    const int o = ((grp - 1) * TM * TN + i * TN + j) * NGRP + t;
-                    mv[o] = acc[i][j];
-                    mi[o] = cidx[i][j];
-                }
+            for (int j = 0; j < TN; j++) {
+                const int o = (((1 - grp) * TMH + (i % TMH)) * TN + j) * NGRP + t;
+                mv[o] = acc[i][j];
+                mi[o] = cidx[i][j];
+            }
         }
         __syncthreads();
-        if (grp > 0) return;
 #pragma unroll
-        for (int q = 0; q < KS - 1; q++)
+        for (int i = 0; i < TM; i++) {
+            if ((i / TMH) != grp) continue;
 #pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++) {
-                    const int o = (q * TM * TN + i * TN + j) * NGRP + t;
-                    const float v = mv[o];
-                    const int ci = mi[o];
-                    if (v > acc[i][j] || (v == acc[i][j] && ci < cidx[i][j])) { acc[i][j] = v; cidx[i][j] = ci; }
-                }
+            for (int j = 0; j < TN; j++) {
+                const int o = ((grp * TMH + (i % TMH)) * TN + j) * NGRP + t;
+                const float v = mv[o];
+                const int ci = mi[o];
+                if (v > acc[i][j] || (v == acc[i][j] && ci < cidx[i][j])) { acc[i][j] = v; cidx[i][j] = ci; }
+            }
+        }
     }
 
     // Locate the argmax inside the recorded chunk and write both outputs.
 #pragma unroll
     for (int i = 0; i < TM; i++) {
+        if (KS == 2 && (i / TMH) != grp) continue;
         const int m = m0 + GEO::row(ty, i);
         if (m >= d.M) continue;
         const RowAddr<CONV> ra(d, m, g);
@@ -121,13 +161,9 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
             int p = 0;
             if (best > 0.f) {
                 const int kb = cidx[i][j] * kChunk;
-                const int ke = min(kb + kChunk, K);
                 const float* xr = input + ra.x + (size_t)kb * ra.xk;
                 const float* wr = weight + ((size_t)g * d.NG + n) * K + kb;
-                for (int k = ke - kb - 1; k >= 0; k--) {  // descending: the lowest match is written last
-                    const float df = xr[(size_t)k * ra.xk] - wr[k];
-                    if (__builtin_fabsf(df) == best) p = (kb + k) | (__float_as_int(df) & 0x80000000);
-                }
+                p = locate_in_chunk<(!CONV && VEC == 4)>(xr, ra.xk, wr, min(kChunk, K - kb), best, kb);
             }
             output[ra.o + (size_t)n * ra.on] = best;
             pos[ra.o + (size_t)n * ra.on] = p;
@@ -148,55 +184,81 @@ struct InfForward {
 };
 
 // ---------------------------------------------------------------------------
-// Few outputs per group (the 10-way classification head): one wave per row m,
-// lanes split k, each lane keeps the exact (value, k) pair per output and the
-// wave reduces with "larger value, then lower k".  Memory bound by design.
+// Few outputs per group (the 10-way classification head): a workgroup takes RW
+// rows m of one group, its 256 lanes split k, each lane keeps the exact
+// (value, k) pair per (row, output), and the pairs are reduced with "larger
+// value, then lower k" first inside each wave, then across the four waves
+// through LDS.  Bound by reading x once and w from L2.
 // ---------------------------------------------------------------------------
-template <int NB>
+__device__ __forceinline__ void take_better(float& v, int& p, float ov, int op) {
+    if (ov > v || (ov == v && (op & 0x7fffffff) < (p & 0x7fffffff))) { v = ov; p = op; }
+}
+
+template <int RW, int NB>
 __global__ void __launch_bounds__(256)
 inf_forward_skinny_kernel(const float* __restrict__ input, const float* __restrict__ weight,
                           float* __restrict__ output, int32_t* __restrict__ pos, Dims d) {
-    const int lane = threadIdx.x & 63;
-    const int wave = (blockIdx.x * 256 + threadIdx.x) >> 6;
-    const int rows = d.M * d.G;
-    if (wave >= rows) return;
-    const int m = wave / d.G, g = wave % d.G;
-    const int b = m / d.HW, hw = m % d.HW;
+    __shared__ float sv[4][RW * NB];
+    __shared__ int sp[4][RW * NB];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int row_blocks = (d.M + RW - 1) / RW;
+    const int g = blockIdx.x / row_blocks;
+    const int m0 = (blockIdx.x % row_blocks) * RW;
     const int K = d.K, xk = d.HW;
-    const float* xr = input + ((size_t)(b * d.G + g) * K) * d.HW + hw;
-    const size_t ooff = ((size_t)(b * d.G + g) * d.NG) * d.HW + hw;
-    for (int nb = 0; nb < d.NG; nb += NB) {
-        float best[NB];
-        int bk[NB];
+    size_t xoff[RW], ooff[RW];
 #pragma unroll
-        for (int j = 0; j < NB; j++) { best[j] = 0.f; bk[j] = 0; }
-        for (int k = lane; k < K; k += 64) {
-            const float xv = xr[(size_t)k * xk];
+    for (int r = 0; r < RW; r++) {
+        const int m = min(m0 + r, d.M - 1);  // rows past the end repeat the last one and are not written
+        const int b = m / d.HW, hw = m % d.HW;
+        xoff[r] = ((size_t)(b * d.G + g) * K) * d.HW + hw;
+        ooff[r] = ((size_t)(b * d.G + g) * d.NG) * d.HW + hw;
+    }
+    for (int nb = 0; nb < d.NG; nb += NB) {
+        float best[RW][NB];
+        int bp[RW][NB];
+#pragma unroll
+        for (int r = 0; r < RW; r++)
+#pragma unroll
+            for (int j = 0; j < NB; j++) { best[r][j] = 0.f; bp[r][j] = 0; }
+        for (int k = tid; k < K; k += 256) {
+            float xv[RW], wv[NB];
+#pragma unroll
+            for (int r = 0; r < RW; r++) xv[r] = input[xoff[r] + (size_t)k * xk];
+#pragma unroll
+            for (int j = 0; j < NB; j++)
+                wv[j] = weight[((size_t)g * d.NG + min(nb + j, d.NG - 1)) * K + k];
+#pragma unroll
+            for (int r = 0; r < RW; r++)
+#pragma unroll
+                for (int j = 0; j < NB; j++) {
+                    const float df = xv[r] - wv[j];
+                    const float a = __builtin_fabsf(df);
+                    if (a > best[r][j]) { best[r][j] = a; bp[r][j] = k | (__float_as_int(df) & 0x80000000); }
+                }
+        }
+#pragma unroll
+        for (int r = 0; r < RW; r++)
 #pragma unroll
             for (int j = 0; j < NB; j++) {
-                if (nb + j < d.NG) {
-                    const float df = xv - weight[((size_t)g * d.NG + nb + j) * K + k];
-                    const float a = __builtin_fabsf(df);
-                    if (a > best[j]) { best[j] = a; bk[j] = k | (__float_as_int(df) & 0x80000000); }
-                }
+                float v = best[r][j];
+                int p = bp[r][j];
+#pragma unroll
+                for (int off = 32; off >= 1; off >>= 1) take_better(v, p, __shfl_xor(v, off, 64), __shfl_xor(p, off, 64));
+                if (lane == 0) { sv[wave][r * NB + j] = v; sp[wave][r * NB + j] = p; }
+            }
+        __syncthreads();
+        if (tid < RW * NB) {
+            float v = sv[0][tid];
+            int p = sp[0][tid];
+#pragma unroll
+            for (int q = 1; q < 4; q++) take_better(v, p, sv[q][tid], sp[q][tid]);
+            const int r = tid / NB, j = tid % NB;
+            if (m0 + r < d.M && nb + j < d.NG) {
+                output[ooff[r] + (size_t)(nb + j) * d.HW] = v;
+                pos[ooff[r] + (size_t)(nb + j) * d.HW] = v > 0.f ? p : 0;
             }
         }
-#pragma unroll
-        for (int j = 0; j < NB; j++) {
-            float v = best[j];
-            int p = bk[j];
-#pragma unroll
-            for (int off = 32; off >= 1; off >>= 1) {
-                const float ov = __shfl_xor(v, off, 64);
-                const int op = __shfl_xor(p, off, 64);
-                const bool take = ov > v || (ov == v && (op & 0x7fffffff) < (p & 0x7fffffff));
-                if (take) { v = ov; p = op; }
-            }
-            if (lane == 0 && nb + j < d.NG) {
-                output[ooff + (size_t)(nb + j) * d.HW] = v;
-                pos[ooff + (size_t)(nb + j) * d.HW] = v > 0.f ? p : 0;
-            }
-        }
+        __syncthreads();
     }
 }
 
@@ -204,10 +266,10 @@ hipError_t inf_forward(const float* input, const float* weight, float* output, i
                        hipStream_t stream) {
     if (pr.NG <= 16) {
         const Dims d = make_dims(pr);
-        const int rows = d.M * d.G;
-        const unsigned grid = (unsigned)((rows + 3) / 4);
-        hipLaunchKernelGGL(inf_forward_skinny_kernel<8>, dim3(grid), dim3(256), 0, stream, input, weight, output, pos,
-                           d);
+        constexpr int RW = 2;
+        const unsigned grid = (unsigned)((d.M + RW - 1) / RW) * d.G;
+        hipLaunchKernelGGL((inf_forward_skinny_kernel<RW, 8>), dim3(grid), dim3(256), 0, stream, input, weight,
+                           output, pos, d);
         return hipGetLastError();
     }
     return dispatch_forward<InfForward>(pr, can_vec4(pr, input, weight), stream, input, weight, output, pos);

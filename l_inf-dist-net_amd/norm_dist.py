@@ -174,7 +174,11 @@ class NormDistConv(nn.Module):
         h, w = x.size(2), x.size(3)
         out_h = (h + 2 * self.padding - self.kernel_size) // self.stride + 1
         out_w = (w + 2 * self.padding - self.kernel_size) // self.stride + 1
-        unfold = lambda t: F.unfold(t, self.kernel_size, self.dilation, self.padding, self.stride)
+        if self.kernel_size == 1 and self.stride == 1 and self.padding == 0:
+            # a 1x1 window is the identity: skip F.unfold, which launches one kernel per image
+            unfold = lambda t: t.reshape(t.size(0), t.size(1), -1)
+        else:
+            unfold = lambda t: F.unfold(t, self.kernel_size, self.dilation, self.padding, self.stride)
         cols = unfold(x)
         weight = self.weight.view(self.weight.size(0), -1)
         y = norm_dist(cols.view(cols.size(0), cols.size(1), -1), weight, self.group, p=self.p, tag=self.tag)

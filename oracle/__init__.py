@@ -116,23 +116,28 @@ def norm_dist_forward(x, weight, group, p, f32_reference_order=False):
     return out
 
 
-def norm_dist_backward_input(grad_output, x, weight, output, group, p):
+def norm_dist_backward_input(grad_output, x, weight, output, group, p, with_abs_terms=False):
+    """with_abs_terms=True also returns sum_n |term| per element (the rounding-error scale)."""
     B, CO, CI, G, HW = _dims(x, weight, group)
     grad_input = torch.empty_like(x)
+    mag = torch.empty_like(x) if with_abs_terms else None
     _check(lib().ldist_oracle_norm_dist_backward_input(_f(grad_output), _f(x), _f(weight), _f(output), B, CO, CI, G,
-                                                        HW, _f(grad_input), ctypes.c_float(p)),
+                                                        HW, _f(grad_input), ctypes.c_float(p),
+                                                        _f(mag) if with_abs_terms else None),
            "norm_dist_backward_input")
-    return grad_input
+    return (grad_input, mag) if with_abs_terms else grad_input
 
 
-def norm_dist_backward_weight(grad_output, x, weight, output, group, p, grad_weight=None):
+def norm_dist_backward_weight(grad_output, x, weight, output, group, p, grad_weight=None, with_abs_terms=False):
     B, CO, CI, G, HW = _dims(x, weight, group)
     if grad_weight is None:
         grad_weight = torch.zeros_like(weight)
+    mag = torch.empty_like(weight) if with_abs_terms else None
     _check(lib().ldist_oracle_norm_dist_backward_weight(_f(grad_output), _f(x), _f(weight), _f(output), B, CO, CI, G,
-                                                         HW, _f(grad_weight), ctypes.c_float(p)),
+                                                         HW, _f(grad_weight), ctypes.c_float(p),
+                                                         _f(mag) if with_abs_terms else None),
            "norm_dist_backward_weight")
-    return grad_weight
+    return (grad_weight, mag) if with_abs_terms else grad_weight
 
 
 # --------------------------------------------------------------------------- #

@@ -378,9 +378,11 @@ int ldist_oracle_norm_dist_forward_f32(const float* input, const float* weight, 
 /*   t = x - w, s = +1 if t > 0 else -1 (:295-296).  Every element is written */
 /*   (:359-360).  Evaluated in double from the float inputs.                  */
 /* ------------------------------------------------------------------------- */
+/*   abs_terms (may be NULL) receives sum_n |g * (|t|/out)^(p-1)|, the scale  */
+/*   against which a float evaluation's rounding error is judged.             */
 int ldist_oracle_norm_dist_backward_input(const float* grad_output, const float* input, const float* weight,
                                           const float* output, int B, int CO, int CI, int G, int HW,
-                                          float* grad_input, float p) {
+                                          float* grad_input, float p, float* abs_terms) {
     int rc = check_dims(B, CO, CI, G, HW);
     if (rc) return rc;
     if (!grad_output || !input || !weight || !output || !grad_input || !(p > 1.0f)) return LDIST_ORACLE_EINVAL;
@@ -392,15 +394,17 @@ int ldist_oracle_norm_dist_backward_input(const float* grad_output, const float*
             const int g = bg % G;
             for (int hw = 0; hw < HW; hw++) {
                 const double x = (double)input[((size_t)bg * K + k) * HW + hw];
-                double acc = 0.0;
+                double acc = 0.0, mag = 0.0;
                 for (int n = 0; n < NG; n++) {
                     size_t o = ((size_t)bg * NG + n) * HW + hw;
                     double t = x - (double)weight[((size_t)g * NG + n) * K + k];
                     double ro = 1.0 / (double)output[o];
                     double v = (double)grad_output[o] * pow(fabs(t) * ro, pm1);
                     acc += t > 0 ? v : -v;
+                    mag += fabs(v);
                 }
                 grad_input[((size_t)bg * K + k) * HW + hw] = (float)acc;
+                if (abs_terms) abs_terms[((size_t)bg * K + k) * HW + hw] = (float)mag;
             }
         }
     }
@@ -413,7 +417,7 @@ int ldist_oracle_norm_dist_backward_input(const float* grad_output, const float*
 /*   zero-filled buffer (:424, model/norm_dist.py:45).                        */
 int ldist_oracle_norm_dist_backward_weight(const float* grad_output, const float* input, const float* weight,
                                            const float* output, int B, int CO, int CI, int G, int HW,
-                                           float* grad_weight, float p) {
+                                           float* grad_weight, float p, float* abs_terms) {
     int rc = check_dims(B, CO, CI, G, HW);
     if (rc) return rc;
     if (!grad_output || !input || !weight || !output || !grad_weight || !(p > 1.0f)) return LDIST_ORACLE_EINVAL;
@@ -424,7 +428,7 @@ int ldist_oracle_norm_dist_backward_weight(const float* grad_output, const float
         for (int k = 0; k < K; k++) {
             const int g = gn / NG;
             const double w = (double)weight[(size_t)gn * K + k];
-            double acc = 0.0;
+            double acc = 0.0, mag = 0.0;
             for (int b = 0; b < B; b++) {
                 const size_t obase = ((size_t)b * CO + gn) * HW;
                 const size_t xbase = ((size_t)(b * G + g) * K + k) * HW;
@@ -433,10 +437,12 @@ int ldist_oracle_norm_dist_backward_weight(const float* grad_output, const float
                     double ro = 1.0 / (double)output[obase + hw];
                     double v = (double)grad_output[obase + hw] * pow(fabs(t) * ro, pm1);
                     acc += t > 0 ? v : -v;
+                    mag += fabs(v);
                 }
             }
             float* dst = grad_weight + (size_t)gn * K + k;
             *dst = (float)((double)*dst + acc);
+            if (abs_terms) abs_terms[(size_t)gn * K + k] = (float)mag;
         }
     }
     return LDIST_ORACLE_OK;

@@ -88,3 +88,22 @@ def dense_inf_backward(grad_out, pos, CI, G):
     grad_x = onehot.sum(dim=2).reshape(B, CI, HW)
     grad_w = -onehot.sum(dim=(0, 4)).reshape(CO, K)
     return grad_x, grad_w
+
+
+def assert_sum_close(got, exact, abs_terms, p=None, rtol=1e-5, atol=1e-6):
+    """Tolerance for a float32 sum of signed terms checked against its exact value.
+
+    |got - exact| <= tol_scale * (rtol*|exact| + atol*max(1, sum|terms|)).
+    The absolute part scales with the size of what was summed: float32 rounding
+    of the terms alone already leaves an error proportional to sum|terms|, for
+    any implementation.  For the p-norm gradients every term is u^(p-1) with u
+    known to about 2e-7 relative, so the terms themselves are only good to
+    (p-1)*2e-7; tol_scale = max(1, p/8) accounts for that above p = 8.
+    """
+    scale = 1.0 if p is None else max(1.0, p / 8.0)
+    err = (got.double() - exact.double()).abs()
+    bound = scale * (rtol * exact.double().abs() + atol * abs_terms.double().clamp_min(1.0))
+    bad = err > bound
+    assert not bool(bad.any()), (
+        f"{int(bad.sum())} of {bad.numel()} elements outside tolerance; worst excess "
+        f"{float((err - bound).max()):.3e} (err {float(err[bad].max()):.3e})")

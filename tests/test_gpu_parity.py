@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import oracle
-from helpers import SIGN, gen, make_inputs
+from helpers import SIGN, assert_sum_close, gen, make_inputs
 
 pytestmark = pytest.mark.gpu
 
@@ -172,16 +172,17 @@ def test_norm_backward(shape, p):
     x, w = make_inputs(B, CO, CI, G, HW, seed=6 + sum(shape))
     go = torch.randn(B, CO, HW, generator=gen(7))
     out = oracle.norm_dist_forward(x, w, G, p)
-    ex = oracle.norm_dist_backward_input(go, x, w, out, G, p)
-    ew = oracle.norm_dist_backward_weight(go, x, w, out, G, p)
+    ex, mx = oracle.norm_dist_backward_input(go, x, w, out, G, p, with_abs_terms=True)
+    ew, mw = oracle.norm_dist_backward_weight(go, x, w, out, G, p, with_abs_terms=True)
     gx = torch.full((B, CI, HW), float("nan"), device=DEV)
     gw = torch.full((CO, CI // G), 0.125, device=DEV)
     args = (go.to(DEV), x.to(DEV), w.to(DEV), out.to(DEV))
     cpp.norm_dist_backward_input(*args, gx, G, p)
     cpp.norm_dist_backward_weight(*args, gw, G, p)
     torch.cuda.synchronize()
-    torch.testing.assert_close(gx.cpu(), ex, rtol=RTOL, atol=ATOL)
-    torch.testing.assert_close(gw.cpu(), ew + 0.125, rtol=RTOL, atol=ATOL)
+    # rel 1e-5 / abs 1e-6, the absolute part relative to the magnitude of the summed terms
+    assert_sum_close(gx.cpu(), ex, mx, p, RTOL, ATOL)
+    assert_sum_close(gw.cpu() - 0.125, ew, mw, p, RTOL, ATOL)
 
 
 def test_error_codes_and_checks():
@@ -198,6 +199,6 @@ def test_error_codes_and_checks():
     with pytest.raises(RuntimeError):
         cpp.inf_dist_forward(x.cpu(), w, out, pos, 1)
     with pytest.raises(RuntimeError):
-        cpp.inf_dist_forward(x.expand(2, 6, 2)[:, :, :1], w, out, pos, 1)  # not contiguous
+        cpp.inf_dist_forward(x, torch.zeros(6, 4, device=DEV).t(), out, pos, 1)  # weight not contiguous
     with pytest.raises(RuntimeError):
         cpp.norm_dist_forward(x, w, out, 1, 0.5)
