@@ -119,19 +119,8 @@ bound_forward_kernel(const float* __restrict__ lower, const float* __restrict__ 
                 }
     }
 
-#pragma unroll
-    for (int i = 0; i < TM; i++) {
-        const int m = m0 + GEO::row(ty, i);
-        if (m >= d.M) continue;
-        const RowAddr<CONV> ra(d, m, g);
-#pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const int n = n0 + GEO::col(tx, j);
-            if (n >= d.NG) continue;
-            out_lower[ra.o + (size_t)n * ra.on] = lo[i][j];
-            out_upper[ra.o + (size_t)n * ra.on] = up[i][j];
-        }
-    }
+    store_patch<GEO, CONV>(out_lower, lo, d, m0, n0, g, tx, ty, 0xFFu, d.ovec != 0);
+    store_patch<GEO, CONV>(out_upper, up, d, m0, n0, g, tx, ty, 0xFFu, d.ovec != 0);
 }
 
 template <class GEO, bool CONV, int VEC>
@@ -149,7 +138,8 @@ struct BoundForward {
 
 hipError_t bound_forward(const float* lower, const float* upper, const float* weight, float* out_lower,
                          float* out_upper, const Problem& pr, hipStream_t stream) {
-    return dispatch_forward<BoundForward>(pr, can_vec4(pr, lower, upper, weight), stream, lower, upper, weight,
+    return dispatch_forward<BoundForward>(pr, can_vec4(pr, lower, upper, weight),
+                                          can_vec4_out(pr, out_lower, out_upper), stream, lower, upper, weight,
                                           out_lower, out_upper);
 }
 

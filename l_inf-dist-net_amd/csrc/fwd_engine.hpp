@@ -4,6 +4,8 @@
 #include "kernels.hpp"
 #include "tile.hpp"
 
+#include <type_traits>
+
 namespace ldist {
 
 // Global -> register -> LDS staging of one pipeline stage: NX input panels
@@ -111,7 +113,80 @@ struct RowAddr {
     }
 };
 
-inline Dims make_dims(const Problem& pr) { return Dims{pr.B, pr.G, pr.K, pr.NG, pr.HW, pr.B * pr.HW, 0, 0}; }
+// Writes one lane's TM x TN patch of a result tensor.  When `vec` is set (base
+// pointer 16-byte aligned, NG % 4 == 0 in the fc layout, HW % 4 == 0 in the conv
+// layout) each run of four values along the contiguous axis (n for fc, the row
+// index for conv) that lies fully inside the tensor goes out as one 128-bit
+// store; everything else falls back to single stores.  `rows` selects which of
+// the lane's rows to write (bit i = row i), in whole runs of four.
+template <class GEO, bool CONV, class T>
+__device__ __forceinline__ void store_patch(T* __restrict__ dst, const T (&val)[GEO::TM][GEO::TN], const Dims& d,
+                                            int m0, int n0, int g, int tx, int ty, unsigned rows, bool vec) {
+    constexpr int TM = GEO::TM, TN = GEO::TN;
+    using V4 = typename std::conditional<std::is_same<T, float>::value, float4, int4>::type;
+    if constexpr (!CONV) {
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            if (!((rows >> i) & 1)) continue;
+            const int m = m0 + GEO::row(ty, i);
+            if (m >= d.M) continue;
+            T* row = dst + ((size_t)m * d.G + g) * d.NG;
+#pragma unroll
+            for (int r = 0; r < TN / 4; r++) {  // the lane's columns come in runs of four
+                const int j = 4 * r;
+                const int n = n0 + GEO::col(tx, j);
+                if (vec && n + 3 < d.NG) {
+                    V4 q;
+                    q.x = val[i][j]; q.y = val[i][j + 1]; q.z = val[i][j + 2]; q.w = val[i][j + 3];
+                    *reinterpret_cast<V4*>(row + n) = q;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (n + e < d.NG) row[n + e] = val[i][j + e];
+                }
+            }
+#pragma unroll
+            for (int j = TN / 4 * 4; j < TN; j++) {
+                const int n = n0 + GEO::col(tx, j);
+                if (n < d.NG) row[n] = val[i][j];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int n = n0 + GEO::col(tx, j);
+            if (n >= d.NG) continue;
+#pragma unroll
+            for (int r = 0; r < TM / 4; r++) {  // the lane's rows come in runs of four
+                const int i = 4 * r;
+                if (((rows >> i) & 0xF) != 0xF) continue;  // a run is written by one k-group as a whole
+                const int m = m0 + GEO::row(ty, i);
+                if (m >= d.M) continue;
+                if (vec && m + 3 < d.M) {  // HW % 4 == 0 keeps the four rows inside one image
+                    const int b = m / d.HW, hw = m % d.HW;
+                    V4 q;
+                    q.x = val[i][j]; q.y = val[i + 1][j]; q.z = val[i + 2][j]; q.w = val[i + 3][j];
+                    *reinterpret_cast<V4*>(dst + ((size_t)(b * d.G + g) * d.NG + n) * d.HW + hw) = q;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int me = m + e;
+                        if (me < d.M) {
+                            const int b = me / d.HW, hw = me % d.HW;
+                            dst[((size_t)(b * d.G + g) * d.NG + n) * d.HW + hw] = val[i + e][j];
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+inline bool can_vec4_out(const Problem& pr, const void* a, const void* b = nullptr) {
+    return aligned16(a) && aligned16(b) && (pr.HW == 1 ? pr.NG % 4 == 0 : pr.HW % 4 == 0);
+}
+
+inline Dims make_dims(const Problem& pr) { return Dims{pr.B, pr.G, pr.K, pr.NG, pr.HW, pr.B * pr.HW, 0, 0, 0}; }
 
 inline bool can_vec4(const Problem& pr, const void* a, const void* b, const void* c = nullptr) {
     return pr.K % 4 == 0 && (pr.HW == 1 || pr.HW % 4 == 0) && aligned16(a) && aligned16(b) && aligned16(c);
@@ -121,8 +196,9 @@ inline bool can_vec4(const Problem& pr, const void* a, const void* b, const void
 // problem.  KERNEL is a class template wrapping the __global__ function so that
 // one dispatcher serves all forward kernels.
 template <template <class, bool, int> class KERNEL, class GEO, class... Args>
-hipError_t launch_forward(const Problem& pr, bool vec4, hipStream_t stream, Args... args) {
+hipError_t launch_forward(const Problem& pr, bool vec4, bool ovec, hipStream_t stream, Args... args) {
     Dims d = make_dims(pr);
+    d.ovec = ovec;
     d.tiles_m = (d.M + GEO::BM - 1) / GEO::BM;
     d.tiles_n = (d.NG + GEO::BN - 1) / GEO::BN;
     const unsigned grid = (unsigned)d.tiles_m * d.tiles_n * d.G;
@@ -134,14 +210,14 @@ hipError_t launch_forward(const Problem& pr, bool vec4, hipStream_t stream, Args
 }
 
 template <template <class, bool, int> class KERNEL, class... Args>
-hipError_t dispatch_forward(const Problem& pr, bool vec4, hipStream_t stream, Args... args) {
+hipError_t dispatch_forward(const Problem& pr, bool vec4, bool ovec, hipStream_t stream, Args... args) {
     switch (choose_tile(pr.B * pr.HW, pr.NG, pr.G, pr.num_cu)) {
         case TileChoice::M128N80K2:
-            return launch_forward<KERNEL, Geo<128, 80, 8, 5, 2>>(pr, vec4, stream, args...);
+            return launch_forward<KERNEL, Geo<128, 80, 8, 5, 2>>(pr, vec4, ovec, stream, args...);
         case TileChoice::M256N32K1:
-            return launch_forward<KERNEL, Geo<256, 32, 8, 4, 1>>(pr, vec4, stream, args...);
+            return launch_forward<KERNEL, Geo<256, 32, 8, 4, 1>>(pr, vec4, ovec, stream, args...);
         default:
-            return launch_forward<KERNEL, Geo<128, 64, 8, 4, 1>>(pr, vec4, stream, args...);
+            return launch_forward<KERNEL, Geo<128, 64, 8, 4, 1>>(pr, vec4, ovec, stream, args...);
     }
 }
 

@@ -146,29 +146,32 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
         }
     }
 
-    // Locate the argmax inside the recorded chunk and write both outputs.
+    // Locate the argmax inside the recorded chunk, then write both outputs.
+    int ppos[TM][TN];
+    unsigned rows = 0;
 #pragma unroll
     for (int i = 0; i < TM; i++) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) ppos[i][j] = 0;
         if (KS == 2 && (i / TMH) != grp) continue;
+        rows |= 1u << i;
         const int m = m0 + GEO::row(ty, i);
         if (m >= d.M) continue;
         const RowAddr<CONV> ra(d, m, g);
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const int n = n0 + GEO::col(tx, j);
-            if (n >= d.NG) continue;
             const float best = acc[i][j];
-            int p = 0;
-            if (best > 0.f) {
+            if (n < d.NG && best > 0.f) {
                 const int kb = cidx[i][j] * kChunk;
                 const float* xr = input + ra.x + (size_t)kb * ra.xk;
                 const float* wr = weight + ((size_t)g * d.NG + n) * K + kb;
-                p = locate_in_chunk<(!CONV && VEC == 4)>(xr, ra.xk, wr, min(kChunk, K - kb), best, kb);
+                ppos[i][j] = locate_in_chunk<(!CONV && VEC == 4)>(xr, ra.xk, wr, min(kChunk, K - kb), best, kb);
             }
-            output[ra.o + (size_t)n * ra.on] = best;
-            pos[ra.o + (size_t)n * ra.on] = p;
         }
     }
+    store_patch<GEO, CONV>(output, acc, d, m0, n0, g, tx, ty, rows, d.ovec != 0);
+    store_patch<GEO, CONV>(pos, ppos, d, m0, n0, g, tx, ty, rows, d.ovec != 0);
 }
 
 template <class GEO, bool CONV, int VEC>
@@ -272,7 +275,8 @@ hipError_t inf_forward(const float* input, const float* weight, float* output, i
                            output, pos, d);
         return hipGetLastError();
     }
-    return dispatch_forward<InfForward>(pr, can_vec4(pr, input, weight), stream, input, weight, output, pos);
+    return dispatch_forward<InfForward>(pr, can_vec4(pr, input, weight), can_vec4_out(pr, output, pos), stream, input,
+                                        weight, output, pos);
 }
 
 }  // namespace ldist

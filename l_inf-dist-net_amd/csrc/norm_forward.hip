@@ -133,17 +133,10 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
 
     const float inv_p = 1.0f / p;
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
-        const int m = m0 + GEO::row(ty, i);
-        if (m >= d.M) continue;
-        const RowAddr<CONV> ra(d, m, g);
+    for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const int n = n0 + GEO::col(tx, j);
-            if (n >= d.NG) continue;
-            output[ra.o + (size_t)n * ra.on] = pow_pos(acc[i][j], inv_p) * mx[i][j];
-        }
-    }
+        for (int j = 0; j < TN; j++) acc[i][j] = pow_pos(acc[i][j], inv_p) * mx[i][j];
+    store_patch<GEO, CONV>(output, acc, d, m0, n0, g, tx, ty, 0xFFu, d.ovec != 0);
 }
 
 template <class GEO, bool CONV, int VEC>
@@ -160,7 +153,8 @@ struct NormForward {
 
 hipError_t norm_forward(const float* input, const float* weight, float* output, float p, const Problem& pr,
                         hipStream_t stream) {
-    return dispatch_forward<NormForward>(pr, can_vec4(pr, input, weight), stream, input, weight, output, p);
+    return dispatch_forward<NormForward>(pr, can_vec4(pr, input, weight), can_vec4_out(pr, output), stream, input,
+                                         weight, output, p);
 }
 
 }  // namespace ldist

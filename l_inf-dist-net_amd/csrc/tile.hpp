@@ -27,6 +27,7 @@ struct Dims {
     int B, G, K, NG, HW;  // K = CI/G, NG = CO/G
     int M;                // B*HW rows
     int tiles_m, tiles_n;
+    int ovec;             // outputs may be written with 128-bit stores
 };
 
 // XOR applied to the m (or n) coordinate of LDS row kk.  It permutes aligned

@@ -1,0 +1,64 @@
+"""The C-ABI library loads on a machine without a GPU, exports every symbol that
+include/ldist.h declares, and rejects bad arguments before touching a device."""
+import ctypes
+import os
+import re
+
+import pytest
+
+import __graft_entry__ as entry
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    pkg = entry.load_package()
+    if not os.path.exists(pkg.LIB_PATH):
+        pkg.build_library()
+    return pkg._lib.lib()
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "ldist.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ldist_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_seven_reference_entry_points():
+    names = declared_symbols()
+    for ref in ("norm_dist_forward", "norm_dist_backward_input", "norm_dist_backward_weight", "inf_dist_forward",
+                "inf_dist_bound_forward", "inf_dist_backward_input", "inf_dist_backward_weight"):
+        assert "ldist_" + ref in names  # reference model/norm_dist.cpp:92-100
+
+
+def test_every_declared_symbol_is_exported(lib):
+    for name in declared_symbols():
+        assert hasattr(lib, name), name
+
+
+def test_binding_signatures_cover_all_compute_entry_points():
+    pkg = entry.load_package()
+    compute = [n for n in declared_symbols() if "_dist_" in n]
+    assert sorted(pkg._lib.SIGNATURES) == sorted(compute)
+
+
+def test_version_and_error_strings(lib):
+    assert lib.ldist_version() == 100
+    for code in (0, -1, -2, -3, -4, -99):
+        assert isinstance(lib.ldist_strerror(code), bytes) and lib.ldist_strerror(code)
+    assert lib.ldist_set_tile_override(7) == -1 and lib.ldist_set_tile_override(-1) == 0
+
+
+def test_argument_checks_need_no_device(lib):
+    one = ctypes.c_void_p(16)  # never dereferenced: the size checks fail first
+    assert lib.ldist_inf_dist_forward(None, one, 1, 1, 1, 1, 1, one, one, None) == -1
+    assert lib.ldist_inf_dist_forward(one, one, 0, 1, 1, 1, 1, one, one, None) == -1
+    assert lib.ldist_inf_dist_forward(one, one, 2, 4, 6, 4, 1, one, one, None) == -1      # CI % G
+    assert lib.ldist_inf_dist_forward(one, one, 2, 6, 4, 4, 1, one, one, None) == -1      # CO % G
+    assert lib.ldist_inf_dist_forward(one, one, 1 << 20, 1 << 12, 8, 1, 1, one, one, None) == -2  # 2^32 outputs
+    assert lib.ldist_norm_dist_forward(one, one, 1, 1, 1, 1, 1, one, 1.0, None) == -1     # p must exceed 1
+    assert lib.ldist_norm_dist_forward(one, one, 1, 1, 1, 1, 1, one, float("inf"), None) == -1
+    assert lib.ldist_norm_dist_backward_weight(one, one, one, one, 1, 1, 1, 1, 1, None, 8.0, None) == -1
+    assert lib.ldist_inf_dist_bound_forward(one, None, one, 1, 1, 1, 1, 1, one, one, None) == -1
+    assert lib.ldist_inf_dist_backward_input_overwrite(one, one, 1, 1, 1, 1, 0, one, None) == -1

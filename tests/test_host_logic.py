@@ -1,0 +1,239 @@
+"""Host-side behaviour of the Python layer (no GPU): dispatch, autograd contract, module semantics.
+
+The native calls are replaced by fakes that run the CPU oracle on CPU tensors, so
+what is tested here is the wrapper logic written from the reference's
+model/norm_dist.py, model/mlp.py and model/bound_module.py -- not the kernels.
+"""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import __graft_entry__ as entry
+import oracle
+from helpers import gen
+
+pkg = entry.load_package()
+import l_inf_dist_net_amd.norm_dist_cpp as cpp  # noqa: E402  (module registered by load_package())
+
+
+@pytest.fixture()
+def fake_native(monkeypatch):
+    calls = []
+
+    def inf_dist_forward(x, w, out, pos, G):
+        calls.append("inf_dist_forward")
+        o, p = oracle.inf_dist_forward(x.contiguous(), w.contiguous(), G)
+        out.copy_(o); pos.copy_(p)
+
+    def inf_dist_bound_forward(lo, up, w, ol, ou, G):
+        calls.append("inf_dist_bound_forward")
+        a, b = oracle.inf_dist_bound_forward(lo.contiguous(), up.contiguous(), w.contiguous(), G)
+        ol.copy_(a); ou.copy_(b)
+
+    def bwd_in_over(go, pos, gi, G):
+        calls.append("inf_dist_backward_input_overwrite")
+        gi.copy_(oracle.inf_dist_backward_input(go, pos, gi.size(1), G))
+
+    def bwd_w_over(go, pos, gw, G):
+        calls.append("inf_dist_backward_weight_overwrite")
+        gw.copy_(oracle.inf_dist_backward_weight(go, pos, gw.size(1) * G, G))
+
+    def norm_dist_forward(x, w, out, G, p):
+        calls.append("norm_dist_forward")
+        out.copy_(oracle.norm_dist_forward(x.contiguous(), w.contiguous(), G, p))
+
+    def norm_bwd_in(go, x, w, out, gi, G, p):
+        calls.append("norm_dist_backward_input")
+        gi.copy_(oracle.norm_dist_backward_input(go, x.contiguous(), w.contiguous(), out.contiguous(), G, p))
+
+    def norm_bwd_w(go, x, w, out, gw, G, p):
+        calls.append("norm_dist_backward_weight")
+        assert torch.count_nonzero(gw) == 0  # the wrapper must hand over a zero-filled buffer
+        oracle.norm_dist_backward_weight(go, x.contiguous(), w.contiguous(), out.contiguous(), G, p, grad_weight=gw)
+
+    for name, fn in [("inf_dist_forward", inf_dist_forward), ("inf_dist_bound_forward", inf_dist_bound_forward),
+                     ("inf_dist_backward_input_overwrite", bwd_in_over),
+                     ("inf_dist_backward_weight_overwrite", bwd_w_over), ("norm_dist_forward", norm_dist_forward),
+                     ("norm_dist_backward_input", norm_bwd_in), ("norm_dist_backward_weight", norm_bwd_w)]:
+        monkeypatch.setattr(cpp, name, fn)
+    return calls
+
+
+def test_binding_rejects_cpu_and_wrong_dtype_tensors():
+    x, w = torch.zeros(2, 4, 1), torch.zeros(3, 4)
+    out, pos = torch.zeros(2, 3, 1), torch.zeros(2, 3, 1, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):   # reference CHECK_CUDA, norm_dist.cpp:3
+        cpp.inf_dist_forward(x, w, out, pos, 1)
+    with pytest.raises(RuntimeError):
+        cpp.norm_dist_forward(x, w, out, 1, 8.0)
+
+
+def test_distf_dispatch_and_errors(fake_native):
+    x = torch.rand(3, 6, 2, generator=gen(0))
+    w = torch.rand(4, 3, generator=gen(1))
+    y = pkg.norm_dist(x, w, 2, float("inf"))
+    assert fake_native == ["inf_dist_forward"] and y.shape == (3, 4, 2)
+    fake_native.clear()
+    pkg.norm_dist(x, w, 2, 8.0)
+    assert fake_native == ["norm_dist_forward"]
+    with pytest.raises(NotImplementedError):       # model/norm_dist.py:21-22
+        pkg.norm_dist(x, w, 2, 1.0)
+    with pytest.raises(AssertionError):            # model/norm_dist.py:12
+        pkg.norm_dist(x, w, 3, 8.0)
+
+
+@pytest.mark.parametrize("p", [float("inf"), 8.0])
+def test_distf_backward_respects_needs_input_grad(fake_native, p):
+    x = torch.rand(3, 6, 2, generator=gen(2))
+    w = torch.rand(4, 3, generator=gen(3))
+    go = torch.randn(3, 4, 2, generator=gen(4))
+    for rx, rw in ((True, True), (True, False), (False, True)):
+        fake_native.clear()
+        xx, ww = x.clone().requires_grad_(rx), w.clone().requires_grad_(rw)
+        y = pkg.norm_dist(xx, ww, 2, p)
+        y.backward(go.transpose(0, 1).contiguous().transpose(0, 1))  # a non-contiguous upstream gradient
+        kinds = [c for c in fake_native if "backward" in c]
+        assert any("input" in c for c in kinds) == rx and any("weight" in c for c in kinds) == rw
+        assert (xx.grad is not None) == rx and (ww.grad is not None) == rw
+
+
+def test_gradients_agree_with_the_dense_torch_formula(fake_native):
+    # the reference's own cross-check: use_custom_cuda_func=False (model/norm_dist.py:52-57)
+    x = torch.rand(4, 6, 3, generator=gen(5))
+    w = torch.rand(4, 3, generator=gen(6))
+    go = torch.randn(4, 4, 3, generator=gen(7))
+    for p in (float("inf"), 6.0):
+        a = [t.clone().requires_grad_(True) for t in (x, w)]
+        b = [t.clone().requires_grad_(True) for t in (x, w)]
+        ya = pkg.norm_dist(a[0], a[1], 2, p)
+        yb = pkg.norm_dist(b[0], b[1], 2, p, use_custom_cuda_func=False)
+        torch.testing.assert_close(ya, yb, rtol=1e-5, atol=1e-6)
+        ya.backward(go); yb.backward(go)
+        torch.testing.assert_close(a[0].grad, b[0].grad, rtol=1e-4, atol=1e-5)
+        torch.testing.assert_close(a[1].grad, b[1].grad, rtol=1e-4, atol=1e-5)
+
+
+def test_inf_dist_bound_matches_its_dense_formula(fake_native):
+    x = torch.rand(4, 6, 3, generator=gen(8))
+    w = torch.rand(4, 3, generator=gen(9))
+    lo, up = (x - 0.1).contiguous(), (x + 0.1).contiguous()
+    a = pkg.inf_dist_bound(lo, up, w, 2)
+    b = pkg.inf_dist_bound(lo, up, w, 2, use_custom_cuda_func=False)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    assert not a[0].requires_grad
+
+
+def test_mean_norm_train_and_eval():
+    mn = pkg.MeanNorm(3, momentum=0.1)
+    x = torch.randn(5, 3, 4, 4, generator=gen(10))
+    mn.train()
+    y = mn(x)
+    mean = x.mean(dim=(0, 2, 3))
+    torch.testing.assert_close(y, x - mean.view(1, 3, 1, 1))
+    torch.testing.assert_close(mn.running_mean, 0.1 * mean)          # (1-m)*0 + m*mean, norm_dist.py:92-93
+    mn.eval()
+    torch.testing.assert_close(mn(x), x - mn.running_mean.view(1, 3, 1, 1))
+    x2 = torch.randn(6, 3, generator=gen(11))                        # 2-D input path (norm_dist.py:90-91)
+    mn.train()
+    torch.testing.assert_close(mn(x2), x2 - x2.mean(dim=0))
+    xg = x.clone().requires_grad_(True)                              # the batch mean carries gradient
+    pkg.MeanNorm(3).train()(xg).sum().backward()
+    torch.testing.assert_close(xg.grad, torch.zeros_like(x), atol=1e-6, rtol=0)
+
+
+def naive_dist_conv(x, weight, stride, padding, group, p):
+    """Direct loops over output positions: the definition the unfold-based layer must reproduce."""
+    B, C, H, W = x.shape
+    CO, CG, k, _ = weight.shape
+    xp = F.pad(x, (padding,) * 4)
+    oh, ow = (H + 2 * padding - k) // stride + 1, (W + 2 * padding - k) // stride + 1
+    out = torch.zeros(B, CO, oh, ow)
+    ng = CO // group
+    for co in range(CO):
+        g = co // ng
+        for i in range(oh):
+            for j in range(ow):
+                patch = xp[:, g * CG:(g + 1) * CG, i * stride:i * stride + k, j * stride:j * stride + k]
+                d = (patch - weight[co]).abs().reshape(B, -1)
+                out[:, co, i, j] = d.max(dim=1)[0] if math.isinf(p) else (d.double() ** p).sum(1) ** (1 / p)
+    return out
+
+
+@pytest.mark.parametrize("p", [float("inf"), 4.0])
+def test_conv_layer_matches_naive_loops(fake_native, p):
+    torch.manual_seed(0)
+    layer = pkg.NormDistConv(4, 6, 3, stride=2, padding=1, group=2, p=p, bias=True, mean_normalize=False)
+    with torch.no_grad():
+        layer.bias.copy_(torch.arange(6.0))
+    x = torch.rand(2, 4, 5, 5, generator=gen(12))
+    y, lo, up = layer(x)
+    assert lo is None and up is None
+    ref = naive_dist_conv(x, layer.weight.detach(), 2, 1, 2, p) + torch.arange(6.0).view(1, 6, 1, 1)
+    torch.testing.assert_close(y, ref.float(), rtol=1e-5, atol=1e-6)
+
+
+def test_fc_layer_is_a_1x1_conv_and_bounds_need_eval_and_inf(fake_native):
+    torch.manual_seed(1)
+    fc = pkg.NormDist(6, 5, p=float("inf"), bias=True, mean_normalize=True)
+    x = torch.rand(4, 6, generator=gen(13))
+    fc.eval()
+    fc.normalize.running_mean.copy_(torch.linspace(-1, 1, 5))
+    y, lo, up = fc(x, x - 0.05, x + 0.05)
+    ev, _ = oracle.inf_dist_forward(x.reshape(4, 6, 1), fc.weight.detach().reshape(5, 6), 1)
+    torch.testing.assert_close(y, ev.reshape(4, 5) - fc.normalize.running_mean + fc.bias)
+    assert bool((lo <= y + 1e-6).all()) and bool((y <= up + 1e-6).all())
+    el, eu = oracle.inf_dist_bound_forward((x - 0.05).reshape(4, 6, 1), (x + 0.05).reshape(4, 6, 1),
+                                           fc.weight.detach().reshape(5, 6), 1)
+    torch.testing.assert_close(lo, el.reshape(4, 5) - fc.normalize.running_mean + fc.bias)   # same shift on the bounds
+    torch.testing.assert_close(up, eu.reshape(4, 5) - fc.normalize.running_mean + fc.bias)
+    fc.train()
+    with pytest.raises(AssertionError):            # model/norm_dist.py:143
+        fc(x, x - 0.05, x + 0.05)
+    fc.eval(); fc.p = 8.0
+    with pytest.raises(AssertionError):
+        fc(x, x - 0.05, x + 0.05)
+
+
+def test_constructor_state_dict_and_p_setters():
+    torch.manual_seed(2)
+    conv = pkg.NormDistConv(4, 8, 3, group=2, bias=True, mean_normalize=True)
+    assert sorted(conv.state_dict()) == ["bias", "normalize.running_mean", "weight"]
+    assert conv.weight.shape == (8, 2, 3, 3) and conv.p == 0
+    for i in range(8):                              # identity init, model/norm_dist.py:118-120
+        assert conv.weight[i, i % 2, 1, 1].item() == -10.0
+    wide = pkg.NormDistConv(8, 4, 1)                # in > out: no identity init
+    assert not bool((wide.weight == -10.0).any())
+    model = torch.nn.Sequential(pkg.NormDist(4, 4), torch.nn.ReLU(), pkg.NormDistConv(4, 4, 1))
+    assert pkg.get_p_norm(model) == 0
+    pkg.set_p_norm(model, 8.0)
+    assert all(m.p == 8.0 for m in model if hasattr(m, "p")) and pkg.get_p_norm(model) == 8.0
+    assert pkg.get_p_norm(torch.nn.Linear(2, 2)) is None
+    t0 = pkg.NormDistConv.tag
+    assert pkg.NormDist(2, 2).tag == t0 + 1
+    # keyword spellings used by the benchmark description
+    alias = pkg.NormDistConv(4, 8, 1, groups=2, mean_shift=True)
+    assert alias.group == 2 and alias.normalize is not None
+    assert pkg.MeanNormDist(4, 8).normalize is not None and pkg.MeanNormDist(4, 8).bias is None
+    assert "in_features=4" in repr(pkg.NormDist(4, 8))
+
+
+def test_mlp_triple_and_certified_margin(fake_native):
+    torch.manual_seed(3)
+    net = pkg.MLP(depth=3, width=1, input_dim=(3, 2, 2), num_classes=4)
+    assert net.fc[0].out_channels == 1024            # width * 1024 hidden units, model/mlp.py:5
+    pkg.set_p_norm(net, float("inf"))
+    net.eval()
+    x = torch.rand(5, 3, 2, 2, generator=gen(14))
+    y, lo, up = net(x, x - 0.01, x + 0.01)
+    assert y.shape == (5, 4) and bool((lo <= y + 1e-6).all()) and bool((y <= up + 1e-6).all())
+    y_only = net(x)
+    assert y_only[1] is None and y_only[2] is None and torch.equal(y_only[0], y)
+    targets = torch.tensor([0, 1, 2, 3, 0])
+    out, res = pkg.BoundFinalIdentity()(y, lo, up, targets)
+    for b in range(5):
+        for j in range(4):
+            expect = 0.0 if j == targets[b] else (up[b, j] - lo[b, targets[b]]).item()
+            assert res[b, j].item() == pytest.approx(expect)
+    assert pkg.BoundFinalIdentity()(y) is y
