@@ -51,6 +51,10 @@ int ldist_last_hip_error(void);
  * tiling of the three forward kernels.  -1 = choose by shape (default), 0 = 128x80
  * tile with two k-groups, 1 = 128x64, 2 = 256x32.  Process-wide; not thread safe. */
 int ldist_set_tile_override(int choice);
+/* Tuning knob, no counterpart in the reference: 1 (default) orders the tiles of
+ * the forward kernels so that each of the 8 XCDs works on one contiguous run of
+ * tiles, 0 keeps the plain order.  Results do not depend on it. */
+int ldist_set_xcd_remap(int on);
 
 /* L_inf forward.  Replaces inf_dist_forward_cuda (model/norm_dist.cpp:13-14,
  * model/inf_dist_cuda.cu:173-180).

@@ -186,7 +186,7 @@ inline bool can_vec4_out(const Problem& pr, const void* a, const void* b = nullp
     return aligned16(a) && aligned16(b) && (pr.HW == 1 ? pr.NG % 4 == 0 : pr.HW % 4 == 0);
 }
 
-inline Dims make_dims(const Problem& pr) { return Dims{pr.B, pr.G, pr.K, pr.NG, pr.HW, pr.B * pr.HW, 0, 0, 0}; }
+inline Dims make_dims(const Problem& pr) { return Dims{pr.B, pr.G, pr.K, pr.NG, pr.HW, pr.B * pr.HW, 0, 0, 0, g_xcd_remap}; }
 
 inline bool can_vec4(const Problem& pr, const void* a, const void* b, const void* c = nullptr) {
     return pr.K % 4 == 0 && (pr.HW == 1 || pr.HW % 4 == 0) && aligned16(a) && aligned16(b) && aligned16(c);

@@ -21,6 +21,7 @@ enum class TileChoice { M128N80K2, M128N64K1, M256N32K1 };
 // M256N32K1 serves grouped layers with few outputs per group.
 // -1 = choose by shape; 0, 1, 2 force M128N80K2, M128N64K1, M256N32K1 (tests and tuning).
 extern int g_tile_override;
+extern int g_xcd_remap;  // 1 (default): XCD-aware tile order; 0: plain order (tuning)
 
 inline TileChoice choose_tile(int M, int NG, int G, int num_cu) {
     if (g_tile_override >= 0 && g_tile_override <= 2) return static_cast<TileChoice>(g_tile_override);

@@ -10,6 +10,7 @@
 
 namespace ldist {
 int g_tile_override = -1;
+int g_xcd_remap = 1;
 }
 
 namespace {
@@ -80,6 +81,11 @@ const char* ldist_strerror(int code) {
 }
 
 int ldist_last_hip_error(void) { return g_last_hip_error; }
+
+int ldist_set_xcd_remap(int on) {
+    ldist::g_xcd_remap = on ? 1 : 0;
+    return LDIST_OK;
+}
 
 int ldist_set_tile_override(int choice) {
     if (choice < -1 || choice > 2) return LDIST_EINVAL;

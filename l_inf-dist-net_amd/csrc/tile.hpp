@@ -28,6 +28,7 @@ struct Dims {
     int M;                // B*HW rows
     int tiles_m, tiles_n;
     int ovec;             // outputs may be written with 128-bit stores
+    int xcd_remap;        // 1: hand each XCD a contiguous run of tiles
 };
 
 // XOR applied to the m (or n) coordinate of LDS row kk.  It permutes aligned
@@ -265,7 +266,7 @@ __device__ __forceinline__ void tile_of_block(const Dims& d, int& tm, int& tn, i
     const int total = gridDim.x;
     int id = blockIdx.x;
     constexpr int XCD = 8;
-    if (total % XCD == 0) id = (id % XCD) * (total / XCD) + id / XCD;
+    if (d.xcd_remap && total % XCD == 0) id = (id % XCD) * (total / XCD) + id / XCD;
     tm = id % d.tiles_m;
     const int r = id / d.tiles_m;
     tn = r % d.tiles_n;
