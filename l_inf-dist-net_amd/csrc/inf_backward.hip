@@ -66,8 +66,8 @@ inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* 
 }
 
 // ---- grad_weight -----------------------------------------------------------
-// Workgroup = (group g, NB consecutive outputs n, KC consecutive k, a slice of
-// the images b).  For one image the NB rows of grad_output/pos are one
+// Workgroup = (group g, NB consecutive outputs n, KC consecutive k -- all of K when
+// a row of bins fits in 64 KB -- and a slice of the images b).  For one image the NB rows of grad_output/pos are one
 // contiguous run of NB*HW elements.  bins[nb][kc].
 // When the images are split over several workgroups (SPLIT) the bins are added
 // to grad_weight with global atomics, otherwise the workgroup is the only
@@ -85,7 +85,14 @@ inf_backward_weight_kernel(const float* __restrict__ grad_output, const int32_t*
     const int kc = min(KC, d.K - k0);
     const int b0 = blockIdx.z * b_per_wg;
     const int b1 = min(d.B, b0 + b_per_wg);
-    for (int e = threadIdx.x; e < nb * kc; e += 256) bins[e] = 0.f;
+    // kc is a multiple of 4 whenever vec is set, so rows of bins and of grad_weight stay 16-byte aligned
+    const bool vec = (kc & 3) == 0 && (d.K & 3) == 0 && (reinterpret_cast<uintptr_t>(grad_weight) & 15u) == 0;
+    if (vec) {
+        float4* b4 = reinterpret_cast<float4*>(bins);
+        for (int e = threadIdx.x; e < nb * kc / 4; e += 256) b4[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+    } else {
+        for (int e = threadIdx.x; e < nb * kc; e += 256) bins[e] = 0.f;
+    }
     __syncthreads();
 
     const int run = nb * d.HW;  // contiguous elements per image
@@ -120,6 +127,16 @@ inf_backward_weight_kernel(const float* __restrict__ grad_output, const int32_t*
     }
     __syncthreads();
 
+    if (vec && OVERWRITE && !SPLIT) {
+        const int kc4 = kc / 4;
+        const float4* b4 = reinterpret_cast<const float4*>(bins);
+        for (int e = threadIdx.x; e < nb * kc4; e += 256) {
+            const int nn = e / kc4, k4 = e - nn * kc4;
+            float* dst = grad_weight + ((size_t)g * d.NG + n0 + nn) * d.K + k0 + k4 * 4;
+            *reinterpret_cast<float4*>(dst) = b4[e];
+        }
+        return;
+    }
     for (int e = threadIdx.x; e < nb * kc; e += 256) {
         const int nn = e / kc, k = e - nn * kc;
         float* dst = grad_weight + ((size_t)g * d.NG + n0 + nn) * d.K + k0 + k;
@@ -170,8 +187,10 @@ hipError_t inf_backward_input(const float* grad_output, const int32_t* pos, floa
 hipError_t inf_backward_weight(const float* grad_output, const int32_t* pos, float* grad_weight, const Problem& pr,
                                bool overwrite, hipStream_t stream) {
     const BwdDims d{pr.B, pr.G, pr.K, pr.NG, pr.HW};
-    const int NB = min(pr.NG, 8);
-    const int KC = min(pr.K, kBinFloats / NB);
+    // One pass over all K channels per workgroup when a row of bins fits: re-reading the strided
+    // grad_output/pos columns for every channel range costs more than the smaller row block.
+    const int KC = min(pr.K, kBinFloats);
+    const int NB = max(1, min(min(pr.NG, 8), kBinFloats / KC));
     const int n_blocks = (pr.NG + NB - 1) / NB;
     const int k_ranges = (pr.K + KC - 1) / KC;
     const long slabs = (long)pr.G * n_blocks * k_ranges;
