@@ -1,16 +1,19 @@
 #!/usr/bin/env python3
 """Benchmark of the distance-neuron hot path on one MI355X.
 
-Workload (BASELINE.json configs[1]): the CIFAR-10-shaped 5-layer L_inf-dist MLP
-3072 -> 5120 -> 5120 -> 5120 -> 5120 -> 10 at p = inf, batch 512, fp32, forward
-plus backward (grad_x of every layer and every grad_w).  A "step" is one
-forward+backward pass over one synthetic batch that already sits in HBM.
+Default workload (BASELINE.json configs[1], the one the metric is quoted on): the
+CIFAR-10-shaped 5-layer L_inf-dist MLP 3072 -> 5120 -> 5120 -> 5120 -> 5120 -> 10 at
+p = inf, batch 512, fp32, forward plus backward (grad_x of every layer and every
+grad_w).  A "step" is one pass of the hot path over one synthetic batch that already
+sits in HBM.  `--workload c0|c2|c3|c4` runs the other BASELINE.json configurations
+with the same output format (they are parity-test cases; the driver's line is c1).
 
-Prints ONE JSON line.  `value` is G dist-ops/s, a dist-op being one (row, output,
-input) triple of a forward pass (48.35 G per step).  `roofline` is measured live
-on the dominant kernel (the tiled L_inf forward) with events on the stream the
-kernels run on; `cpu_baseline` times the CPU oracle on a bounded row sample of
-the same workload.
+Prints ONE JSON line.  `value` is G dist-ops/s; a dist-op is one (row, output,
+input) triple of one pass (forward, grad-input or grad-weight for the p-norm paths;
+the forward only at p = inf, whose backward is a byte-bound scatter).  `roofline`
+is measured live on the workload's dominant kernel with events on the stream the
+kernels run on; `cpu_baseline` times the CPU oracle on a bounded row sample of the
+same workload.
 """
 import argparse
 import json
@@ -24,64 +27,63 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 LAYERS = [3072, 5120, 5120, 5120, 5120, 10]
-BATCH = 512
 CIFAR_MEAN = (0.4914, 0.4822, 0.4465)
 CIFAR_STD = 0.2009
-FP32_PEAK_TFLOPS = 157.3          # MI355X vector fp32 (packed FMA) peak
-VALU_ISSUE_PEAK_T = 39.3          # 256 CU x 64 lanes x 2.4 GHz lane-instructions per second
-FLOPS_PER_DIST_OP = 2             # sub, max; abs/compare/index bookkeeping count as zero
+EPS = 8 / 255
+FP32_PEAK_TFLOPS = 157.3          # MI355X vector fp32 peak (counts packed FMA)
+INF = float("inf")
 
 
-def dist_ops_per_forward(batch):
+def stack_ops(batch):
     return sum(batch * a * b for a, b in zip(LAYERS[:-1], LAYERS[1:]))
 
 
-def make_inputs(batch, seed=0):
+def normalise(x):
     import torch
-    g = torch.Generator().manual_seed(seed)
-    x = torch.rand(batch, 3, 32, 32, generator=g)
     mean = torch.tensor(CIFAR_MEAN).view(1, 3, 1, 1)
-    x = ((x - mean) / CIFAR_STD).reshape(batch, -1).contiguous()
-    ws = [torch.randn(o, i, generator=g) / math.sqrt(i) for i, o in zip(LAYERS[:-1], LAYERS[1:])]
-    upstream = torch.randn(batch, LAYERS[-1], generator=g)
-    return x, ws, upstream
+    return ((x - mean) / CIFAR_STD).reshape(x.size(0), -1).contiguous()
 
 
-def build_model(pkg, ws, dev):
+def stack_weights(g):
+    import torch
+    return [torch.randn(o, i, generator=g) / math.sqrt(i) for i, o in zip(LAYERS[:-1], LAYERS[1:])]
+
+
+def build_mlp(pkg, ws, dev, p, train):
     import torch
     model = pkg.MLP(depth=5, width=5, input_dim=3072, num_classes=10, head_mean_normalize=True)
     with torch.no_grad():
         for layer, w in zip(list(model.fc) + [model.fc_last], ws):
             layer.weight.copy_(w.view_as(layer.weight))
-    pkg.set_p_norm(model, float("inf"))
-    return model.to(dev).train()
+    pkg.set_p_norm(model, p)
+    model = model.to(dev)
+    return model.train() if train else model.eval()
 
 
 class KernelTimer:
-    """Brackets every tiled L_inf forward launch with events on the current stream."""
+    """Brackets every launch of one binding function with events on the current stream."""
 
-    def __init__(self, cpp, torch):
-        self.cpp, self.torch = cpp, torch
-        self.orig = cpp.inf_dist_forward
+    def __init__(self, cpp, torch, name, flops_of, accept):
+        self.cpp, self.torch, self.name, self.flops_of, self.accept = cpp, torch, name, flops_of, accept
+        self.orig = getattr(cpp, name)
         self.records = []
         self.enabled = False
 
     def __enter__(self):
-        def timed(input, weight, output, pos, G):
-            if not self.enabled or weight.size(0) // G <= 16:   # the 10-way head runs a different kernel
-                return self.orig(input, weight, output, pos, G)
+        def timed(*args):
+            if not self.enabled or not self.accept(*args):
+                return self.orig(*args)
             a = self.torch.cuda.Event(enable_timing=True)
             b = self.torch.cuda.Event(enable_timing=True)
             a.record()
-            self.orig(input, weight, output, pos, G)
+            self.orig(*args)
             b.record()
-            flops = FLOPS_PER_DIST_OP * input.size(0) * input.size(2) * weight.size(0) * weight.size(1)
-            self.records.append((a, b, flops))
-        self.cpp.inf_dist_forward = timed
+            self.records.append((a, b, self.flops_of(*args)))
+        setattr(self.cpp, self.name, timed)
         return self
 
     def __exit__(self, *exc):
-        self.cpp.inf_dist_forward = self.orig
+        setattr(self.cpp, self.name, self.orig)
 
     def summary(self):
         ms = sum(a.elapsed_time(b) for a, b, _ in self.records)
@@ -90,42 +92,183 @@ class KernelTimer:
         return n, ms / max(n, 1), flops / max(n, 1)
 
 
-def cpu_baseline(target_seconds=12.0):
-    """C1 forward+backward with the CPU oracle (C, OpenMP) on a row subset sized to ~target_seconds."""
-    import torch
-    import oracle
-    x, ws, upstream = make_inputs(BATCH)
+def mnk(x, w):
+    return x.size(0) * x.size(2) * w.size(0) * w.size(1)
 
-    def run(rows):
-        t0 = time.perf_counter()
+
+# --------------------------------------------------------------------------- #
+# Workloads.  Each gives: step(), dist-ops per step, images per step, a CPU     #
+# sample function, and the kernel to time for the roofline: (binding name,      #
+# flops per launch, launch filter, description, algorithmic flops per dist-op). #
+# --------------------------------------------------------------------------- #
+def workload_c0(pkg, torch, dev):
+    g = torch.Generator().manual_seed(0)
+    x = torch.rand(512, 784, generator=g).reshape(512, 784, 1).contiguous()
+    w = (torch.randn(5120, 784, generator=g) / math.sqrt(784)).contiguous()
+    xd, wd = x.to(dev), w.to(dev)
+    out = torch.empty(512, 5120, 1, device=dev)
+    pos = torch.empty(512, 5120, 1, device=dev, dtype=torch.int32)
+    cpp = pkg.norm_dist_cpp
+
+    def step():
+        cpp.inf_dist_forward(xd, wd, out, pos, 1)
+
+    def cpu(oracle, rows):
+        oracle.inf_dist_forward(x[:rows].contiguous(), w, 1)
+        return rows * 784 * 5120
+
+    return dict(step=step, ops=512 * 784 * 5120, images=512, full_rows=512, cpu=cpu,
+                name="configs[0]: single L_inf-dist fc layer forward, 512 x 784 -> 5120, values + argmax",
+                kernel=("inf_dist_forward", lambda x_, w_, *_: 2 * mnk(x_, w_), lambda *a: True,
+                        "inf_forward_kernel (tiled L_inf forward)", 2))
+
+
+def mlp_workload(pkg, torch, dev, p):
+    g = torch.Generator().manual_seed(0)
+    x = normalise(torch.rand(512, 3, 32, 32, generator=g))
+    ws = stack_weights(g)
+    upstream = torch.randn(512, 10, generator=g)
+    model = build_mlp(pkg, ws, dev, p, train=True)
+    xd = x.to(dev).requires_grad_(True)
+    up = upstream.to(dev)
+
+    def step():
+        xd.grad = None
+        for prm in model.parameters():
+            prm.grad = None
+        y, _, _ = model(xd)
+        y.backward(up)
+
+    def cpu(oracle, rows):
         h = x[:rows].reshape(rows, -1, 1).contiguous()
         saved = []
         for w in ws:
-            out, pos = oracle.inf_dist_forward(h, w, 1)
-            saved.append((h.size(1), pos))
+            if math.isinf(p):
+                out, pos = oracle.inf_dist_forward(h, w, 1)
+            else:
+                out, pos = oracle.norm_dist_forward(h, w, 1, p), None
+            saved.append((h, w, out, pos))
             h = (out - out.mean(dim=0, keepdim=True)).contiguous()
-        g = upstream[:rows].reshape(rows, -1, 1).contiguous()
-        for (ci, pos), w in zip(reversed(saved), reversed(ws)):
-            g = (g - g.mean(dim=0, keepdim=True)).contiguous()
-            oracle.inf_dist_backward_weight(g, pos, ci, 1)
-            g = oracle.inf_dist_backward_input(g, pos, ci, 1)
-        return time.perf_counter() - t0
+        gr = upstream[:rows].reshape(rows, -1, 1).contiguous()
+        for (hin, w, out, pos) in reversed(saved):
+            gr = (gr - gr.mean(dim=0, keepdim=True)).contiguous()
+            if math.isinf(p):
+                oracle.inf_dist_backward_weight(gr, pos, hin.size(1), 1)
+                gr = oracle.inf_dist_backward_input(gr, pos, hin.size(1), 1)
+            else:
+                oracle.norm_dist_backward_weight(gr, hin, w, out, 1, p)
+                gr = oracle.norm_dist_backward_input(gr, hin, w, out, 1, p)
+        return stack_ops(rows) * (1 if math.isinf(p) else 3)
 
-    probe_rows = 8
-    t = run(probe_rows)
-    rows = int(max(probe_rows, min(BATCH, probe_rows * target_seconds / max(t, 1e-3))))
-    t = run(rows)
-    reps = 1
-    while t < target_seconds and reps < 64:      # fast hosts: repeat the pass until the sample is long enough
-        t += run(rows)
+    return step, cpu
+
+
+def workload_c1(pkg, torch, dev):
+    step, cpu = mlp_workload(pkg, torch, dev, INF)
+    return dict(step=step, ops=stack_ops(512), images=512, full_rows=512, cpu=cpu,
+                name="configs[1]: 5-layer L_inf-dist MLP 3072-5120-5120-5120-5120-10, p=inf, batch 512, "
+                     "forward+backward (all grad_x and grad_w), mean shift in training mode",
+                kernel=("inf_dist_forward", lambda x_, w_, *_: 2 * mnk(x_, w_),
+                        lambda x_, w_, o_, p_, G: w_.size(0) // G > 16,   # the 10-way head runs another kernel
+                        "inf_forward_kernel (tiled L_inf forward)", 2))
+
+
+def workload_c2(pkg, torch, dev):
+    step, cpu = mlp_workload(pkg, torch, dev, 8.0)
+    return dict(step=step, ops=3 * stack_ops(512), images=512, full_rows=512, cpu=cpu,
+                name="configs[2]: the same MLP at p=8, forward+backward (3 dist-op passes per layer)",
+                kernel=("norm_dist_backward_input", lambda go, x_, w_, *_: 7 * mnk(x_, w_),
+                        lambda go, x_, w_, *_: w_.size(0) > 16, "norm_backward_kernel (grad_input)", 7))
+
+
+def workload_c3(pkg, torch, dev):
+    g = torch.Generator().manual_seed(0)
+    img = torch.rand(1024, 3, 32, 32, generator=g)
+    x, lo, up = normalise(img), normalise((img - EPS).clamp(0, 1)), normalise((img + EPS).clamp(0, 1))
+    ws = stack_weights(g)
+    means = [torch.randn(o, generator=g) * 0.1 for o in LAYERS[1:]]
+    model = build_mlp(pkg, ws, dev, INF, train=False)
+    with torch.no_grad():
+        for layer, m in zip(list(model.fc) + [model.fc_last], means):
+            layer.normalize.running_mean.copy_(m)
+    targets = torch.randint(0, 10, (1024,), generator=g).to(dev)
+    final = pkg.BoundFinalIdentity()
+    xd, lod, upd = x.to(dev), lo.to(dev), up.to(dev)
+
+    def step():
+        with torch.no_grad():
+            y, l, u = model(xd, lod, upd)
+            return final(y, l, u, targets)
+
+    def cpu(oracle, rows):
+        h, l, u = (t[:rows].reshape(rows, -1, 1).contiguous() for t in (x, lo, up))
+        for w, m in zip(ws, means):
+            out, _ = oracle.inf_dist_forward(h, w, 1)
+            ol, ou = oracle.inf_dist_bound_forward(l, u, w, 1)
+            h, l, u = ((t - m.view(1, -1, 1)).contiguous() for t in (out, ol, ou))
+        return 2 * stack_ops(rows)
+
+    return dict(step=step, ops=2 * stack_ops(1024), images=1024, full_rows=1024, cpu=cpu,
+                name="configs[3]: interval-bound certification forward through the MLP, batch 1024, eps=8/255: "
+                     "value path + lower/upper bounds + certified margins (bound-ops and dist-ops both counted)",
+                kernel=("inf_dist_bound_forward", lambda l_, u_, w_, *_: 6 * mnk(l_, w_),
+                        lambda l_, u_, w_, *_: True, "bound_forward_kernel", 6))
+
+
+def workload_c4(pkg, torch, dev):
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(0)
+    img = torch.rand(128, 128, 32, 32, generator=g)
+    w = (torch.randn(128, 32, 3, 3, generator=g) / math.sqrt(288)).reshape(128, 288).contiguous()
+    go = torch.randn(128, 128, 1024, generator=g)
+    cols = F.unfold(img, 3, padding=1).contiguous()        # (128, 1152, 1024), outside the timed region
+    xd = cols.to(dev).requires_grad_(True)
+    wd = w.to(dev).requires_grad_(True)
+    god = go.to(dev)
+
+    def step():
+        xd.grad = None
+        wd.grad = None
+        y = pkg.norm_dist(xd, wd, 4, INF)
+        y.backward(god)
+
+    def cpu(oracle, rows):
+        xs, gs = cols[:rows].contiguous(), go[:rows].contiguous()
+        _, pos = oracle.inf_dist_forward(xs, w, 4)
+        oracle.inf_dist_backward_input(gs, pos, 1152, 4)
+        oracle.inf_dist_backward_weight(gs, pos, 1152, 4)
+        return rows * 1024 * 128 * 288
+
+    return dict(step=step, ops=128 * 1024 * 128 * 288, images=128, full_rows=128, cpu=cpu,
+                name="configs[4]: unfolded 3x3 L_inf-dist conv layer, batch 128, 128->128 channels, 32x32, groups 4, "
+                     "forward+backward (unfold outside the timed region)",
+                kernel=("inf_dist_forward", lambda x_, w_, *_: 2 * mnk(x_, w_), lambda *a: True,
+                        "inf_forward_kernel (conv layout, k tracked in the loop)", 2))
+
+
+WORKLOADS = {"c0": workload_c0, "c1": workload_c1, "c2": workload_c2, "c3": workload_c3, "c4": workload_c4}
+
+
+def cpu_baseline(wl, target_seconds=12.0):
+    """The CPU oracle (C, OpenMP) on a row subset of the same workload, sized to about target_seconds."""
+    import oracle
+    probe = max(1, min(8, wl["full_rows"]))
+    t0 = time.perf_counter()
+    wl["cpu"](oracle, probe)
+    t = time.perf_counter() - t0
+    rows = int(max(probe, min(wl["full_rows"], probe * target_seconds / max(t, 1e-3))))
+    ops, t, reps = 0, 0.0, 0
+    while reps == 0 or (t < target_seconds and reps < 64):   # fast hosts: repeat until the sample is long enough
+        t0 = time.perf_counter()
+        ops += wl["cpu"](oracle, rows)
+        t += time.perf_counter() - t0
         reps += 1
-    ops = dist_ops_per_forward(rows) * reps
     return {
         "value": round(ops / t / 1e9, 3),
         "unit": "G dist-ops/s",
         "cores": oracle.num_threads(),
         "kind": "port",
-        "sample": f"C oracle (OpenMP), forward+backward of the same 5-layer stack on {rows} of {BATCH} rows, "
+        "sample": f"C oracle (OpenMP) on {rows} of {wl['full_rows']} rows of the same workload, "
                   f"{reps} pass(es), {t:.1f} s",
     }
 
@@ -135,6 +278,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c1")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run three plain 256 MiB device copies, the known-size kernel that "
@@ -151,19 +295,11 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
-    x, ws, upstream = make_inputs(BATCH)
-    model = build_model(pkg, ws, dev)
-    xd = x.to(dev).requires_grad_(True)
-    up = upstream.to(dev)
+    wl = WORKLOADS[args.workload](pkg, torch, dev)
+    step = wl["step"]
+    kname, flops_of, accept, kdesc, flops_per_op = wl["kernel"]
 
-    def step():
-        xd.grad = None
-        for prm in model.parameters():
-            prm.grad = None
-        y, _, _ = model(xd)
-        y.backward(up)
-
-    with KernelTimer(pkg.norm_dist_cpp, torch) as kt:
+    with KernelTimer(pkg.norm_dist_cpp, torch, kname, flops_of, accept) as kt:
         for _ in range(args.warmup):
             step()
         torch.cuda.synchronize()
@@ -183,7 +319,7 @@ def main():
         torch.cuda.synchronize()
 
     ms_per_step = elapsed * 1e3 / args.steps
-    ops = dist_ops_per_forward(BATCH)
+    ops = wl["ops"]
     value = ops / (ms_per_step * 1e-3) / 1e9
     achieved = k_flops / (k_ms * 1e-3) / 1e12 if k_ms > 0 else 0.0
     out = {
@@ -199,29 +335,35 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "configs[1]: 5-layer L_inf-dist MLP 3072-5120-5120-5120-5120-10, p=inf, batch 512, "
-                               "forward+backward (all grad_x and grad_w), mean shift in training mode",
-                   "batch": BATCH, "dist_ops_per_step": ops},
-        "img_per_s": round(BATCH / (ms_per_step * 1e-3), 1),
-        "pct_fp32_valu_peak": round(100 * value * 1e9 * FLOPS_PER_DIST_OP / (FP32_PEAK_TFLOPS * 1e12), 2),
+        "config": {"workload": wl["name"], "dist_ops_per_step": ops},
+        "img_per_s": round(wl["images"] / (ms_per_step * 1e-3), 1),
+        "pct_fp32_valu_peak": round(100 * value * 1e9 * flops_per_op / (FP32_PEAK_TFLOPS * 1e12), 2),
         "roofline": {
             "bound": "mfma",
-            "kernel": "inf_forward_kernel (tiled L_inf forward, VALU only: the max-plus reduction cannot use MFMA; "
-                      "'mfma' here names the compute roof, priced at the fp32 vector peak)",
+            "kernel": kdesc + " -- VALU only: a max / power-sum reduction has no multiply-accumulate for MFMA; "
+                              "'mfma' names the compute roof, priced at the fp32 vector peak",
             "achieved": round(achieved, 2),
             "peak": FP32_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / FP32_PEAK_TFLOPS, 4),
-            "frac_of_valu_issue_peak": round(achieved * 1e12 / FLOPS_PER_DIST_OP / (VALU_ISSUE_PEAK_T * 1e12), 4),
+            "dist_ops_per_s_T": round(achieved / flops_per_op, 3),
             "launches_timed": n_launch,
             "avg_launch_ms": round(k_ms, 4),
             "avg_flops_per_launch": k_flops,
             "traffic": None,
         },
     }
+    if args.workload == "c1":
+        # HBM bytes per launch, average over the step's four tiled forward launches, from two
+        # rocprofv3 --pmc runs of this command (profiles/): FETCH_SIZE x 2.0 (copy-probe factor)
+        # + WRITE_SIZE x 1.0
+        out["roofline"]["traffic"] = TRAFFIC_C1_BYTES
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline()
+        out["cpu_baseline"] = cpu_baseline(wl)
     print(json.dumps(out))
+
+
+TRAFFIC_C1_BYTES = 3.5e8
 
 
 if __name__ == "__main__":

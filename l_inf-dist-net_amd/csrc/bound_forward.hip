@@ -11,6 +11,7 @@
 // infinity anywhere in its panels is reduced with the reference's literal
 // predicate instead, so results match the reference for every input.
 #include "fwd_engine.hpp"
+#include "skinny.hpp"
 
 namespace ldist {
 
@@ -53,7 +54,7 @@ bound_forward_kernel(const float* __restrict__ lower, const float* __restrict__ 
         const float* xp = stage + grp * kChunk * GEO::SM;
         const float* wp = stage + 2 * GEO::XS + grp * kChunk * GEO::SN;
         if (!irregular) {
-            sweep_chunk<GEO, 2, 1>(xp, wp, tx, ty, [&](const Frag<GEO, 2, 1>& f) {
+            sweep_chunk<GEO, 2, 1>(xp, wp, tx, ty, [&](const Frag<GEO, 2, 1>& f, int) {
 #pragma unroll
                 for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -68,7 +69,7 @@ bound_forward_kernel(const float* __restrict__ lower, const float* __restrict__ 
                     }
             });
         } else {
-            sweep_chunk<GEO, 2, 1>(xp, wp, tx, ty, [&](const Frag<GEO, 2, 1>& f) {
+            sweep_chunk<GEO, 2, 1>(xp, wp, tx, ty, [&](const Frag<GEO, 2, 1>& f, int) {
 #pragma unroll
                 for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -123,6 +124,64 @@ bound_forward_kernel(const float* __restrict__ lower, const float* __restrict__ 
     store_patch<GEO, CONV>(out_upper, up, d, m0, n0, g, tx, ty, 0xFFu, d.ovec != 0);
 }
 
+// Few outputs per group: lanes split k and apply the reference's literal predicate.
+template <int RW, int NB>
+__global__ void __launch_bounds__(256)
+bound_forward_skinny_kernel(const float* __restrict__ lower, const float* __restrict__ upper,
+                            const float* __restrict__ weight, float* __restrict__ out_lower,
+                            float* __restrict__ out_upper, Dims d) {
+    __shared__ float sl[4][RW * NB], su[4][RW * NB];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    SkinnyRows<RW> rows;
+    rows.init(d);
+    const int K = d.K, xk = d.HW;
+    for (int nb = 0; nb < d.NG; nb += NB) {
+        float lo[RW][NB], up[RW][NB];
+#pragma unroll
+        for (int r = 0; r < RW; r++)
+#pragma unroll
+            for (int j = 0; j < NB; j++) { lo[r][j] = 0.f; up[r][j] = 0.f; }
+        for (int k = tid; k < K; k += 256) {
+            float lv[RW], uv[RW], wv[NB];
+#pragma unroll
+            for (int r = 0; r < RW; r++) {
+                lv[r] = lower[rows.xoff[r] + (size_t)k * xk];
+                uv[r] = upper[rows.xoff[r] + (size_t)k * xk];
+            }
+#pragma unroll
+            for (int j = 0; j < NB; j++) wv[j] = weight[((size_t)rows.g * d.NG + min(nb + j, d.NG - 1)) * K + k];
+#pragma unroll
+            for (int r = 0; r < RW; r++)
+#pragma unroll
+                for (int j = 0; j < NB; j++) {
+                    const float tl = lv[r] - wv[j], tu = uv[r] - wv[j];
+                    const float al = __builtin_fabsf(tl), au = __builtin_fabsf(tu);
+                    up[r][j] = __builtin_fmaxf(up[r][j], __builtin_fmaxf(al, au));
+                    if (!(tl < 0.f && tu > 0.f)) lo[r][j] = __builtin_fmaxf(lo[r][j], __builtin_fminf(al, au));
+                }
+        }
+#pragma unroll
+        for (int r = 0; r < RW; r++)
+#pragma unroll
+            for (int j = 0; j < NB; j++) {
+                const float l = wave_max(lo[r][j]), u = wave_max(up[r][j]);
+                if (lane == 0) { sl[wave][r * NB + j] = l; su[wave][r * NB + j] = u; }
+            }
+        __syncthreads();
+        if (tid < RW * NB) {
+            float l = sl[0][tid], u = su[0][tid];
+#pragma unroll
+            for (int q = 1; q < 4; q++) { l = __builtin_fmaxf(l, sl[q][tid]); u = __builtin_fmaxf(u, su[q][tid]); }
+            const int r = tid / NB, j = tid % NB;
+            if (rows.m0 + r < d.M && nb + j < d.NG) {
+                out_lower[rows.ooff[r] + (size_t)(nb + j) * d.HW] = l;
+                out_upper[rows.ooff[r] + (size_t)(nb + j) * d.HW] = u;
+            }
+        }
+        __syncthreads();
+    }
+}
+
 template <class GEO, bool CONV, int VEC>
 struct BoundForward {
     static hipError_t launch(unsigned grid, const Dims& d, int device, hipStream_t stream, const float* lower,
@@ -138,6 +197,13 @@ struct BoundForward {
 
 hipError_t bound_forward(const float* lower, const float* upper, const float* weight, float* out_lower,
                          float* out_upper, const Problem& pr, hipStream_t stream) {
+    if (pr.NG <= kSkinnyMaxNG) {
+        const Dims d = make_dims(pr);
+        constexpr int RW = 2;
+        hipLaunchKernelGGL((bound_forward_skinny_kernel<RW, 8>), dim3(skinny_grid(d, RW)), dim3(256), 0, stream, lower,
+                           upper, weight, out_lower, out_upper, d);
+        return hipGetLastError();
+    }
     return dispatch_forward<BoundForward>(pr, can_vec4(pr, lower, upper, weight),
                                           can_vec4_out(pr, out_lower, out_upper), stream, lower, upper, weight,
                                           out_lower, out_upper);

@@ -11,10 +11,16 @@
 // first k to reach it).
 #include "fwd_engine.hpp"
 #include "inf_locate.hpp"
+#include "skinny.hpp"
 
 namespace ldist {
 
-template <class GEO, bool CONV, int VEC>
+// EXACT = false: track the chunk of the maximum and locate k afterwards (1.5 + 3/32 VALU
+// instructions per element, plus one re-read of a 32-wide chunk per output).
+// EXACT = true: track k itself (subtract, compare, two selects = 4 instructions per
+// element, no re-read).  That pays in the conv layout with short K, where the re-read is a
+// strided gather that costs more than the whole reduction.
+template <class GEO, bool CONV, int VEC, bool EXACT>
 __global__ void __launch_bounds__(GEO::NT, 2)
 inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ weight, float* __restrict__ output,
                    int32_t* __restrict__ pos, Dims d) {
@@ -56,24 +62,40 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
         for (int i = 0; i < TM; i++)
 #pragma unroll
             for (int j = 0; j < TN; j++) cm[i][j] = 0.f;
-        sweep_chunk<GEO, 1, 2>(stage + grp * kChunk * GEO::SM, stage + GEO::XS + grp * kChunk * GEO::SN, tx, ty,
-                            [&](const Frag<GEO, 1, 2>& f) {
-#pragma unroll
-                                for (int i = 0; i < TM; i++)
-#pragma unroll
-                                    for (int j = 0; j < TN; j++) {
-                                        const float d0 = __builtin_fabsf(f.x[0][0][i] - f.w[0][j]);
-                                        const float d1 = __builtin_fabsf(f.x[0][1][i] - f.w[1][j]);
-                                        cm[i][j] = __builtin_fmaxf(__builtin_fmaxf(cm[i][j], d0), d1);
-                                    }
-                            });
+        const float* xp = stage + grp * kChunk * GEO::SM;
+        const float* wp = stage + GEO::XS + grp * kChunk * GEO::SN;
         const int c = s * KS + grp;
+        if constexpr (EXACT) {
+            sweep_chunk<GEO, 1, 2>(xp, wp, tx, ty, [&](const Frag<GEO, 1, 2>& f, int kk) {
+                const int k0 = c * kChunk + kk;
 #pragma unroll
-        for (int i = 0; i < TM; i++)
+                for (int i = 0; i < TM; i++)
 #pragma unroll
-            for (int j = 0; j < TN; j++) {
-                if (cm[i][j] > acc[i][j]) { acc[i][j] = cm[i][j]; cidx[i][j] = c; }
-            }
+                    for (int j = 0; j < TN; j++) {
+                        const float d0 = __builtin_fabsf(f.x[0][0][i] - f.w[0][j]);
+                        const float d1 = __builtin_fabsf(f.x[0][1][i] - f.w[1][j]);
+                        if (d0 > acc[i][j]) { acc[i][j] = d0; cidx[i][j] = k0; }
+                        if (d1 > acc[i][j]) { acc[i][j] = d1; cidx[i][j] = k0 + 1; }
+                    }
+            });
+        } else {
+            sweep_chunk<GEO, 1, 2>(xp, wp, tx, ty, [&](const Frag<GEO, 1, 2>& f, int) {
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) {
+                        const float d0 = __builtin_fabsf(f.x[0][0][i] - f.w[0][j]);
+                        const float d1 = __builtin_fabsf(f.x[0][1][i] - f.w[1][j]);
+                        cm[i][j] = __builtin_fmaxf(__builtin_fmaxf(cm[i][j], d0), d1);
+                    }
+            });
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    if (cm[i][j] > acc[i][j]) { acc[i][j] = cm[i][j]; cidx[i][j] = c; }
+                }
+        }
         if (NBUF == 1) __syncthreads();  // everyone is done reading the only buffer
         if (s + 1 < nstage) st.store(lds + ((s + 1) % NBUF) * STAGE);
         __syncthreads();
@@ -81,7 +103,7 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
 
     // Merge the two k-groups.  Each group finishes half of the lane's rows, so it needs the
     // other group's candidates for that half only: the larger value wins, equal values keep
-    // the lower chunk.
+    // the lower chunk (or the lower k when k itself was tracked).
     static_assert(KS == 1 || KS == 2, "the merge below pairs two k-groups");
     constexpr int TMH = TM / KS;          // rows finished by each group
     if constexpr (KS == 2) {
@@ -129,10 +151,16 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
             const int n = n0 + GEO::col(tx, j);
             const float best = acc[i][j];
             if (n < d.NG && best > 0.f) {
-                const int kb = cidx[i][j] * kChunk;
-                const float* xr = input + ra.x + (size_t)kb * ra.xk;
-                const float* wr = weight + ((size_t)g * d.NG + n) * K + kb;
-                ppos[i][j] = locate_in_chunk<(!CONV && VEC == 4)>(xr, ra.xk, wr, min(kChunk, K - kb), best, kb);
+                if constexpr (EXACT) {
+                    const int k = cidx[i][j];  // only the sign of the difference is missing
+                    const float df = input[ra.x + (size_t)k * ra.xk] - weight[((size_t)g * d.NG + n) * K + k];
+                    ppos[i][j] = k | (__float_as_int(df) & 0x80000000);
+                } else {
+                    const int kb = cidx[i][j] * kChunk;
+                    const float* xr = input + ra.x + (size_t)kb * ra.xk;
+                    const float* wr = weight + ((size_t)g * d.NG + n) * K + kb;
+                    ppos[i][j] = locate_in_chunk<(!CONV && VEC == 4)>(xr, ra.xk, wr, min(kChunk, K - kb), best, kb);
+                }
             }
         }
     }
@@ -140,15 +168,26 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
     store_patch<GEO, CONV>(pos, ppos, d, m0, n0, g, tx, ty, rows, d.ovec != 0);
 }
 
+// Above this K the chunk re-read is cheaper than tracking k in the loop (conv layout).
+constexpr int kExactMaxK = 1024;
+
 template <class GEO, bool CONV, int VEC>
 struct InfForward {
-    static hipError_t launch(unsigned grid, const Dims& d, int device, hipStream_t stream, const float* input,
-                             const float* weight, float* output, int32_t* pos) {
+    template <bool EXACT>
+    static hipError_t go(unsigned grid, const Dims& d, int device, hipStream_t stream, const float* input,
+                         const float* weight, float* output, int32_t* pos) {
         const size_t lds = Stager<GEO, CONV, VEC, 1>::LDS_BYTES;
-        auto kern = inf_forward_kernel<GEO, CONV, VEC>;
+        auto kern = inf_forward_kernel<GEO, CONV, VEC, EXACT>;
         if (hipError_t e = allow_lds(kern, lds, device); e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(grid), dim3(GEO::NT), lds, stream, input, weight, output, pos, d);
         return hipGetLastError();
+    }
+    static hipError_t launch(unsigned grid, const Dims& d, int device, hipStream_t stream, const float* input,
+                             const float* weight, float* output, int32_t* pos) {
+        if constexpr (CONV) {
+            if (d.K <= kExactMaxK) return go<true>(grid, d, device, stream, input, weight, output, pos);
+        }
+        return go<false>(grid, d, device, stream, input, weight, output, pos);
     }
 };
 
@@ -233,7 +272,7 @@ inf_forward_skinny_kernel(const float* __restrict__ input, const float* __restri
 
 hipError_t inf_forward(const float* input, const float* weight, float* output, int32_t* pos, const Problem& pr,
                        hipStream_t stream) {
-    if (pr.NG <= 16) {
+    if (pr.NG <= kSkinnyMaxNG) {
         const Dims d = make_dims(pr);
         constexpr int RW = 2;
         const unsigned grid = (unsigned)((d.M + RW - 1) / RW) * d.G;

@@ -18,7 +18,7 @@ struct NbDims {
     int B, G, K, NG, HW, M;
 };
 
-constexpr int BA = 64, BKO = 64, RB = 32, LDP = 65;  // tile, stage depth, padded LDS row
+constexpr int BKO = 64, RB = 32, LDP = 65;  // tile width, stage depth, padded LDS row
 
 // WEIGHT = false: grad_input.  WEIGHT = true: grad_weight.
 template <bool WEIGHT, bool CONV>
@@ -39,7 +39,9 @@ struct Views {
     }
 };
 
-template <bool WEIGHT, bool CONV, bool SPLIT>
+// BA = rows of P per workgroup (64, or 32 when 64 would leave the device short of
+// workgroups); a lane owns BA/16 rows x 4 columns.
+template <bool WEIGHT, bool CONV, bool SPLIT, int BA>
 __global__ void __launch_bounds__(256)
 norm_backward_kernel(const float* __restrict__ grad_output, const float* __restrict__ input,
                      const float* __restrict__ weight, const float* __restrict__ output, float* __restrict__ grad,
@@ -58,16 +60,17 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
     const int R = WEIGHT ? d.M : d.NG;
     const int r_begin = blockIdx.y * r_per_wg;
     const int r_end = min(R, r_begin + r_per_wg);
-    const int tx = tid & 15, ty = tid >> 4;  // lane's patch: rows a0 + ty*4.., columns k0 + tx*4..
+    constexpr int PA = BA / 16;              // rows per lane
+    const int tx = tid & 15, ty = tid >> 4;  // lane's patch: rows a0 + ty*PA.., columns k0 + tx*4..
     const float e = p - 1.0f;
     const int ie = small_int_power(e);
 
-    float q[4][4], acc[4][4];
+    float q[PA][4], acc[PA][4];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < PA; i++)
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const int a = a0 + ty * 4 + i, k = k0 + tx * 4 + j;
+            const int a = a0 + ty * PA + i, k = k0 + tx * 4 + j;
             acc[i][j] = 0.f;
             q[i][j] = (a < A && k < d.K) ? (WEIGHT ? weight[v.w_at(a, k)] : input[v.x_at(a, k)]) : 0.f;
         }
@@ -80,19 +83,21 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
     for (int r0 = r_begin; r0 < r_end; r0 += RB) {
         __syncthreads();
 #pragma unroll
-        for (int it = 0; it < RB * 64 / 256; it++) {
+        for (int it = 0; it < RB * BKO / 256; it++) {
+            const int id = tid + it * 256;
+            const int rr = O_K_CONTIG ? id / BKO : id & (RB - 1);
+            const int cc = O_K_CONTIG ? id % BKO : id / RB;
+            const int r = r0 + rr, k = k0 + cc;
+            float val = 0.f;
+            if (r < r_end && k < d.K) val = WEIGHT ? input[v.x_at(r, k)] : weight[v.w_at(r, k)];
+            Os[rr * LDP + cc] = val;
+        }
+#pragma unroll
+        for (int it = 0; it < RB * BA / 256; it++) {
             const int id = tid + it * 256;
             {
-                const int rr = O_K_CONTIG ? id >> 6 : id & (RB - 1);
-                const int cc = O_K_CONTIG ? id & 63 : id >> 5;
-                const int r = r0 + rr, k = k0 + cc;
-                float val = 0.f;
-                if (r < r_end && k < d.K) val = WEIGHT ? input[v.x_at(r, k)] : weight[v.w_at(r, k)];
-                Os[rr * LDP + cc] = val;
-            }
-            {
-                const int rr = C_A_CONTIG ? id >> 6 : id & (RB - 1);
-                const int cc = C_A_CONTIG ? id & 63 : id >> 5;
+                const int rr = C_A_CONTIG ? id / BA : id & (RB - 1);
+                const int cc = C_A_CONTIG ? id % BA : id / RB;
                 const int r = r0 + rr, a = a0 + cc;
                 float c = 0.f, ri = 0.f;
                 if (r < r_end && a < A) {
@@ -108,13 +113,13 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
         auto reduce = [&](auto power) {
 #pragma unroll 2
             for (int rr = 0; rr < RB; rr++) {
-                float o[4], c[4], ri[4];
+                float o[4], c[PA], ri[PA];
 #pragma unroll
                 for (int j = 0; j < 4; j++) o[j] = Os[rr * LDP + tx * 4 + j];
 #pragma unroll
-                for (int i = 0; i < 4; i++) { c[i] = Cs[rr * LDP + ty * 4 + i]; ri[i] = Rs[rr * LDP + ty * 4 + i]; }
+                for (int i = 0; i < PA; i++) { c[i] = Cs[rr * LDP + ty * PA + i]; ri[i] = Rs[rr * LDP + ty * PA + i]; }
 #pragma unroll
-                for (int i = 0; i < 4; i++)
+                for (int i = 0; i < PA; i++)
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
                         const float t = q[i][j] - o[j];
@@ -134,10 +139,10 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
     }
 
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < PA; i++)
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const int a = a0 + ty * 4 + i, k = k0 + tx * 4 + j;
+            const int a = a0 + ty * PA + i, k = k0 + tx * 4 + j;
             if (a < A && k < d.K) {
                 if (WEIGHT) {
                     float* dst = grad + v.w_at(a, k);
@@ -150,10 +155,10 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
         }
 }
 
-template <bool WEIGHT>
-static hipError_t launch_norm_backward(const float* grad_output, const float* input, const float* weight,
-                                       const float* output, float* grad, float p, const Problem& pr,
-                                       hipStream_t stream) {
+template <bool WEIGHT, int BA>
+static hipError_t launch_norm_backward_ba(const float* grad_output, const float* input, const float* weight,
+                                          const float* output, float* grad, float p, const Problem& pr,
+                                          hipStream_t stream) {
     const NbDims d{pr.B, pr.G, pr.K, pr.NG, pr.HW, pr.B * pr.HW};
     const int A = WEIGHT ? d.NG : d.M;
     const int R = WEIGHT ? d.M : d.NG;
@@ -171,7 +176,7 @@ static hipError_t launch_norm_backward(const float* grad_output, const float* in
     const dim3 grid((unsigned)tiles, (unsigned)splits);
     const bool conv = pr.HW != 1;
 #define LDIST_LAUNCH(W, C, S)                                                                                      \
-    hipLaunchKernelGGL((norm_backward_kernel<W, C, S>), grid, dim3(256), 0, stream, grad_output, input, weight,    \
+    hipLaunchKernelGGL((norm_backward_kernel<W, C, S, BA>), grid, dim3(256), 0, stream, grad_output, input, weight,    \
                        output, grad, p, d, tiles_a, tiles_k, r_per_wg)
     if (WEIGHT) {
         if (splits > 1) { if (conv) LDIST_LAUNCH(WEIGHT, true, true); else LDIST_LAUNCH(WEIGHT, false, true); }
@@ -181,6 +186,18 @@ static hipError_t launch_norm_backward(const float* grad_output, const float* in
     }
 #undef LDIST_LAUNCH
     return hipGetLastError();
+}
+
+template <bool WEIGHT>
+static hipError_t launch_norm_backward(const float* grad_output, const float* input, const float* weight,
+                                       const float* output, float* grad, float p, const Problem& pr,
+                                       hipStream_t stream) {
+    // 64-row tiles unless they would give fewer than four workgroups per CU (and the rows allow halving)
+    const int A = WEIGHT ? pr.NG : pr.B * pr.HW;
+    const long tiles64 = (long)((A + 63) / 64) * ((pr.K + BKO - 1) / BKO) * pr.G;
+    if (tiles64 < 4L * pr.num_cu && A > 32)
+        return launch_norm_backward_ba<WEIGHT, 32>(grad_output, input, weight, output, grad, p, pr, stream);
+    return launch_norm_backward_ba<WEIGHT, 64>(grad_output, input, weight, output, grad, p, pr, stream);
 }
 
 hipError_t norm_backward_input(const float* grad_output, const float* input, const float* weight,

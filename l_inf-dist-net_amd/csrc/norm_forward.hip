@@ -9,6 +9,7 @@
 // p goes through v_log_f32 / v_exp_f32.
 #include "fwd_engine.hpp"
 #include "pow.hpp"
+#include "skinny.hpp"
 
 namespace ldist {
 
@@ -55,7 +56,7 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
         for (int i = 0; i < TM; i++)
 #pragma unroll
             for (int j = 0; j < TN; j++) cm[i][j] = 0.f;
-        sweep_chunk<GEO, 1, 2>(xp, wp, tx, ty, [&](const Frag<GEO, 1, 2>& f) {
+        sweep_chunk<GEO, 1, 2>(xp, wp, tx, ty, [&](const Frag<GEO, 1, 2>& f, int) {
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -76,7 +77,7 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
                 cm[i][j] = __builtin_amdgcn_rcpf(mx[i][j]);
             }
         auto add_powers = [&](auto power) {
-            sweep_chunk<GEO, 1, 2>(xp, wp, tx, ty, [&](const Frag<GEO, 1, 2>& f) {
+            sweep_chunk<GEO, 1, 2>(xp, wp, tx, ty, [&](const Frag<GEO, 1, 2>& f, int) {
 #pragma unroll
                 for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -139,6 +140,75 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
     store_patch<GEO, CONV>(output, acc, d, m0, n0, g, tx, ty, 0xFFu, d.ovec != 0);
 }
 
+// Few outputs per group: two passes over k, first the exact maximum per (row, output),
+// then the sum of (|x-w| / max)^p; lanes split k in both.
+template <int RW, int NB>
+__global__ void __launch_bounds__(256)
+norm_forward_skinny_kernel(const float* __restrict__ input, const float* __restrict__ weight,
+                           float* __restrict__ output, float p, Dims d) {
+    __shared__ float red[4][RW * NB];
+    __shared__ float bcast[RW * NB];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    SkinnyRows<RW> rows;
+    rows.init(d);
+    const int K = d.K, xk = d.HW;
+    for (int nb = 0; nb < d.NG; nb += NB) {
+        float acc[RW][NB], rmx[RW][NB];
+        // pass 0: maximum; pass 1: power sum
+        for (int pass = 0; pass < 2; pass++) {
+#pragma unroll
+            for (int r = 0; r < RW; r++)
+#pragma unroll
+                for (int j = 0; j < NB; j++) acc[r][j] = 0.f;
+            for (int k = tid; k < K; k += 256) {
+                float xv[RW], wv[NB];
+#pragma unroll
+                for (int r = 0; r < RW; r++) xv[r] = input[rows.xoff[r] + (size_t)k * xk];
+#pragma unroll
+                for (int j = 0; j < NB; j++) wv[j] = weight[((size_t)rows.g * d.NG + min(nb + j, d.NG - 1)) * K + k];
+#pragma unroll
+                for (int r = 0; r < RW; r++)
+#pragma unroll
+                    for (int j = 0; j < NB; j++) {
+                        const float a = __builtin_fabsf(xv[r] - wv[j]);
+                        if (pass == 0) acc[r][j] = __builtin_fmaxf(acc[r][j], a);
+                        else acc[r][j] += pow_pos(a * rmx[r][j], p);
+                    }
+            }
+#pragma unroll
+            for (int r = 0; r < RW; r++)
+#pragma unroll
+                for (int j = 0; j < NB; j++) {
+                    const float v = pass == 0 ? wave_max(acc[r][j]) : wave_sum(acc[r][j]);
+                    if (lane == 0) red[wave][r * NB + j] = v;
+                }
+            __syncthreads();
+            if (tid < RW * NB) {
+                float v = red[0][tid];
+#pragma unroll
+                for (int q = 1; q < 4; q++) v = pass == 0 ? __builtin_fmaxf(v, red[q][tid]) : v + red[q][tid];
+                if (pass == 0) {
+                    bcast[tid] = __builtin_fmaxf(v, 1e-10f);   // the reference's seed for the maximum
+                } else {
+                    const float mx = bcast[tid];
+                    const float sum = v + 1e-10f * pow_pos(1e-10f * __builtin_amdgcn_rcpf(mx), p);  // seeded sum
+                    const int r = tid / NB, j = tid % NB;
+                    if (rows.m0 + r < d.M && nb + j < d.NG)
+                        output[rows.ooff[r] + (size_t)(nb + j) * d.HW] = pow_pos(sum, 1.0f / p) * mx;
+                }
+            }
+            __syncthreads();
+            if (pass == 0) {
+#pragma unroll
+                for (int r = 0; r < RW; r++)
+#pragma unroll
+                    for (int j = 0; j < NB; j++) rmx[r][j] = __builtin_amdgcn_rcpf(bcast[r * NB + j]);
+            }
+            __syncthreads();
+        }
+    }
+}
+
 template <class GEO, bool CONV, int VEC>
 struct NormForward {
     static hipError_t launch(unsigned grid, const Dims& d, int device, hipStream_t stream, const float* input,
@@ -153,6 +223,13 @@ struct NormForward {
 
 hipError_t norm_forward(const float* input, const float* weight, float* output, float p, const Problem& pr,
                         hipStream_t stream) {
+    if (pr.NG <= kSkinnyMaxNG) {
+        const Dims d = make_dims(pr);
+        constexpr int RW = 2;
+        hipLaunchKernelGGL((norm_forward_skinny_kernel<RW, 8>), dim3(skinny_grid(d, RW)), dim3(256), 0, stream, input,
+                           weight, output, p, d);
+        return hipGetLastError();
+    }
     return dispatch_forward<NormForward>(pr, can_vec4(pr, input, weight), can_vec4_out(pr, output), stream, input,
                                          weight, output, p);
 }

@@ -121,7 +121,8 @@ struct Frag {
     }
 };
 
-// Walks one 32-row chunk of the panels and calls f(frag) once per KP k rows.
+// Walks one 32-row chunk of the panels and calls f(frag, kk) once per KP k rows
+// (kk = first row of the fragment inside the chunk, ascending).
 // 2*KP rows per trip, as two fragments: the operands of the next fragment are
 // fetched from LDS while the current one is being reduced.  The loop is kept
 // rolled on purpose: unrolled, the compiler hoists every LDS read of the chunk
@@ -137,10 +138,10 @@ __device__ __forceinline__ void sweep_chunk(const float* xp, const float* wp, in
 #pragma unroll 1
     for (int kk = 0; kk < kChunk; kk += 2 * KP) {
         b.read(cur, KP, XSTRIDE);
-        f(a);
+        f(a, kk);
         nxt.set(xp, wp, (kk + 2 * KP) & (kChunk - 1), tx, ty);  // the last trip re-reads row 0; harmless
         a.read(nxt, 0, XSTRIDE);
-        f(b);
+        f(b, kk + KP);
         cur = nxt;
     }
 }
