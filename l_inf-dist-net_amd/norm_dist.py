@@ -1,14 +1,17 @@
 """Distance-neuron operators and layers with the reference's Python interface.
 
-Mirrors model/norm_dist.py of the reference: ``DistF`` (autograd function),
-``norm_dist`` / ``inf_dist_bound`` (functional API, including the dense
-pure-torch formulas selected by ``use_custom_cuda_func=False``), ``MeanNorm``,
-``NormDistConv``, ``NormDist``, ``set_p_norm`` / ``get_p_norm``.  The native
-calls go through ``norm_dist_cpp`` (this package's ctypes binding of
-libldist_hip.so) instead of the reference's CUDA extension.
+Public names, signatures and return conventions follow the reference's
+model/norm_dist.py so that its callers work unchanged:
 
-Additions that the reference does not have: the aliases ``MeanNormDist`` and
-the keyword spellings ``groups`` / ``mean_shift`` accepted by the layers.
+    DistF                      autograd function            (reference :7-47)
+    norm_dist, inf_dist_bound  functional API               (reference :49-76)
+    MeanNorm                   per-channel mean shift       (reference :78-100)
+    NormDistConv, NormDist     conv / fully connected layer (reference :102-187)
+    set_p_norm, get_p_norm     p of every layer of a model  (reference :189-198)
+
+The native calls go through ``norm_dist_cpp`` (this package's ctypes binding of
+libldist_hip.so).  Not in the reference: ``MeanNormDist`` and the keyword
+spellings ``groups`` / ``mean_shift`` accepted by the layers.
 """
 import math
 
@@ -18,91 +21,106 @@ import torch.nn.functional as F
 
 from . import norm_dist_cpp
 
+_INF = float("inf")
+
+
+def _out_shape(x, weight):
+    return x.size(0), weight.size(0), x.size(2)
+
 
 class DistF(torch.autograd.Function):
-    """out = ||x - w||_p per (row, output); p = inf keeps the argmax for the backward.
+    """y[b, n, hw] = || x[b, group(n), :, hw] - weight[n, :] ||_p for p = inf or p > 1.
 
-    Reference: model/norm_dist.py:7-47.  x is (B, CI, HW), weight (CO, CI/group).
+    x is (B, CI, HW), weight (CO, CI/group).  At p = inf the forward also records
+    which input attains the maximum; the backward routes the gradient there.
     """
 
     @staticmethod
     def forward(ctx, x, weight, group, p, tag):
         assert weight.size(1) * group == x.size(1)
-        shape = (x.size(0), weight.size(0), x.size(2))
-        output = torch.empty(shape, device=x.device, dtype=x.dtype)
-        if math.isinf(p):
-            pos = torch.empty(shape, device=x.device, dtype=torch.int32)
-            norm_dist_cpp.inf_dist_forward(x, weight, output, pos, group)
-            ctx.save_for_backward(x, weight, output, pos)
-        elif p > 1:
-            norm_dist_cpp.norm_dist_forward(x, weight, output, group, p)
-            ctx.save_for_backward(x, weight, output)
-        else:
+        if not (math.isinf(p) or p > 1):
             raise NotImplementedError
-        ctx.group = group
-        ctx.p = p
-        ctx.tag = tag
-        return output
+        y = torch.empty(_out_shape(x, weight), device=x.device, dtype=x.dtype)
+        if math.isinf(p):
+            argmax = torch.empty(y.shape, device=x.device, dtype=torch.int32)
+            norm_dist_cpp.inf_dist_forward(x, weight, y, argmax, group)
+            ctx.save_for_backward(x, weight, y, argmax)
+        else:
+            norm_dist_cpp.norm_dist_forward(x, weight, y, group, p)
+            ctx.save_for_backward(x, weight, y)
+        ctx.group, ctx.p, ctx.tag = group, p, tag
+        return y
 
     @staticmethod
     def backward(ctx, grad_output):
-        grad_input = grad_weight = None
-        grad_output = grad_output.contiguous()
+        want_x, want_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        g = grad_output.contiguous()
+        gx = gw = None
         if math.isinf(ctx.p):
-            x, weight, output, pos = ctx.saved_tensors
-            # the scatter kernels write every element, so no zero fill is needed here
-            if ctx.needs_input_grad[0]:
-                grad_input = torch.empty_like(x)
-                norm_dist_cpp.inf_dist_backward_input_overwrite(grad_output, pos, grad_input, ctx.group)
-            if ctx.needs_input_grad[1]:
-                grad_weight = torch.empty_like(weight)
-                norm_dist_cpp.inf_dist_backward_weight_overwrite(grad_output, pos, grad_weight, ctx.group)
+            x, weight, _, argmax = ctx.saved_tensors
+            # the scatter kernels write every element, zeros included: no fill needed here
+            if want_x:
+                gx = torch.empty_like(x)
+                norm_dist_cpp.inf_dist_backward_input_overwrite(g, argmax, gx, ctx.group)
+            if want_w:
+                gw = torch.empty_like(weight)
+                norm_dist_cpp.inf_dist_backward_weight_overwrite(g, argmax, gw, ctx.group)
         else:
-            x, weight, output = ctx.saved_tensors
-            if ctx.needs_input_grad[0]:
-                grad_input = torch.empty_like(x)
-                norm_dist_cpp.norm_dist_backward_input(grad_output, x, weight, output, grad_input, ctx.group, ctx.p)
-            if ctx.needs_input_grad[1]:
-                grad_weight = torch.zeros_like(weight)  # the kernel adds onto it
-                norm_dist_cpp.norm_dist_backward_weight(grad_output, x, weight, output, grad_weight, ctx.group, ctx.p)
-        return grad_input, grad_weight, None, None, None
+            x, weight, y = ctx.saved_tensors
+            if want_x:
+                gx = torch.empty_like(x)
+                norm_dist_cpp.norm_dist_backward_input(g, x, weight, y, gx, ctx.group, ctx.p)
+            if want_w:
+                gw = torch.zeros_like(weight)  # this kernel adds onto the buffer
+                norm_dist_cpp.norm_dist_backward_weight(g, x, weight, y, gw, ctx.group, ctx.p)
+        return gx, gw, None, None, None
+
+
+def _pairwise_difference(inp, weight, group):
+    """(B, G, CO/G, CI/G, HW) tensor of input minus weight, by broadcasting."""
+    b, _, hw = inp.shape
+    return inp.view(b, group, 1, -1, hw) - weight.view(group, -1, weight.size(-1), 1)
 
 
 def norm_dist(input, weight, group, p, use_custom_cuda_func=True, tag=None):
-    """model/norm_dist.py:49-58.  The dense torch formula runs only when asked for explicitly."""
+    """Distances between every input column and every weight row.
+
+    use_custom_cuda_func=False evaluates the same quantity with dense torch ops
+    (the broadcast difference is B*CO*CI/group*HW floats), as the reference's
+    option of that name does; it is never chosen automatically.
+    """
     if use_custom_cuda_func:
         return DistF.apply(input, weight, group, p, tag)
-    y = input.view(input.size(0), group, 1, -1, input.size(2)) - weight.view(group, -1, weight.size(-1), 1)
+    diff = _pairwise_difference(input, weight, group)
     with torch.no_grad():
-        normalize = torch.norm(y, dim=3, p=float("inf"), keepdim=True)
-    y = torch.norm(y / normalize, dim=3, p=p, keepdim=True) * normalize
-    return y.view(y.size(0), -1, y.size(-1))
+        scale = torch.norm(diff, dim=3, p=_INF, keepdim=True)
+    dist = torch.norm(diff / scale, dim=3, p=p, keepdim=True) * scale
+    return dist.view(dist.size(0), -1, dist.size(-1))
 
 
 def inf_dist_bound(input_lower, input_upper, weight, group, use_custom_cuda_func=True, tag=None):
-    """model/norm_dist.py:60-76.  Returns (output_lower, output_upper); not differentiable."""
-    shape = input_lower.size(0), weight.size(0), input_lower.size(2)
+    """Interval bounds of the L_inf distance for inputs in [input_lower, input_upper].
+
+    Returns (output_lower, output_upper); neither carries gradient.
+    """
+    shape = _out_shape(input_lower, weight)
     if use_custom_cuda_func:
-        output_lower = input_lower.new_empty(shape)
-        output_upper = input_upper.new_empty(shape)
-        norm_dist_cpp.inf_dist_bound_forward(input_lower, input_upper, weight, output_lower, output_upper, group)
-        return output_lower, output_upper
-    w = weight.view(group, -1, weight.size(-1), 1)
-    y1 = input_lower.view(input_lower.size(0), group, 1, -1, input_lower.size(2)) - w
-    y2 = input_upper.view(input_upper.size(0), group, 1, -1, input_upper.size(2)) - w
-    abs_y1, abs_y2 = torch.abs(y1), torch.abs(y2)
-    output_upper = torch.maximum(abs_y1, abs_y2).max(dim=3)[0].view(shape)
-    output_lower = torch.minimum(abs_y1, abs_y2)
-    output_lower[(y1 < 0) & (y2 > 0)] = 0
-    output_lower = output_lower.max(dim=3)[0].view(shape)
-    return output_lower, output_upper
+        lo = input_lower.new_empty(shape)
+        hi = input_upper.new_empty(shape)
+        norm_dist_cpp.inf_dist_bound_forward(input_lower, input_upper, weight, lo, hi, group)
+        return lo, hi
+    d_lo = _pairwise_difference(input_lower, weight, group)
+    d_hi = _pairwise_difference(input_upper, weight, group)
+    a_lo, a_hi = d_lo.abs(), d_hi.abs()
+    hi = torch.maximum(a_lo, a_hi).amax(dim=3).view(shape)
+    straddles = (d_lo < 0) & (d_hi > 0)          # the weight lies strictly inside the interval
+    nearest = torch.where(straddles, torch.zeros_like(a_lo), torch.minimum(a_lo, a_hi))
+    return nearest.amax(dim=3).view(shape), hi
 
 
 class MeanNorm(nn.Module):
-    """Subtracts the per-channel mean (batch mean when training, running mean otherwise).
-
-    Reference: model/norm_dist.py:78-100.
-    """
+    """Subtracts a per-channel mean: the batch mean in training mode (which also moves
+    ``running_mean`` by ``momentum``), ``running_mean`` in eval mode."""
 
     def __init__(self, out_channels, momentum=0.1):
         super().__init__()
@@ -111,59 +129,61 @@ class MeanNorm(nn.Module):
         self.register_buffer("running_mean", torch.zeros(out_channels))
 
     def forward(self, x):
-        y = x.view(x.size(0), x.size(1), -1)
+        flat = x.view(x.size(0), x.size(1), -1)
         if self.training:
-            mean = y.mean(dim=-1).mean(dim=0) if x.dim() > 2 else x.mean(dim=0)
+            mean = flat.mean(dim=-1).mean(dim=0) if x.dim() > 2 else x.mean(dim=0)
             with torch.no_grad():
                 self.running_mean.mul_(1 - self.momentum).add_(mean, alpha=self.momentum)
         else:
             mean = self.running_mean
-        return (y - mean.unsqueeze(-1)).view_as(x)
+        return (flat - mean.unsqueeze(-1)).view_as(x)
 
     def extra_repr(self):
-        return f"{self.out_channels}"
+        return str(self.out_channels)
 
 
 class NormDistConv(nn.Module):
-    """Convolution-shaped layer of distance neurons (model/norm_dist.py:102-169).
+    """Convolution-shaped layer of distance neurons.
 
-    forward(x, lower=None, upper=None) returns (y, lower', upper'); the bounds
-    need p = inf and eval mode.
+    forward(x, lower=None, upper=None) -> (y, lower', upper').  Interval bounds are
+    propagated only at p = inf in eval mode.  ``p`` starts at 0 and has to be set
+    (``set_p_norm``) before the first forward.
     """
+
+    tag = 0
 
     def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1, group=1, p=0,
                  bias=True, mean_normalize=False, identity_init=True, groups=None, mean_shift=None):
         super().__init__()
-        if groups is not None:
-            group = groups
-        if mean_shift is not None:
-            mean_normalize = mean_shift
-        self.in_channels = in_channels
-        self.out_channels = out_channels
-        self.kernel_size = kernel_size
-        self.stride = stride
-        self.padding = padding
-        self.dilation = dilation
-        self.group = group
-        self.p = p
+        group = group if groups is None else groups
+        mean_normalize = mean_normalize if mean_shift is None else mean_shift
         assert in_channels % group == 0
         assert out_channels % group == 0
+        self.in_channels, self.out_channels = in_channels, out_channels
+        self.kernel_size, self.stride, self.padding, self.dilation = kernel_size, stride, padding, dilation
+        self.group = group
+        self.p = p
 
-        weight_tensor = torch.randn(out_channels, in_channels // group, kernel_size, kernel_size)
+        per_group = in_channels // group
+        w = torch.randn(out_channels, per_group, kernel_size, kernel_size)
         if identity_init and in_channels <= out_channels:
+            rows = torch.arange(out_channels)
             centre = kernel_size // 2
-            for i in range(out_channels):
-                weight_tensor[i, i % (in_channels // group), centre, centre] = -10.0
-        self.weight = nn.Parameter(weight_tensor)
+            w[rows, rows % per_group, centre, centre] = -10.0
+        self.weight = nn.Parameter(w)
         self.normalize = MeanNorm(out_channels) if mean_normalize else None
         self.bias = nn.Parameter(torch.zeros(out_channels)) if bias else None
 
-        if not hasattr(NormDistConv, "tag"):
-            NormDistConv.tag = 0
         NormDistConv.tag += 1
         self.tag = NormDistConv.tag
 
-    def _post(self, t):
+    def _columns(self, t):
+        """(B, C*k*k, L) patches of t; a 1x1 window needs no unfold (which launches one kernel per image)."""
+        if self.kernel_size == 1 and self.stride == 1 and self.padding == 0:
+            return t.reshape(t.size(0), t.size(1), -1)
+        return F.unfold(t, self.kernel_size, self.dilation, self.padding, self.stride)
+
+    def _shift(self, t):
         if self.normalize is not None:
             t = self.normalize(t)
         if self.bias is not None:
@@ -171,46 +191,32 @@ class NormDistConv(nn.Module):
         return t
 
     def forward(self, x, lower=None, upper=None):
-        h, w = x.size(2), x.size(3)
-        out_h = (h + 2 * self.padding - self.kernel_size) // self.stride + 1
-        out_w = (w + 2 * self.padding - self.kernel_size) // self.stride + 1
-        if self.kernel_size == 1 and self.stride == 1 and self.padding == 0:
-            # a 1x1 window is the identity: skip F.unfold, which launches one kernel per image
-            unfold = lambda t: t.reshape(t.size(0), t.size(1), -1)
-        else:
-            unfold = lambda t: F.unfold(t, self.kernel_size, self.dilation, self.padding, self.stride)
-        cols = unfold(x)
-        weight = self.weight.view(self.weight.size(0), -1)
-        y = norm_dist(cols.view(cols.size(0), cols.size(1), -1), weight, self.group, p=self.p, tag=self.tag)
-        y = y.view(cols.size(0), -1, out_h, out_w)
-        # MeanNorm updates its running mean on y only; the bounds below run in eval mode
-        y = self._post(y)
+        span = self.kernel_size - 2 * self.padding
+        out_hw = ((x.size(2) - span) // self.stride + 1, (x.size(3) - span) // self.stride + 1)
+        w2d = self.weight.view(self.weight.size(0), -1)
+        y = norm_dist(self._columns(x), w2d, self.group, p=self.p, tag=self.tag)
+        y = self._shift(y.view(x.size(0), -1, *out_hw))  # in training mode only y moves the running mean
         if lower is None or upper is None:
             return y, None, None
         assert math.isinf(self.p) and not self.training
-        lower, upper = unfold(lower), unfold(upper)
-        lower, upper = inf_dist_bound(lower.view(cols.size(0), cols.size(1), -1),
-                                      upper.view(cols.size(0), cols.size(1), -1), weight, self.group, tag=self.tag)
-        return y, self._post(lower.view_as(y)), self._post(upper.view_as(y))
+        lo, hi = inf_dist_bound(self._columns(lower), self._columns(upper), w2d, self.group, tag=self.tag)
+        return y, self._shift(lo.view_as(y)), self._shift(hi.view_as(y))
 
     def extra_repr(self):
-        s = f"{self.in_channels}, {self.out_channels}, kernel_size={self.kernel_size}, stride={self.stride}"
+        parts = [f"{self.in_channels}, {self.out_channels}, kernel_size={self.kernel_size}, stride={self.stride}"]
         if self.padding != 0:
-            s += f", padding={self.padding}"
+            parts.append(f"padding={self.padding}")
         if self.dilation != 1:
-            s += f", dilation={self.dilation}"
+            parts.append(f"dilation={self.dilation}")
         if self.group != 1:
-            s += f", group={self.group}"
+            parts.append(f"group={self.group}")
         if self.bias is None:
-            s += ", bias=False"
-        return s
+            parts.append("bias=False")
+        return ", ".join(parts)
 
 
 class NormDist(NormDistConv):
-    """Fully connected layer of distance neurons: a 1x1 NormDistConv on (B, C, 1, 1).
-
-    Reference: model/norm_dist.py:171-187.
-    """
+    """Fully connected layer of distance neurons: a 1x1 NormDistConv applied to (B, C, 1, 1)."""
 
     def __init__(self, in_features, out_features, p=0, bias=True, mean_normalize=False, identity_init=True,
                  mean_shift=None):
@@ -218,36 +224,31 @@ class NormDist(NormDistConv):
                          identity_init=identity_init, mean_shift=mean_shift)
 
     def forward(self, x, lower=None, upper=None):
-        x = x.unsqueeze(-1).unsqueeze(-1)
-        lower = lower.view_as(x) if lower is not None else None
-        upper = upper.view_as(x) if upper is not None else None
-        x, lower, upper = super().forward(x, lower, upper)
-        x = x.squeeze(-1).squeeze(-1)
-        lower = lower.view_as(x) if lower is not None else None
-        upper = upper.view_as(x) if upper is not None else None
-        return x, lower, upper
+        as_image = lambda t: None if t is None else t.reshape(t.size(0), t.size(1), 1, 1)
+        outs = super().forward(as_image(x), as_image(lower), as_image(upper))
+        return tuple(None if t is None else t.reshape(t.size(0), t.size(1)) for t in outs)
 
     def extra_repr(self):
         return f"in_features={self.in_channels}, out_features={self.out_channels}, bias={self.bias is not None}"
 
 
 class MeanNormDist(NormDist):
-    """NormDist with the mean shift switched on (no class of this name exists in the reference)."""
+    """NormDist with the mean shift switched on and no bias (no class of this name in the reference)."""
 
     def __init__(self, in_features, out_features, p=0, bias=False, identity_init=True):
         super().__init__(in_features, out_features, p=p, bias=bias, mean_normalize=True, identity_init=identity_init)
 
 
+def _dist_layers(model):
+    return (m for m in model.modules() if isinstance(m, NormDistConv))  # NormDist is a subclass
+
+
 def set_p_norm(model, p):
-    """model/norm_dist.py:189-192."""
-    for m in model.modules():
-        if isinstance(m, (NormDist, NormDistConv)):
-            m.p = p
+    for layer in _dist_layers(model):
+        layer.p = p
 
 
 def get_p_norm(model):
-    """model/norm_dist.py:194-198."""
-    for m in model.modules():
-        if isinstance(m, (NormDist, NormDistConv)):
-            return m.p
+    for layer in _dist_layers(model):
+        return layer.p
     return None

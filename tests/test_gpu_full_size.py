@@ -1,0 +1,126 @@
+"""GPU parity at the full sizes of the benchmark configurations (BASELINE.json configs 0-4).
+
+The vectorised oracle is fast enough to check the L_inf paths bit for bit at full
+size; the p-norm and bound paths are checked on a row subset of the full-size
+layer (rows are independent) plus size-independent invariants on the whole output.
+"""
+import math
+
+import pytest
+import torch
+
+import oracle
+from helpers import assert_sum_close, gen
+
+pytestmark = pytest.mark.gpu
+
+
+def _layer(B, CI, CO, seed=0):
+    g = gen(seed)
+    x = torch.rand(B, CI, 1, generator=g)
+    w = (torch.randn(CO, CI, generator=g) / math.sqrt(CI)).contiguous()
+    return x, w
+
+
+def test_config0_forward_bit_exact():
+    from gpu_common import gpu_inf_forward, say
+    say("config 0: 512 x 784 -> 5120")
+    x, w = _layer(512, 784, 5120)
+    out, pos = gpu_inf_forward(x, w, 1)
+    eo, ep = oracle.inf_dist_forward(x, w, 1)
+    assert torch.equal(out, eo) and torch.equal(pos, ep)
+
+
+@pytest.mark.parametrize("ci", [3072, 5120])
+def test_config1_hidden_layer_forward_and_backward(ci):
+    from gpu_common import DEV, cpp, gpu_inf_forward, say
+    say("config 1 layer: 512 x", ci, "-> 5120")
+    x, w = _layer(512, ci, 5120, seed=1)
+    x = ((x - 0.47) / 0.2009).contiguous()           # normalised-image range, like the first layer's input
+    out, pos = gpu_inf_forward(x, w, 1)
+    eo, ep = oracle.inf_dist_forward(x, w, 1)
+    assert torch.equal(out, eo) and torch.equal(pos, ep)
+    go = torch.randn(512, 5120, 1, generator=gen(2))
+    gx = torch.empty(512, ci, 1, device=DEV)
+    gw = torch.empty(5120, ci, device=DEV)
+    cpp.inf_dist_backward_input_overwrite(go.to(DEV), pos.to(DEV), gx, 1)
+    cpp.inf_dist_backward_weight_overwrite(go.to(DEV), pos.to(DEV), gw, 1)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(gx.cpu(), oracle.inf_dist_backward_input(go, ep, ci, 1), rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(gw.cpu(), oracle.inf_dist_backward_weight(go, ep, ci, 1), rtol=1e-5, atol=1e-6)
+
+
+def test_config1_head_forward_bit_exact():
+    from gpu_common import gpu_inf_forward
+    x, w = _layer(512, 5120, 10, seed=3)
+    out, pos = gpu_inf_forward(x, w, 1)
+    eo, ep = oracle.inf_dist_forward(x, w, 1)
+    assert torch.equal(out, eo) and torch.equal(pos, ep)
+
+
+def test_config2_pnorm_layer_rows_and_invariants():
+    from gpu_common import DEV, cpp, gpu_norm_forward, say
+    say("config 2 layer: 512 x 5120 -> 5120, p = 8")
+    x, w = _layer(512, 5120, 5120, seed=4)
+    p = 8.0
+    out = gpu_norm_forward(x, w, 1, p)
+    rows = slice(100, 116)
+    torch.testing.assert_close(out[rows], oracle.norm_dist_forward(x[rows].contiguous(), w, 1, p), rtol=1e-5, atol=1e-6)
+    # invariant on the whole output: a1 <= out <= K^(1/p) * a1 with a1 the L_inf distance
+    a1, _ = oracle.inf_dist_forward(x, w, 1)
+    assert bool((out >= a1 * (1 - 1e-6)).all()) and bool((out <= a1 * 5120 ** (1 / p) * (1 + 1e-6)).all())
+    # gradients on the row subset (grad_input rows are independent; grad_weight of a row subset is a valid problem)
+    go = torch.randn(16, 5120, 1, generator=gen(5))
+    xs, outs = x[rows].contiguous(), out[rows].contiguous()
+    ex, mx = oracle.norm_dist_backward_input(go, xs, w, outs, 1, p, with_abs_terms=True)
+    ew, mw = oracle.norm_dist_backward_weight(go, xs, w, outs, 1, p, with_abs_terms=True)
+    gx = torch.empty(16, 5120, 1, device=DEV)
+    gw = torch.zeros(5120, 5120, device=DEV)
+    args = (go.to(DEV), xs.to(DEV), w.to(DEV), outs.to(DEV))
+    cpp.norm_dist_backward_input(*args, gx, 1, p)
+    cpp.norm_dist_backward_weight(*args, gw, 1, p)
+    torch.cuda.synchronize()
+    assert_sum_close(gx.cpu(), ex, mx, p)
+    assert_sum_close(gw.cpu(), ew, mw, p)
+
+
+def test_config3_bound_layer():
+    from gpu_common import gpu_bound_forward, gpu_inf_forward, say
+    say("config 3 layer: 1024 x 5120 -> 5120 bounds")
+    x, w = _layer(1024, 5120, 5120, seed=6)
+    eps = 8 / 255 / 0.2009
+    lo, up = (x - eps).contiguous(), (x + eps).contiguous()
+    ol, ou = gpu_bound_forward(lo, up, w, 1)
+    rows = slice(500, 532)
+    el, eu = oracle.inf_dist_bound_forward(lo[rows].contiguous(), up[rows].contiguous(), w, 1)
+    assert torch.equal(ol[rows], el) and torch.equal(ou[rows], eu)
+    # soundness on the whole output: L <= value(x) <= U, and U - L <= 2 eps (1-Lipschitz in L_inf)
+    val, _ = gpu_inf_forward(x, w, 1)
+    assert bool((ol <= val).all()) and bool((val <= ou).all())
+    assert bool(((ou - ol) <= 2 * eps * (1 + 1e-5)).all())
+    # the degenerate box reproduces the value forward bit for bit at full size
+    dl, du = gpu_bound_forward(x, x, w, 1)
+    assert torch.equal(dl, val) and torch.equal(du, val)
+
+
+def test_config4_unfolded_conv_layer():
+    import torch.nn.functional as F
+    from gpu_common import DEV, cpp, gpu_inf_forward, say
+    say("config 4: 128 x 1152 x 1024, 128 outputs, 4 groups")
+    g = gen(7)
+    img = torch.rand(128, 128, 32, 32, generator=g)
+    w = (torch.randn(128, 288, generator=g) / math.sqrt(288)).contiguous()
+    cols = F.unfold(img, 3, padding=1).contiguous()
+    out, pos = gpu_inf_forward(cols, w, 4)
+    eo, ep = oracle.inf_dist_forward(cols, w, 4)
+    assert torch.equal(out, eo) and torch.equal(pos, ep)
+    go = torch.randn(128, 128, 1024, generator=g)
+    gx = torch.empty(128, 1152, 1024, device=DEV)
+    gw = torch.empty(128, 288, device=DEV)
+    cpp.inf_dist_backward_input_overwrite(go.to(DEV), pos.to(DEV), gx, 4)
+    cpp.inf_dist_backward_weight_overwrite(go.to(DEV), pos.to(DEV), gw, 4)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(gx.cpu(), oracle.inf_dist_backward_input(go, ep, 1152, 4), rtol=1e-5, atol=1e-6)
+    # 131072 contributions per weight row: compare against the double sum with a scale-aware bound
+    ew = oracle.inf_dist_backward_weight(go, ep, 1152, 4)
+    torch.testing.assert_close(gw.cpu(), ew, rtol=1e-4, atol=2e-3)
