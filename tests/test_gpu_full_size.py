@@ -15,6 +15,14 @@ from helpers import assert_sum_close, gen
 pytestmark = pytest.mark.gpu
 
 
+def _scatter_magnitudes(go, pos, ci, G):
+    """Sum of |g| landing on every gradient element: the scale of float32 rounding in the scatter sums."""
+    mag_pos = pos & 0x7FFFFFFF                       # sign bit cleared: every contribution counts as +|g|
+    mx = oracle.inf_dist_backward_input(go.abs(), mag_pos, ci, G)
+    mw = -oracle.inf_dist_backward_weight(go.abs(), mag_pos, ci, G)
+    return mx, mw
+
+
 def _layer(B, CI, CO, seed=0):
     g = gen(seed)
     x = torch.rand(B, CI, 1, generator=g)
@@ -46,8 +54,10 @@ def test_config1_hidden_layer_forward_and_backward(ci):
     cpp.inf_dist_backward_input_overwrite(go.to(DEV), pos.to(DEV), gx, 1)
     cpp.inf_dist_backward_weight_overwrite(go.to(DEV), pos.to(DEV), gw, 1)
     torch.cuda.synchronize()
-    torch.testing.assert_close(gx.cpu(), oracle.inf_dist_backward_input(go, ep, ci, 1), rtol=1e-5, atol=1e-6)
-    torch.testing.assert_close(gw.cpu(), oracle.inf_dist_backward_weight(go, ep, ci, 1), rtol=1e-5, atol=1e-6)
+    # thousands of O(1) gradients can land on one input here: rel 1e-5 / abs 1e-6 relative to sum|g|
+    mx, mw = _scatter_magnitudes(go, ep, ci, 1)
+    assert_sum_close(gx.cpu(), oracle.inf_dist_backward_input(go, ep, ci, 1), mx)
+    assert_sum_close(gw.cpu(), oracle.inf_dist_backward_weight(go, ep, ci, 1), mw)
 
 
 def test_config1_head_forward_bit_exact():
@@ -120,7 +130,7 @@ def test_config4_unfolded_conv_layer():
     cpp.inf_dist_backward_input_overwrite(go.to(DEV), pos.to(DEV), gx, 4)
     cpp.inf_dist_backward_weight_overwrite(go.to(DEV), pos.to(DEV), gw, 4)
     torch.cuda.synchronize()
-    torch.testing.assert_close(gx.cpu(), oracle.inf_dist_backward_input(go, ep, 1152, 4), rtol=1e-5, atol=1e-6)
-    # 131072 contributions per weight row: compare against the double sum with a scale-aware bound
-    ew = oracle.inf_dist_backward_weight(go, ep, 1152, 4)
-    torch.testing.assert_close(gw.cpu(), ew, rtol=1e-4, atol=2e-3)
+    # 131072 contributions per weight row: rel 1e-5 / abs 1e-6 relative to sum|g| per element
+    mx, mw = _scatter_magnitudes(go, ep, 1152, 4)
+    assert_sum_close(gx.cpu(), oracle.inf_dist_backward_input(go, ep, 1152, 4), mx)
+    assert_sum_close(gw.cpu(), oracle.inf_dist_backward_weight(go, ep, 1152, 4), mw)
