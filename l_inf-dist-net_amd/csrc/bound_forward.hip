@@ -120,8 +120,8 @@ bound_forward_kernel(const float* __restrict__ lower, const float* __restrict__ 
                 }
     }
 
-    store_patch<GEO, CONV>(out_lower, lo, d, m0, n0, g, tx, ty, 0xFFu, d.ovec != 0);
-    store_patch<GEO, CONV>(out_upper, up, d, m0, n0, g, tx, ty, 0xFFu, d.ovec != 0);
+    store_patch<GEO, CONV>(out_lower, lo, d, m0, n0, g, tx, ty, d.ovec != 0);
+    store_patch<GEO, CONV>(out_upper, up, d, m0, n0, g, tx, ty, d.ovec != 0);
 }
 
 // Few outputs per group: lanes split k and apply the reference's literal predicate.

@@ -113,72 +113,79 @@ struct RowAddr {
     }
 };
 
-// Writes one lane's TM x TN patch of a result tensor.  When `vec` is set (base
-// pointer 16-byte aligned, NG % 4 == 0 in the fc layout, HW % 4 == 0 in the conv
-// layout) each run of four values along the contiguous axis (n for fc, the row
-// index for conv) that lies fully inside the tensor goes out as one 128-bit
-// store; everything else falls back to single stores.  `rows` selects which of
-// the lane's rows to write (bit i = row i), in whole runs of four.
+// Writes one run of four consecutive rows (global rows m_first .. m_first+3) times the
+// lane's TN columns of a result tensor.  When `vec` is set (base pointer 16-byte aligned,
+// NG % 4 == 0 in the fc layout, HW % 4 == 0 in the conv layout) every group of four values
+// along the contiguous axis (n for fc, the row index for conv) that lies fully inside the
+// tensor goes out as one 128-bit store; everything else falls back to single stores.
 template <class GEO, bool CONV, class T>
-__device__ __forceinline__ void store_patch(T* __restrict__ dst, const T (&val)[GEO::TM][GEO::TN], const Dims& d,
-                                            int m0, int n0, int g, int tx, int ty, unsigned rows, bool vec) {
-    constexpr int TM = GEO::TM, TN = GEO::TN;
+__device__ __forceinline__ void store_run(T* __restrict__ dst, const T (&val)[4][GEO::TN], const Dims& d, int m_first,
+                                          int n0, int g, int tx, bool vec) {
+    constexpr int TN = GEO::TN;
     using V4 = typename std::conditional<std::is_same<T, float>::value, float4, int4>::type;
     if constexpr (!CONV) {
 #pragma unroll
-        for (int i = 0; i < TM; i++) {
-            if (!((rows >> i) & 1)) continue;
-            const int m = m0 + GEO::row(ty, i);
+        for (int e = 0; e < 4; e++) {
+            const int m = m_first + e;
             if (m >= d.M) continue;
             T* row = dst + ((size_t)m * d.G + g) * d.NG;
 #pragma unroll
-            for (int r = 0; r < TN / 4; r++) {  // the lane's columns come in runs of four
+            for (int r = 0; r < TN / 4; r++) {  // the lane's columns come in groups of four
                 const int j = 4 * r;
                 const int n = n0 + GEO::col(tx, j);
                 if (vec && n + 3 < d.NG) {
                     V4 q;
-                    q.x = val[i][j]; q.y = val[i][j + 1]; q.z = val[i][j + 2]; q.w = val[i][j + 3];
+                    q.x = val[e][j]; q.y = val[e][j + 1]; q.z = val[e][j + 2]; q.w = val[e][j + 3];
                     *reinterpret_cast<V4*>(row + n) = q;
                 } else {
 #pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        if (n + e < d.NG) row[n + e] = val[i][j + e];
+                    for (int c = 0; c < 4; c++)
+                        if (n + c < d.NG) row[n + c] = val[e][j + c];
                 }
             }
 #pragma unroll
             for (int j = TN / 4 * 4; j < TN; j++) {
                 const int n = n0 + GEO::col(tx, j);
-                if (n < d.NG) row[n] = val[i][j];
+                if (n < d.NG) row[n] = val[e][j];
             }
         }
     } else {
+        if (m_first >= d.M) return;
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const int n = n0 + GEO::col(tx, j);
             if (n >= d.NG) continue;
+            if (vec && m_first + 3 < d.M) {  // HW % 4 == 0 keeps the four rows inside one image
+                const int b = m_first / d.HW, hw = m_first % d.HW;
+                V4 q;
+                q.x = val[0][j]; q.y = val[1][j]; q.z = val[2][j]; q.w = val[3][j];
+                *reinterpret_cast<V4*>(dst + ((size_t)(b * d.G + g) * d.NG + n) * d.HW + hw) = q;
+            } else {
 #pragma unroll
-            for (int r = 0; r < TM / 4; r++) {  // the lane's rows come in runs of four
-                const int i = 4 * r;
-                if (((rows >> i) & 0xF) != 0xF) continue;  // a run is written by one k-group as a whole
-                const int m = m0 + GEO::row(ty, i);
-                if (m >= d.M) continue;
-                if (vec && m + 3 < d.M) {  // HW % 4 == 0 keeps the four rows inside one image
-                    const int b = m / d.HW, hw = m % d.HW;
-                    V4 q;
-                    q.x = val[i][j]; q.y = val[i + 1][j]; q.z = val[i + 2][j]; q.w = val[i + 3][j];
-                    *reinterpret_cast<V4*>(dst + ((size_t)(b * d.G + g) * d.NG + n) * d.HW + hw) = q;
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const int me = m + e;
-                        if (me < d.M) {
-                            const int b = me / d.HW, hw = me % d.HW;
-                            dst[((size_t)(b * d.G + g) * d.NG + n) * d.HW + hw] = val[i + e][j];
-                        }
+                for (int e = 0; e < 4; e++) {
+                    const int me = m_first + e;
+                    if (me < d.M) {
+                        const int b = me / d.HW, hw = me % d.HW;
+                        dst[((size_t)(b * d.G + g) * d.NG + n) * d.HW + hw] = val[e][j];
                     }
                 }
             }
         }
+    }
+}
+
+// Writes a lane's whole TM x TN patch (its rows come in runs of four, see Geo::row).
+template <class GEO, bool CONV, class T>
+__device__ __forceinline__ void store_patch(T* __restrict__ dst, const T (&val)[GEO::TM][GEO::TN], const Dims& d,
+                                            int m0, int n0, int g, int tx, int ty, bool vec) {
+#pragma unroll
+    for (int r = 0; r < GEO::TM / 4; r++) {
+        T run[4][GEO::TN];
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+#pragma unroll
+            for (int j = 0; j < GEO::TN; j++) run[e][j] = val[4 * r + e][j];
+        store_run<GEO, CONV>(dst, run, d, m0 + GEO::row(ty, 4 * r), n0, g, tx, vec);
     }
 }
 

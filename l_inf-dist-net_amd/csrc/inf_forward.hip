@@ -101,71 +101,146 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
         __syncthreads();
     }
 
-    // Merge the two k-groups.  Each group finishes half of the lane's rows, so it needs the
-    // other group's candidates for that half only: the larger value wins, equal values keep
-    // the lower chunk (or the lower k when k itself was tracked).
+    // Merge the two k-groups.  Each group finishes half of the lane's rows (one run of four),
+    // so it needs the other group's candidates for that half only: the larger value wins,
+    // equal values keep the lower chunk (or the lower k when k itself was tracked).
     static_assert(KS == 1 || KS == 2, "the merge below pairs two k-groups");
+    static_assert(TM == 8, "a lane's rows are two runs of four");
     constexpr int TMH = TM / KS;          // rows finished by each group
+    float best[TMH][TN];                  // this group's share, compacted
+    int where[TMH][TN];
     if constexpr (KS == 2) {
         float* mv = lds;  // [2 groups][TMH*TN][NGRP] values, then as many chunk ids
         int* mi = reinterpret_cast<int*>(lds) + 2 * TMH * TN * NGRP;
 #pragma unroll
-        for (int i = 0; i < TM; i++) {
-            const bool mine = (i / TMH) == grp;
-            if (mine) continue;  // rows of the other group: hand my candidates over
+        for (int ii = 0; ii < TMH; ii++)
 #pragma unroll
             for (int j = 0; j < TN; j++) {
-                const int o = (((1 - grp) * TMH + (i % TMH)) * TN + j) * NGRP + t;
-                mv[o] = acc[i][j];
-                mi[o] = cidx[i][j];
+                // hand over my candidates for the rows the other group finishes, keep the rest
+                const int o = (((1 - grp) * TMH + ii) * TN + j) * NGRP + t;
+                mv[o] = grp ? acc[ii][j] : acc[TMH + ii][j];
+                mi[o] = grp ? cidx[ii][j] : cidx[TMH + ii][j];
+                best[ii][j] = grp ? acc[TMH + ii][j] : acc[ii][j];
+                where[ii][j] = grp ? cidx[TMH + ii][j] : cidx[ii][j];
             }
-        }
         __syncthreads();
 #pragma unroll
-        for (int i = 0; i < TM; i++) {
-            if ((i / TMH) != grp) continue;
+        for (int ii = 0; ii < TMH; ii++)
 #pragma unroll
             for (int j = 0; j < TN; j++) {
-                const int o = ((grp * TMH + (i % TMH)) * TN + j) * NGRP + t;
+                const int o = ((grp * TMH + ii) * TN + j) * NGRP + t;
                 const float v = mv[o];
                 const int ci = mi[o];
-                if (v > acc[i][j] || (v == acc[i][j] && ci < cidx[i][j])) { acc[i][j] = v; cidx[i][j] = ci; }
+                if (v > best[ii][j] || (v == best[ii][j] && ci < where[ii][j])) { best[ii][j] = v; where[ii][j] = ci; }
             }
-        }
+    } else {
+#pragma unroll
+        for (int ii = 0; ii < TMH; ii++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) { best[ii][j] = acc[ii][j]; where[ii][j] = cidx[ii][j]; }
     }
+    const int i_first = KS == 2 ? grp * TMH : 0;   // first of the lane's rows this group finishes
 
-    // Locate the argmax inside the recorded chunk, then write both outputs.
-    int ppos[TM][TN];
-    unsigned rows = 0;
+    // Turn the recorded chunk (or k) into the reference's pos, then write both outputs.
+    int ppos[TMH][TN];
+    auto row_of = [&](int ii) { return m0 + GEO::row(ty, i_first + ii); };
+    if constexpr (!EXACT && !CONV && VEC == 4) {
+        // fc layout: both 32-wide rows are contiguous and 16-byte aligned.  The lane's outputs are
+        // walked in a rolled loop, two per trip, and the 16 loads of the next output are in flight
+        // while the current one is searched.  A rolled loop needs run-time indexing, so each lane
+        // parks its (value, chunk) pairs in LDS (free by now) as park[o][lane] and puts the
+        // resulting pos back in place of the chunk.  Rows and columns past the edge of the tensor
+        // read a clamped, valid address and are never stored.
+        constexpr int NOUT = TMH * TN;
+        static_assert(NOUT % 2 == 0, "two outputs per trip");
+        __syncthreads();   // everyone is done with the merge area
+        float* park_v = lds;
+        int* park_c = reinterpret_cast<int*>(lds) + NOUT * GEO::NT;
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
+        for (int ii = 0; ii < TMH; ii++)
 #pragma unroll
-        for (int j = 0; j < TN; j++) ppos[i][j] = 0;
-        if (KS == 2 && (i / TMH) != grp) continue;
-        rows |= 1u << i;
-        const int m = m0 + GEO::row(ty, i);
-        if (m >= d.M) continue;
-        const RowAddr<CONV> ra(d, m, g);
+            for (int j = 0; j < TN; j++) {
+                park_v[(ii * TN + j) * GEO::NT + tid] = best[ii][j];
+                park_c[(ii * TN + j) * GEO::NT + tid] = where[ii][j];
+            }
+        struct Slot { float4 x[kChunk / 4], w[kChunk / 4]; };
+        auto issue = [&](int o, Slot& sl) {
+            const int ii = o / TN, j = o - ii * TN;
+            const int m = min(row_of(ii), d.M - 1), n = min(n0 + GEO::col(tx, j), d.NG - 1);
+            const int kb = park_c[o * GEO::NT + tid] * kChunk;
+            const int len = min(kChunk, K - kb);
+            const float4* xr = reinterpret_cast<const float4*>(input + ((size_t)m * d.G + g) * K + kb);
+            const float4* wr = reinterpret_cast<const float4*>(weight + ((size_t)g * d.NG + n) * K + kb);
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const int n = n0 + GEO::col(tx, j);
-            const float best = acc[i][j];
-            if (n < d.NG && best > 0.f) {
-                if constexpr (EXACT) {
-                    const int k = cidx[i][j];  // only the sign of the difference is missing
-                    const float df = input[ra.x + (size_t)k * ra.xk] - weight[((size_t)g * d.NG + n) * K + k];
-                    ppos[i][j] = k | (__float_as_int(df) & 0x80000000);
-                } else {
-                    const int kb = cidx[i][j] * kChunk;
-                    const float* xr = input + ra.x + (size_t)kb * ra.xk;
-                    const float* wr = weight + ((size_t)g * d.NG + n) * K + kb;
-                    ppos[i][j] = locate_in_chunk<(!CONV && VEC == 4)>(xr, ra.xk, wr, min(kChunk, K - kb), best, kb);
+            for (int q = 0; q < kChunk / 4; q++) {
+                const int qq = q * 4 < len ? q : 0;   // past the end of the row: re-read the start, masked below
+                sl.x[q] = xr[qq];
+                sl.w[q] = wr[qq];
+            }
+        };
+        auto finish = [&](int o, const Slot& sl) {
+            const int kb = park_c[o * GEO::NT + tid] * kChunk;
+            const int len = min(kChunk, K - kb);
+            const float target = park_v[o * GEO::NT + tid];
+            int p = 0;
+#pragma unroll
+            for (int k = kChunk - 1; k >= 0; k--) {  // descending: the lowest match is written last
+                const float4 xq = sl.x[k / 4], wq = sl.w[k / 4];
+                const float xv = k % 4 == 0 ? xq.x : k % 4 == 1 ? xq.y : k % 4 == 2 ? xq.z : xq.w;
+                const float wv = k % 4 == 0 ? wq.x : k % 4 == 1 ? wq.y : k % 4 == 2 ? wq.z : wq.w;
+                const float df = xv - wv;
+                if (k < len && __builtin_fabsf(df) == target) p = (kb + k) | (__float_as_int(df) & 0x80000000);
+            }
+            park_c[o * GEO::NT + tid] = target > 0.f ? p : 0;
+        };
+        Slot sa, sb;
+        issue(0, sa);
+#pragma unroll 1
+        for (int o = 0; o < NOUT; o += 2) {
+            issue(o + 1, sb);
+            finish(o, sa);
+            issue(min(o + 2, NOUT - 1), sa);   // the last trip fetches a spare copy and drops it
+            finish(o + 1, sb);
+        }
+#pragma unroll
+        for (int ii = 0; ii < TMH; ii++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) ppos[ii][j] = park_c[(ii * TN + j) * GEO::NT + tid];
+    } else {
+#pragma unroll
+        for (int ii = 0; ii < TMH; ii++) {
+            const int m = row_of(ii);
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                const int n = n0 + GEO::col(tx, j);
+                ppos[ii][j] = 0;
+                if (m < d.M && n < d.NG && best[ii][j] > 0.f) {
+                    const RowAddr<CONV> ra(d, m, g);
+                    if constexpr (EXACT) {
+                        const int k = where[ii][j];  // only the sign of the difference is missing
+                        const float df = input[ra.x + (size_t)k * ra.xk] - weight[((size_t)g * d.NG + n) * K + k];
+                        ppos[ii][j] = k | (__float_as_int(df) & 0x80000000);
+                    } else {
+                        const int kb = where[ii][j] * kChunk;
+                        ppos[ii][j] = locate_in_chunk<false>(input + ra.x + (size_t)kb * ra.xk, ra.xk,
+                                                             weight + ((size_t)g * d.NG + n) * K + kb,
+                                                             min(kChunk, K - kb), best[ii][j], kb);
+                    }
                 }
             }
         }
     }
-    store_patch<GEO, CONV>(output, acc, d, m0, n0, g, tx, ty, rows, d.ovec != 0);
-    store_patch<GEO, CONV>(pos, ppos, d, m0, n0, g, tx, ty, rows, d.ovec != 0);
+#pragma unroll
+    for (int r = 0; r < TMH / 4; r++) {
+        float vrun[4][TN];
+        int prun[4][TN];
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) { vrun[e][j] = best[4 * r + e][j]; prun[e][j] = ppos[4 * r + e][j]; }
+        store_run<GEO, CONV>(output, vrun, d, row_of(4 * r), n0, g, tx, d.ovec != 0);
+        store_run<GEO, CONV>(pos, prun, d, row_of(4 * r), n0, g, tx, d.ovec != 0);
+    }
 }
 
 // Above this K the chunk re-read is cheaper than tracking k in the loop (conv layout).
@@ -176,7 +251,10 @@ struct InfForward {
     template <bool EXACT>
     static hipError_t go(unsigned grid, const Dims& d, int device, hipStream_t stream, const float* input,
                          const float* weight, float* output, int32_t* pos) {
-        const size_t lds = Stager<GEO, CONV, VEC, 1>::LDS_BYTES;
+        // pipeline buffers, or the per-lane (value, chunk) parking area of the epilogue if larger
+        constexpr size_t park = (size_t)(GEO::TM / GEO::KS) * GEO::TN * GEO::NT * 2 * sizeof(float);
+        constexpr size_t pipe = Stager<GEO, CONV, VEC, 1>::LDS_BYTES;
+        const size_t lds = (!EXACT && !CONV && VEC == 4 && park > pipe) ? park : pipe;
         auto kern = inf_forward_kernel<GEO, CONV, VEC, EXACT>;
         if (hipError_t e = allow_lds(kern, lds, device); e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(grid), dim3(GEO::NT), lds, stream, input, weight, output, pos, d);

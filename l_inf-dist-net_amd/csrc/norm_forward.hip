@@ -137,7 +137,7 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
     for (int i = 0; i < TM; i++)
 #pragma unroll
         for (int j = 0; j < TN; j++) acc[i][j] = pow_pos(acc[i][j], inv_p) * mx[i][j];
-    store_patch<GEO, CONV>(output, acc, d, m0, n0, g, tx, ty, 0xFFu, d.ovec != 0);
+    store_patch<GEO, CONV>(output, acc, d, m0, n0, g, tx, ty, d.ovec != 0);
 }
 
 // Few outputs per group: two passes over k, first the exact maximum per (row, output),
