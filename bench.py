@@ -363,7 +363,7 @@ def main():
     print(json.dumps(out))
 
 
-TRAFFIC_C1_BYTES = 3.5e8
+TRAFFIC_C1_BYTES = 3.35e8
 
 
 if __name__ == "__main__":
