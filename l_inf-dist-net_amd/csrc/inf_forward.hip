@@ -145,67 +145,85 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
     int ppos[TMH][TN];
     auto row_of = [&](int ii) { return m0 + GEO::row(ty, i_first + ii); };
     if constexpr (!EXACT && !CONV && VEC == 4) {
-        // fc layout: both 32-wide rows are contiguous and 16-byte aligned.  The lane's outputs are
-        // walked in a rolled loop, two per trip, and the 16 loads of the next output are in flight
-        // while the current one is searched.  A rolled loop needs run-time indexing, so each lane
-        // parks its (value, chunk) pairs in LDS (free by now) as park[o][lane] and puts the
-        // resulting pos back in place of the chunk.  Rows and columns past the edge of the tensor
-        // read a clamped, valid address and are never stored.
-        constexpr int NOUT = TMH * TN;
-        static_assert(NOUT % 2 == 0, "two outputs per trip");
+        // fc layout: a recorded chunk is 128 contiguous, 16-byte aligned bytes of the x row and of
+        // the w row.  Eight neighbouring lanes take one output: each loads 16 bytes of both rows,
+        // so a wave's load instruction touches 8 whole lines instead of 64 partial ones (a lane
+        // that walks its own outputs alone is bound by the tag look-ups of the vector cache, not
+        // by bytes).  The lowest matching k is the match of the lowest lane that has one: a ballot
+        // tells every lane whether a lower lane of its eight matched.  The (value, chunk) pairs of
+        // the whole tile are parked in LDS (free by now) as cand[row][col]; pos replaces the chunk.
+        // Rows and columns past the edge of the tensor read a clamped, valid address and are never
+        // stored.
+        constexpr int LPO = kChunk / 4;             // lanes per output
+        constexpr int NGQ = GEO::NT / LPO;          // outputs in flight per trip of the workgroup
+        constexpr int NIT = BM * BN / NGQ;          // trips
+        constexpr int DEPTH = 4;                    // outputs per lane group whose loads are issued together
+        static_assert(BM * BN % NGQ == 0 && NIT % (2 * DEPTH) == 0, "whole batches");
         __syncthreads();   // everyone is done with the merge area
-        float* park_v = lds;
-        int* park_c = reinterpret_cast<int*>(lds) + NOUT * GEO::NT;
+        float* cand_v = lds;
+        int* cand_c = reinterpret_cast<int*>(lds) + BM * BN;
 #pragma unroll
         for (int ii = 0; ii < TMH; ii++)
 #pragma unroll
             for (int j = 0; j < TN; j++) {
-                park_v[(ii * TN + j) * GEO::NT + tid] = best[ii][j];
-                park_c[(ii * TN + j) * GEO::NT + tid] = where[ii][j];
+                const int o = GEO::row(ty, i_first + ii) * BN + GEO::col(tx, j);
+                cand_v[o] = best[ii][j];
+                cand_c[o] = where[ii][j];
             }
-        struct Slot { float4 x[kChunk / 4], w[kChunk / 4]; };
-        auto issue = [&](int o, Slot& sl) {
-            const int ii = o / TN, j = o - ii * TN;
-            const int m = min(row_of(ii), d.M - 1), n = min(n0 + GEO::col(tx, j), d.NG - 1);
-            const int kb = park_c[o * GEO::NT + tid] * kChunk;
-            const int len = min(kChunk, K - kb);
-            const float4* xr = reinterpret_cast<const float4*>(input + ((size_t)m * d.G + g) * K + kb);
-            const float4* wr = reinterpret_cast<const float4*>(weight + ((size_t)g * d.NG + n) * K + kb);
-#pragma unroll
-            for (int q = 0; q < kChunk / 4; q++) {
-                const int qq = q * 4 < len ? q : 0;   // past the end of the row: re-read the start, masked below
-                sl.x[q] = xr[qq];
-                sl.w[q] = wr[qq];
-            }
+        __syncthreads();
+        const int sub = tid % LPO, gq = tid / LPO;
+        const int shift = (tid & 63) - sub;         // bit of this lane group's first lane in a ballot
+        const float* xg = input + (size_t)g * K + 4 * sub;
+        const float* wg = weight + (size_t)g * d.NG * K + 4 * sub;
+        struct Slot { float4 x, w; int kb; };
+        // element offsets fit 32 bits: the entry point rejects tensors of 2^31 elements or more
+        const unsigned ldx = (unsigned)d.G * K;
+        auto issue = [&](int it, Slot& sl) {
+            if (it >= NIT) return;                       // the last trip has nothing left to prefetch
+            const int o = it * NGQ + gq;
+            const int ml = o / BN, nl = o - ml * BN;
+            const unsigned m = min(m0 + ml, d.M - 1), n = min(n0 + nl, d.NG - 1);
+            const int kb = cand_c[o] * kChunk;
+            const unsigned off = kb + 4 * sub < K ? kb : kb - 4 * sub;   // past the end of the row: its first 16 bytes, masked below
+            sl.kb = kb;
+            sl.x = *reinterpret_cast<const float4*>(xg + (m * ldx + off));
+            sl.w = *reinterpret_cast<const float4*>(wg + (n * (unsigned)K + off));
         };
-        auto finish = [&](int o, const Slot& sl) {
-            const int kb = park_c[o * GEO::NT + tid] * kChunk;
-            const int len = min(kChunk, K - kb);
-            const float target = park_v[o * GEO::NT + tid];
-            int p = 0;
-#pragma unroll
-            for (int k = kChunk - 1; k >= 0; k--) {  // descending: the lowest match is written last
-                const float4 xq = sl.x[k / 4], wq = sl.w[k / 4];
-                const float xv = k % 4 == 0 ? xq.x : k % 4 == 1 ? xq.y : k % 4 == 2 ? xq.z : xq.w;
-                const float wv = k % 4 == 0 ? wq.x : k % 4 == 1 ? wq.y : k % 4 == 2 ? wq.z : wq.w;
-                const float df = xv - wv;
-                if (k < len && __builtin_fabsf(df) == target) p = (kb + k) | (__float_as_int(df) & 0x80000000);
-            }
-            park_c[o * GEO::NT + tid] = target > 0.f ? p : 0;
+        auto finish = [&](int it, const Slot& sl) {
+            const int o = it * NGQ + gq;
+            const float target = cand_v[o];
+            const float d0 = sl.x.x - sl.w.x, d1 = sl.x.y - sl.w.y, d2 = sl.x.z - sl.w.z, d3 = sl.x.w - sl.w.w;
+            int q = -1;
+            float df = 0.f;
+            if (__builtin_fabsf(d3) == target) { q = 3; df = d3; }   // descending: the lowest match is kept
+            if (__builtin_fabsf(d2) == target) { q = 2; df = d2; }
+            if (__builtin_fabsf(d1) == target) { q = 1; df = d1; }
+            if (__builtin_fabsf(d0) == target) { q = 0; df = d0; }
+            const int k = sl.kb + 4 * sub + q;
+            const bool hit = q >= 0 && sl.kb + 4 * sub < K && target > 0.f;
+            const unsigned mine = (unsigned)(__builtin_amdgcn_ballot_w64(hit) >> shift) & ((1u << LPO) - 1);
+            if (hit && (mine & ((1u << sub) - 1)) == 0) cand_c[o] = k | (__float_as_int(df) & 0x80000000);
+            if (sub == 0 && mine == 0) cand_c[o] = 0;
         };
-        Slot sa, sb;
-        issue(0, sa);
+        Slot sa[DEPTH], sb[DEPTH];
+#pragma unroll
+        for (int e = 0; e < DEPTH; e++) issue(e, sa[e]);
 #pragma unroll 1
-        for (int o = 0; o < NOUT; o += 2) {
-            issue(o + 1, sb);
-            finish(o, sa);
-            issue(min(o + 2, NOUT - 1), sa);   // the last trip fetches a spare copy and drops it
-            finish(o + 1, sb);
+        for (int it = 0; it < NIT; it += 2 * DEPTH) {
+#pragma unroll
+            for (int e = 0; e < DEPTH; e++) issue(it + DEPTH + e, sb[e]);
+#pragma unroll
+            for (int e = 0; e < DEPTH; e++) finish(it + e, sa[e]);
+#pragma unroll
+            for (int e = 0; e < DEPTH; e++) issue(it + 2 * DEPTH + e, sa[e]);
+#pragma unroll
+            for (int e = 0; e < DEPTH; e++) finish(it + DEPTH + e, sb[e]);
         }
+        __syncthreads();
 #pragma unroll
         for (int ii = 0; ii < TMH; ii++)
 #pragma unroll
-            for (int j = 0; j < TN; j++) ppos[ii][j] = park_c[(ii * TN + j) * GEO::NT + tid];
+            for (int j = 0; j < TN; j++) ppos[ii][j] = cand_c[GEO::row(ty, i_first + ii) * BN + GEO::col(tx, j)];
     } else {
 #pragma unroll
         for (int ii = 0; ii < TMH; ii++) {
@@ -251,8 +269,8 @@ struct InfForward {
     template <bool EXACT>
     static hipError_t go(unsigned grid, const Dims& d, int device, hipStream_t stream, const float* input,
                          const float* weight, float* output, int32_t* pos) {
-        // pipeline buffers, or the per-lane (value, chunk) parking area of the epilogue if larger
-        constexpr size_t park = (size_t)(GEO::TM / GEO::KS) * GEO::TN * GEO::NT * 2 * sizeof(float);
+        // pipeline buffers, or the tile's (value, chunk) parking area of the epilogue if larger
+        constexpr size_t park = (size_t)GEO::BM * GEO::BN * 2 * sizeof(float);
         constexpr size_t pipe = Stager<GEO, CONV, VEC, 1>::LDS_BYTES;
         const size_t lds = (!EXACT && !CONV && VEC == 4 && park > pipe) ? park : pipe;
         auto kern = inf_forward_kernel<GEO, CONV, VEC, EXACT>;
