@@ -69,7 +69,8 @@ bound_forward_kernel(const float* __restrict__ lower, const float* __restrict__ 
                     }
             });
         } else {
-            sweep_chunk<GEO, 2, 1>(xp, wp, tx, ty, [&](const Frag<GEO, 2, 1>& f, int) {
+            // rare path, kept lean: a second pipelined sweep here would push the hot loop into scratch
+            sweep_chunk_plain<GEO, 2>(xp, wp, tx, ty, [&](const Frag<GEO, 2, 1>& f, int) {
 #pragma unroll
                 for (int i = 0; i < TM; i++)
 #pragma unroll

@@ -126,7 +126,9 @@ struct Frag {
 // 2*KP rows per trip, as two fragments: the operands of the next fragment are
 // fetched from LDS while the current one is being reduced.  The loop is kept
 // rolled on purpose: unrolled, the compiler hoists every LDS read of the chunk
-// above the arithmetic and spills the accumulators.
+// above the arithmetic and spills the accumulators.  Without the scheduling
+// barriers it sinks each fetch down to its first use, which puts the LDS
+// latency back on the critical path.
 template <class GEO, int NX, int KP, class F>
 __device__ __forceinline__ void sweep_chunk(const float* xp, const float* wp, int tx, int ty, F&& f) {
     static_assert(KP == 1 || KP == 2, "a trip must stay inside one aligned run of four rows");
@@ -138,11 +140,27 @@ __device__ __forceinline__ void sweep_chunk(const float* xp, const float* wp, in
 #pragma unroll 1
     for (int kk = 0; kk < kChunk; kk += 2 * KP) {
         b.read(cur, KP, XSTRIDE);
+        __builtin_amdgcn_sched_barrier(0);   // keep each fetch ahead of the arithmetic it overlaps with
         f(a, kk);
         nxt.set(xp, wp, (kk + 2 * KP) & (kChunk - 1), tx, ty);  // the last trip re-reads row 0; harmless
         a.read(nxt, 0, XSTRIDE);
+        __builtin_amdgcn_sched_barrier(0);
         f(b, kk + KP);
         cur = nxt;
+    }
+}
+
+// Same walk without the operand prefetch, one k row per trip: for rarely taken
+// paths that must not add to the register budget of the hot loop.
+template <class GEO, int NX, class F>
+__device__ __forceinline__ void sweep_chunk_plain(const float* xp, const float* wp, int tx, int ty, F&& f) {
+#pragma unroll 1
+    for (int kk = 0; kk < kChunk; kk++) {
+        LanePtr<GEO> lp;
+        lp.set(xp, wp, kk & ~3, tx, ty);
+        Frag<GEO, NX, 1> a;
+        a.read(lp, kk & 3, GEO::XS);
+        f(a, kk);
     }
 }
 
