@@ -28,7 +28,6 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
     constexpr int NGRP = GEO::NGRP;
     using Stage = Stager<GEO, CONV, VEC, 1>;
     constexpr int STAGE = Stage::STAGE, NBUF = Stage::NBUF;
-    static_assert(KS == 1 || 2 * TM * TN * NGRP <= NBUF * STAGE, "merge area fits in the panels");
     extern __shared__ __align__(16) float lds[];
 
     int tm, tn, g;
@@ -101,83 +100,52 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
         __syncthreads();
     }
 
-    // Merge the two k-groups.  Each group finishes half of the lane's rows (one run of four),
-    // so it needs the other group's candidates for that half only: the larger value wins,
-    // equal values keep the lower chunk (or the lower k when k itself was tracked).
-    static_assert(KS == 1 || KS == 2, "the merge below pairs two k-groups");
-    static_assert(TM == 8, "a lane's rows are two runs of four");
-    constexpr int TMH = TM / KS;          // rows finished by each group
-    float best[TMH][TN];                  // this group's share, compacted
-    int where[TMH][TN];
-    if constexpr (KS == 2) {
-        float* mv = lds;  // [2 groups][TMH*TN][NGRP] values, then as many chunk ids
-        int* mi = reinterpret_cast<int*>(lds) + 2 * TMH * TN * NGRP;
+    // Epilogue, independent of the lane patch: the tile's (value, chunk or k) pairs are parked in
+    // LDS (free by now), k-groups merge there in turn, the whole workgroup turns the recorded
+    // chunk into the reference's pos, and the tile goes out with stores along the contiguous axis.
+    // cand index of tile-local (row ml, column nl): the contiguous output axis is innermost.
+    auto slot = [](int ml, int nl) { return CONV ? nl * BM + ml : ml * BN + nl; };
+    float* cand_v = lds;
+    int* cand_c = reinterpret_cast<int*>(lds) + BM * BN;
+#pragma unroll 1
+    for (int turn = 0; turn < KS; turn++) {
+        if (grp == turn) {
 #pragma unroll
-        for (int ii = 0; ii < TMH; ii++)
+            for (int i = 0; i < TM; i++)
 #pragma unroll
-            for (int j = 0; j < TN; j++) {
-                // hand over my candidates for the rows the other group finishes, keep the rest
-                const int o = (((1 - grp) * TMH + ii) * TN + j) * NGRP + t;
-                mv[o] = grp ? acc[ii][j] : acc[TMH + ii][j];
-                mi[o] = grp ? cidx[ii][j] : cidx[TMH + ii][j];
-                best[ii][j] = grp ? acc[TMH + ii][j] : acc[ii][j];
-                where[ii][j] = grp ? cidx[TMH + ii][j] : cidx[ii][j];
-            }
+                for (int j = 0; j < TN; j++) {
+                    const int o = slot(GEO::row(ty, i), GEO::col(tx, j));
+                    bool take = true;
+                    if (turn > 0) {   // larger value wins; equal values keep the lower chunk (or k)
+                        const float v = cand_v[o];
+                        take = acc[i][j] > v || (acc[i][j] == v && cidx[i][j] < cand_c[o]);
+                    }
+                    if (take) { cand_v[o] = acc[i][j]; cand_c[o] = cidx[i][j]; }
+                }
+        }
         __syncthreads();
-#pragma unroll
-        for (int ii = 0; ii < TMH; ii++)
-#pragma unroll
-            for (int j = 0; j < TN; j++) {
-                const int o = ((grp * TMH + ii) * TN + j) * NGRP + t;
-                const float v = mv[o];
-                const int ci = mi[o];
-                if (v > best[ii][j] || (v == best[ii][j] && ci < where[ii][j])) { best[ii][j] = v; where[ii][j] = ci; }
-            }
-    } else {
-#pragma unroll
-        for (int ii = 0; ii < TMH; ii++)
-#pragma unroll
-            for (int j = 0; j < TN; j++) { best[ii][j] = acc[ii][j]; where[ii][j] = cidx[ii][j]; }
     }
-    const int i_first = KS == 2 ? grp * TMH : 0;   // first of the lane's rows this group finishes
 
-    // Turn the recorded chunk (or k) into the reference's pos, then write both outputs.
-    int ppos[TMH][TN];
-    auto row_of = [&](int ii) { return m0 + GEO::row(ty, i_first + ii); };
     if constexpr (!EXACT && !CONV && VEC == 4) {
         // fc layout: a recorded chunk is 128 contiguous, 16-byte aligned bytes of the x row and of
         // the w row.  Eight neighbouring lanes take one output: each loads 16 bytes of both rows,
         // so a wave's load instruction touches 8 whole lines instead of 64 partial ones (a lane
         // that walks its own outputs alone is bound by the tag look-ups of the vector cache, not
         // by bytes).  The lowest matching k is the match of the lowest lane that has one: a ballot
-        // tells every lane whether a lower lane of its eight matched.  The (value, chunk) pairs of
-        // the whole tile are parked in LDS (free by now) as cand[row][col]; pos replaces the chunk.
-        // Rows and columns past the edge of the tensor read a clamped, valid address and are never
-        // stored.
+        // tells every lane whether a lower lane of its eight matched.  Rows and columns past the
+        // edge of the tensor read a clamped, valid address and are never stored.
         constexpr int LPO = kChunk / 4;             // lanes per output
         constexpr int NGQ = GEO::NT / LPO;          // outputs in flight per trip of the workgroup
         constexpr int NIT = BM * BN / NGQ;          // trips
         constexpr int DEPTH = 4;                    // outputs per lane group whose loads are issued together
         static_assert(BM * BN % NGQ == 0 && NIT % (2 * DEPTH) == 0, "whole batches");
-        __syncthreads();   // everyone is done with the merge area
-        float* cand_v = lds;
-        int* cand_c = reinterpret_cast<int*>(lds) + BM * BN;
-#pragma unroll
-        for (int ii = 0; ii < TMH; ii++)
-#pragma unroll
-            for (int j = 0; j < TN; j++) {
-                const int o = GEO::row(ty, i_first + ii) * BN + GEO::col(tx, j);
-                cand_v[o] = best[ii][j];
-                cand_c[o] = where[ii][j];
-            }
-        __syncthreads();
         const int sub = tid % LPO, gq = tid / LPO;
         const int shift = (tid & 63) - sub;         // bit of this lane group's first lane in a ballot
         const float* xg = input + (size_t)g * K + 4 * sub;
         const float* wg = weight + (size_t)g * d.NG * K + 4 * sub;
-        struct Slot { float4 x, w; int kb; };
         // element offsets fit 32 bits: the entry point rejects tensors of 2^31 elements or more
         const unsigned ldx = (unsigned)d.G * K;
+        struct Slot { float4 x, w; int kb; };
         auto issue = [&](int it, Slot& sl) {
             if (it >= NIT) return;                       // the last trip has nothing left to prefetch
             const int o = it * NGQ + gq;
@@ -219,45 +187,74 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
 #pragma unroll
             for (int e = 0; e < DEPTH; e++) finish(it + DEPTH + e, sb[e]);
         }
-        __syncthreads();
-#pragma unroll
-        for (int ii = 0; ii < TMH; ii++)
-#pragma unroll
-            for (int j = 0; j < TN; j++) ppos[ii][j] = cand_c[GEO::row(ty, i_first + ii) * BN + GEO::col(tx, j)];
     } else {
-#pragma unroll
-        for (int ii = 0; ii < TMH; ii++) {
-            const int m = row_of(ii);
-#pragma unroll
-            for (int j = 0; j < TN; j++) {
-                const int n = n0 + GEO::col(tx, j);
-                ppos[ii][j] = 0;
-                if (m < d.M && n < d.NG && best[ii][j] > 0.f) {
-                    const RowAddr<CONV> ra(d, m, g);
-                    if constexpr (EXACT) {
-                        const int k = where[ii][j];  // only the sign of the difference is missing
-                        const float df = input[ra.x + (size_t)k * ra.xk] - weight[((size_t)g * d.NG + n) * K + k];
-                        ppos[ii][j] = k | (__float_as_int(df) & 0x80000000);
-                    } else {
-                        const int kb = where[ii][j] * kChunk;
-                        ppos[ii][j] = locate_in_chunk<false>(input + ra.x + (size_t)kb * ra.xk, ra.xk,
-                                                             weight + ((size_t)g * d.NG + n) * K + kb,
-                                                             min(kChunk, K - kb), best[ii][j], kb);
-                    }
+        // Other layouts: every lane takes outputs tid, tid + NT, ... of the tile on its own.
+#pragma unroll 1
+        for (int o = tid; o < BM * BN; o += GEO::NT) {
+            const int ml = CONV ? o % BM : o / BN, nl = CONV ? o / BM : o % BN;
+            const int m = m0 + ml, n = n0 + nl;
+            const float v = cand_v[o];
+            int p = 0;
+            if (m < d.M && n < d.NG && v > 0.f) {
+                const RowAddr<CONV> ra(d, m, g);
+                const float* wr = weight + ((size_t)g * d.NG + n) * K;
+                if constexpr (EXACT) {
+                    const int k = cand_c[o];  // only the sign of the difference is missing
+                    const float df = input[ra.x + (size_t)k * ra.xk] - wr[k];
+                    p = k | (__float_as_int(df) & 0x80000000);
+                } else {
+                    const int kb = cand_c[o] * kChunk;
+                    p = locate_in_chunk<false>(input + ra.x + (size_t)kb * ra.xk, ra.xk, wr + kb, min(kChunk, K - kb),
+                                               v, kb);
                 }
             }
+            cand_c[o] = p;
         }
     }
+    __syncthreads();
+
+    // Tile -> global.  Groups of four along the contiguous axis (n for fc, the row index for conv)
+    // go out as one 128-bit store where the tensor allows it (d.ovec: bases 16-byte aligned and
+    // NG % 4 == 0, resp. HW % 4 == 0 which keeps four rows inside one image).
+    constexpr int CW = CONV ? BM : BN;              // tile extent along the contiguous axis
+    static_assert(CW % 4 == 0, "");
+#pragma unroll 1
+    for (int q = tid; q < BM * BN / 4; q += GEO::NT) {
+        const int outer = q / (CW / 4), inner = (q % (CW / 4)) * 4;
+        const int ml = CONV ? inner : outer, nl = CONV ? outer : inner;
+        const int m = m0 + ml, n = n0 + nl;
+        if (m >= d.M || n >= d.NG) continue;
+        const float4 v4 = *reinterpret_cast<const float4*>(cand_v + 4 * q);
+        const int4 p4 = *reinterpret_cast<const int4*>(cand_c + 4 * q);
+        const float vs[4] = {v4.x, v4.y, v4.z, v4.w};
+        const int ps[4] = {p4.x, p4.y, p4.z, p4.w};
+        if constexpr (!CONV) {
+            const size_t at = ((size_t)m * d.G + g) * d.NG + n;
+            if (d.ovec && n + 3 < d.NG) {
+                *reinterpret_cast<float4*>(output + at) = v4;
+                *reinterpret_cast<int4*>(pos + at) = p4;
+            } else {
 #pragma unroll
-    for (int r = 0; r < TMH / 4; r++) {
-        float vrun[4][TN];
-        int prun[4][TN];
+                for (int e = 0; e < 4; e++)
+                    if (n + e < d.NG) { output[at + e] = vs[e]; pos[at + e] = ps[e]; }
+            }
+        } else {
+            if (d.ovec && m + 3 < d.M) {
+                const int b = m / d.HW, hw = m % d.HW;
+                const size_t at = ((size_t)(b * d.G + g) * d.NG + n) * d.HW + hw;
+                *reinterpret_cast<float4*>(output + at) = v4;
+                *reinterpret_cast<int4*>(pos + at) = p4;
+            } else {
 #pragma unroll
-        for (int e = 0; e < 4; e++)
-#pragma unroll
-            for (int j = 0; j < TN; j++) { vrun[e][j] = best[4 * r + e][j]; prun[e][j] = ppos[4 * r + e][j]; }
-        store_run<GEO, CONV>(output, vrun, d, row_of(4 * r), n0, g, tx, d.ovec != 0);
-        store_run<GEO, CONV>(pos, prun, d, row_of(4 * r), n0, g, tx, d.ovec != 0);
+                for (int e = 0; e < 4; e++)
+                    if (m + e < d.M) {
+                        const int b = (m + e) / d.HW, hw = (m + e) % d.HW;
+                        const size_t at = ((size_t)(b * d.G + g) * d.NG + n) * d.HW + hw;
+                        output[at] = vs[e];
+                        pos[at] = ps[e];
+                    }
+            }
+        }
     }
 }
 
@@ -272,7 +269,7 @@ struct InfForward {
         // pipeline buffers, or the tile's (value, chunk) parking area of the epilogue if larger
         constexpr size_t park = (size_t)GEO::BM * GEO::BN * 2 * sizeof(float);
         constexpr size_t pipe = Stager<GEO, CONV, VEC, 1>::LDS_BYTES;
-        const size_t lds = (!EXACT && !CONV && VEC == 4 && park > pipe) ? park : pipe;
+        const size_t lds = park > pipe ? park : pipe;
         auto kern = inf_forward_kernel<GEO, CONV, VEC, EXACT>;
         if (hipError_t e = allow_lds(kern, lds, device); e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(grid), dim3(GEO::NT), lds, stream, input, weight, output, pos, d);
