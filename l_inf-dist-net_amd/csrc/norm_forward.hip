@@ -3,17 +3,30 @@
 // that no power can overflow for any p.  Semantics follow the reference kernel
 // model/norm_dist_cuda.cu:228-292: mx and the sum are seeded with 1e-10 (:232-233),
 // and whenever a block of k raises mx the sum is rescaled by (mx_old/mx_new)^p
-// (:257-261).  Here the block is a 32-wide chunk: sweep one finds the chunk
-// maximum (sub + half a max3 per element), the rescale runs once per output,
-// sweep two adds (|x-w| / mx)^p.  p = 2, 3, 4, 8 use multiplies only; any other
-// p goes through v_log_f32 / v_exp_f32.
+// (:257-261).  Here the block is a 32-wide chunk.  For p <= 16 a chunk is normally
+// swept once with the scale left by earlier chunks (see the kernel); otherwise
+// sweep one finds the chunk maximum (sub + half a max3 per element), the rescale
+// runs once per output, sweep two adds (|x-w| / mx)^p.  p = 2, 3, 4, 8 use
+// multiplies only; any other p goes through v_log_f32 / v_exp_f32.
 #include "fwd_engine.hpp"
 #include "pow.hpp"
 #include "skinny.hpp"
 
 namespace ldist {
 
-template <class GEO, bool CONV, int VEC>
+// IP: the exponent when it is one of the multiply-only cases (2, 3, 4, 8), else 0.  A template
+// parameter rather than a run-time switch: one kernel holding all five power sweeps next to
+// the maximum sweep pushed the hot loops into scratch.
+//
+// ONE = true (p <= kOneSweepMaxP): a chunk is swept once.  Any scale s gives the same result,
+// out = s * (sum_k (|x-w|/s)^p)^(1/p); the maximum only keeps the powers in range.  So a chunk
+// adds (|x-w| / s)^p with the scale s left by earlier chunks, and only a wave that sees a chunk
+// sum overflow (or turn NaN) goes back over that chunk the long way: find its maximum, move
+// the scale there as the reference does, add the powers again.  The first chunk always takes
+// that road (the scale starts at the reference's seed 1e-10).  With p <= 16 a chunk may exceed
+// the scale by a factor of 70 before that happens.  ONE = false: every chunk is swept twice
+// (maximum, then powers), for exponents so large that almost any increase would overflow.
+template <class GEO, bool CONV, int VEC, int IP, bool ONE>
 __global__ void __launch_bounds__(GEO::NT, 2)
 norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ weight, float* __restrict__ output,
                     float p, Dims d) {
@@ -30,17 +43,21 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
     const int tid = threadIdx.x;
     const int grp = tid / NGRP, t = tid % NGRP;
     const int tx = t % GEO::TX, ty = t / GEO::TX;
-    const int ip = small_int_power(p);
+    auto power = [p](float v) {
+        if constexpr (IP > 0) return pow_int<IP>(v);
+        else return pow_pos(v, p);
+    };
 
     Stage st;
     const float* const ins[1] = {input};
     st.init(ins, weight, d, m0, n0, g, tid);
 
-    float acc[TM][TN], mx[TM][TN];
+    // acc = sum of (|x-w| * rs)^p over the k seen so far; rs = 1 / scale.  Seeds as in the reference.
+    float acc[TM][TN], rs[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++) { acc[i][j] = grp == 0 ? 1e-10f : 0.f; mx[i][j] = 1e-10f; }
+        for (int j = 0; j < TN; j++) { acc[i][j] = grp == 0 ? 1e-10f : 0.f; rs[i][j] = 1e10f; }
 
     const int nstage = (d.K + KK - 1) / KK;
     st.load(0);
@@ -51,60 +68,96 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
         if (s + 1 < nstage) st.load((s + 1) * KK);
         const float* xp = stage + grp * kChunk * GEO::SM;
         const float* wp = stage + GEO::XS + grp * kChunk * GEO::SN;
-        float cm[TM][TN];  // chunk maximum, then 1 / running maximum
+        float cs[TM][TN];  // chunk maximum, or chunk sum
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
-            for (int j = 0; j < TN; j++) cm[i][j] = 0.f;
-        sweep_chunk<GEO, 1, 2>(xp, wp, tx, ty, [&](const Frag<GEO, 1, 2>& f, int) {
+            for (int j = 0; j < TN; j++) cs[i][j] = 0.f;
+        // moves the scale of every output whose chunk maximum (in cs) exceeds it
+        auto raise_scale = [&]() {
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int j = 0; j < TN; j++) {
-                    const float d0 = __builtin_fabsf(f.x[0][0][i] - f.w[0][j]);
-                    const float d1 = __builtin_fabsf(f.x[0][1][i] - f.w[1][j]);
-                    cm[i][j] = __builtin_fmaxf(__builtin_fmaxf(cm[i][j], d0), d1);
+                    const float r = cs[i][j] * rs[i][j];
+                    if (r > 1.f) {
+                        acc[i][j] *= pow_pos(__builtin_amdgcn_rcpf(r), p);
+                        rs[i][j] = __builtin_amdgcn_rcpf(cs[i][j]);
+                    }
+                    cs[i][j] = 0.f;
                 }
-        });
-#pragma unroll
-        for (int i = 0; i < TM; i++)
-#pragma unroll
-            for (int j = 0; j < TN; j++) {
-                if (cm[i][j] > mx[i][j]) {
-                    acc[i][j] *= pow_pos(mx[i][j] * __builtin_amdgcn_rcpf(cm[i][j]), p);
-                    mx[i][j] = cm[i][j];
-                }
-                cm[i][j] = __builtin_amdgcn_rcpf(mx[i][j]);
-            }
-        auto add_powers = [&](auto power) {
+        };
+        if constexpr (ONE) {
             sweep_chunk<GEO, 1, 2>(xp, wp, tx, ty, [&](const Frag<GEO, 1, 2>& f, int) {
 #pragma unroll
                 for (int i = 0; i < TM; i++)
 #pragma unroll
                     for (int j = 0; j < TN; j++) {
-                        const float v0 = __builtin_fabsf(f.x[0][0][i] - f.w[0][j]) * cm[i][j];
-                        const float v1 = __builtin_fabsf(f.x[0][1][i] - f.w[1][j]) * cm[i][j];
-                        acc[i][j] += power(v0);
-                        acc[i][j] += power(v1);
+                        cs[i][j] += power(__builtin_fabsf(f.x[0][0][i] - f.w[0][j]) * rs[i][j]);
+                        cs[i][j] += power(__builtin_fabsf(f.x[0][1][i] - f.w[1][j]) * rs[i][j]);
                     }
             });
-        };
-        switch (ip) {
-            case 2: add_powers([](float v) { return pow_int<2>(v); }); break;
-            case 3: add_powers([](float v) { return pow_int<3>(v); }); break;
-            case 4: add_powers([](float v) { return pow_int<4>(v); }); break;
-            case 8: add_powers([](float v) { return pow_int<8>(v); }); break;
-            default: add_powers([p](float v) { return pow_pos(v, p); }); break;
+            bool redo = false;
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) redo |= !(cs[i][j] < 1e30f);
+            if (__builtin_amdgcn_ballot_w64(redo) != 0) {   // rare: kept lean, no operand prefetch
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) cs[i][j] = 0.f;
+                sweep_chunk_plain<GEO, 1>(xp, wp, tx, ty, [&](const Frag<GEO, 1, 1>& f, int) {
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int j = 0; j < TN; j++)
+                            cs[i][j] = __builtin_fmaxf(cs[i][j], __builtin_fabsf(f.x[0][0][i] - f.w[0][j]));
+                });
+                raise_scale();
+                sweep_chunk_plain<GEO, 1>(xp, wp, tx, ty, [&](const Frag<GEO, 1, 1>& f, int) {
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int j = 0; j < TN; j++)
+                            cs[i][j] += power(__builtin_fabsf(f.x[0][0][i] - f.w[0][j]) * rs[i][j]);
+                });
+            }
+        } else {
+            sweep_chunk<GEO, 1, 2>(xp, wp, tx, ty, [&](const Frag<GEO, 1, 2>& f, int) {
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) {
+                        const float d0 = __builtin_fabsf(f.x[0][0][i] - f.w[0][j]);
+                        const float d1 = __builtin_fabsf(f.x[0][1][i] - f.w[1][j]);
+                        cs[i][j] = __builtin_fmaxf(__builtin_fmaxf(cs[i][j], d0), d1);
+                    }
+            });
+            raise_scale();
+            sweep_chunk<GEO, 1, 2>(xp, wp, tx, ty, [&](const Frag<GEO, 1, 2>& f, int) {
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) {
+                        cs[i][j] += power(__builtin_fabsf(f.x[0][0][i] - f.w[0][j]) * rs[i][j]);
+                        cs[i][j] += power(__builtin_fabsf(f.x[0][1][i] - f.w[1][j]) * rs[i][j]);
+                    }
+            });
         }
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) acc[i][j] += cs[i][j];
         if (NBUF == 1) __syncthreads();  // everyone is done reading the only buffer
         if (s + 1 < nstage) st.store(lds + ((s + 1) % NBUF) * STAGE);
         __syncthreads();
     }
 
-    // Merge the k-groups onto the common maximum.
+    // Merge the k-groups onto the larger scale.
     if constexpr (KS > 1) {
-        float* ma = lds;  // [KS-1][TM*TN][NGRP] sums, then as many maxima
-        float* mm = lds + (KS - 1) * TM * TN * NGRP;
+        float* ma = lds;  // [KS-1][TM*TN][NGRP] sums, then as many reciprocal scales
+        float* mr = lds + (KS - 1) * TM * TN * NGRP;
         if (grp > 0) {
 #pragma unroll
             for (int i = 0; i < TM; i++)
@@ -112,7 +165,7 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
                 for (int j = 0; j < TN; j++) {
                     const int o = ((grp - 1) * TM * TN + i * TN + j) * NGRP + t;
                     ma[o] = acc[i][j];
-                    mm[o] = mx[i][j];
+                    mr[o] = rs[i][j];
                 }
         }
         __syncthreads();
@@ -124,11 +177,11 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
 #pragma unroll
                 for (int j = 0; j < TN; j++) {
                     const int o = (q * TM * TN + i * TN + j) * NGRP + t;
-                    const float a2 = ma[o], m2 = mm[o];
-                    const float m = __builtin_fmaxf(mx[i][j], m2);
-                    const float r = __builtin_amdgcn_rcpf(m);
-                    acc[i][j] = acc[i][j] * pow_pos(mx[i][j] * r, p) + a2 * pow_pos(m2 * r, p);
-                    mx[i][j] = m;
+                    const float a2 = ma[o], r2 = mr[o];
+                    const float r = __builtin_fminf(rs[i][j], r2);   // the larger scale
+                    acc[i][j] = acc[i][j] * pow_pos(r * __builtin_amdgcn_rcpf(rs[i][j]), p) +
+                                a2 * pow_pos(r * __builtin_amdgcn_rcpf(r2), p);
+                    rs[i][j] = r;
                 }
     }
 
@@ -136,9 +189,12 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++) acc[i][j] = pow_pos(acc[i][j], inv_p) * mx[i][j];
+        for (int j = 0; j < TN; j++) acc[i][j] = pow_pos(acc[i][j], inv_p) * __builtin_amdgcn_rcpf(rs[i][j]);
     store_patch<GEO, CONV>(output, acc, d, m0, n0, g, tx, ty, d.ovec != 0);
 }
+
+// Largest exponent for the one-sweep kernel: 70^16 is about 3e29, inside the overflow test.
+constexpr float kOneSweepMaxP = 16.f;
 
 // Few outputs per group: two passes over k, first the exact maximum per (row, output),
 // then the sum of (|x-w| / max)^p; lanes split k in both.
@@ -211,13 +267,26 @@ norm_forward_skinny_kernel(const float* __restrict__ input, const float* __restr
 
 template <class GEO, bool CONV, int VEC>
 struct NormForward {
-    static hipError_t launch(unsigned grid, const Dims& d, int device, hipStream_t stream, const float* input,
-                             const float* weight, float* output, float p) {
+    template <int IP, bool ONE>
+    static hipError_t go(unsigned grid, const Dims& d, int device, hipStream_t stream, const float* input,
+                         const float* weight, float* output, float p) {
         const size_t lds = Stager<GEO, CONV, VEC, 1>::LDS_BYTES;
-        auto kern = norm_forward_kernel<GEO, CONV, VEC>;
+        auto kern = norm_forward_kernel<GEO, CONV, VEC, IP, ONE>;
         if (hipError_t e = allow_lds(kern, lds, device); e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(grid), dim3(GEO::NT), lds, stream, input, weight, output, p, d);
         return hipGetLastError();
+    }
+    static hipError_t launch(unsigned grid, const Dims& d, int device, hipStream_t stream, const float* input,
+                             const float* weight, float* output, float p) {
+        switch (small_int_power(p)) {
+            case 2: return go<2, true>(grid, d, device, stream, input, weight, output, p);
+            case 3: return go<3, true>(grid, d, device, stream, input, weight, output, p);
+            case 4: return go<4, true>(grid, d, device, stream, input, weight, output, p);
+            case 8: return go<8, true>(grid, d, device, stream, input, weight, output, p);
+            default:
+                return p <= kOneSweepMaxP ? go<0, true>(grid, d, device, stream, input, weight, output, p)
+                                          : go<0, false>(grid, d, device, stream, input, weight, output, p);
+        }
     }
 };
 

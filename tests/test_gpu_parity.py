@@ -163,6 +163,35 @@ def test_norm_forward_scale_robust_and_seeded():
                                atol=0)
 
 
+@pytest.mark.parametrize("tile", [-1, 0, 1])
+@pytest.mark.parametrize("p", [2.0, 3.0, 8.0, 3.5, 16.0, 16.5])
+@pytest.mark.parametrize("profile", ["growing", "shrinking", "spike", "tiny"])
+def test_norm_forward_magnitude_jumps_between_chunks(profile, p, tile):
+    """|x - w| changes by orders of magnitude from one 32-wide chunk of k to the next: the kernel
+    that sweeps a chunk once with the scale of earlier chunks has to notice the overflow and go
+    back over the chunk (growing, spike), and must not lose small later terms (shrinking)."""
+    from gpu_common import gpu_norm_forward, say, set_tile
+    B, CO, K = 70, 90, 416
+    say("norm_forward magnitude jumps", profile, "p", p, "tile", tile)
+    x, w = make_inputs(B, CO, K, 1, 1, seed=11)
+    chunk = torch.arange(K) // 32
+    if profile == "growing":
+        mag = 10.0 ** (2.0 * chunk.float() - 6.0)            # 1e-6 ... 1e18
+    elif profile == "shrinking":
+        mag = 10.0 ** (6.0 - 1.0 * chunk.float())
+    elif profile == "spike":
+        mag = torch.ones(K)
+        mag[200:203] = 1e9
+    else:
+        mag = torch.full((K,), 1e-12)                         # the 1e-10 seeds of the reference matter here
+    xs = (x * mag.view(1, K, 1)).contiguous()
+    ws = (w * mag.view(1, K)).contiguous()
+    set_tile(tile)
+    out = gpu_norm_forward(xs, ws, 1, p)
+    set_tile(-1)
+    torch.testing.assert_close(out, oracle.norm_dist_forward(xs, ws, 1, p), rtol=RTOL, atol=0)
+
+
 @pytest.mark.parametrize("shape", PNORM_SHAPES)
 @pytest.mark.parametrize("p", [8.0, 2.0, 3.0, 4.0, 5.5, 100.0])
 def test_norm_backward(shape, p):
