@@ -110,7 +110,9 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
             }
         }
         __syncthreads();
-        auto reduce = [&](auto power) {
+        // spower(u) = sign(u) * |u|^(p-1) for the signed, normalised difference u = (Q - O) * rinv.
+        // Odd integer exponents keep the sign by themselves, even ones take one factor as |u|.
+        auto reduce = [&](auto spower) {
 #pragma unroll 2
             for (int rr = 0; rr < RB; rr++) {
                 float o[4], c[PA], ri[PA];
@@ -121,20 +123,17 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
 #pragma unroll
                 for (int i = 0; i < PA; i++)
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        const float t = q[i][j] - o[j];
-                        const float pw = power(__builtin_fabsf(t) * ri[i]);
-                        // sign(t) * pw; at t == 0 the power is 0 and the sign is irrelevant
-                        acc[i][j] += c[i] * __builtin_copysignf(pw, t);
-                    }
+                    for (int j = 0; j < 4; j++) acc[i][j] += c[i] * spower((q[i][j] - o[j]) * ri[i]);
             }
         };
         switch (ie) {
             case 1: reduce([](float u) { return u; }); break;
-            case 2: reduce([](float u) { return pow_int<2>(u); }); break;
+            case 2: reduce([](float u) { return u * __builtin_fabsf(u); }); break;
             case 3: reduce([](float u) { return pow_int<3>(u); }); break;
             case 7: reduce([](float u) { return pow_int<7>(u); }); break;
-            default: reduce([e](float u) { return pow_pos(u, e); }); break;
+            default:   // at u == 0 the power is 0 and the sign is irrelevant
+                reduce([e](float u) { return __builtin_copysignf(pow_pos(__builtin_fabsf(u), e), u); });
+                break;
         }
     }
 
