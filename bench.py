@@ -212,7 +212,8 @@ def workload_c3(pkg, torch, dev):
                 name="configs[3]: interval-bound certification forward through the MLP, batch 1024, eps=8/255: "
                      "value path + lower/upper bounds + certified margins (bound-ops and dist-ops both counted)",
                 kernel=("inf_dist_bound_forward", lambda l_, u_, w_, *_: 6 * mnk(l_, w_),
-                        lambda l_, u_, w_, *_: True, "bound_forward_kernel", 6))
+                        lambda l_, u_, w_, *_: w_.size(0) > 16,   # the 10-way head runs another kernel
+                        "bound_forward_kernel (tiled interval-bound forward)", 6))
 
 
 def workload_c4(pkg, torch, dev):

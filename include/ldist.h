@@ -5,9 +5,11 @@
  * DEVICE pointer to float32 / int32 data on the current HIP device, `stream`
  * is a hipStream_t passed as void* (NULL = the default stream).  All calls are
  * asynchronous with respect to the host: they enqueue kernels on `stream` and
- * return.  The library allocates nothing, keeps no state between calls and
- * never frees or retains the caller's buffers, like the reference launchers
- * (model/norm_dist.py:10-15,34,37,42,45,63-64 allocate everything in Python).
+ * return.  The library allocates no device memory and never frees or retains
+ * the caller's buffers, like the reference launchers (model/norm_dist.py:10-15,
+ * 34,37,42,45,63-64 allocate everything in Python).  The only state it keeps
+ * between calls is process-wide: the two tuning knobs below, a cache of device
+ * properties, and which kernels have had their LDS limit raised on a device.
  *
  * Each of the seven core entry points replaces one `*_cuda` launcher declared
  * in the reference's binding (model/norm_dist.cpp:7-20) and keeps its argument

@@ -118,6 +118,29 @@ def inf_dist_bound(input_lower, input_upper, weight, group, use_custom_cuda_func
     return nearest.amax(dim=3).view(shape), hi
 
 
+class _BatchMeanShift(torch.autograd.Function):
+    """flat (B, C, L) minus its per-channel mean over B and L; also returns that mean.
+
+    The forward is the reference's expression (model/norm_dist.py:87-96).  The backward is
+    written out, gx = gy - mean(gy), instead of being left to autograd, whose chain through
+    mean / unsqueeze / sub costs about twice as many small kernels per layer.
+    """
+
+    @staticmethod
+    def _channel_mean(flat):
+        return flat.mean(dim=-1).mean(dim=0) if flat.size(-1) > 1 else flat.squeeze(-1).mean(dim=0)
+
+    @staticmethod
+    def forward(ctx, flat):
+        mean = _BatchMeanShift._channel_mean(flat)
+        ctx.mark_non_differentiable(mean)
+        return flat - mean.unsqueeze(-1), mean
+
+    @staticmethod
+    def backward(ctx, grad_y, _grad_mean):
+        return grad_y - _BatchMeanShift._channel_mean(grad_y).unsqueeze(-1)
+
+
 class MeanNorm(nn.Module):
     """Subtracts a per-channel mean: the batch mean in training mode (which also moves
     ``running_mean`` by ``momentum``), ``running_mean`` in eval mode."""
@@ -131,12 +154,11 @@ class MeanNorm(nn.Module):
     def forward(self, x):
         flat = x.view(x.size(0), x.size(1), -1)
         if self.training:
-            mean = flat.mean(dim=-1).mean(dim=0) if x.dim() > 2 else x.mean(dim=0)
+            shifted, mean = _BatchMeanShift.apply(flat)
             with torch.no_grad():
                 self.running_mean.mul_(1 - self.momentum).add_(mean, alpha=self.momentum)
-        else:
-            mean = self.running_mean
-        return (flat - mean.unsqueeze(-1)).view_as(x)
+            return shifted.view_as(x)
+        return (flat - self.running_mean.unsqueeze(-1)).view_as(x)
 
     def extra_repr(self):
         return str(self.out_channels)

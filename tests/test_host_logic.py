@@ -141,6 +141,15 @@ def test_mean_norm_train_and_eval():
     xg = x.clone().requires_grad_(True)                              # the batch mean carries gradient
     pkg.MeanNorm(3).train()(xg).sum().backward()
     torch.testing.assert_close(xg.grad, torch.zeros_like(x), atol=1e-6, rtol=0)
+    # the hand-written backward of the shift against autograd through the plain formula, float64
+    for shape in ((5, 3, 4, 4), (6, 3)):
+        xa = torch.randn(*shape, generator=gen(12), dtype=torch.float64).requires_grad_(True)
+        xb = xa.detach().clone().requires_grad_(True)
+        up = torch.randn(*shape, generator=gen(13), dtype=torch.float64)
+        pkg.MeanNorm(3).double().train()(xa).backward(up)
+        dims = (0, 2, 3) if len(shape) == 4 else (0,)
+        (xb - xb.mean(dim=dims, keepdim=True)).backward(up)
+        torch.testing.assert_close(xa.grad, xb.grad, rtol=1e-12, atol=1e-12)
 
 
 def naive_dist_conv(x, weight, stride, padding, group, p):
