@@ -364,7 +364,7 @@ def main():
     print(json.dumps(out))
 
 
-TRAFFIC_C1_BYTES = 3.35e8
+TRAFFIC_C1_BYTES = 3.21e8
 
 
 if __name__ == "__main__":
