@@ -133,17 +133,32 @@ template <class GEO, int NX, int KP, class F>
 __device__ __forceinline__ void sweep_chunk(const float* xp, const float* wp, int tx, int ty, F&& f) {
     static_assert(KP == 1 || KP == 2, "a trip must stay inside one aligned run of four rows");
     constexpr int XSTRIDE = GEO::XS;
+    // LDS instructions of one fragment read: 128-bit reads of x and w, plus the fifth column
+    // (its KP 32-bit reads merge into one ds_read2_b32).  LDS returns in order, so waiting until
+    // that many are outstanding means: the fragment fetched before this one has arrived.  The
+    // explicit wait is only a hint that keeps the compiler from waiting for everything
+    // (lgkmcnt(0)) right after a fetch; it still adds whatever wait correctness needs.
+    constexpr int FRAG_LDS = NX * KP * (GEO::TM / 4) + KP * (GEO::TN == 8 ? 2 : 1) + (GEO::TN == 5 ? 1 : 0);
+    constexpr int WAIT_PREV = 0xc07f | (FRAG_LDS << 8);   // vmcnt, expcnt at their maxima; lgkmcnt = FRAG_LDS
+    static_assert(FRAG_LDS < 16, "lgkmcnt field");
     Frag<GEO, NX, KP> a, b;
     LanePtr<GEO> cur, nxt;
     cur.set(xp, wp, 0, tx, ty);
+    // Nothing but this sweep's own LDS reads may be in flight inside the loop: a scalar load left
+    // pending here (they return out of order) would force lgkmcnt(0) at the top of every trip.
+    __builtin_amdgcn_s_waitcnt(0xc07f);
     a.read(cur, 0, XSTRIDE);
 #pragma unroll 1
     for (int kk = 0; kk < kChunk; kk += 2 * KP) {
         b.read(cur, KP, XSTRIDE);
         __builtin_amdgcn_sched_barrier(0);   // keep each fetch ahead of the arithmetic it overlaps with
+        __builtin_amdgcn_s_waitcnt(WAIT_PREV);
+        __builtin_amdgcn_sched_barrier(0);
         f(a, kk);
         nxt.set(xp, wp, (kk + 2 * KP) & (kChunk - 1), tx, ty);  // the last trip re-reads row 0; harmless
         a.read(nxt, 0, XSTRIDE);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(WAIT_PREV);
         __builtin_amdgcn_sched_barrier(0);
         f(b, kk + KP);
         cur = nxt;
