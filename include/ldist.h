@@ -125,6 +125,16 @@ int ldist_inf_dist_backward_input_overwrite(const float* grad_output, const int3
 int ldist_inf_dist_backward_weight_overwrite(const float* grad_output, const int32_t* pos, int B, int CO, int CI,
                                              int G, int HW, float* grad_weight, ldist_stream_t stream);
 
+/* Per-channel mean shift of a contiguous (B, C, L) tensor in one kernel:
+ *   mean[c] = mean over b and l of x[b,c,l];   y[b,c,l] = x[b,c,l] - mean[c]
+ *   running_mean[c] = (1 - momentum) * running_mean[c] + momentum * mean[c]   (when running_mean != NULL)
+ * No native counterpart in the reference: this is the training-mode arithmetic of its MeanNorm
+ * module (model/norm_dist.py:85-96), which runs as five small torch kernels per layer; the backward
+ * pass is the same operation on the gradient (gx = gy - mean(gy)).  mean_out (C floats) and
+ * running_mean may be NULL; y must not overlap x. */
+int ldist_mean_shift(const float* x, int B, int C, int L, float* y, float* mean_out, float* running_mean,
+                     float momentum, ldist_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -70,4 +70,7 @@ hipError_t norm_backward_weight(const float* grad_output, const float* input, co
                                 const float* output, float* grad_weight, float p, const Problem& pr,
                                 hipStream_t stream);
 
+hipError_t mean_shift(const float* x, float* y, float* mean_out, float* running_mean, float momentum, int B, int C,
+                      int L, hipStream_t stream);
+
 }  // namespace ldist

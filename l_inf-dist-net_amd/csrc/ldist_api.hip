@@ -175,4 +175,13 @@ int ldist_norm_dist_backward_weight(const float* grad_output, const float* input
                                               (hipStream_t)stream));
 }
 
+int ldist_mean_shift(const float* x, int B, int C, int L, float* y, float* mean_out, float* running_mean,
+                     float momentum, ldist_stream_t stream) {
+    if (!x || !y || B <= 0 || C <= 0 || L <= 0 || !(momentum >= 0.0f && momentum <= 1.0f)) return LDIST_EINVAL;
+    if ((long long)B * C * L >= (1LL << 31)) return LDIST_ERANGE;
+    ldist::Problem pr{};
+    if (int rc = current_device(pr)) return rc;
+    return finish(ldist::mean_shift(x, y, mean_out, running_mean, momentum, B, C, L, (hipStream_t)stream));
+}
+
 }  // extern "C"

@@ -118,27 +118,46 @@ def inf_dist_bound(input_lower, input_upper, weight, group, use_custom_cuda_func
     return nearest.amax(dim=3).view(shape), hi
 
 
-class _BatchMeanShift(torch.autograd.Function):
-    """flat (B, C, L) minus its per-channel mean over B and L; also returns that mean.
+def _channel_mean(flat):
+    # the reference's expression (model/norm_dist.py:88-91)
+    return flat.mean(dim=-1).mean(dim=0) if flat.size(-1) > 1 else flat.squeeze(-1).mean(dim=0)
 
-    The forward is the reference's expression (model/norm_dist.py:87-96).  The backward is
-    written out, gx = gy - mean(gy), instead of being left to autograd, whose chain through
-    mean / unsqueeze / sub costs about twice as many small kernels per layer.
+
+def _native_shift(flat):
+    return flat.is_cuda and flat.dtype == torch.float32
+
+
+class _BatchMeanShift(torch.autograd.Function):
+    """flat (B, C, L) minus its per-channel mean over B and L; moves owner.running_mean.
+
+    float32 CUDA tensors go through one native kernel per direction (``norm_dist_cpp.mean_shift``);
+    the reference's torch expressions (model/norm_dist.py:87-96) cost five small kernels per layer
+    forward and, through autograd, as many backward.  Other tensors take those torch expressions,
+    with the backward gx = gy - mean(gy) written out.
     """
 
     @staticmethod
-    def _channel_mean(flat):
-        return flat.mean(dim=-1).mean(dim=0) if flat.size(-1) > 1 else flat.squeeze(-1).mean(dim=0)
+    def forward(ctx, flat, owner):
+        ctx.set_materialize_grads(False)
+        if _native_shift(flat):
+            flat = flat.contiguous()
+            shifted = torch.empty_like(flat)
+            norm_dist_cpp.mean_shift(flat, shifted, None, owner.running_mean, owner.momentum)
+            return shifted
+        mean = _channel_mean(flat)
+        owner.running_mean.mul_(1 - owner.momentum).add_(mean, alpha=owner.momentum)
+        return flat - mean.unsqueeze(-1)
 
     @staticmethod
-    def forward(ctx, flat):
-        mean = _BatchMeanShift._channel_mean(flat)
-        ctx.mark_non_differentiable(mean)
-        return flat - mean.unsqueeze(-1), mean
-
-    @staticmethod
-    def backward(ctx, grad_y, _grad_mean):
-        return grad_y - _BatchMeanShift._channel_mean(grad_y).unsqueeze(-1)
+    def backward(ctx, grad_y):
+        if grad_y is None:
+            return None, None
+        if _native_shift(grad_y):
+            grad_y = grad_y.contiguous()
+            grad_x = torch.empty_like(grad_y)
+            norm_dist_cpp.mean_shift(grad_y, grad_x)
+            return grad_x, None
+        return grad_y - _channel_mean(grad_y).unsqueeze(-1), None
 
 
 class MeanNorm(nn.Module):
@@ -154,10 +173,7 @@ class MeanNorm(nn.Module):
     def forward(self, x):
         flat = x.view(x.size(0), x.size(1), -1)
         if self.training:
-            shifted, mean = _BatchMeanShift.apply(flat)
-            with torch.no_grad():
-                self.running_mean.mul_(1 - self.momentum).add_(mean, alpha=self.momentum)
-            return shifted.view_as(x)
+            return _BatchMeanShift.apply(flat, self).view_as(x)
         return (flat - self.running_mean.unsqueeze(-1)).view_as(x)
 
     def extra_repr(self):

@@ -160,3 +160,26 @@ def inf_dist_backward_input_overwrite(grad_output, pos, grad_input, G):
 
 def inf_dist_backward_weight_overwrite(grad_output, pos, grad_weight, G):
     _inf_backward_weight("ldist_inf_dist_backward_weight_overwrite", grad_output, pos, grad_weight, G)
+
+
+def mean_shift(x, y, mean_out=None, running_mean=None, momentum=0.0):
+    """y = x minus its per-channel mean over dims 0 and 2 of a (B, C, L) tensor, in one kernel.
+
+    Not in the reference's binding: there the same arithmetic is MeanNorm's torch code
+    (model/norm_dist.py:85-96).  ``mean_out`` (C) receives the mean, ``running_mean`` (C) is moved
+    by ``momentum`` in place; both are optional.
+    """
+    _check_input(x, "x")
+    _check_input(y, "y")
+    _expect(x.dim() == 3 and y.shape == x.shape, "x and y must be (B, C, L) tensors of one shape")
+    _expect(y.data_ptr() != x.data_ptr(), "y must not alias x")
+    tensors = [x, y]
+    for t, n in ((mean_out, "mean_out"), (running_mean, "running_mean")):
+        if t is not None:
+            _check_input(t, n)
+            _expect(t.numel() == x.size(1), f"{n} must have C elements")
+            tensors.append(t)
+    dev = _same_device(*tensors)
+    _call("ldist_mean_shift", dev, _p(x), x.size(0), x.size(1), x.size(2), _p(y),
+          None if mean_out is None else _p(mean_out), None if running_mean is None else _p(running_mean),
+          float(momentum))

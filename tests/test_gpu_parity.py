@@ -214,6 +214,53 @@ def test_norm_backward(shape, p):
     assert_sum_close(gw.cpu() - 0.125, ew, mw, p, RTOL, ATOL)
 
 
+@pytest.mark.parametrize("shape", [(512, 5120, 1), (37, 10, 1), (1030, 50, 1), (600, 36, 1), (6, 5, 12), (4, 3, 7),
+                                   (16, 8, 1024)])
+def test_mean_shift_kernel(shape):
+    """One-kernel per-channel mean shift (training-mode MeanNorm, reference model/norm_dist.py:85-96)
+    against the closed form in float64; also the mean it reports and the running mean it moves."""
+    from gpu_common import DEV, cpp, say
+    say("mean_shift", shape)
+    B, C, L = shape
+    x = torch.randn(B, C, L, generator=gen(21)) + torch.linspace(-3, 3, C).view(1, C, 1)
+    running = torch.linspace(-1, 1, C)
+    mean64 = x.double().mean(dim=(0, 2))
+    xd = x.to(DEV)
+    y = torch.full_like(xd, float("nan"))
+    mean_out = torch.empty(C, device=DEV)
+    rm = running.to(DEV)
+    cpp.mean_shift(xd, y, mean_out, rm, 0.1)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(mean_out.cpu().double(), mean64, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(y.cpu().double(), x.double() - mean64.view(1, C, 1), rtol=1e-6, atol=2e-6)
+    torch.testing.assert_close(rm.cpu().double(), 0.9 * running.double() + 0.1 * mean64, rtol=1e-6, atol=1e-6)
+    y2 = torch.empty_like(xd)                      # the optional outputs left out
+    cpp.mean_shift(xd, y2)
+    torch.cuda.synchronize()
+    assert torch.equal(y2, y)
+
+
+def test_mean_norm_module_on_gpu_matches_cpu_module():
+    from gpu_common import DEV, pkg
+    for shape in ((64, 12), (8, 6, 5, 5)):
+        x = torch.randn(*shape, generator=gen(22))
+        up = torch.randn(*shape, generator=gen(23))
+        ref, dev = pkg.MeanNorm(shape[1]).train(), pkg.MeanNorm(shape[1]).train().to(DEV)
+        xa, xb = x.clone().requires_grad_(True), x.to(DEV).requires_grad_(True)
+        ref(xa).backward(up)
+        out = dev(xb)
+        out.backward(up.to(DEV))
+        torch.cuda.synchronize()
+        torch.testing.assert_close(out.detach().cpu(), ref(x).detach(), rtol=1e-6, atol=1e-6)
+        torch.testing.assert_close(xb.grad.cpu(), xa.grad, rtol=1e-6, atol=1e-6)
+        # two training-mode calls on the CPU module, one on the GPU module
+        torch.testing.assert_close(dev.running_mean.cpu(), 0.1 * x.mean(dim=tuple(d for d in range(x.dim()) if d != 1)),
+                                   rtol=1e-5, atol=1e-6)
+        dev.eval()
+        torch.testing.assert_close(dev(x.to(DEV)).cpu(), x - dev.running_mean.cpu().view(1, -1, *([1] * (x.dim() - 2))),
+                                   rtol=1e-6, atol=1e-6)
+
+
 def test_error_codes_and_checks():
     from gpu_common import DEV, cpp, pkg
     lib = pkg._lib.lib()
