@@ -21,10 +21,11 @@ struct BwdDims {
 // Workgroup = (image b, group g, TH consecutive hw, KC consecutive k).
 // bins[kc][th]; element (k, hw) of the slab lives at ((b*G+g)*K + k)*HW + hw.
 template <bool OVERWRITE>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(1024)
 inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* __restrict__ pos,
-                          float* __restrict__ grad_input, BwdDims d, int th_log2, int KC, int hw_tiles) {
-    extern __shared__ float bins[];
+                          float* __restrict__ grad_input, BwdDims d, int th_log2, int KC, int hw_tiles, int vec) {
+    extern __shared__ __align__(16) float bins[];
+    const int NT = blockDim.x;
     const int TH = 1 << th_log2;
     const int tile = blockIdx.x % hw_tiles;
     const int bg = blockIdx.x / hw_tiles;  // b*G + g
@@ -32,12 +33,49 @@ inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* 
     const int k0 = blockIdx.y * KC;
     const int kc = min(KC, d.K - k0);
     const int nb = kc * TH;
-    for (int e = threadIdx.x; e < nb; e += 256) bins[e] = 0.f;
+    const size_t obase = (size_t)bg * d.NG * d.HW;
+    const size_t xbase = ((size_t)bg * d.K + k0) * d.HW;
+
+    if (vec) {
+        // fc layout (TH == 1) with NG, K, kc multiples of 4 and 16-byte aligned tensors: the rows of
+        // pos / grad_output and the slab of grad_input are contiguous, so everything moves 128 bits
+        // at a time; the loads of a lane's four elements are in flight together.
+        float4* b4 = reinterpret_cast<float4*>(bins);
+        for (int e = threadIdx.x; e < kc / 4; e += NT) b4[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+        __syncthreads();
+        const int4* p4 = reinterpret_cast<const int4*>(pos + obase);
+        const float4* g4 = reinterpret_cast<const float4*>(grad_output + obase);
+        for (int e = threadIdx.x; e < d.NG / 4; e += NT) {
+            const int4 pv = p4[e];
+            const float4 gv = g4[e];
+            const int ps[4] = {pv.x, pv.y, pv.z, pv.w};
+            const float gs[4] = {gv.x, gv.y, gv.z, gv.w};
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int idx = (ps[q] & 0x7fffffff) - k0;
+                if (idx >= 0 && idx < kc) atomicAdd(&bins[idx], ps[q] >= 0 ? gs[q] : -gs[q]);
+            }
+        }
+        __syncthreads();
+        float4* dst = reinterpret_cast<float4*>(grad_input + xbase);
+        for (int e = threadIdx.x; e < kc / 4; e += NT) {
+            const float4 v = b4[e];
+            if (OVERWRITE) {
+                dst[e] = v;
+            } else if (v.x != 0.f || v.y != 0.f || v.z != 0.f || v.w != 0.f) {
+                float4 o = dst[e];
+                o.x += v.x; o.y += v.y; o.z += v.z; o.w += v.w;
+                dst[e] = o;
+            }
+        }
+        return;
+    }
+
+    for (int e = threadIdx.x; e < nb; e += NT) bins[e] = 0.f;
     __syncthreads();
 
-    const size_t obase = (size_t)bg * d.NG * d.HW;
     const int total = d.NG * TH;
-    for (int e = threadIdx.x; e < total; e += 256) {
+    for (int e = threadIdx.x; e < total; e += NT) {
         const int n = e >> th_log2, j = e & (TH - 1);
         const int hw = hw0 + j;
         if (hw < d.HW) {
@@ -52,8 +90,7 @@ inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* 
     }
     __syncthreads();
 
-    const size_t xbase = ((size_t)bg * d.K + k0) * d.HW;
-    for (int e = threadIdx.x; e < nb; e += 256) {
+    for (int e = threadIdx.x; e < nb; e += NT) {
         const int k = e >> th_log2, j = e & (TH - 1);
         const int hw = hw0 + j;
         if (hw < d.HW) {
@@ -175,12 +212,21 @@ hipError_t inf_backward_input(const float* grad_output, const int32_t* pos, floa
     const int hw_tiles = (pr.HW + TH - 1) / TH;
     const dim3 grid((unsigned)pr.B * pr.G * hw_tiles, (unsigned)((pr.K + KC - 1) / KC));
     const size_t lds = (size_t)KC * TH * sizeof(float);
+    // fc layout, everything a multiple of four floats and 16-byte aligned: 128-bit path
+    const int vec = pr.HW == 1 && pr.NG % 4 == 0 && pr.K % 4 == 0 && KC % 4 == 0 && aligned16(grad_output) &&
+                    aligned16(pos) && aligned16(grad_input);
+    // few workgroups (one per image and group in the fc layout): more lanes each keep more loads in flight
+    const long wgs = (long)grid.x * grid.y;
+    const long work = pr.HW == 1 ? pr.NG : (long)pr.NG * TH;        // elements scanned per workgroup
+    int threads = 256;
+    if (wgs < 8L * pr.num_cu && work >= 4096) threads = 512;
+    if (wgs < 4L * pr.num_cu && work >= 16384) threads = 1024;
     if (overwrite)
-        hipLaunchKernelGGL(inf_backward_input_kernel<true>, grid, dim3(256), lds, stream, grad_output, pos,
-                           grad_input, d, th_log2, KC, hw_tiles);
+        hipLaunchKernelGGL(inf_backward_input_kernel<true>, grid, dim3(threads), lds, stream, grad_output, pos,
+                           grad_input, d, th_log2, KC, hw_tiles, vec);
     else
-        hipLaunchKernelGGL(inf_backward_input_kernel<false>, grid, dim3(256), lds, stream, grad_output, pos,
-                           grad_input, d, th_log2, KC, hw_tiles);
+        hipLaunchKernelGGL(inf_backward_input_kernel<false>, grid, dim3(threads), lds, stream, grad_output, pos,
+                           grad_input, d, th_log2, KC, hw_tiles, vec);
     return hipGetLastError();
 }
 
