@@ -3,7 +3,7 @@
 // that no power can overflow for any p.  Semantics follow the reference kernel
 // model/norm_dist_cuda.cu:228-292: mx and the sum are seeded with 1e-10 (:232-233),
 // and whenever a block of k raises mx the sum is rescaled by (mx_old/mx_new)^p
-// (:257-261).  Here the block is a 32-wide chunk.  For p <= 16 a chunk is normally
+// (:257-261).  Here the block is a 32-wide chunk.  For p <= 64 a chunk is normally
 // swept once with the scale left by earlier chunks (see the kernel); otherwise
 // sweep one finds the chunk maximum (sub + half a max3 per element), the rescale
 // runs once per output, sweep two adds (|x-w| / mx)^p.  p = 2, 3, 4, 8 use
@@ -23,8 +23,7 @@ namespace ldist {
 // adds (|x-w| / s)^p with the scale s left by earlier chunks, and only a wave that sees a chunk
 // sum overflow (or turn NaN) goes back over that chunk the long way: find its maximum, move
 // the scale there as the reference does, add the powers again.  The first chunk always takes
-// that road (the scale starts at the reference's seed 1e-10).  With p <= 16 a chunk may exceed
-// the scale by a factor of 70 before that happens.  ONE = false: every chunk is swept twice
+// that road (the scale starts at the reference's seed 1e-10).  ONE = false: every chunk is swept twice
 // (maximum, then powers), for exponents so large that almost any increase would overflow.
 template <class GEO, bool CONV, int VEC, int IP, bool ONE>
 __global__ void __launch_bounds__(GEO::NT, 2)
@@ -193,8 +192,11 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
     store_patch<GEO, CONV>(output, acc, d, m0, n0, g, tx, ty, d.ovec != 0);
 }
 
-// Largest exponent for the one-sweep kernel: 70^16 is about 3e29, inside the overflow test.
-constexpr float kOneSweepMaxP = 16.f;
+// Largest exponent for the one-sweep kernel.  A chunk goes back the long way once it exceeds the
+// scale by 10^(30/p): a factor of 70 at p = 16, still 2.9 at p = 64, which later chunks rarely
+// do.  Beyond that nearly every new maximum would overflow and the retries would cost more than
+// sweeping every chunk twice.
+constexpr float kOneSweepMaxP = 64.f;
 
 // Few outputs per group: two passes over k, first the exact maximum per (row, output),
 // then the sum of (|x-w| / max)^p; lanes split k in both.

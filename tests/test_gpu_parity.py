@@ -164,7 +164,7 @@ def test_norm_forward_scale_robust_and_seeded():
 
 
 @pytest.mark.parametrize("tile", [-1, 0, 1])
-@pytest.mark.parametrize("p", [2.0, 3.0, 8.0, 3.5, 16.0, 16.5])
+@pytest.mark.parametrize("p", [2.0, 3.0, 8.0, 3.5, 16.5, 37.0, 64.0, 64.5])
 @pytest.mark.parametrize("profile", ["growing", "shrinking", "spike", "tiny"])
 def test_norm_forward_magnitude_jumps_between_chunks(profile, p, tile):
     """|x - w| changes by orders of magnitude from one 32-wide chunk of k to the next: the kernel
