@@ -117,7 +117,11 @@ def workload_c0(pkg, torch, dev):
         oracle.inf_dist_forward(x[:rows].contiguous(), w, 1)
         return rows * 784 * 5120
 
-    return dict(step=step, ops=512 * 784 * 5120, images=512, full_rows=512, cpu=cpu,
+    def formula(rows):
+        pkg.norm_dist(x[:rows].contiguous(), w, 1, INF, use_custom_cuda_func=False)
+        return rows * 784 * 5120
+
+    return dict(step=step, ops=512 * 784 * 5120, images=512, full_rows=512, cpu=cpu, formula=formula,
                 name="configs[0]: single L_inf-dist fc layer forward, 512 x 784 -> 5120, values + argmax",
                 kernel=("inf_dist_forward", lambda x_, w_, *_: 2 * mnk(x_, w_), lambda *a: True,
                         "inf_forward_kernel (tiled L_inf forward)", 2))
@@ -160,12 +164,25 @@ def mlp_workload(pkg, torch, dev, p):
                 gr = oracle.norm_dist_backward_input(gr, hin, w, out, 1, p)
         return stack_ops(rows) * (1 if math.isinf(p) else 3)
 
-    return step, cpu
+    def formula(rows):
+        # forward + backward through the dense torch formula (what the reference runs with
+        # use_custom_cuda_func=False), autograd doing the backward
+        import torch
+        h = x[:rows].reshape(rows, -1, 1).clone().requires_grad_(True)
+        params = [w.clone().requires_grad_(True) for w in ws]
+        out = h
+        for w in params:
+            out = pkg.norm_dist(out, w, 1, p, use_custom_cuda_func=False)
+            out = out - out.mean(dim=0, keepdim=True)
+        out.backward(upstream[:rows].reshape(rows, -1, 1))
+        return stack_ops(rows) * (1 if math.isinf(p) else 3)
+
+    return step, cpu, formula
 
 
 def workload_c1(pkg, torch, dev):
-    step, cpu = mlp_workload(pkg, torch, dev, INF)
-    return dict(step=step, ops=stack_ops(512), images=512, full_rows=512, cpu=cpu,
+    step, cpu, formula = mlp_workload(pkg, torch, dev, INF)
+    return dict(step=step, ops=stack_ops(512), images=512, full_rows=512, cpu=cpu, formula=formula,
                 name="configs[1]: 5-layer L_inf-dist MLP 3072-5120-5120-5120-5120-10, p=inf, batch 512, "
                      "forward+backward (all grad_x and grad_w), mean shift in training mode",
                 kernel=("inf_dist_forward", lambda x_, w_, *_: 2 * mnk(x_, w_),
@@ -174,8 +191,8 @@ def workload_c1(pkg, torch, dev):
 
 
 def workload_c2(pkg, torch, dev):
-    step, cpu = mlp_workload(pkg, torch, dev, 8.0)
-    return dict(step=step, ops=3 * stack_ops(512), images=512, full_rows=512, cpu=cpu,
+    step, cpu, formula = mlp_workload(pkg, torch, dev, 8.0)
+    return dict(step=step, ops=3 * stack_ops(512), images=512, full_rows=512, cpu=cpu, formula=formula,
                 name="configs[2]: the same MLP at p=8, forward+backward (3 dist-op passes per layer)",
                 kernel=("norm_dist_backward_input", lambda go, x_, w_, *_: 7 * mnk(x_, w_),
                         lambda go, x_, w_, *_: w_.size(0) > 16, "norm_backward_kernel (grad_input)", 7))
@@ -208,7 +225,15 @@ def workload_c3(pkg, torch, dev):
             h, l, u = ((t - m.view(1, -1, 1)).contiguous() for t in (out, ol, ou))
         return 2 * stack_ops(rows)
 
-    return dict(step=step, ops=2 * stack_ops(1024), images=1024, full_rows=1024, cpu=cpu,
+    def formula(rows):
+        h, l, u = (t[:rows].reshape(rows, -1, 1).contiguous() for t in (x, lo, up))
+        for w, m in zip(ws, means):
+            out = pkg.norm_dist(h, w, 1, INF, use_custom_cuda_func=False)
+            ol, ou = pkg.inf_dist_bound(l, u, w, 1, use_custom_cuda_func=False)
+            h, l, u = ((t - m.view(1, -1, 1)).contiguous() for t in (out, ol, ou))
+        return 2 * stack_ops(rows)
+
+    return dict(step=step, ops=2 * stack_ops(1024), images=1024, full_rows=1024, cpu=cpu, formula=formula,
                 name="configs[3]: interval-bound certification forward through the MLP, batch 1024, eps=8/255: "
                      "value path + lower/upper bounds + certified margins (bound-ops and dist-ops both counted)",
                 kernel=("inf_dist_bound_forward", lambda l_, u_, w_, *_: 6 * mnk(l_, w_),
@@ -240,7 +265,22 @@ def workload_c4(pkg, torch, dev):
         oracle.inf_dist_backward_weight(gs, pos, 1152, 4)
         return rows * 1024 * 128 * 288
 
-    return dict(step=step, ops=128 * 1024 * 128 * 288, images=128, full_rows=128, cpu=cpu,
+    def formula(rows):
+        xs = cols[:rows].clone().requires_grad_(True)
+        wr = w.clone().requires_grad_(True)
+        pkg.norm_dist(xs, wr, 4, INF, use_custom_cuda_func=False).backward(go[:rows])
+        return rows * 1024 * 128 * 288
+
+    imgd = img.to(dev)
+
+    def step_with_unfold():
+        wd.grad = None
+        xi = imgd.detach().requires_grad_(True)
+        y = pkg.norm_dist(F.unfold(xi, 3, padding=1), wd, 4, INF)
+        y.backward(god)
+
+    return dict(step=step, ops=128 * 1024 * 128 * 288, images=128, full_rows=128, cpu=cpu, formula=formula,
+                step_alt=("ms_per_step_incl_unfold_and_fold", step_with_unfold),
                 name="configs[4]: unfolded 3x3 L_inf-dist conv layer, batch 128, 128->128 channels, 32x32, groups 4, "
                      "forward+backward (unfold outside the timed region)",
                 kernel=("inf_dist_forward", lambda x_, w_, *_: 2 * mnk(x_, w_), lambda *a: True,
@@ -271,6 +311,30 @@ def cpu_baseline(wl, target_seconds=12.0):
         "kind": "port",
         "sample": f"C oracle (OpenMP) on {rows} of {wl['full_rows']} rows of the same workload, "
                   f"{reps} pass(es), {t:.1f} s",
+    }
+
+
+def cpu_formula_baseline(wl, target_seconds=5.0):
+    """The dense torch formula of the reference's use_custom_cuda_func=False path on the host CPU,
+    on a few rows of the same workload (it materialises rows x N x K floats per layer)."""
+    import torch
+    rows = 1 if wl["full_rows"] <= 128 else 2
+    t0 = time.perf_counter()
+    ops = wl["formula"](rows)
+    t = time.perf_counter() - t0
+    reps = 1
+    while t < target_seconds and reps < 256:
+        t0 = time.perf_counter()
+        ops += wl["formula"](rows)
+        t += time.perf_counter() - t0
+        reps += 1
+    return {
+        "value": round(ops / t / 1e9, 3),
+        "unit": "G dist-ops/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"dense torch formula (the reference's use_custom_cuda_func=False arithmetic) on {rows} of "
+                  f"{wl['full_rows']} rows of the same workload, {reps} pass(es), {t:.1f} s",
     }
 
 
@@ -359,8 +423,19 @@ def main():
         # rocprofv3 --pmc runs of this command (profiles/): FETCH_SIZE x 2.0 (copy-probe factor)
         # + WRITE_SIZE x 1.0
         out["roofline"]["traffic"] = TRAFFIC_C1_BYTES
+    if "step_alt" in wl:
+        label, alt = wl["step_alt"]
+        for _ in range(args.warmup):
+            alt()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            alt()
+        torch.cuda.synchronize()
+        out[label] = round((time.perf_counter() - t0) * 1e3 / args.steps, 4)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(wl)
+        out["cpu_reference_formula"] = cpu_formula_baseline(wl)
     print(json.dumps(out))
 
 
