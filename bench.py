@@ -190,6 +190,30 @@ def workload_c1(pkg, torch, dev):
                         "inf_forward_kernel (tiled L_inf forward)", 2))
 
 
+def workload_c1t(pkg, torch, dev):
+    # configs[1] followed by the optimizer: one complete training step of the reference's recipe
+    # (main.py: forward, backward, AdamW with l_inf weight decay), on the same synthetic batch
+    g = torch.Generator().manual_seed(0)
+    x = normalise(torch.rand(512, 3, 32, 32, generator=g))
+    ws = stack_weights(g)
+    upstream = torch.randn(512, 10, generator=g)
+    model = build_mlp(pkg, ws, dev, INF, train=True)
+    opt = pkg.AdamW(model, lr=1e-3, weight_decay=5e-3)
+    xd, up = x.to(dev), upstream.to(dev)
+
+    def step():
+        for prm in model.parameters():
+            prm.grad = None
+        y, _, _ = model(xd)
+        y.backward(up)
+        opt.step()
+
+    base = workload_c1(pkg, torch, dev)
+    return dict(base, step=step,
+                name="configs[1] plus the AdamW step with l_inf weight decay: one full training step "
+                     "(forward, backward, optimizer) of the 5-layer MLP, batch 512")
+
+
 def workload_c2(pkg, torch, dev):
     step, cpu, formula = mlp_workload(pkg, torch, dev, 8.0)
     return dict(step=step, ops=3 * stack_ops(512), images=512, full_rows=512, cpu=cpu, formula=formula,
@@ -287,7 +311,8 @@ def workload_c4(pkg, torch, dev):
                         "inf_forward_kernel (conv layout, k tracked in the loop)", 2))
 
 
-WORKLOADS = {"c0": workload_c0, "c1": workload_c1, "c2": workload_c2, "c3": workload_c3, "c4": workload_c4}
+WORKLOADS = {"c0": workload_c0, "c1": workload_c1, "c1t": workload_c1t, "c2": workload_c2, "c3": workload_c3,
+             "c4": workload_c4}
 
 
 def cpu_baseline(wl, target_seconds=12.0):

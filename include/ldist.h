@@ -135,6 +135,24 @@ int ldist_inf_dist_backward_weight_overwrite(const float* grad_output, const int
 int ldist_mean_shift(const float* x, int B, int C, int L, float* y, float* mean_out, float* running_mean,
                      float momentum, ldist_stream_t stream);
 
+/* One AdamW step with row-wise l_p weight decay on a contiguous (rows, cols) parameter, in place
+ * and in one kernel.  No native counterpart in the reference: it is the arithmetic of its
+ * optimizer (adamw.py:36-85), about sixteen elementwise torch kernels per tensor there.
+ * Decay first, on the parameter itself, chosen by p_norm (the p of the owning module):
+ *   p_norm <= 0 or NaN  (module without p, :42-43):  w *= 1 - lr*weight_decay
+ *   finite p_norm > 0   (:44-50):  a = w^2 + eps, s = a / max_row(a), q = s^(p/2 - 1),
+ *                                  w += -lr*weight_decay * (sum_row s*q)^(2/p - 1) * q * w
+ *   p_norm = +inf       (:51-55):  only the first element of largest |w| in each row decays
+ * then Adam on the decayed value (:73-85) with bias corrections for the 1-based `step`:
+ *   m = beta1*m + (1-beta1)*g,  v = beta2*v + (1-beta2)*g*g,
+ *   w -= lr/(1-beta1^step) * m / (sqrt(v)/sqrt(1-beta2^step) + eps)
+ * grad == NULL: the decay alone (exp_avg, exp_avg_sq are not touched and may be NULL).
+ * The hyper-parameters are doubles, as in the reference's Python: 1 - beta2 = 0.001 loses five
+ * digits when beta2 is first rounded to float. */
+int ldist_adamw_lp_step(float* param, const float* grad, float* exp_avg, float* exp_avg_sq, int rows, int cols,
+                        double p_norm, double lr, double beta1, double beta2, double eps, double weight_decay,
+                        int step, ldist_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -14,6 +14,7 @@ _I = ctypes.c_void_p   # const int32_t* / int32_t* (device)
 _S = ctypes.c_void_p   # hipStream_t
 _i = ctypes.c_int
 _f = ctypes.c_float
+_d = ctypes.c_double
 
 # name -> argument types, in the order of include/ldist.h
 SIGNATURES = {
@@ -27,6 +28,7 @@ SIGNATURES = {
     "ldist_norm_dist_backward_input": [_F, _F, _F, _F, _i, _i, _i, _i, _i, _F, _f, _S],
     "ldist_norm_dist_backward_weight": [_F, _F, _F, _F, _i, _i, _i, _i, _i, _F, _f, _S],
     "ldist_mean_shift": [_F, _i, _i, _i, _F, _F, _F, _f, _S],
+    "ldist_adamw_lp_step": [_F, _F, _F, _F, _i, _i, _d, _d, _d, _d, _d, _d, _i, _S],
 }
 
 _lib = None

@@ -73,4 +73,8 @@ hipError_t norm_backward_weight(const float* grad_output, const float* input, co
 hipError_t mean_shift(const float* x, float* y, float* mean_out, float* running_mean, float momentum, int B, int C,
                       int L, hipStream_t stream);
 
+hipError_t adamw_lp_step(float* param, const float* grad, float* exp_avg, float* exp_avg_sq, int rows, int cols,
+                         double p_norm, double lr, double beta1, double beta2, double eps, double weight_decay, int step,
+                         hipStream_t stream);
+
 }  // namespace ldist

@@ -184,4 +184,19 @@ int ldist_mean_shift(const float* x, int B, int C, int L, float* y, float* mean_
     return finish(ldist::mean_shift(x, y, mean_out, running_mean, momentum, B, C, L, (hipStream_t)stream));
 }
 
+int ldist_adamw_lp_step(float* param, const float* grad, float* exp_avg, float* exp_avg_sq, int rows, int cols,
+                        double p_norm, double lr, double beta1, double beta2, double eps, double weight_decay, int step,
+                        ldist_stream_t stream) {
+    if (!param || rows <= 0 || cols <= 0 || step < 1) return LDIST_EINVAL;
+    if (grad && (!exp_avg || !exp_avg_sq)) return LDIST_EINVAL;
+    if (!(lr >= 0.0) || !(eps >= 0.0) || !(weight_decay >= 0.0) || !(beta1 >= 0.0 && beta1 < 1.0) ||
+        !(beta2 >= 0.0 && beta2 < 1.0))
+        return LDIST_EINVAL;   // the reference constructor's checks, adamw.py:15-24
+    if ((long long)rows * cols >= (1LL << 31)) return LDIST_ERANGE;
+    ldist::Problem pr{};
+    if (int rc = current_device(pr)) return rc;
+    return finish(ldist::adamw_lp_step(param, grad, exp_avg, exp_avg_sq, rows, cols, p_norm, lr, beta1, beta2, eps,
+                                       weight_decay, step, (hipStream_t)stream));
+}
+
 }  // extern "C"

@@ -183,3 +183,22 @@ def mean_shift(x, y, mean_out=None, running_mean=None, momentum=0.0):
     _call("ldist_mean_shift", dev, _p(x), x.size(0), x.size(1), x.size(2), _p(y),
           None if mean_out is None else _p(mean_out), None if running_mean is None else _p(running_mean),
           float(momentum))
+
+
+def adamw_lp_step(param, grad, exp_avg, exp_avg_sq, p_norm, lr, beta1, beta2, eps, weight_decay, step):
+    """One AdamW step with row-wise l_p weight decay, in place, in one kernel (reference adamw.py:36-85).
+
+    ``param`` is viewed as (param.size(0), rest); ``p_norm`` is None for a module without p, else the
+    module's p (float, may be inf).  Not in the reference's binding: there this is torch code.
+    """
+    tensors = [param, grad, exp_avg, exp_avg_sq]
+    for t, n in zip(tensors, ("param", "grad", "exp_avg", "exp_avg_sq")):
+        _check_input(t, n)
+        _expect(t.shape == param.shape, f"{n} must have the shape of param")
+    dev = _same_device(*tensors)
+    rows = param.size(0) if param.dim() > 0 else 1
+    cols = param.numel() // max(rows, 1)
+    _expect(param.numel() > 0, "param must not be empty")
+    _call("ldist_adamw_lp_step", dev, _p(param), _p(grad), _p(exp_avg), _p(exp_avg_sq), rows, cols,
+          -1.0 if p_norm is None else float(p_norm), float(lr), float(beta1), float(beta2), float(eps),
+          float(weight_decay), int(step))

@@ -200,3 +200,27 @@ def fallback_inf_dist_values(x, weight, group, rows_per_chunk=None):
 
 def is_inf(p):
     return math.isinf(p)
+
+
+def mean_shift(x, running_mean=None, momentum=0.1):
+    """(y, mean) of the per-channel mean shift of a (B, C, L) tensor; moves running_mean in place if given."""
+    B, C, L = x.shape
+    y = torch.empty_like(x)
+    mean = torch.empty(C, dtype=torch.float32)
+    _check(lib().ldist_oracle_mean_shift(_f(x), B, C, L, _f(y), _f(mean),
+                                         None if running_mean is None else _f(running_mean),
+                                         ctypes.c_float(momentum)), "mean_shift")
+    return y, mean
+
+
+def adamw_lp_step(param, grad, exp_avg, exp_avg_sq, p_norm, lr, betas, eps, weight_decay, step):
+    """In place on param (2-D view rows x cols), exp_avg, exp_avg_sq.  p_norm None = the module has no p."""
+    rows = param.size(0)
+    cols = param.numel() // rows
+    pn = -1.0 if p_norm is None else float(p_norm)
+    _check(lib().ldist_oracle_adamw_lp_step(_f(param), None if grad is None else _f(grad),
+                                            None if exp_avg is None else _f(exp_avg),
+                                            None if exp_avg_sq is None else _f(exp_avg_sq), rows, cols,
+                                            ctypes.c_double(pn), ctypes.c_double(lr), ctypes.c_double(betas[0]),
+                                            ctypes.c_double(betas[1]), ctypes.c_double(eps),
+                                            ctypes.c_double(weight_decay), int(step)), "adamw_lp_step")

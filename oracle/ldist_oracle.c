@@ -447,3 +447,89 @@ int ldist_oracle_norm_dist_backward_weight(const float* grad_output, const float
     }
     return LDIST_ORACLE_OK;
 }
+
+/* Per-channel mean shift of a (B, C, L) tensor: the training-mode arithmetic of the reference's */
+/* MeanNorm (model/norm_dist.py:85-96): mean over b and l, y = x - mean, running mean moved by   */
+/* momentum.  Sums are taken in double.  mean_out and running_mean may be NULL.                  */
+int ldist_oracle_mean_shift(const float* x, int B, int C, int L, float* y, float* mean_out, float* running_mean,
+                            float momentum) {
+    if (!x || !y || B <= 0 || C <= 0 || L <= 0) return LDIST_ORACLE_EINVAL;
+#pragma omp parallel for schedule(static)
+    for (int c = 0; c < C; c++) {
+        double s = 0.0;
+        for (int b = 0; b < B; b++)
+            for (int l = 0; l < L; l++) s += (double)x[((size_t)b * C + c) * L + l];
+        const double mean = s / ((double)B * (double)L);
+        for (int b = 0; b < B; b++)
+            for (int l = 0; l < L; l++) {
+                const size_t at = ((size_t)b * C + c) * L + l;
+                y[at] = (float)((double)x[at] - mean);
+            }
+        if (mean_out) mean_out[c] = (float)mean;
+        if (running_mean) running_mean[c] = (float)((1.0 - (double)momentum) * (double)running_mean[c] + (double)momentum * mean);
+    }
+    return LDIST_ORACLE_OK;
+}
+
+/* One AdamW step with row-wise l_p weight decay on a (rows, cols) parameter: reference           */
+/* adamw.py:36-85.  The decay comes first and acts on the parameter itself (:40-56):              */
+/*   p_norm <= 0 ("the module has no p", :42-43):  w *= 1 - lr*wd                                  */
+/*   finite p_norm (:44-50):  a = w^2 + eps,  s = a / max_row(a),  q = s^(p/2 - 1),                */
+/*                            w += -lr*wd * (sum_row s*q)^(2/p - 1) * q * w                         */
+/*   p_norm = +inf (:51-55):  only the first element of largest |w| in the row: w -= lr*wd * w     */
+/* then Adam on the decayed parameter (:73-85): m = b1*m + (1-b1)*g, v = b2*v + (1-b2)*g*g,        */
+/*   w -= lr / (1 - b1^step) * m / (sqrt(v) / sqrt(1 - b2^step) + eps).  `step` counts from 1.     */
+/* grad == NULL: the decay alone.  Everything is evaluated in double and rounded once.            */
+int ldist_oracle_adamw_lp_step(float* param, const float* grad, float* exp_avg, float* exp_avg_sq, int rows, int cols,
+                               double p_norm, double lr, double beta1, double beta2, double eps, double weight_decay,
+                               int step) {
+    if (!param || rows <= 0 || cols <= 0 || step < 1) return LDIST_ORACLE_EINVAL;
+    if (grad && (!exp_avg || !exp_avg_sq)) return LDIST_ORACLE_EINVAL;
+    const double lw = lr * weight_decay;
+    const double bc1 = 1.0 - pow(beta1, (double)step), bc2 = 1.0 - pow(beta2, (double)step);
+#pragma omp parallel for schedule(static)
+    for (int r = 0; r < rows; r++) {
+        float* w = param + (size_t)r * cols;
+        double* nw = (double*)malloc(sizeof(double) * (size_t)cols);
+        if (!nw) continue;
+        if (!(p_norm > 0.0)) {
+            for (int i = 0; i < cols; i++) nw[i] = (double)w[i] * (1.0 - lw);
+        } else if (isinf(p_norm)) {
+            int best = 0;
+            for (int i = 1; i < cols; i++)
+                if (fabsf(w[i]) > fabsf(w[best])) best = i;
+            for (int i = 0; i < cols; i++) nw[i] = (double)w[i];
+            nw[best] = (double)w[best] - lw * (double)w[best];
+        } else {
+            const double p = p_norm;
+            double mx = 0.0, sum = 0.0;
+            for (int i = 0; i < cols; i++) {
+                const double a = (double)w[i] * (double)w[i] + eps;
+                if (a > mx) mx = a;
+            }
+            for (int i = 0; i < cols; i++) {
+                const double s = ((double)w[i] * (double)w[i] + eps) / mx;
+                sum += s * pow(s, p / 2.0 - 1.0);
+            }
+            const double c = pow(sum, 2.0 / p - 1.0);
+            for (int i = 0; i < cols; i++) {
+                const double s = ((double)w[i] * (double)w[i] + eps) / mx;
+                nw[i] = (double)w[i] - lw * c * pow(s, p / 2.0 - 1.0) * (double)w[i];
+            }
+        }
+        for (int i = 0; i < cols; i++) {
+            if (grad) {
+                const size_t at = (size_t)r * cols + i;
+                const double g = (double)grad[at];
+                const double m = beta1 * (double)exp_avg[at] + (1.0 - beta1) * g;
+                const double v = beta2 * (double)exp_avg_sq[at] + (1.0 - beta2) * g * g;
+                exp_avg[at] = (float)m;
+                exp_avg_sq[at] = (float)v;
+                nw[i] -= lr / bc1 * m / (sqrt(v) / sqrt(bc2) + eps);
+            }
+            w[i] = (float)nw[i];
+        }
+        free(nw);
+    }
+    return LDIST_ORACLE_OK;
+}

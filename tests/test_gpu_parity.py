@@ -261,6 +261,56 @@ def test_mean_norm_module_on_gpu_matches_cpu_module():
                                    rtol=1e-6, atol=1e-6)
 
 
+@pytest.mark.parametrize("shape", [(64, 5120), (37, 50), (128, 288), (10, 5120), (33, 1), (5, 3, 3, 3), (300, 7)])
+@pytest.mark.parametrize("p", [None, 2.0, 4.0, 8.0, 3.5, 37.0, 1000.0, float("inf")])
+def test_adamw_lp_step_kernel(shape, p):
+    """The fused optimizer step (reference adamw.py:36-85) against the double-precision oracle over
+    three steps; moments and parameter within float32 rounding."""
+    from gpu_common import DEV, cpp, say
+    say("adamw_lp_step", shape, "p", p)
+    g = gen(41)
+    w = torch.randn(*shape, generator=g) * 0.5
+    if len(shape) == 2 and shape[1] >= 50:
+        w[1, 7], w[1, 30] = 3.0, -3.0                     # a tie for the largest entry: the first decays at p = inf
+    m, v = torch.zeros_like(w), torch.zeros_like(w)
+    wd_, md, vd = w.to(DEV), m.to(DEV), v.to(DEV)
+    hp = dict(lr=0.03, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.25)
+    for step in (1, 2, 3):
+        grad = torch.randn(*shape, generator=g)
+        rows = w.view(w.size(0), -1)
+        oracle.adamw_lp_step(rows, grad.view_as(rows), m.view_as(rows), v.view_as(rows), p, hp["lr"], hp["betas"],
+                             hp["eps"], hp["weight_decay"], step)
+        cpp.adamw_lp_step(wd_, grad.to(DEV), md, vd, p, hp["lr"], hp["betas"][0], hp["betas"][1], hp["eps"],
+                          hp["weight_decay"], step)
+        torch.cuda.synchronize()
+        torch.testing.assert_close(md.cpu(), m, rtol=1e-6, atol=2e-7)      # 0.9 m + 0.1 g can cancel
+        torch.testing.assert_close(vd.cpu(), v, rtol=1e-6, atol=1e-9)
+        torch.testing.assert_close(wd_.cpu(), w, rtol=1e-5, atol=1e-6)
+
+
+def test_adamw_optimizer_on_gpu_follows_the_cpu_optimizer():
+    from gpu_common import DEV, pkg
+    for p in (8.0, float("inf")):
+        torch.manual_seed(5)
+        cpu_model = pkg.MLP(depth=3, width=1, input_dim=48, num_classes=10)
+        gpu_model = pkg.MLP(depth=3, width=1, input_dim=48, num_classes=10)
+        gpu_model.load_state_dict(cpu_model.state_dict())
+        gpu_model = gpu_model.to(DEV)
+        for mdl in (cpu_model, gpu_model):
+            pkg.set_p_norm(mdl, p)
+        oc, og = pkg.AdamW(cpu_model, lr=0.01, weight_decay=0.1), pkg.AdamW(gpu_model, lr=0.01, weight_decay=0.1)
+        g = gen(43)
+        for _ in range(3):
+            for a, b in zip(cpu_model.parameters(), gpu_model.parameters()):
+                a.grad = torch.randn(a.shape, generator=g)
+                b.grad = a.grad.to(DEV)
+            oc.step()
+            og.step()
+        torch.cuda.synchronize()
+        for a, b in zip(cpu_model.parameters(), gpu_model.parameters()):
+            torch.testing.assert_close(b.detach().cpu(), a.detach(), rtol=2e-5, atol=2e-6)
+
+
 def test_error_codes_and_checks():
     from gpu_common import DEV, cpp, pkg
     lib = pkg._lib.lib()

@@ -246,3 +246,59 @@ def test_mlp_triple_and_certified_margin(fake_native):
             expect = 0.0 if j == targets[b] else (up[b, j] - lo[b, targets[b]]).item()
             assert res[b, j].item() == pytest.approx(expect)
     assert pkg.BoundFinalIdentity()(y) is y
+
+
+def _tiny_model():
+    torch.manual_seed(3)
+    model = pkg.MLP(depth=2, width=1, input_dim=12, num_classes=5)
+    model.extra = torch.nn.Linear(4, 3)            # a module without p: plain decay (reference adamw.py:42-43)
+    return model
+
+
+@pytest.mark.parametrize("p", [8.0, 2.0, 3.5, float("inf")])
+def test_adamw_cpu_path_matches_oracle_per_parameter(p):
+    """The optimizer's torch expressions (CPU tensors) against the C oracle, parameter by parameter,
+    over three steps: group layout, step counter, state tensors, decay chosen by the owner's p."""
+    import oracle
+    model = _tiny_model()
+    pkg.set_p_norm(model, p)
+    opt = pkg.AdamW(model, lr=0.02, betas=(0.8, 0.95), eps=1e-7, weight_decay=0.4)
+    owners = {id(g["params"][0]): g["module"] for g in opt.param_groups}
+    assert len(opt.param_groups) == len(list(model.parameters()))           # one group per parameter
+    mirror = {id(q): (q.detach().clone(), torch.zeros_like(q), torch.zeros_like(q)) for q in model.parameters()}
+    g = gen(31)
+    for step in (1, 2, 3):
+        for q in model.parameters():
+            q.grad = torch.randn(q.shape, generator=g)
+        skipped = model.extra.bias
+        skipped.grad = None                                                   # no gradient: untouched, no state
+        before = skipped.detach().clone()
+        opt.step()
+        assert torch.equal(skipped.detach(), before) and len(opt.state[skipped]) == 0
+        for q in model.parameters():
+            if q.grad is None:
+                continue
+            w, m, v = mirror[id(q)]
+            w2 = w.view(w.size(0), -1).contiguous()
+            oracle.adamw_lp_step(w2, q.grad.reshape(w2.shape).contiguous(), m.view_as(w2), v.view_as(w2),
+                                 pkg.get_p_norm(owners[id(q)]), 0.02, (0.8, 0.95), 1e-7, 0.4, step)
+            w.copy_(w2.view_as(w))
+            torch.testing.assert_close(q.detach(), w, rtol=2e-5, atol=1e-6)
+            assert opt.state[q]["step"] == step
+    assert pkg.get_p_norm(model.extra) is None
+
+
+def test_adamw_constructor_checks_and_closure():
+    model = _tiny_model()
+    for bad in (dict(lr=-1.0), dict(eps=-1e-8), dict(betas=(1.0, 0.9)), dict(betas=(0.9, -0.1)), dict(weight_decay=-0.1)):
+        with pytest.raises(ValueError):
+            pkg.AdamW(model, **bad)
+    pkg.set_p_norm(model, 8.0)
+    opt = pkg.AdamW(model)
+    calls = []
+
+    def closure():
+        calls.append(1)
+        return torch.tensor(3.0)
+
+    assert opt.step(closure).item() == 3.0 and calls == [1]
