@@ -153,6 +153,29 @@ int ldist_adamw_lp_step(float* param, const float* grad, float* exp_avg, float* 
                         double p_norm, double lr, double beta1, double beta2, double eps, double weight_decay,
                         int step, ldist_stream_t stream);
 
+/* Patch extraction for the convolution-shaped layer, with torch's F.unfold layout, which the
+ * reference uses to turn an image into the layer's input (model/norm_dist.py:132,144-145):
+ *   cols[b, (c*KH + i)*KW + j, h*WO + w] = img[b, c, h*stride + i*dilation - padding, w*stride + j*dilation - padding]
+ * (0 outside the image); HO = (H + 2*padding - dilation*(KH-1) - 1)/stride + 1, WO likewise.
+ * img is (B, C, H, W), cols is (B, C*KH*KW, HO*WO).  No native counterpart in the reference. */
+int ldist_unfold(const float* img, int B, int C, int H, int W, int KH, int KW, int stride, int padding, int dilation,
+                 float* cols, ldist_stream_t stream);
+
+/* Adjoint of ldist_unfold (what autograd does behind F.unfold): every element of grad_img is written
+ * with the sum of the grad_cols entries that were copied from it. */
+int ldist_fold(const float* grad_cols, int B, int C, int H, int W, int KH, int KW, int stride, int padding,
+               int dilation, float* grad_img, ldist_stream_t stream);
+
+/* ldist_inf_dist_backward_input_overwrite composed with ldist_fold: the gradient of the L_inf layer
+ * with respect to the IMAGE, without the (B, C*KH*KW, HO*WO) gradient of the columns in between.
+ * grad_output and pos are (B, CO, HO*WO) as produced for the unfolded input; pos & 0x7fffffff is the
+ * in-group row (c*KH + i)*KW + j of the columns.  Every element of grad_img (B, C, H, W) is written;
+ * contributions whose argmax lies in the padding vanish, as they do in fold.
+ * LDIST_ERANGE if (C/G)*W exceeds 16384 floats (use the two separate calls then). */
+int ldist_inf_dist_backward_input_folded(const float* grad_output, const int32_t* pos, int B, int CO, int C, int G,
+                                         int H, int W, int KH, int KW, int stride, int padding, int dilation,
+                                         float* grad_img, ldist_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -77,4 +77,15 @@ hipError_t adamw_lp_step(float* param, const float* grad, float* exp_avg, float*
                          double p_norm, double lr, double beta1, double beta2, double eps, double weight_decay, int step,
                          hipStream_t stream);
 
+// Geometry of a convolution-shaped layer working on an image tensor (B, C, H, W).
+struct ConvGeom {
+    int B, C, H, W;        // image
+    int KH, KW, S, P, D;   // window, stride, padding, dilation
+    int HO, WO;            // output positions
+};
+hipError_t unfold(const float* img, float* cols, const ConvGeom& q, hipStream_t stream);
+hipError_t fold(const float* gcols, float* gimg, const ConvGeom& q, hipStream_t stream);
+hipError_t inf_backward_input_folded(const float* grad_output, const int32_t* pos, float* grad_img, const ConvGeom& q,
+                                     int G, int CO, hipStream_t stream);
+
 }  // namespace ldist

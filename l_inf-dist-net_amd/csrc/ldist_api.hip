@@ -63,6 +63,21 @@ int finish(hipError_t e) {
 
 bool valid_p(float p) { return p > 1.0f && std::isfinite(p); }
 
+// Fills q from the image and window sizes; the number of output positions follows torch's unfold.
+int conv_geometry(int B, int C, int H, int W, int KH, int KW, int stride, int padding, int dilation, ldist::ConvGeom& q) {
+    if (B <= 0 || C <= 0 || H <= 0 || W <= 0 || KH <= 0 || KW <= 0 || stride <= 0 || padding < 0 || dilation <= 0)
+        return LDIST_EINVAL;
+    const long long ho = ((long long)H + 2LL * padding - (long long)dilation * (KH - 1) - 1) / stride + 1;
+    const long long wo = ((long long)W + 2LL * padding - (long long)dilation * (KW - 1) - 1) / stride + 1;
+    if ((long long)H + 2LL * padding < (long long)dilation * (KH - 1) + 1 ||
+        (long long)W + 2LL * padding < (long long)dilation * (KW - 1) + 1)
+        return LDIST_EINVAL;   // the window does not fit the padded image
+    const long long lim = 1LL << 31;
+    if ((long long)B * C * H * W >= lim || (long long)B * C * KH * KW * ho * wo >= lim) return LDIST_ERANGE;
+    q = ldist::ConvGeom{B, C, H, W, KH, KW, stride, padding, dilation, (int)ho, (int)wo};
+    return LDIST_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -197,6 +212,40 @@ int ldist_adamw_lp_step(float* param, const float* grad, float* exp_avg, float* 
     if (int rc = current_device(pr)) return rc;
     return finish(ldist::adamw_lp_step(param, grad, exp_avg, exp_avg_sq, rows, cols, p_norm, lr, beta1, beta2, eps,
                                        weight_decay, step, (hipStream_t)stream));
+}
+
+int ldist_unfold(const float* img, int B, int C, int H, int W, int KH, int KW, int stride, int padding, int dilation,
+                 float* cols, ldist_stream_t stream) {
+    ldist::ConvGeom q{};
+    if (!img || !cols) return LDIST_EINVAL;
+    if (int rc = conv_geometry(B, C, H, W, KH, KW, stride, padding, dilation, q)) return rc;
+    ldist::Problem pr{};
+    if (int rc = current_device(pr)) return rc;
+    return finish(ldist::unfold(img, cols, q, (hipStream_t)stream));
+}
+
+int ldist_fold(const float* grad_cols, int B, int C, int H, int W, int KH, int KW, int stride, int padding,
+               int dilation, float* grad_img, ldist_stream_t stream) {
+    ldist::ConvGeom q{};
+    if (!grad_cols || !grad_img) return LDIST_EINVAL;
+    if (int rc = conv_geometry(B, C, H, W, KH, KW, stride, padding, dilation, q)) return rc;
+    ldist::Problem pr{};
+    if (int rc = current_device(pr)) return rc;
+    return finish(ldist::fold(grad_cols, grad_img, q, (hipStream_t)stream));
+}
+
+int ldist_inf_dist_backward_input_folded(const float* grad_output, const int32_t* pos, int B, int CO, int C, int G,
+                                         int H, int W, int KH, int KW, int stride, int padding, int dilation,
+                                         float* grad_img, ldist_stream_t stream) {
+    ldist::ConvGeom q{};
+    if (!grad_output || !pos || !grad_img || CO <= 0 || G <= 0) return LDIST_EINVAL;
+    if (int rc = conv_geometry(B, C, H, W, KH, KW, stride, padding, dilation, q)) return rc;
+    if (C % G != 0 || CO % G != 0) return LDIST_EINVAL;
+    if ((long long)B * CO * q.HO * q.WO >= (1LL << 31)) return LDIST_ERANGE;
+    if ((long long)(C / G) * W > 16384) return LDIST_ERANGE;   // one image row of a group must fit the LDS bins
+    ldist::Problem pr{};
+    if (int rc = current_device(pr)) return rc;
+    return finish(ldist::inf_backward_input_folded(grad_output, pos, grad_img, q, G, CO, (hipStream_t)stream));
 }
 
 }  // extern "C"

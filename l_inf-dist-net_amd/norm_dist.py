@@ -76,6 +76,58 @@ class DistF(torch.autograd.Function):
         return gx, gw, None, None, None
 
 
+class _Unfold(torch.autograd.Function):
+    """F.unfold for float32 GPU images as one native kernel, with the native fold as its backward."""
+
+    @staticmethod
+    def forward(ctx, img, kernel_size, dilation, padding, stride):
+        img = img.contiguous()
+        ho, wo = norm_dist_cpp.conv_output_size(img.size(2), img.size(3), kernel_size, stride, padding, dilation)
+        cols = torch.empty(img.size(0), img.size(1) * kernel_size * kernel_size, ho * wo, device=img.device,
+                           dtype=img.dtype)
+        norm_dist_cpp.unfold(img, cols, kernel_size, stride, padding, dilation)
+        ctx.geometry = (img.shape, kernel_size, stride, padding, dilation)
+        return cols
+
+    @staticmethod
+    def backward(ctx, grad_cols):
+        shape, kernel_size, stride, padding, dilation = ctx.geometry
+        grad_img = torch.empty(shape, device=grad_cols.device, dtype=grad_cols.dtype)
+        norm_dist_cpp.fold(grad_cols.contiguous(), grad_img, kernel_size, stride, padding, dilation)
+        return grad_img, None, None, None, None
+
+
+class _ConvInfDist(torch.autograd.Function):
+    """The L_inf layer on an image: unfold, distance forward, and in the backward pass the gradient
+    with respect to the image directly (scatter and fold fused), so that neither the columns nor
+    their nine times larger gradient outlive the call.  Same results as unfold + DistF."""
+
+    @staticmethod
+    def forward(ctx, img, weight, group, kernel_size, dilation, padding, stride):
+        cols = _Unfold.forward(ctx, img, kernel_size, dilation, padding, stride)
+        y = torch.empty(_out_shape(cols, weight), device=img.device, dtype=img.dtype)
+        argmax = torch.empty(y.shape, device=img.device, dtype=torch.int32)
+        norm_dist_cpp.inf_dist_forward(cols, weight, y, argmax, group)
+        ctx.save_for_backward(argmax)
+        ctx.group, ctx.weight_shape = group, weight.shape
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        (argmax,) = ctx.saved_tensors
+        shape, kernel_size, stride, padding, dilation = ctx.geometry
+        g = grad_output.contiguous()
+        grad_img = grad_w = None
+        if ctx.needs_input_grad[0]:
+            grad_img = torch.empty(shape, device=g.device, dtype=g.dtype)
+            norm_dist_cpp.inf_dist_backward_input_folded(g, argmax, grad_img, ctx.group, kernel_size, stride, padding,
+                                                         dilation)
+        if ctx.needs_input_grad[1]:
+            grad_w = torch.empty(ctx.weight_shape, device=g.device, dtype=g.dtype)
+            norm_dist_cpp.inf_dist_backward_weight_overwrite(g, argmax, grad_w, ctx.group)
+        return grad_img, grad_w, None, None, None, None, None
+
+
 def _pairwise_difference(inp, weight, group):
     """(B, G, CO/G, CI/G, HW) tensor of input minus weight, by broadcasting."""
     b, _, hw = inp.shape
@@ -219,7 +271,16 @@ class NormDistConv(nn.Module):
         """(B, C*k*k, L) patches of t; a 1x1 window needs no unfold (which launches one kernel per image)."""
         if self.kernel_size == 1 and self.stride == 1 and self.padding == 0:
             return t.reshape(t.size(0), t.size(1), -1)
+        if t.is_cuda and t.dtype == torch.float32:
+            return _Unfold.apply(t, self.kernel_size, self.dilation, self.padding, self.stride)
         return F.unfold(t, self.kernel_size, self.dilation, self.padding, self.stride)
+
+    def _fused_inf_conv(self, x):
+        """True when the image-space L_inf path applies: a real window, p = inf, float32 on the GPU, and one
+        image row of a group small enough for the fused backward kernel."""
+        return (math.isinf(self.p) and x.is_cuda and x.dtype == torch.float32 and
+                not (self.kernel_size == 1 and self.stride == 1 and self.padding == 0) and
+                (self.in_channels // self.group) * x.size(3) <= norm_dist_cpp.FOLDED_MAX_ROW_FLOATS)
 
     def _shift(self, t):
         if self.normalize is not None:
@@ -232,7 +293,10 @@ class NormDistConv(nn.Module):
         span = self.kernel_size - 2 * self.padding
         out_hw = ((x.size(2) - span) // self.stride + 1, (x.size(3) - span) // self.stride + 1)
         w2d = self.weight.view(self.weight.size(0), -1)
-        y = norm_dist(self._columns(x), w2d, self.group, p=self.p, tag=self.tag)
+        if self._fused_inf_conv(x):
+            y = _ConvInfDist.apply(x, w2d, self.group, self.kernel_size, self.dilation, self.padding, self.stride)
+        else:
+            y = norm_dist(self._columns(x), w2d, self.group, p=self.p, tag=self.tag)
         y = self._shift(y.view(x.size(0), -1, *out_hw))  # in training mode only y moves the running mean
         if lower is None or upper is None:
             return y, None, None

@@ -202,3 +202,54 @@ def adamw_lp_step(param, grad, exp_avg, exp_avg_sq, p_norm, lr, beta1, beta2, ep
     _call("ldist_adamw_lp_step", dev, _p(param), _p(grad), _p(exp_avg), _p(exp_avg_sq), rows, cols,
           -1.0 if p_norm is None else float(p_norm), float(lr), float(beta1), float(beta2), float(eps),
           float(weight_decay), int(step))
+
+
+def _conv_args(img, kernel_size, stride, padding, dilation):
+    _expect(img.dim() == 4, "img must be (B, C, H, W)")
+    B, C, H, W = img.shape
+    return B, C, H, W, int(kernel_size), int(kernel_size), int(stride), int(padding), int(dilation)
+
+
+def conv_output_size(H, W, kernel_size, stride=1, padding=0, dilation=1):
+    span = dilation * (kernel_size - 1) + 1
+    return (H + 2 * padding - span) // stride + 1, (W + 2 * padding - span) // stride + 1
+
+
+def unfold(img, cols, kernel_size, stride=1, padding=0, dilation=1):
+    """cols (B, C*k*k, HO*WO) = torch.nn.functional.unfold(img, k, dilation, padding, stride), in one kernel."""
+    _check_input(img, "img")
+    _check_input(cols, "cols")
+    dev = _same_device(img, cols)
+    B, C, H, W, KH, KW, S, P, D = _conv_args(img, kernel_size, stride, padding, dilation)
+    HO, WO = conv_output_size(H, W, KH, S, P, D)
+    _expect(cols.shape == (B, C * KH * KW, HO * WO), "cols must be (B, C*k*k, HO*WO)")
+    _call("ldist_unfold", dev, _p(img), B, C, H, W, KH, KW, S, P, D, _p(cols))
+
+
+def fold(grad_cols, grad_img, kernel_size, stride=1, padding=0, dilation=1):
+    """grad_img (B, C, H, W) = the adjoint of unfold applied to grad_cols; every element is written."""
+    _check_input(grad_cols, "grad_cols")
+    _check_input(grad_img, "grad_img")
+    dev = _same_device(grad_cols, grad_img)
+    B, C, H, W, KH, KW, S, P, D = _conv_args(grad_img, kernel_size, stride, padding, dilation)
+    HO, WO = conv_output_size(H, W, KH, S, P, D)
+    _expect(grad_cols.shape == (B, C * KH * KW, HO * WO), "grad_cols must be (B, C*k*k, HO*WO)")
+    _call("ldist_fold", dev, _p(grad_cols), B, C, H, W, KH, KW, S, P, D, _p(grad_img))
+
+
+FOLDED_MAX_ROW_FLOATS = 16384   # (C/G) * W must fit the kernel's LDS bins
+
+
+def inf_dist_backward_input_folded(grad_output, pos, grad_img, G, kernel_size, stride=1, padding=0, dilation=1):
+    """Gradient of the L_inf layer with respect to the image: inf_dist_backward_input followed by fold, fused."""
+    _check_input(grad_output, "grad_output")
+    _check_input(pos, "pos", torch.int32)
+    _check_input(grad_img, "grad_img")
+    dev = _same_device(grad_output, pos, grad_img)
+    B, C, H, W, KH, KW, S, P, D = _conv_args(grad_img, kernel_size, stride, padding, dilation)
+    HO, WO = conv_output_size(H, W, KH, S, P, D)
+    CO = grad_output.size(1)
+    _expect(grad_output.dim() == 3 and grad_output.shape == pos.shape and grad_output.size(0) == B and
+            grad_output.size(2) == HO * WO, "grad_output and pos must be (B, CO, HO*WO)")
+    _call("ldist_inf_dist_backward_input_folded", dev, _p(grad_output), _p(pos), B, CO, C, G, H, W, KH, KW, S, P, D,
+          _p(grad_img))

@@ -39,7 +39,7 @@ def test_every_declared_symbol_is_exported(lib):
 
 def test_binding_signatures_cover_all_compute_entry_points():
     pkg = entry.load_package()
-    compute = [n for n in declared_symbols() if "_dist_" in n or n in ("ldist_mean_shift", "ldist_adamw_lp_step")]
+    compute = [n for n in declared_symbols() if "_dist_" in n or n in ("ldist_mean_shift", "ldist_adamw_lp_step", "ldist_unfold", "ldist_fold")]
     assert sorted(pkg._lib.SIGNATURES) == sorted(compute)
 
 

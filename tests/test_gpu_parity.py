@@ -311,6 +311,85 @@ def test_adamw_optimizer_on_gpu_follows_the_cpu_optimizer():
             torch.testing.assert_close(b.detach().cpu(), a.detach(), rtol=2e-5, atol=2e-6)
 
 
+CONV_CASES = [  # B, C, H, W, k, stride, padding, dilation
+    (2, 4, 8, 8, 3, 1, 1, 1), (3, 6, 9, 7, 3, 1, 0, 1), (2, 8, 12, 12, 3, 2, 1, 1), (1, 3, 11, 13, 5, 1, 2, 1),
+    (2, 4, 10, 10, 3, 1, 2, 2), (4, 16, 32, 32, 3, 1, 1, 1), (2, 2, 6, 6, 2, 2, 0, 1),
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_unfold_and_fold_kernels(case):
+    """Native patch extraction against torch.nn.functional.unfold (bit-equal: it only copies), and its
+    adjoint against autograd through F.unfold."""
+    import torch.nn.functional as F
+    from gpu_common import DEV, cpp, say
+    say("unfold/fold", case)
+    B, C, H, W, k, s_, p_, d_ = case
+    img = torch.randn(B, C, H, W, generator=gen(51))
+    ref = F.unfold(img, k, d_, p_, s_)
+    cols = torch.full(ref.shape, float("nan"), device=DEV)
+    cpp.unfold(img.to(DEV), cols, k, s_, p_, d_)
+    torch.cuda.synchronize()
+    assert torch.equal(cols.cpu(), ref)
+    gcols = torch.randn(ref.shape, generator=gen(52))
+    leaf = img.double().requires_grad_(True)
+    F.unfold(leaf, k, d_, p_, s_).backward(gcols.double())
+    gimg = torch.full(img.shape, float("nan"), device=DEV)
+    cpp.fold(gcols.to(DEV), gimg, k, s_, p_, d_)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(gimg.cpu().double(), leaf.grad, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("group", [1, 2])
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_inf_backward_input_folded(case, group):
+    """Scatter and fold fused, against the oracle's scatter into the columns followed by torch's fold."""
+    import torch.nn.functional as F
+    from gpu_common import DEV, cpp, say
+    B, C, H, W, k, s_, p_, d_ = case
+    if C % group:
+        pytest.skip("channels do not divide into the groups")
+    say("inf_backward_input_folded", case, "group", group)
+    CO = 6 * group
+    img = torch.randn(B, C, H, W, generator=gen(53))
+    w = torch.randn(CO, C // group * k * k, generator=gen(54)) * 0.5
+    cols = F.unfold(img, k, d_, p_, s_).contiguous()
+    _, pos = oracle.inf_dist_forward(cols, w, group)
+    go = torch.randn(B, CO, cols.size(2), generator=gen(55))
+    gcols = oracle.inf_dist_backward_input(go, pos, cols.size(1), group)
+    expect = F.fold(gcols.double(), (H, W), k, d_, p_, s_)
+    gimg = torch.full(img.shape, float("nan"), device=DEV)
+    cpp.inf_dist_backward_input_folded(go.to(DEV), pos.to(DEV), gimg, group, k, s_, p_, d_)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(gimg.cpu().double(), expect, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("p", [float("inf"), 8.0])
+def test_conv_layer_image_path_matches_column_path(p):
+    """NormDistConv on the GPU (native unfold; for p = inf the fused image-space backward) against the same
+    layer evaluated through F.unfold + norm_dist with autograd folding the gradient."""
+    import torch.nn.functional as F
+    from gpu_common import DEV, pkg
+    torch.manual_seed(7)
+    layer = pkg.NormDistConv(8, 12, 3, stride=1, padding=1, group=2, p=p, bias=True, mean_normalize=True).to(DEV).train()
+    x = torch.randn(4, 8, 10, 10, generator=gen(56)).to(DEV)
+    up = torch.randn(4, 12, 10, 10, generator=gen(57)).to(DEV)
+    xa = x.clone().requires_grad_(True)
+    ya, _, _ = layer(xa)
+    ya.backward(up)
+    ga, gwa = xa.grad.clone(), layer.weight.grad.clone()
+    layer.weight.grad = None
+    xb = x.clone().requires_grad_(True)
+    yb = pkg.norm_dist(F.unfold(xb, 3, 1, 1, 1), layer.weight.view(12, -1), 2, p).view(4, 12, 10, 10)
+    yb = layer._shift(yb)
+    yb.backward(up)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(ya, yb, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(ga, xb.grad, rtol=RTOL, atol=ATOL)
+    # each weight gradient sums 400 terms of order one, in an order the LDS atomics do not fix
+    torch.testing.assert_close(gwa, layer.weight.grad, rtol=1e-4, atol=5e-5)
+
+
 def test_error_codes_and_checks():
     from gpu_common import DEV, cpp, pkg
     lib = pkg._lib.lib()
