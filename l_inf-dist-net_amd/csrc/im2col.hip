@@ -13,35 +13,83 @@
 
 namespace ldist {
 
-// One lane = four consecutive output positions of one (b, row of cols).  4-wide stores need L % 4 == 0.
+// Exact n / d for 0 <= n < 65536 by one multiply-high (d >= 1): q = (n * ceil(2^32 / d)) >> 32.
+// Larger n take the plain division.
+struct SmallDiv {
+    unsigned d, magic;
+    __host__ explicit SmallDiv(int div = 1) : d((unsigned)div), magic((unsigned)((0x100000000ULL + div - 1) / div)) {}
+    __device__ __forceinline__ int div(int n) const {
+        return d == 1 ? n : ((unsigned)n < 65536u ? (int)__umulhi((unsigned)n, magic) : (int)((unsigned)n / d));
+    }
+};
+
+// A lane takes VEC consecutive output positions of one image plane (b, c) and writes them to all
+// KH*KW rows of cols that belong to that plane: the window positions overlap, so the loads of one
+// lane mostly hit the lines its previous window position fetched, and a wave's stores to one row are
+// one contiguous kilobyte.  4-wide stores need L % 4 == 0.
 template <int VEC>
 __global__ void __launch_bounds__(256)
-unfold_kernel(const float* __restrict__ img, float* __restrict__ cols, ConvGeom q) {
+unfold_kernel(const float* __restrict__ img, float* __restrict__ cols, ConvGeom q, int blocks_per_plane,
+              SmallDiv by_wo) {
     const int L = q.HO * q.WO;
-    const int per_row = (L + VEC - 1) / VEC;
-    const long long total = (long long)q.B * q.C * q.KH * q.KW * per_row;
-    for (long long id = (long long)blockIdx.x * 256 + threadIdx.x; id < total; id += (long long)gridDim.x * 256) {
-        const int v = (int)(id % per_row);
-        const long long row = id / per_row;                 // b * (C*KH*KW) + (c*KH + i)*KW + j
-        const int j = (int)(row % q.KW);
-        const long long r1 = row / q.KW;
-        const int i = (int)(r1 % q.KH);
-        const long long bc = r1 / q.KH;                     // b * C + c
-        const float* plane = img + bc * q.H * q.W;
-        float out[VEC];
+    const long long bc = blockIdx.x / blocks_per_plane;       // b * C + c
+    const int v = (blockIdx.x % blocks_per_plane) * 256 + threadIdx.x;
+    if ((long long)v * VEC >= L) return;
+    const float* plane = img + bc * q.H * q.W;
+    int y0[VEC], x0[VEC];
 #pragma unroll
-        for (int e = 0; e < VEC; e++) {
-            const int l = v * VEC + e;
-            const int h = l / q.WO, w = l - h * q.WO;
-            const int y = h * q.S + i * q.D - q.P, x = w * q.S + j * q.D - q.P;
-            out[e] = (l < L && (unsigned)y < (unsigned)q.H && (unsigned)x < (unsigned)q.W) ? plane[y * q.W + x] : 0.f;
+    for (int e = 0; e < VEC; e++) {
+        const int l = min(v * VEC + e, L - 1);
+        const int h = by_wo.div(l), w = l - h * q.WO;
+        y0[e] = h * q.S - q.P;
+        x0[e] = w * q.S - q.P;
+    }
+    float* dst = cols + bc * q.KH * q.KW * L + (long long)v * VEC;
+    for (int i = 0; i < q.KH; i++)
+        for (int j = 0; j < q.KW; j++) {
+            float out[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                const int y = y0[e] + i * q.D, x = x0[e] + j * q.D;
+                out[e] = ((unsigned)y < (unsigned)q.H && (unsigned)x < (unsigned)q.W) ? plane[y * q.W + x] : 0.f;
+            }
+            float* row = dst + (long long)(i * q.KW + j) * L;
+            if constexpr (VEC == 4) {
+                *reinterpret_cast<float4*>(row) = make_float4(out[0], out[1], out[2], out[3]);
+            } else {
+                row[0] = out[0];
+            }
         }
-        float* dst = cols + row * L + (long long)v * VEC;
-        if constexpr (VEC == 4) {
-            *reinterpret_cast<float4*>(dst) = make_float4(out[0], out[1], out[2], out[3]);
-        } else {
-            dst[0] = out[0];
+}
+
+// The common window: 3 x 3, stride 1, dilation 1, padding 1, W % 4 == 0, 16-byte aligned tensors.
+// A lane takes four neighbouring pixels of one image row; per window row it needs the aligned
+// float4 of those pixels and the two pixels next to it, and writes three float4 (the j = 0, 1, 2
+// rows of cols): 9 loads for 9 stores instead of 36.
+__global__ void __launch_bounds__(256)
+unfold_3x3_kernel(const float* __restrict__ img, float* __restrict__ cols, int planes, int H, int W) {
+    const int L = H * W, quads = L / 4;
+    const long long id = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (id >= (long long)planes * quads) return;
+    const long long bc = id / quads;
+    const int v = (int)(id - bc * quads);
+    const int l = v * 4, h = l / W, w = l - h * W;
+    const float* plane = img + bc * L;
+    float* dst = cols + bc * 9 * L + l;
+#pragma unroll
+    for (int i = 0; i < 3; i++) {
+        const int y = h + i - 1;
+        float4 mid = make_float4(0.f, 0.f, 0.f, 0.f);
+        float left = 0.f, right = 0.f;
+        if ((unsigned)y < (unsigned)H) {
+            const float* r = plane + y * W + w;
+            mid = *reinterpret_cast<const float4*>(r);
+            if (w > 0) left = r[-1];
+            if (w + 4 < W) right = r[4];
         }
+        *reinterpret_cast<float4*>(dst + (long long)(i * 3 + 0) * L) = make_float4(left, mid.x, mid.y, mid.z);
+        *reinterpret_cast<float4*>(dst + (long long)(i * 3 + 1) * L) = mid;
+        *reinterpret_cast<float4*>(dst + (long long)(i * 3 + 2) * L) = make_float4(mid.y, mid.z, mid.w, right);
     }
 }
 
@@ -80,7 +128,8 @@ fold_kernel(const float* __restrict__ gcols, float* __restrict__ gimg, ConvGeom 
 // workgroups, each keeping only what lands in its own rows.
 __global__ void __launch_bounds__(256)
 inf_backward_input_folded_kernel(const float* __restrict__ grad_output, const int32_t* __restrict__ pos,
-                                 float* __restrict__ grad_img, ConvGeom q, int G, int NG, int R, int row_tiles) {
+                                 float* __restrict__ grad_img, ConvGeom q, int G, int NG, int R, int row_tiles,
+                                 SmallDiv by_khw, SmallDiv by_kw, SmallDiv by_wo) {
     extern __shared__ float bins[];
     const int CG = q.C / G;
     const int tile = blockIdx.x % row_tiles;
@@ -100,16 +149,17 @@ inf_backward_input_folded_kernel(const float* __restrict__ grad_output, const in
     const int span = (h_hi - h_lo + 1) * q.WO;      // contiguous run of output positions per output channel
     if (span > 0) {
         const size_t obase = ((size_t)bg * NG) * L + (size_t)h_lo * q.WO;
-        const int total = NG * span;
         const int khw = q.KH * q.KW;
-        for (int e = threadIdx.x; e < total; e += 256) {
-            const int n = e / span, t = e - n * span;
+        // lanes run along the positions of one output channel, channels are shared out over the waves
+        for (int n = threadIdx.x >> 6; n < NG; n += 4)
+        for (int t = threadIdx.x & 63; t < span; t += 64) {
             const size_t o = obase + (size_t)n * L + t;
             const int p = pos[o];
             const int k = p & 0x7fffffff;
-            const int c = k / khw, r = k - c * khw;
-            const int i = r / q.KW, j = r - i * q.KW;
-            const int h = h_lo + t / q.WO, w = t % q.WO;
+            const int c = by_khw.div(k), r = k - c * khw;
+            const int i = by_kw.div(r), j = r - i * q.KW;
+            const int th = by_wo.div(t);
+            const int h = h_lo + th, w = t - th * q.WO;
             const int y = h * q.S + i * q.D - q.P - y0, x = w * q.S + j * q.D - q.P;
             if ((unsigned)y < (unsigned)rows && (unsigned)x < (unsigned)q.W && c < CG) {
                 const float gv = grad_output[o];
@@ -134,11 +184,23 @@ static unsigned grid_for(long long items) {
 
 hipError_t unfold(const float* img, float* cols, const ConvGeom& q, hipStream_t stream) {
     const int L = q.HO * q.WO;
-    const long long rows = (long long)q.B * q.C * q.KH * q.KW;
+    const long long planes = (long long)q.B * q.C;
+    if (q.KH == 3 && q.KW == 3 && q.S == 1 && q.D == 1 && q.P == 1 && q.W % 4 == 0 && aligned16(img) &&
+        aligned16(cols)) {
+        const long long lanes = planes * (q.H * q.W / 4);
+        hipLaunchKernelGGL(unfold_3x3_kernel, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, stream, img, cols,
+                           (int)planes, q.H, q.W);
+        return hipGetLastError();
+    }
+    const SmallDiv by_wo(q.WO);
     if (L % 4 == 0 && aligned16(cols)) {
-        hipLaunchKernelGGL(unfold_kernel<4>, dim3(grid_for(rows * (L / 4))), dim3(256), 0, stream, img, cols, q);
+        const int bpp = (L / 4 + 255) / 256;
+        hipLaunchKernelGGL(unfold_kernel<4>, dim3((unsigned)(planes * bpp)), dim3(256), 0, stream, img, cols, q, bpp,
+                           by_wo);
     } else {
-        hipLaunchKernelGGL(unfold_kernel<1>, dim3(grid_for(rows * L)), dim3(256), 0, stream, img, cols, q);
+        const int bpp = (L + 255) / 256;
+        hipLaunchKernelGGL(unfold_kernel<1>, dim3((unsigned)(planes * bpp)), dim3(256), 0, stream, img, cols, q, bpp,
+                           by_wo);
     }
     return hipGetLastError();
 }
@@ -159,7 +221,8 @@ hipError_t inf_backward_input_folded(const float* grad_output, const int32_t* po
     const int row_tiles = (q.H + R - 1) / R;
     const size_t lds = (size_t)CG * R * q.W * sizeof(float);
     hipLaunchKernelGGL(inf_backward_input_folded_kernel, dim3((unsigned)(q.B * G * row_tiles)), dim3(256), lds, stream,
-                       grad_output, pos, grad_img, q, G, NG, R, row_tiles);
+                       grad_output, pos, grad_img, q, G, NG, R, row_tiles, SmallDiv(q.KH * q.KW), SmallDiv(q.KW),
+                       SmallDiv(q.WO));
     return hipGetLastError();
 }
 
