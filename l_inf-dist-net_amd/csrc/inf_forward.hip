@@ -141,8 +141,8 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
         static_assert(BM * BN % NGQ == 0 && NIT % (2 * DEPTH) == 0, "whole batches");
         const int sub = tid % LPO, gq = tid / LPO;
         const int shift = (tid & 63) - sub;         // bit of this lane group's first lane in a ballot
-        const float* xg = input + (size_t)g * K + 4 * sub;
-        const float* wg = weight + (size_t)g * d.NG * K + 4 * sub;
+        const float* xg = input + (size_t)g * K;
+        const float* wg = weight + (size_t)g * d.NG * K;
         // element offsets fit 32 bits: the entry point rejects tensors of 2^31 elements or more
         const unsigned ldx = (unsigned)d.G * K;
         struct Slot { float4 x, w; int kb; };
@@ -152,7 +152,9 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
             const int ml = o / BN, nl = o - ml * BN;
             const unsigned m = min(m0 + ml, d.M - 1), n = min(n0 + nl, d.NG - 1);
             const int kb = cand_c[o] * kChunk;
-            const unsigned off = kb + 4 * sub < K ? kb : kb - 4 * sub;   // past the end of the row: its first 16 bytes, masked below
+            // a lane whose 16 bytes lie past the end of the row reads the chunk's first 16 instead (masked
+            // below); the offset must never go negative, it is added as an unsigned 32-bit quantity
+            const unsigned off = kb + 4 * sub < K ? kb + 4 * sub : kb;
             sl.kb = kb;
             sl.x = *reinterpret_cast<const float4*>(xg + (m * ldx + off));
             sl.w = *reinterpret_cast<const float4*>(wg + (n * (unsigned)K + off));

@@ -19,6 +19,8 @@ SHAPES = [
     (5, 7, 3, 1, 1),          # tiny, few outputs (one-wave-per-row kernel)
     (33, 100, 77, 1, 1),      # K % 4 != 0: scalar loads, ragged M / N / K
     (130, 70, 260, 1, 1),     # vector loads, M and N tails, K tail inside a chunk
+    (20, 40, 12, 1, 1),       # vector loads with K shorter than one chunk of 32
+    (9, 24, 36, 1, 1),        # vector loads, second chunk holds a single group of four
     (64, 96, 96, 3, 1),       # groups, K = 32 exactly one chunk
     (64, 48, 96, 3, 1),       # groups with 16 outputs each
     (256, 160, 784, 1, 1),    # MNIST-sized K, two N tiles of 80
@@ -358,10 +360,12 @@ def test_inf_backward_input_folded(case, group):
     go = torch.randn(B, CO, cols.size(2), generator=gen(55))
     gcols = oracle.inf_dist_backward_input(go, pos, cols.size(1), group)
     expect = F.fold(gcols.double(), (H, W), k, d_, p_, s_)
+    terms = F.fold(oracle.inf_dist_backward_input(go.abs(), pos & ~SIGN, cols.size(1), group).double(), (H, W), k, d_,
+                   p_, s_).abs()   # sum of |term| per pixel: the float32 sum is good to 1e-6 of that, in any order
     gimg = torch.full(img.shape, float("nan"), device=DEV)
     cpp.inf_dist_backward_input_folded(go.to(DEV), pos.to(DEV), gimg, group, k, s_, p_, d_)
     torch.cuda.synchronize()
-    torch.testing.assert_close(gimg.cpu().double(), expect, rtol=RTOL, atol=ATOL)
+    assert_sum_close(gimg.cpu(), expect, terms, rtol=RTOL, atol=ATOL)
 
 
 @pytest.mark.parametrize("p", [float("inf"), 8.0])
