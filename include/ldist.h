@@ -39,7 +39,8 @@ enum {
     LDIST_EINVAL = -1,  /* null pointer, non-positive size, CI % G or CO % G non-zero, p <= 1 or NaN */
     LDIST_ERANGE = -2,  /* a tensor has 2^31 or more elements (kernels index with 32 bits) */
     LDIST_ELAUNCH = -3, /* the HIP runtime reported an error at launch (see ldist_last_hip_error) */
-    LDIST_EDEVICE = -4  /* the current device is not a gfx950 the library was built for */
+    LDIST_EDEVICE = -4, /* the current device is not a gfx950 the library was built for */
+    LDIST_EUNSUPPORTED = -5 /* a specialised entry point does not cover this geometry: use the general one */
 };
 
 typedef void* ldist_stream_t; /* hipStream_t */
@@ -160,6 +161,24 @@ int ldist_adamw_lp_step(float* param, const float* grad, float* exp_avg, float* 
  * img is (B, C, H, W), cols is (B, C*KH*KW, HO*WO).  No native counterpart in the reference. */
 int ldist_unfold(const float* img, int B, int C, int H, int W, int KH, int KW, int stride, int padding, int dilation,
                  float* cols, ldist_stream_t stream);
+
+/* L_inf forward of the convolution-shaped layer straight from the image, without the unfolded tensor:
+ * what ldist_unfold followed by ldist_inf_dist_forward computes (the reference: F.unfold at
+ * model/norm_dist.py:132, then inf_dist_forward_cuda), bit for bit, reading the image once.
+ *   img (B, C, H, W), weight (CO, C/G*KH*KW), output and pos (B, CO, HO*WO).
+ * Covers 3x3 windows with dilation 1, stride 1 or 2, WO % 8 == 0, and a group's image rows fitting
+ * LDS; ldist_inf_dist_conv_forward_supported returns 1 for such a geometry, 0 otherwise, and
+ * ldist_inf_dist_conv_forward returns LDIST_EUNSUPPORTED for the rest (nothing is enqueued). */
+int ldist_inf_dist_conv_forward_supported(int C, int H, int W, int CO, int G, int KH, int KW, int stride, int padding,
+                                          int dilation);
+int ldist_inf_dist_conv_forward(const float* img, const float* weight, int B, int C, int H, int W, int CO, int G,
+                                int KH, int KW, int stride, int padding, int dilation, float* output, int32_t* pos,
+                                ldist_stream_t stream);
+/* Testing and tuning knob, no counterpart in the reference: output rows per workgroup of
+ * ldist_inf_dist_conv_forward; 0 (default) = chosen by shape.  A positive value is clamped to what the
+ * geometry allows and also switches off the rule that leaves small or channel-heavy layers, which
+ * would keep too few waves on a CU, to the general path.  Process-wide; not thread safe. */
+int ldist_set_conv_rows_override(int rows);
 
 /* Adjoint of ldist_unfold (what autograd does behind F.unfold): every element of grad_img is written
  * with the sum of the grad_cols entries that were copied from it. */

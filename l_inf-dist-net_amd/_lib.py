@@ -29,6 +29,8 @@ SIGNATURES = {
     "ldist_norm_dist_backward_weight": [_F, _F, _F, _F, _i, _i, _i, _i, _i, _F, _f, _S],
     "ldist_mean_shift": [_F, _i, _i, _i, _F, _F, _F, _f, _S],
     "ldist_unfold": [_F, _i, _i, _i, _i, _i, _i, _i, _i, _i, _F, _S],
+    "ldist_inf_dist_conv_forward_supported": [_i, _i, _i, _i, _i, _i, _i, _i, _i, _i],
+    "ldist_inf_dist_conv_forward": [_F, _F, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _F, _I, _S],
     "ldist_fold": [_F, _i, _i, _i, _i, _i, _i, _i, _i, _i, _F, _S],
     "ldist_inf_dist_backward_input_folded": [_F, _I, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _F, _S],
     "ldist_adamw_lp_step": [_F, _F, _F, _F, _i, _i, _d, _d, _d, _d, _d, _d, _i, _S],
@@ -58,6 +60,8 @@ def lib():
             fn.restype = ctypes.c_int
         handle.ldist_set_tile_override.argtypes = [ctypes.c_int]
         handle.ldist_set_tile_override.restype = ctypes.c_int
+        handle.ldist_set_conv_rows_override.argtypes = [ctypes.c_int]
+        handle.ldist_set_conv_rows_override.restype = ctypes.c_int
         handle.ldist_version.restype = ctypes.c_int
         handle.ldist_strerror.restype = ctypes.c_char_p
         handle.ldist_strerror.argtypes = [ctypes.c_int]

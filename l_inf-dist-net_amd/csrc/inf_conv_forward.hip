@@ -1,0 +1,336 @@
+// L_inf distance layer on an image without the unfolded tensor (the reference unfolds with F.unfold,
+// model/norm_dist.py:132, and then calls inf_dist_forward_cuda on the nine times larger columns):
+//   out[b, g*NG + n, h*WO + w] = max_k |x_k - weight[g*NG + n, k]|,  k = (c*3 + i)*3 + j,
+//   x_k = img[b, g*CG + c, h*S + i - P, w*S + j - P]   (0 outside the image),
+// pos as in the column kernel (lowest k of the maximum, bit 31 = sign of the difference, 0 for a zero maximum).
+// Values and indices equal the column path's bit for bit: the same fp32 subtractions of the same numbers.
+//
+// A workgroup owns R output rows of one (image, group) and BN of the group's outputs.  The image rows those
+// positions look at, all CG channels of them, are copied once into LDS with the zero padding materialised, and
+// stay there; the weights stream through a double-buffered LDS stage of CC channels (9*CC values of k), stored
+// k-major so that a lane's four outputs are one 128-bit read.  A lane owns 8 neighbouring positions of one
+// output row times 4 outputs.  For a window row (c, i) it reads the 8 + 2 pixels its positions cover for
+// j = 0, 1, 2 with three (stride 2: five) aligned 128-bit reads, so 12 LDS words serve 24 differences.
+// The loop keeps the maximum per channel and records the channel of the running maximum (subtract + half a
+// v_max3 per difference, three instructions per channel and output); the lowest k inside the recorded
+// channel is found afterwards from the image rows still in LDS.
+#include "kernels.hpp"
+
+namespace ldist {
+
+int g_conv_rows_override = 0;   // > 0: output rows per workgroup forced (tests and tuning)
+
+namespace {
+
+constexpr int kTM = 8, kTN = 4;   // positions x outputs per lane
+constexpr int kCC = 4;            // channels per weight stage
+constexpr int kTrack = 1;         // channels per recorded unit
+constexpr int kKC = kCC * 9;      // k values per weight stage
+constexpr int kMaxThreads = 256;
+constexpr int kBNP = 68;          // row length of the weight stage: 64 outputs + 4, a constant so that reads take immediate offsets
+constexpr int kWRegs = 9;         // weight words a lane carries from global to LDS per stage (64 outputs x 36 / 256)
+
+struct ConvFwd {
+    int B, G, CG, NG, K;         // images, groups, channels and outputs per group, K = 9*CG
+    int H, W, HO, WO, P;         // image, output positions, padding
+    int R, NR, WP, CGP;          // output rows per workgroup, image rows held, padded row length, CG rounded up to kCC
+    int SEG, ML, NL, BN;         // 8-position segments per output row, lanes along positions / outputs, outputs per
+                                 // workgroup
+    int tiles_h, tiles_n;
+    int vec_in, vec_out;         // 128-bit global loads of image rows / stores of results allowed
+};
+
+template <int S>
+__global__ void __launch_bounds__(kMaxThreads, 2)
+inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__ weight, float* __restrict__ out,
+                        int32_t* __restrict__ pos, ConvFwd a) {
+    constexpr int NXR = (7 * S + 2) / 4 + 1;          // 128-bit reads per window row: pixels 0 .. 7*S + 2
+    extern __shared__ __align__(16) float lds[];
+    float* tile = lds;                                  // [CGP][NR][WP]
+    float* wst = lds + a.CGP * a.NR * a.WP;             // 2 x [kKC][kBNP]
+    const int tid = threadIdx.x, NT = blockDim.x;
+
+    int id = blockIdx.x;
+    const int tn = id % a.tiles_n; id /= a.tiles_n;
+    const int th = id % a.tiles_h; id /= a.tiles_h;
+    const int g = id % a.G, b = id / a.G;
+    const int h0 = th * a.R, n0 = tn * a.BN;
+    const int y0 = h0 * S - a.P;
+    const int NR = a.NR, WP = a.WP, K = a.K;
+    constexpr int BNP = kBNP;
+
+    // ---- weights: global -> registers -> LDS stage, k-major ----
+    const float* wgrp = weight + ((size_t)g * a.NG + n0) * K;
+    const int nvalid = min(a.NG - n0, a.BN);            // outputs of this tile that exist
+    float wreg[kWRegs];
+    auto wload = [&](int ch) {
+        const int kb = ch * kKC;
+#pragma unroll
+        for (int r = 0; r < kWRegs; r++) {
+            const int idx = tid + r * NT;
+            const int n = idx / kKC, kk = idx - n * kKC;
+            // branch-free: an entry that does not exist reads the tile's first weight and is replaced by zero
+            const bool real = n < nvalid && kb + kk < K;
+            const float v = wgrp[real ? (unsigned)(n * K + kb + kk) : 0u];
+            wreg[r] = real ? v : 0.f;
+        }
+    };
+    auto wstore = [&](float* stage) {
+#pragma unroll
+        for (int r = 0; r < kWRegs; r++) {
+            const int idx = tid + r * NT;
+            const int n = idx / kKC, kk = idx - n * kKC;
+            stage[kk * BNP + n] = wreg[r];   // n <= 63 (idx < kWRegs * 256 = 36 * 64): inside the stage, zeros beyond BN
+        }
+    };
+    // A workgroup too small to carry a whole stage in kWRegs words per lane (tiny images) moves the rest
+    // directly; with 256 lanes this loop is empty.
+    auto wrest = [&](int ch, float* stage) {
+        const int kb = ch * kKC;
+        for (int idx = tid + kWRegs * NT; idx < kKC * a.BN; idx += NT) {
+            const int n = idx / kKC, kk = idx - n * kKC;
+            const bool real = n < nvalid && kb + kk < K;
+            stage[kk * BNP + n] = real ? wgrp[(unsigned)(n * K + kb + kk)] : 0.f;
+        }
+    };
+    wload(0);
+
+    // ---- image rows -> LDS, padding as zeros ----
+    {
+        const int words = a.CGP * NR * WP;
+        for (int i = tid * 4; i < words; i += NT * 4) *reinterpret_cast<float4*>(tile + i) = make_float4(0.f, 0.f, 0.f, 0.f);
+        __syncthreads();
+        const float* src = img + ((size_t)b * a.G + g) * a.CG * a.H * a.W;
+        const int rows = a.CG * NR;
+        if (a.vec_in) {
+            const int QW = a.W / 4;
+            for (int i = tid; i < rows * QW; i += NT) {
+                const int row = i / QW, xq = i - row * QW;
+                const int c = row / NR, r = row - c * NR;
+                const int y = y0 + r;
+                if ((unsigned)y < (unsigned)a.H) {
+                    const float4 v = *reinterpret_cast<const float4*>(src + ((size_t)c * a.H + y) * a.W + 4 * xq);
+                    float* dst = tile + (c * NR + r) * WP + a.P + 4 * xq;
+                    dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+                }
+            }
+        } else {
+            for (int i = tid; i < rows * a.W; i += NT) {
+                const int row = i / a.W, x = i - row * a.W;
+                const int c = row / NR, r = row - c * NR;
+                const int y = y0 + r;
+                if ((unsigned)y < (unsigned)a.H) tile[(c * NR + r) * WP + a.P + x] = src[((size_t)c * a.H + y) * a.W + x];
+            }
+        }
+    }
+    wstore(wst);
+    wrest(0, wst);
+    __syncthreads();
+
+    // ---- lane geometry ----
+    const int nl = tid % a.NL, ml = tid / a.NL;
+    const int hr = ml / a.SEG, w0 = (ml - hr * a.SEG) * kTM;
+    const float* xlane = tile + (hr * S) * WP + w0 * S;        // + (c*NR + i)*WP: 16-byte aligned (WP % 4 == 0)
+
+    float acc[kTM][kTN];
+    int unit[kTM][kTN];
+#pragma unroll
+    for (int e = 0; e < kTM; e++)
+#pragma unroll
+        for (int t = 0; t < kTN; t++) { acc[e][t] = 0.f; unit[e][t] = 0; }
+
+    const int nstage = a.CGP / kCC;
+    const float* xch = xlane;
+    for (int ch = 0; ch < nstage; ch++) {
+        if (ch + 1 < nstage) wload(ch + 1);
+        const float* wrow = wst + (ch & 1) * kKC * BNP + kTN * nl;   // walks down the 9*kCC rows of the stage
+        const float* xrow = xch;                                     // walks down the window rows of its channels
+        // The loops over units, channels and window rows stay rolled: one trip is 6 LDS reads and 144
+        // arithmetic instructions, and its registers are all the compiler has to keep.
+#pragma unroll 1
+        for (int u = 0; u < kCC / kTrack; u++) {
+            float cm[kTM][kTN];
+#pragma unroll
+            for (int e = 0; e < kTM; e++)
+#pragma unroll
+                for (int t = 0; t < kTN; t++) cm[e][t] = 0.f;
+            // The 3*kTrack window rows of the unit, unrolled, with the reads of a row issued before the
+            // arithmetic of the row before it.
+            struct Row { float x[NXR * 4]; float w[3][kTN]; };
+            auto fetch = [&](Row& f, int r) {     // r = cc*3 + i: window row i of the unit's channel cc
+                const float* xp = xrow + ((r / 3) * NR + r % 3) * WP;
+#pragma unroll
+                for (int q = 0; q < NXR; q++) {
+                    const float4 v = *reinterpret_cast<const float4*>(xp + 4 * q);
+                    f.x[4 * q] = v.x; f.x[4 * q + 1] = v.y; f.x[4 * q + 2] = v.z; f.x[4 * q + 3] = v.w;
+                }
+#pragma unroll
+                for (int j = 0; j < 3; j++) {
+                    const float4 w4 = *reinterpret_cast<const float4*>(wrow + (3 * r + j) * BNP);
+                    f.w[j][0] = w4.x; f.w[j][1] = w4.y; f.w[j][2] = w4.z; f.w[j][3] = w4.w;
+                }
+            };
+            Row fa, fb;
+            fetch(fa, 0);
+#pragma unroll
+            for (int r = 0; r < 3 * kTrack; r++) {
+                Row& cur = (r & 1) ? fb : fa;
+                Row& nxt = (r & 1) ? fa : fb;
+                if (r + 1 < 3 * kTrack) fetch(nxt, r + 1);
+#pragma unroll
+                for (int j = 0; j < 3; j++)
+#pragma unroll
+                    for (int e = 0; e < kTM; e++)
+#pragma unroll
+                        for (int t = 0; t < kTN; t++)
+                            cm[e][t] = __builtin_fmaxf(cm[e][t], __builtin_fabsf(cur.x[e * S + j] - cur.w[j][t]));
+            }
+            xrow += kTrack * NR * WP;
+            wrow += 9 * kTrack * BNP;
+            const int un = ch * (kCC / kTrack) + u;
+#pragma unroll
+            for (int e = 0; e < kTM; e++)
+#pragma unroll
+                for (int t = 0; t < kTN; t++)
+                    if (cm[e][t] > acc[e][t]) { acc[e][t] = cm[e][t]; unit[e][t] = un; }
+        }
+        xch += kCC * NR * WP;
+        if (ch + 1 < nstage) {
+            wstore(wst + ((ch + 1) & 1) * kKC * BNP);
+            wrest(ch + 1, wst + ((ch + 1) & 1) * kKC * BNP);
+        }
+        __syncthreads();
+    }
+
+    // ---- the lowest k of the recorded unit, from the image rows in LDS and the weight rows in cache ----
+    const int h = h0 + hr;
+    if (h >= a.HO) return;
+    const int L = a.HO * a.WO;
+    // Per output the recorded channel's nine weights are contiguous: two 16-byte loads at 4-byte alignment
+    // and one word instead of one load per candidate, issued for the lane's eight positions together.
+    typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
+    static_assert(kTrack == 1, "a unit is one channel: nine candidates");
+#pragma unroll
+    for (int t = 0; t < kTN; t++) {
+        const int n = n0 + kTN * nl + t;
+        if (n >= a.NG) break;
+        const float* wn = weight + ((size_t)g * a.NG + n) * K;
+        float wq[kTM][9];
+#pragma unroll
+        for (int e = 0; e < kTM; e++) {
+            const float* wp = wn + unit[e][t] * 9;           // a recorded unit is a real channel: inside the row
+            const f4u q0 = *reinterpret_cast<const f4u*>(wp), q1 = *reinterpret_cast<const f4u*>(wp + 4);
+            wq[e][0] = q0.x; wq[e][1] = q0.y; wq[e][2] = q0.z; wq[e][3] = q0.w;
+            wq[e][4] = q1.x; wq[e][5] = q1.y; wq[e][6] = q1.z; wq[e][7] = q1.w;
+            wq[e][8] = wp[8];
+        }
+        int ps[kTM];
+#pragma unroll
+        for (int e = 0; e < kTM; e++) {
+            const float target = acc[e][t];
+            const float* xe = xlane + e * S + unit[e][t] * NR * WP;
+            int q = 0;
+            float dq = 0.f;
+#pragma unroll
+            for (int r = 8; r >= 0; r--) {                    // descending: the lowest match is the one kept
+                const float df = xe[(r / 3) * WP + r % 3] - wq[e][r];
+                if (__builtin_fabsf(df) == target) { q = r; dq = df; }
+            }
+            ps[e] = target > 0.f ? ((unit[e][t] * 9 + q) | (__float_as_int(dq) & 0x80000000)) : 0;
+        }
+        const size_t at = (((size_t)b * a.G + g) * a.NG + n) * L + (size_t)h * a.WO + w0;
+        if (a.vec_out) {
+            *reinterpret_cast<float4*>(out + at) = make_float4(acc[0][t], acc[1][t], acc[2][t], acc[3][t]);
+            *reinterpret_cast<float4*>(out + at + 4) = make_float4(acc[4][t], acc[5][t], acc[6][t], acc[7][t]);
+            *reinterpret_cast<int4*>(pos + at) = make_int4(ps[0], ps[1], ps[2], ps[3]);
+            *reinterpret_cast<int4*>(pos + at + 4) = make_int4(ps[4], ps[5], ps[6], ps[7]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < kTM; e++) { out[at + e] = acc[e][t]; pos[at + e] = ps[e]; }
+        }
+    }
+}
+
+constexpr size_t kLdsLimit = 160 * 1024;
+
+// Fills the launch shape; false when this kernel does not cover the geometry.
+bool plan(const ConvGeom& q, int G, int CO, ConvFwd& a) {
+    if (q.KH != 3 || q.KW != 3 || q.D != 1 || (q.S != 1 && q.S != 2)) return false;
+    if (q.WO % kTM != 0 || G <= 0 || q.C % G != 0 || CO % G != 0) return false;
+    const int S = q.S, NXR = (7 * S + 2) / 4 + 1;
+    a.B = q.B; a.G = G; a.CG = q.C / G; a.NG = CO / G; a.K = a.CG * 9;
+    a.H = q.H; a.W = q.W; a.HO = q.HO; a.WO = q.WO; a.P = q.P;
+    a.CGP = (a.CG + kCC - 1) / kCC * kCC;
+    a.SEG = q.WO / kTM;
+    // the last lane of a row reads NXR*4 words from column (WO-8)*S; the image with its padding is W + 2P wide
+    int wp = (q.WO - kTM) * S + NXR * 4;
+    if (q.W + 2 * q.P > wp) wp = q.W + 2 * q.P;
+    a.WP = (wp + 3) / 4 * 4;
+    if (a.WP % 32 == 0) a.WP += 4;                     // rows of one lane's window in different banks
+    // Outputs per workgroup: at most 64, split evenly over the tiles; more tiles when a workgroup of that
+    // width would have too many lanes (wide images) or too few to carry a weight stage (small images).
+    const int quads = (a.NG + kTN - 1) / kTN;
+    for (int tiles_n = (quads + 15) / 16; tiles_n <= quads; tiles_n++) {
+        const int NL = (quads + tiles_n - 1) / tiles_n;
+        if (a.SEG * NL > kMaxThreads) continue;
+        const int BN = NL * kTN;
+        // rows per workgroup: the choice that keeps most lanes busy on a CU (LDS limit, 8 waves of this
+        // register footprint, rows computed past the image bottom count as idle); ties take more rows
+        int bestR = 0;
+        double bestScore = -1.0;
+        const int maxR = kMaxThreads / (a.SEG * NL);
+        int forced = g_conv_rows_override;
+        if (forced > maxR) forced = maxR;
+        if (forced > q.HO) forced = q.HO;
+        for (int R = 1; R <= maxR && R <= q.HO; R++) {
+            if (forced > 0 && R != forced) continue;
+            const int NR = (R - 1) * S + 3;
+            const size_t lds = ((size_t)a.CGP * NR * a.WP + 2 * (size_t)kKC * kBNP) * sizeof(float);
+            if (lds > kLdsLimit) break;
+            const int NT = R * a.SEG * NL;
+            const long waves_wg = (NT + 63) / 64;
+            long wgs = (long)(kLdsLimit / lds);
+            if (wgs * waves_wg > 8) wgs = 8 / waves_wg;
+            const int tiles_h = (q.HO + R - 1) / R;
+            const double score = (double)wgs * NT * q.HO / ((double)tiles_h * R);
+            if (score >= bestScore) { bestScore = score; bestR = R; }
+        }
+        // below six resident waves per CU the column kernels, which stream the channels, do better
+        if (bestR == 0 || (bestScore < 384.0 && forced <= 0)) continue;
+        a.NL = NL; a.BN = BN; a.tiles_n = (quads + NL - 1) / NL;
+        a.R = bestR; a.NR = (bestR - 1) * S + 3; a.ML = bestR * a.SEG;
+        a.tiles_h = (q.HO + bestR - 1) / bestR;
+        return (long long)q.B * G * a.tiles_h * a.tiles_n < (1LL << 31);
+    }
+    return false;
+}
+
+}  // namespace
+
+bool inf_conv_forward_supported(const ConvGeom& q, int G, int CO) {
+    ConvFwd a{};
+    return plan(q, G, CO, a);
+}
+
+hipError_t inf_conv_forward(const float* img, const float* weight, float* out, int32_t* pos, const ConvGeom& q, int G,
+                            int CO, int device, hipStream_t stream) {
+    ConvFwd a{};
+    if (!plan(q, G, CO, a)) return hipErrorInvalidValue;   // the API layer asks inf_conv_forward_supported first
+    a.vec_in = q.W % 4 == 0 && aligned16(img);
+    a.vec_out = aligned16(out) && aligned16(pos);           // WO % 8 == 0 keeps every run of 8 positions aligned
+    const size_t lds = ((size_t)a.CGP * a.NR * a.WP + 2 * (size_t)kKC * kBNP) * sizeof(float);
+    static bool raised[64][2] = {};
+    const int si = q.S - 1;
+    auto kern = q.S == 1 ? inf_conv_forward_kernel<1> : inf_conv_forward_kernel<2>;
+    if (!(device >= 0 && device < 64 && raised[device][si])) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)kLdsLimit);
+        if (e != hipSuccess) return e;
+        if (device >= 0 && device < 64) raised[device][si] = true;
+    }
+    const unsigned grid = (unsigned)((long long)q.B * G * a.tiles_h * a.tiles_n);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(a.ML * a.NL), lds, stream, img, weight, out, pos, a);
+    return hipGetLastError();
+}
+
+}  // namespace ldist

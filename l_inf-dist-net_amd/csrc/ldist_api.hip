@@ -91,6 +91,7 @@ const char* ldist_strerror(int code) {
         case LDIST_ERANGE: return "tensor too large (2^31 or more elements)";
         case LDIST_ELAUNCH: return "HIP runtime error at launch";
         case LDIST_EDEVICE: return "current device is not gfx950";
+        case LDIST_EUNSUPPORTED: return "this entry point does not cover the geometry (use the general path)";
         default: return "unknown error";
     }
 }
@@ -222,6 +223,35 @@ int ldist_unfold(const float* img, int B, int C, int H, int W, int KH, int KW, i
     ldist::Problem pr{};
     if (int rc = current_device(pr)) return rc;
     return finish(ldist::unfold(img, cols, q, (hipStream_t)stream));
+}
+
+int ldist_inf_dist_conv_forward_supported(int C, int H, int W, int CO, int G, int KH, int KW, int stride, int padding,
+                                          int dilation) {
+    ldist::ConvGeom q{};
+    if (CO <= 0 || G <= 0) return 0;
+    if (conv_geometry(1, C, H, W, KH, KW, stride, padding, dilation, q) != LDIST_OK) return 0;
+    return ldist::inf_conv_forward_supported(q, G, CO) ? 1 : 0;
+}
+
+int ldist_inf_dist_conv_forward(const float* img, const float* weight, int B, int C, int H, int W, int CO, int G,
+                                int KH, int KW, int stride, int padding, int dilation, float* output, int32_t* pos,
+                                ldist_stream_t stream) {
+    ldist::ConvGeom q{};
+    if (!img || !weight || !output || !pos || CO <= 0 || G <= 0) return LDIST_EINVAL;
+    if (int rc = conv_geometry(B, C, H, W, KH, KW, stride, padding, dilation, q)) return rc;
+    if (C % G != 0 || CO % G != 0) return LDIST_EINVAL;
+    if ((long long)B * CO * q.HO * q.WO >= (1LL << 31) || (long long)CO * (C / G) * KH * KW >= (1LL << 31))
+        return LDIST_ERANGE;
+    if (!ldist::inf_conv_forward_supported(q, G, CO)) return LDIST_EUNSUPPORTED;
+    ldist::Problem pr{};
+    if (int rc = current_device(pr)) return rc;
+    return finish(ldist::inf_conv_forward(img, weight, output, pos, q, G, CO, pr.device, (hipStream_t)stream));
+}
+
+int ldist_set_conv_rows_override(int rows) {
+    if (rows < 0) return LDIST_EINVAL;
+    ldist::g_conv_rows_override = rows;
+    return LDIST_OK;
 }
 
 int ldist_fold(const float* grad_cols, int B, int C, int H, int W, int KH, int KW, int stride, int padding,

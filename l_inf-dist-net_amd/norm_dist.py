@@ -98,16 +98,26 @@ class _Unfold(torch.autograd.Function):
 
 
 class _ConvInfDist(torch.autograd.Function):
-    """The L_inf layer on an image: unfold, distance forward, and in the backward pass the gradient
-    with respect to the image directly (scatter and fold fused), so that neither the columns nor
-    their nine times larger gradient outlive the call.  Same results as unfold + DistF."""
+    """The L_inf layer on an image.  Forward: the kernel that reads the image directly where it covers the
+    geometry, else unfold + distance forward.  Backward: the gradient with respect to the image directly
+    (scatter and fold fused), so the nine times larger gradient of the columns never exists.  Same results
+    as unfold + DistF."""
 
     @staticmethod
     def forward(ctx, img, weight, group, kernel_size, dilation, padding, stride):
-        cols = _Unfold.forward(ctx, img, kernel_size, dilation, padding, stride)
-        y = torch.empty(_out_shape(cols, weight), device=img.device, dtype=img.dtype)
-        argmax = torch.empty(y.shape, device=img.device, dtype=torch.int32)
-        norm_dist_cpp.inf_dist_forward(cols, weight, y, argmax, group)
+        if norm_dist_cpp.inf_dist_conv_forward_supported(img.size(1), img.size(2), img.size(3), weight.size(0), group,
+                                                         kernel_size, stride, padding, dilation):
+            img = img.contiguous()
+            ho, wo = norm_dist_cpp.conv_output_size(img.size(2), img.size(3), kernel_size, stride, padding, dilation)
+            y = torch.empty(img.size(0), weight.size(0), ho * wo, device=img.device, dtype=img.dtype)
+            argmax = torch.empty(y.shape, device=img.device, dtype=torch.int32)
+            norm_dist_cpp.inf_dist_conv_forward(img, weight, y, argmax, group, kernel_size, stride, padding, dilation)
+            ctx.geometry = (img.shape, kernel_size, stride, padding, dilation)
+        else:
+            cols = _Unfold.forward(ctx, img, kernel_size, dilation, padding, stride)
+            y = torch.empty(_out_shape(cols, weight), device=img.device, dtype=img.dtype)
+            argmax = torch.empty(y.shape, device=img.device, dtype=torch.int32)
+            norm_dist_cpp.inf_dist_forward(cols, weight, y, argmax, group)
         ctx.save_for_backward(argmax)
         ctx.group, ctx.weight_shape = group, weight.shape
         return y

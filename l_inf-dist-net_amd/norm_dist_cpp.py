@@ -253,3 +253,27 @@ def inf_dist_backward_input_folded(grad_output, pos, grad_img, G, kernel_size, s
             grad_output.size(2) == HO * WO, "grad_output and pos must be (B, CO, HO*WO)")
     _call("ldist_inf_dist_backward_input_folded", dev, _p(grad_output), _p(pos), B, CO, C, G, H, W, KH, KW, S, P, D,
           _p(grad_img))
+
+
+def inf_dist_conv_forward_supported(C, H, W, CO, G, kernel_size, stride=1, padding=0, dilation=1):
+    """True when inf_dist_conv_forward covers the geometry (3x3, dilation 1, stride 1 or 2, output width a
+    multiple of 8, a group's image rows fitting LDS); otherwise unfold + inf_dist_forward is the way."""
+    k = int(kernel_size)
+    return bool(_lib.lib().ldist_inf_dist_conv_forward_supported(int(C), int(H), int(W), int(CO), int(G), k, k,
+                                                                  int(stride), int(padding), int(dilation)))
+
+
+def inf_dist_conv_forward(img, weight, output, pos, G, kernel_size, stride=1, padding=0, dilation=1):
+    """L_inf forward of the conv-shaped layer straight from the image: output, pos (B, CO, HO*WO) equal to
+    inf_dist_forward on F.unfold(img, ...), without building the columns."""
+    for t, n in ((img, "img"), (weight, "weight"), (output, "output")):
+        _check_input(t, n)
+    _check_input(pos, "pos", torch.int32)
+    dev = _same_device(img, weight, output, pos)
+    B, C, H, W, KH, KW, S, P, D = _conv_args(img, kernel_size, stride, padding, dilation)
+    HO, WO = conv_output_size(H, W, KH, S, P, D)
+    _expect(weight.dim() == 2 and C % G == 0 and weight.size(1) == C // G * KH * KW, "weight must be (CO, C/G*k*k)")
+    CO = weight.size(0)
+    _expect(output.shape == (B, CO, HO * WO) and pos.shape == output.shape, "output and pos must be (B, CO, HO*WO)")
+    _call("ldist_inf_dist_conv_forward", dev, _p(img), _p(weight), B, C, H, W, CO, G, KH, KW, S, P, D, _p(output),
+          _p(pos))

@@ -45,7 +45,7 @@ def test_binding_signatures_cover_all_compute_entry_points():
 
 def test_version_and_error_strings(lib):
     assert lib.ldist_version() == 100
-    for code in (0, -1, -2, -3, -4, -99):
+    for code in (0, -1, -2, -3, -4, -5, -99):
         assert isinstance(lib.ldist_strerror(code), bytes) and lib.ldist_strerror(code)
     assert lib.ldist_set_tile_override(7) == -1 and lib.ldist_set_tile_override(-1) == 0
 
@@ -62,3 +62,20 @@ def test_argument_checks_need_no_device(lib):
     assert lib.ldist_norm_dist_backward_weight(one, one, one, one, 1, 1, 1, 1, 1, None, 8.0, None) == -1
     assert lib.ldist_inf_dist_bound_forward(one, None, one, 1, 1, 1, 1, 1, one, one, None) == -1
     assert lib.ldist_inf_dist_backward_input_overwrite(one, one, 1, 1, 1, 1, 0, one, None) == -1
+
+
+def test_conv_forward_geometry_query_needs_no_device(lib):
+    ok = lib.ldist_inf_dist_conv_forward_supported
+    assert ok(128, 32, 32, 128, 4, 3, 3, 1, 1, 1) == 1      # the benchmark layer
+    assert ok(3, 32, 32, 96, 1, 3, 3, 1, 1, 1) == 1         # the CIFAR conv net's first layer
+    assert ok(16, 32, 32, 64, 1, 3, 3, 2, 1, 1) == 1        # a stride-2 layer
+    assert ok(96, 32, 32, 96, 1, 3, 3, 1, 1, 1) == 0        # 96 channels in one group: too few rows fit LDS
+    assert ok(4, 28, 28, 8, 1, 3, 3, 1, 1, 1) == 0          # output width not a multiple of 8
+    assert ok(4, 16, 16, 8, 1, 5, 5, 1, 2, 1) == 0          # window
+    assert ok(4, 16, 16, 8, 1, 3, 3, 1, 2, 2) == 0          # dilation
+    assert ok(4, 16, 16, 8, 3, 3, 3, 1, 1, 1) == 0          # channels do not divide into the groups
+    assert ok(4096, 64, 64, 8, 1, 3, 3, 1, 1, 1) == 0       # three image rows of a group exceed LDS
+    one = ctypes.c_void_p(16)
+    assert lib.ldist_inf_dist_conv_forward(one, one, 1, 4, 28, 28, 8, 1, 3, 3, 1, 1, 1, one, one, None) == -5
+    assert lib.ldist_inf_dist_conv_forward(None, one, 1, 4, 32, 32, 8, 1, 3, 3, 1, 1, 1, one, one, None) == -1
+    assert lib.ldist_set_conv_rows_override(-1) == -1 and lib.ldist_set_conv_rows_override(0) == 0

@@ -36,9 +36,10 @@ TILES = [-1, 0, 1, 2]
 
 @pytest.fixture(autouse=True)
 def _reset_tile():
-    from gpu_common import set_tile
+    from gpu_common import pkg, set_tile
     yield
     set_tile(-1)
+    pkg._lib.lib().ldist_set_conv_rows_override(0)
 
 
 @pytest.mark.parametrize("tile", TILES)
@@ -366,6 +367,90 @@ def test_inf_backward_input_folded(case, group):
     cpp.inf_dist_backward_input_folded(go.to(DEV), pos.to(DEV), gimg, group, k, s_, p_, d_)
     torch.cuda.synchronize()
     assert_sum_close(gimg.cpu(), expect, terms, rtol=RTOL, atol=ATOL)
+
+
+IMPLICIT_CASES = [  # B, C, H, W, CO, G, stride, padding
+    (2, 4, 8, 8, 8, 1, 1, 1),        # one 8-wide segment per row
+    (2, 8, 16, 16, 24, 2, 1, 1),     # groups, 12 outputs each
+    (3, 6, 9, 16, 10, 1, 1, 1),      # odd height, channels padded up to the stage of four, ragged outputs
+    (2, 3, 32, 32, 20, 1, 1, 1),     # first layer of the CIFAR net: 3 channels
+    (2, 8, 16, 16, 16, 1, 2, 1),     # stride 2
+    (2, 5, 17, 17, 12, 1, 2, 0),     # stride 2 without padding, odd image
+    (1, 16, 32, 32, 96, 1, 1, 1),    # 96 outputs: two tiles of 48
+    (2, 128, 32, 32, 128, 4, 1, 1),  # the benchmark layer at a small batch
+    (2, 4, 10, 10, 8, 1, 1, 0),      # no padding
+    (2, 4, 6, 6, 8, 1, 1, 2),        # padding wider than the window needs
+    (1, 8, 8, 64, 40, 1, 1, 1),      # wide rows: eight segments
+    (2, 72, 16, 16, 72, 1, 1, 1),    # many channels in one group
+]
+
+
+@pytest.mark.parametrize("rows", [0, 2])
+@pytest.mark.parametrize("quant", [None, 8])
+@pytest.mark.parametrize("case", IMPLICIT_CASES)
+def test_inf_conv_forward_matches_column_path_bit_exact(case, quant, rows):
+    """The kernel that reads the image directly against the oracle on torch's unfolded columns: values and
+    first-argmax indices bit for bit (quantised inputs force ties, so the first index is what is checked)."""
+    import torch.nn.functional as F
+    from gpu_common import DEV, cpp, pkg, say
+    B, C, H, W, CO, G, s_, p_ = case
+    say("inf_conv_forward", case, "quant", quant, "rows", rows)
+    lib = pkg._lib.lib()
+    assert lib.ldist_set_conv_rows_override(rows) == 0   # 0: the library's choice; 2: forced, small layers included
+    if not cpp.inf_dist_conv_forward_supported(C, H, W, CO, G, 3, s_, p_, 1):
+        assert rows == 0
+        pytest.skip("left to the column path by the library")
+    img = torch.randn(B, C, H, W, generator=gen(61))
+    w = torch.randn(CO, C // G * 9, generator=gen(62)) * 0.7
+    if quant:
+        img, w = (img * quant).round() / quant, (w * quant).round() / quant
+    cols = F.unfold(img, 3, 1, p_, s_).contiguous()
+    eo, ep = oracle.inf_dist_forward(cols, w, G)
+    out = torch.full(eo.shape, float("nan"), device=DEV)
+    pos = torch.full(eo.shape, -7, device=DEV, dtype=torch.int32)
+    cpp.inf_dist_conv_forward(img.to(DEV), w.to(DEV), out, pos, G, 3, s_, p_, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu(), eo)
+    assert torch.equal(pos.cpu(), ep)
+
+
+@pytest.mark.parametrize("rows", [1, 2, 3, 5, 8])
+def test_inf_conv_forward_any_rows_per_workgroup(rows):
+    """Forcing the number of output rows a workgroup owns (tails at the image bottom included) changes nothing."""
+    import torch.nn.functional as F
+    from gpu_common import DEV, cpp, pkg, say
+    say("inf_conv_forward rows", rows)
+    B, C, H, W, CO, G = 2, 8, 12, 16, 16, 2
+    img = torch.randn(B, C, H, W, generator=gen(63))
+    img[0, 1, 3, 4] = float("nan")
+    img[1, 2, 0, 0] = float("inf")
+    w = torch.randn(CO, C // G * 9, generator=gen(64))
+    eo, ep = oracle.inf_dist_forward(F.unfold(img, 3, 1, 1, 1).contiguous(), w, G, literal=True)
+    out = torch.empty(eo.shape, device=DEV)
+    pos = torch.empty(eo.shape, device=DEV, dtype=torch.int32)
+    lib = pkg._lib.lib()
+    assert lib.ldist_set_conv_rows_override(rows) == 0
+    try:
+        cpp.inf_dist_conv_forward(img.to(DEV), w.to(DEV), out, pos, G, 3, 1, 1, 1)
+        torch.cuda.synchronize()
+    finally:
+        lib.ldist_set_conv_rows_override(0)
+    assert torch.equal(out.cpu(), eo)
+    assert torch.equal(pos.cpu(), ep)
+
+
+def test_inf_conv_forward_refuses_what_it_does_not_cover():
+    from gpu_common import DEV, cpp, pkg
+    assert not cpp.inf_dist_conv_forward_supported(4, 28, 28, 8, 1, 3, 1, 1, 1)    # output width 28
+    assert not cpp.inf_dist_conv_forward_supported(4, 16, 16, 8, 1, 5, 1, 2, 1)    # 5x5 window
+    assert not cpp.inf_dist_conv_forward_supported(4, 16, 16, 8, 1, 3, 1, 2, 2)    # dilation
+    img = torch.zeros(1, 4, 28, 28, device=DEV)
+    w = torch.zeros(8, 36, device=DEV)
+    out = torch.empty(1, 8, 784, device=DEV)
+    pos = torch.empty(1, 8, 784, device=DEV, dtype=torch.int32)
+    rc = pkg._lib.lib().ldist_inf_dist_conv_forward(img.data_ptr(), w.data_ptr(), 1, 4, 28, 28, 8, 1, 3, 3, 1, 1, 1,
+                                                    out.data_ptr(), pos.data_ptr(), None)
+    assert rc == -5
 
 
 @pytest.mark.parametrize("p", [float("inf"), 8.0])
