@@ -224,16 +224,22 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
             wq[e][4] = q1.x; wq[e][5] = q1.y; wq[e][6] = q1.z; wq[e][7] = q1.w;
             wq[e][8] = wp[8];
         }
+        float xq[kTM][9];                                     // all LDS reads first: one wait instead of 72
+#pragma unroll
+        for (int e = 0; e < kTM; e++) {
+            const float* xe = xlane + e * S + unit[e][t] * NR * WP;
+#pragma unroll
+            for (int r = 0; r < 9; r++) xq[e][r] = xe[(r / 3) * WP + r % 3];
+        }
         int ps[kTM];
 #pragma unroll
         for (int e = 0; e < kTM; e++) {
             const float target = acc[e][t];
-            const float* xe = xlane + e * S + unit[e][t] * NR * WP;
             int q = 0;
             float dq = 0.f;
 #pragma unroll
             for (int r = 8; r >= 0; r--) {                    // descending: the lowest match is the one kept
-                const float df = xe[(r / 3) * WP + r % 3] - wq[e][r];
+                const float df = xq[e][r] - wq[e][r];
                 if (__builtin_fabsf(df) == target) { q = r; dq = df; }
             }
             ps[e] = target > 0.f ? ((unit[e][t] * 9 + q) | (__float_as_int(dq) & 0x80000000)) : 0;
