@@ -33,6 +33,8 @@ extern "C" {
 #endif
 
 #define LDIST_VERSION 100 /* major*10000 + minor*100 + patch */
+/* The library is built with hidden visibility; only the entry points below are exported. */
+#define LDIST_API __attribute__((visibility("default")))
 
 enum {
     LDIST_OK = 0,
@@ -45,19 +47,19 @@ enum {
 
 typedef void* ldist_stream_t; /* hipStream_t */
 
-int ldist_version(void);
-const char* ldist_strerror(int code);
+LDIST_API int ldist_version(void);
+LDIST_API const char* ldist_strerror(int code);
 /* hipError_t of the last failed launch made by the calling thread (0 if none). */
-int ldist_last_hip_error(void);
+LDIST_API int ldist_last_hip_error(void);
 
 /* Testing and tuning knob, no counterpart in the reference: forces the workgroup
  * tiling of the three forward kernels.  -1 = choose by shape (default), 0 = 128x80
  * tile with two k-groups, 1 = 128x64, 2 = 256x32.  Process-wide; not thread safe. */
-int ldist_set_tile_override(int choice);
+LDIST_API int ldist_set_tile_override(int choice);
 /* Tuning knob, no counterpart in the reference: 1 (default) orders the tiles of
  * the forward kernels so that each of the 8 XCDs works on one contiguous run of
  * tiles, 0 keeps the plain order.  Results do not depend on it. */
-int ldist_set_xcd_remap(int on);
+LDIST_API int ldist_set_xcd_remap(int on);
 
 /* L_inf forward.  Replaces inf_dist_forward_cuda (model/norm_dist.cpp:13-14,
  * model/inf_dist_cuda.cu:173-180).
@@ -66,14 +68,14 @@ int ldist_set_xcd_remap(int on);
  *                 x[m,k*] - w[n,k*] < 0; 0 when the maximum is 0.
  * A NaN difference never wins.  Values and indices are bit-exact with the
  * reference rule "scan k ascending, update on strict >" (inf_dist_cuda.cu:36-43). */
-int ldist_inf_dist_forward(const float* input, const float* weight, int B, int CO, int CI, int G, int HW,
+LDIST_API int ldist_inf_dist_forward(const float* input, const float* weight, int B, int CO, int CI, int G, int HW,
                            float* output, int32_t* pos, ldist_stream_t stream);
 
 /* Interval-bound forward.  Replaces inf_dist_bound_forward_cuda
  * (model/norm_dist.cpp:15-16, model/inf_dist_cuda.cu:181-188).
  *   output_upper = max_k max(|l-w|, |u-w|)
  *   output_lower = max_k min(|l-w|, |u-w|) over the k where not (l-w < 0 < u-w), else 0 */
-int ldist_inf_dist_bound_forward(const float* input_lower, const float* input_upper, const float* weight, int B,
+LDIST_API int ldist_inf_dist_bound_forward(const float* input_lower, const float* input_upper, const float* weight, int B,
                                  int CO, int CI, int G, int HW, float* output_lower, float* output_upper,
                                  ldist_stream_t stream);
 
@@ -82,14 +84,14 @@ int ldist_inf_dist_bound_forward(const float* input_lower, const float* input_up
  *   grad_input[b, g*K + idx, hw] += (pos >= 0 ? g : -g),  idx = pos & 0x7fffffff
  * grad_input must hold zeros (or the values to accumulate onto) on entry,
  * as the reference requires (model/norm_dist.py:34). */
-int ldist_inf_dist_backward_input(const float* grad_output, const int32_t* pos, int B, int CO, int CI, int G, int HW,
+LDIST_API int ldist_inf_dist_backward_input(const float* grad_output, const int32_t* pos, int B, int CO, int CI, int G, int HW,
                                   float* grad_input, ldist_stream_t stream);
 
 /* L_inf backward w.r.t. weight.  Replaces inf_dist_backward_weight_cuda
  * (model/norm_dist.cpp:19-20, model/inf_dist_cuda.cu:197-204).
  *   grad_weight[g*NG + n, idx] += (pos < 0 ? g : -g), summed over b and hw
  * grad_weight must hold zeros (or the values to accumulate onto) on entry (model/norm_dist.py:37). */
-int ldist_inf_dist_backward_weight(const float* grad_output, const int32_t* pos, int B, int CO, int CI, int G, int HW,
+LDIST_API int ldist_inf_dist_backward_weight(const float* grad_output, const int32_t* pos, int B, int CO, int CI, int G, int HW,
                                    float* grad_weight, ldist_stream_t stream);
 
 /* p-norm forward, p > 1.  Replaces norm_dist_forward_cuda
@@ -97,14 +99,14 @@ int ldist_inf_dist_backward_weight(const float* grad_output, const int32_t* pos,
  *   output = m * (1e-10*(1e-10/m)^p + sum_k (|x-w|/m)^p)^(1/p),  m = max(1e-10, max_k |x-w|)
  * i.e. (sum |x-w|^p)^(1/p) evaluated with the reference's max-normalised
  * stabilisation and seeds (norm_dist_cuda.cu:232-233,253-264,289). */
-int ldist_norm_dist_forward(const float* input, const float* weight, int B, int CO, int CI, int G, int HW,
+LDIST_API int ldist_norm_dist_forward(const float* input, const float* weight, int B, int CO, int CI, int G, int HW,
                             float* output, float p, ldist_stream_t stream);
 
 /* p-norm backward w.r.t. input.  Replaces norm_dist_backward_input_cuda
  * (model/norm_dist.cpp:9-10, model/norm_dist_cuda.cu:438-448).
  *   grad_input[m,k] = sum_n g[m,n] * (|x-w| / output[m,n])^(p-1) * (x-w > 0 ? 1 : -1)
  * Every element of grad_input is written; it may be uninitialised on entry (model/norm_dist.py:42). */
-int ldist_norm_dist_backward_input(const float* grad_output, const float* input, const float* weight,
+LDIST_API int ldist_norm_dist_backward_input(const float* grad_output, const float* input, const float* weight,
                                    const float* output, int B, int CO, int CI, int G, int HW, float* grad_input,
                                    float p, ldist_stream_t stream);
 
@@ -112,7 +114,7 @@ int ldist_norm_dist_backward_input(const float* grad_output, const float* input,
  * (model/norm_dist.cpp:11-12, model/norm_dist_cuda.cu:449-459).
  *   grad_weight[n,k] += sum_{b,hw} g * (|w-x| / output)^(p-1) * (w-x > 0 ? 1 : -1)
  * grad_weight must hold zeros (or the values to accumulate onto) on entry (model/norm_dist.py:45). */
-int ldist_norm_dist_backward_weight(const float* grad_output, const float* input, const float* weight,
+LDIST_API int ldist_norm_dist_backward_weight(const float* grad_output, const float* input, const float* weight,
                                     const float* output, int B, int CO, int CI, int G, int HW, float* grad_weight,
                                     float p, ldist_stream_t stream);
 
@@ -121,9 +123,9 @@ int ldist_norm_dist_backward_weight(const float* grad_output, const float* input
  * memory and skip its own zero fill.  No counterpart in the reference, which
  * needs torch.zeros_like first (model/norm_dist.py:34,37); results are equal
  * to zero-fill followed by the accumulate entry points above. */
-int ldist_inf_dist_backward_input_overwrite(const float* grad_output, const int32_t* pos, int B, int CO, int CI,
+LDIST_API int ldist_inf_dist_backward_input_overwrite(const float* grad_output, const int32_t* pos, int B, int CO, int CI,
                                             int G, int HW, float* grad_input, ldist_stream_t stream);
-int ldist_inf_dist_backward_weight_overwrite(const float* grad_output, const int32_t* pos, int B, int CO, int CI,
+LDIST_API int ldist_inf_dist_backward_weight_overwrite(const float* grad_output, const int32_t* pos, int B, int CO, int CI,
                                              int G, int HW, float* grad_weight, ldist_stream_t stream);
 
 /* Per-channel mean shift of a contiguous (B, C, L) tensor in one kernel:
@@ -133,7 +135,7 @@ int ldist_inf_dist_backward_weight_overwrite(const float* grad_output, const int
  * module (model/norm_dist.py:85-96), which runs as five small torch kernels per layer; the backward
  * pass is the same operation on the gradient (gx = gy - mean(gy)).  mean_out (C floats) and
  * running_mean may be NULL; y must not overlap x. */
-int ldist_mean_shift(const float* x, int B, int C, int L, float* y, float* mean_out, float* running_mean,
+LDIST_API int ldist_mean_shift(const float* x, int B, int C, int L, float* y, float* mean_out, float* running_mean,
                      float momentum, ldist_stream_t stream);
 
 /* One AdamW step with row-wise l_p weight decay on a contiguous (rows, cols) parameter, in place
@@ -150,7 +152,7 @@ int ldist_mean_shift(const float* x, int B, int C, int L, float* y, float* mean_
  * grad == NULL: the decay alone (exp_avg, exp_avg_sq are not touched and may be NULL).
  * The hyper-parameters are doubles, as in the reference's Python: 1 - beta2 = 0.001 loses five
  * digits when beta2 is first rounded to float. */
-int ldist_adamw_lp_step(float* param, const float* grad, float* exp_avg, float* exp_avg_sq, int rows, int cols,
+LDIST_API int ldist_adamw_lp_step(float* param, const float* grad, float* exp_avg, float* exp_avg_sq, int rows, int cols,
                         double p_norm, double lr, double beta1, double beta2, double eps, double weight_decay,
                         int step, ldist_stream_t stream);
 
@@ -159,7 +161,7 @@ int ldist_adamw_lp_step(float* param, const float* grad, float* exp_avg, float* 
  *   cols[b, (c*KH + i)*KW + j, h*WO + w] = img[b, c, h*stride + i*dilation - padding, w*stride + j*dilation - padding]
  * (0 outside the image); HO = (H + 2*padding - dilation*(KH-1) - 1)/stride + 1, WO likewise.
  * img is (B, C, H, W), cols is (B, C*KH*KW, HO*WO).  No native counterpart in the reference. */
-int ldist_unfold(const float* img, int B, int C, int H, int W, int KH, int KW, int stride, int padding, int dilation,
+LDIST_API int ldist_unfold(const float* img, int B, int C, int H, int W, int KH, int KW, int stride, int padding, int dilation,
                  float* cols, ldist_stream_t stream);
 
 /* L_inf forward of the convolution-shaped layer straight from the image, without the unfolded tensor:
@@ -169,20 +171,20 @@ int ldist_unfold(const float* img, int B, int C, int H, int W, int KH, int KW, i
  * Covers 3x3 windows with dilation 1, stride 1 or 2, WO % 8 == 0, and a group's image rows fitting
  * LDS; ldist_inf_dist_conv_forward_supported returns 1 for such a geometry, 0 otherwise, and
  * ldist_inf_dist_conv_forward returns LDIST_EUNSUPPORTED for the rest (nothing is enqueued). */
-int ldist_inf_dist_conv_forward_supported(int C, int H, int W, int CO, int G, int KH, int KW, int stride, int padding,
+LDIST_API int ldist_inf_dist_conv_forward_supported(int C, int H, int W, int CO, int G, int KH, int KW, int stride, int padding,
                                           int dilation);
-int ldist_inf_dist_conv_forward(const float* img, const float* weight, int B, int C, int H, int W, int CO, int G,
+LDIST_API int ldist_inf_dist_conv_forward(const float* img, const float* weight, int B, int C, int H, int W, int CO, int G,
                                 int KH, int KW, int stride, int padding, int dilation, float* output, int32_t* pos,
                                 ldist_stream_t stream);
 /* Testing and tuning knob, no counterpart in the reference: output rows per workgroup of
  * ldist_inf_dist_conv_forward; 0 (default) = chosen by shape.  A positive value is clamped to what the
  * geometry allows and also switches off the rule that leaves small or channel-heavy layers, which
  * would keep too few waves on a CU, to the general path.  Process-wide; not thread safe. */
-int ldist_set_conv_rows_override(int rows);
+LDIST_API int ldist_set_conv_rows_override(int rows);
 
 /* Adjoint of ldist_unfold (what autograd does behind F.unfold): every element of grad_img is written
  * with the sum of the grad_cols entries that were copied from it. */
-int ldist_fold(const float* grad_cols, int B, int C, int H, int W, int KH, int KW, int stride, int padding,
+LDIST_API int ldist_fold(const float* grad_cols, int B, int C, int H, int W, int KH, int KW, int stride, int padding,
                int dilation, float* grad_img, ldist_stream_t stream);
 
 /* ldist_inf_dist_backward_input_overwrite composed with ldist_fold: the gradient of the L_inf layer
@@ -191,7 +193,7 @@ int ldist_fold(const float* grad_cols, int B, int C, int H, int W, int KH, int K
  * in-group row (c*KH + i)*KW + j of the columns.  Every element of grad_img (B, C, H, W) is written;
  * contributions whose argmax lies in the padding vanish, as they do in fold.
  * LDIST_ERANGE if (C/G)*W exceeds 16384 floats (use the two separate calls then). */
-int ldist_inf_dist_backward_input_folded(const float* grad_output, const int32_t* pos, int B, int CO, int C, int G,
+LDIST_API int ldist_inf_dist_backward_input_folded(const float* grad_output, const int32_t* pos, int B, int CO, int C, int G,
                                          int H, int W, int KH, int KW, int stride, int padding, int dilation,
                                          float* grad_img, ldist_stream_t stream);
 

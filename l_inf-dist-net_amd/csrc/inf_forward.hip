@@ -273,7 +273,8 @@ struct InfForward {
         constexpr size_t pipe = Stager<GEO, CONV, VEC, 1>::LDS_BYTES;
         const size_t lds = park > pipe ? park : pipe;
         auto kern = inf_forward_kernel<GEO, CONV, VEC, EXACT>;
-        if (hipError_t e = allow_lds(kern, lds, device); e != hipSuccess) return e;
+        static bool lds_allowed[64] = {};   // per instantiation of this launcher, i.e. per kernel
+        if (hipError_t e = allow_lds(kern, lds, device, lds_allowed); e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(grid), dim3(GEO::NT), lds, stream, input, weight, output, pos, d);
         return hipGetLastError();
     }

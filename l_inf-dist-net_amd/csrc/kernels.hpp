@@ -42,10 +42,11 @@ inline TileChoice choose_tile(int M, int NG, int G, int num_cu) {
     return pick;
 }
 
-// Sets the dynamic-LDS limit of a kernel once per device.
+// Sets the dynamic-LDS limit of a kernel once per device.  `done` is the caller's record for that one
+// kernel (a function-local static of the launcher instantiated per kernel): kernels share their
+// function-pointer type, so a record kept here per type would be shared between them.
 template <class Kern>
-inline hipError_t allow_lds(Kern kern, size_t bytes, int device) {
-    static bool done[64] = {};
+inline hipError_t allow_lds(Kern kern, size_t bytes, int device, bool (&done)[64]) {
     if (device >= 0 && device < 64 && done[device]) return hipSuccess;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
