@@ -168,8 +168,9 @@ LDIST_API int ldist_unfold(const float* img, int B, int C, int H, int W, int KH,
  * what ldist_unfold followed by ldist_inf_dist_forward computes (the reference: F.unfold at
  * model/norm_dist.py:132, then inf_dist_forward_cuda), bit for bit, reading the image once.
  *   img (B, C, H, W), weight (CO, C/G*KH*KW), output and pos (B, CO, HO*WO).
- * Covers 3x3 windows with dilation 1, stride 1 or 2, WO % 8 == 0, and a group's image rows fitting
- * LDS; ldist_inf_dist_conv_forward_supported returns 1 for such a geometry, 0 otherwise, and
+ * Covers 3x3 windows with dilation 1, stride 1 or 2 and WO % 8 == 0, where a group's channels are few
+ * enough for their image rows to stay in LDS or a multiple of four (then they are staged);
+ * ldist_inf_dist_conv_forward_supported returns 1 for such a geometry, 0 otherwise, and
  * ldist_inf_dist_conv_forward returns LDIST_EUNSUPPORTED for the rest (nothing is enqueued). */
 LDIST_API int ldist_inf_dist_conv_forward_supported(int C, int H, int W, int CO, int G, int KH, int KW, int stride, int padding,
                                           int dilation);
@@ -181,6 +182,11 @@ LDIST_API int ldist_inf_dist_conv_forward(const float* img, const float* weight,
  * geometry allows and also switches off the rule that leaves small or channel-heavy layers, which
  * would keep too few waves on a CU, to the general path.  Process-wide; not thread safe. */
 LDIST_API int ldist_set_conv_rows_override(int rows);
+/* Testing and tuning knob, no counterpart in the reference: how ldist_inf_dist_conv_forward keeps the
+ * image rows in LDS.  0 (default) = by shape; 1 = only the variant that holds all channels of a group;
+ * 2 = only the variant that stages four channels at a time (needs C/G % 4 == 0).  A geometry the forced
+ * variant cannot take becomes unsupported.  Process-wide; not thread safe. */
+LDIST_API int ldist_set_conv_staging_override(int mode);
 
 /* Adjoint of ldist_unfold (what autograd does behind F.unfold): every element of grad_img is written
  * with the sum of the grad_cols entries that were copied from it. */

@@ -62,6 +62,8 @@ def lib():
         handle.ldist_set_tile_override.restype = ctypes.c_int
         handle.ldist_set_conv_rows_override.argtypes = [ctypes.c_int]
         handle.ldist_set_conv_rows_override.restype = ctypes.c_int
+        handle.ldist_set_conv_staging_override.argtypes = [ctypes.c_int]
+        handle.ldist_set_conv_staging_override.restype = ctypes.c_int
         handle.ldist_version.restype = ctypes.c_int
         handle.ldist_strerror.restype = ctypes.c_char_p
         handle.ldist_strerror.argtypes = [ctypes.c_int]

@@ -5,20 +5,24 @@
 // pos as in the column kernel (lowest k of the maximum, bit 31 = sign of the difference, 0 for a zero maximum).
 // Values and indices equal the column path's bit for bit: the same fp32 subtractions of the same numbers.
 //
-// A workgroup owns R output rows of one (image, group) and BN of the group's outputs.  The image rows those
-// positions look at, all CG channels of them, are copied once into LDS with the zero padding materialised, and
-// stay there; the weights stream through a double-buffered LDS stage of CC channels (9*CC values of k), stored
-// k-major so that a lane's four outputs are one 128-bit read.  A lane owns 8 neighbouring positions of one
-// output row times 4 outputs.  For a window row (c, i) it reads the 8 + 2 pixels its positions cover for
-// j = 0, 1, 2 with three (stride 2: five) aligned 128-bit reads, so 12 LDS words serve 24 differences.
-// The loop keeps the maximum per channel and records the channel of the running maximum (subtract + half a
-// v_max3 per difference, three instructions per channel and output); the lowest k inside the recorded
-// channel is found afterwards from the image rows still in LDS.
+// A workgroup owns R output rows of one (image, group) and BN of the group's outputs.  The weights stream
+// through a double-buffered LDS stage of CC channels (9*CC values of k), stored k-major so that a lane's four
+// outputs are one 128-bit read.  The image rows those positions look at, zero padding materialised, are in LDS
+// too, in one of two ways:
+//   RESIDENT  all CG channels are copied once and stay (few channels per group: they fit);
+//   staged    CC channels at a time travel through a second double-buffered stage beside the weights.
+// A lane owns 8 neighbouring positions of one output row times 4 outputs.  For a window row (c, i) it reads the
+// 8 + 2 pixels its positions cover for j = 0, 1, 2 with three (stride 2: five) aligned 128-bit reads, so 12 LDS
+// words serve 24 differences.  The loop keeps the maximum per channel and records the channel of the running
+// maximum (subtract + half a v_max3 per difference, three instructions per channel and output); the lowest k
+// inside the recorded channel is found afterwards from nine pixels (LDS when RESIDENT, else the image in
+// global memory) and the channel's nine contiguous weights.
 #include "kernels.hpp"
 
 namespace ldist {
 
-int g_conv_rows_override = 0;   // > 0: output rows per workgroup forced (tests and tuning)
+int g_conv_rows_override = 0;      // > 0: output rows per workgroup forced (tests and tuning)
+int g_conv_staging_override = 0;   // 1: image rows resident in LDS only; 2: staged only; 0: by shape
 
 namespace {
 
@@ -29,6 +33,7 @@ constexpr int kKC = kCC * 9;      // k values per weight stage
 constexpr int kMaxThreads = 256;
 constexpr int kBNP = 68;          // row length of the weight stage: 64 outputs + 4, a constant so that reads take immediate offsets
 constexpr int kWRegs = 9;         // weight words a lane carries from global to LDS per stage (64 outputs x 36 / 256)
+constexpr int kXRegs = 10;        // image words a lane carries per stage when the channels are staged
 
 struct ConvFwd {
     int B, G, CG, NG, K;         // images, groups, channels and outputs per group, K = 9*CG
@@ -38,16 +43,18 @@ struct ConvFwd {
                                  // workgroup
     int tiles_h, tiles_n;
     int vec_in, vec_out;         // 128-bit global loads of image rows / stores of results allowed
+    int resident;                // 1: all channels of the image rows stay in LDS; 0: staged kCC channels at a time
+    int xwords;                  // floats of the image area in LDS
 };
 
-template <int S>
+template <int S, bool RESIDENT>
 __global__ void __launch_bounds__(kMaxThreads, 2)
 inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__ weight, float* __restrict__ out,
                         int32_t* __restrict__ pos, ConvFwd a) {
     constexpr int NXR = (7 * S + 2) / 4 + 1;          // 128-bit reads per window row: pixels 0 .. 7*S + 2
     extern __shared__ __align__(16) float lds[];
-    float* tile = lds;                                  // [CGP][NR][WP]
-    float* wst = lds + a.CGP * a.NR * a.WP;             // 2 x [kKC][kBNP]
+    float* tile = lds;                                  // RESIDENT: [CGP][NR][WP]; staged: 2 x [xwords / 2]
+    float* wst = lds + a.xwords;                        // 2 x [kKC][kBNP]
     const int tid = threadIdx.x, NT = blockDim.x;
 
     int id = blockIdx.x;
@@ -95,12 +102,54 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
     };
     wload(0);
 
-    // ---- image rows -> LDS, padding as zeros ----
-    {
+    const float* src = img + ((size_t)b * a.G + g) * a.CG * a.H * a.W;   // the group's channels of this image
+    // ---- staged: what each lane moves per stage is the same every time, only the channel base advances ----
+    const int xhalf = a.xwords / 2;                     // one stage buffer: at least kCC*NR*WP and kXRegs*NT words
+    int goff[kXRegs];                                   // element offset inside the stage's kCC channels; -1 = padding
+    float xreg[kXRegs];
+    if constexpr (!RESIDENT) {
+        const int plane = NR * WP;
+#pragma unroll
+        for (int r = 0; r < kXRegs; r++) {
+            const int idx = tid + r * NT;
+            const int c = idx / plane, rem = idx - c * plane;
+            const int row = rem / WP, col = rem - row * WP;
+            const int y = y0 + row, x = col - a.P;
+            const bool real = c < kCC && (unsigned)y < (unsigned)a.H && (unsigned)x < (unsigned)a.W;
+            goff[r] = real ? (c * a.H + y) * a.W + x : -1;
+        }
+    }
+    auto xload = [&](int ch) {
+        const float* base = src + (size_t)ch * kCC * a.H * a.W;
+#pragma unroll
+        for (int r = 0; r < kXRegs; r++) {
+            const float v = base[goff[r] < 0 ? 0 : goff[r]];   // branch-free: padding reads a valid word, replaced by 0
+            xreg[r] = goff[r] < 0 ? 0.f : v;
+        }
+    };
+    auto xstore = [&](float* stage) {
+#pragma unroll
+        for (int r = 0; r < kXRegs; r++) stage[tid + r * NT] = xreg[r];   // < kXRegs*NT <= xhalf
+    };
+    // A workgroup too small to carry a whole stage in kXRegs words per lane (tiny images) moves the rest
+    // directly; with 256 lanes this loop is empty.
+    auto xrest = [&](int ch, float* stage) {
+        const float* base = src + (size_t)ch * kCC * a.H * a.W;
+        const int plane = NR * WP;
+        for (int idx = tid + kXRegs * NT; idx < kCC * plane; idx += NT) {
+            const int c = idx / plane, rem = idx - c * plane;
+            const int row = rem / WP, col = rem - row * WP;
+            const int y = y0 + row, x = col - a.P;
+            const bool real = (unsigned)y < (unsigned)a.H && (unsigned)x < (unsigned)a.W;
+            stage[idx] = real ? base[(c * a.H + y) * a.W + x] : 0.f;
+        }
+    };
+
+    // ---- RESIDENT: image rows -> LDS once, padding as zeros ----
+    if constexpr (RESIDENT) {
         const int words = a.CGP * NR * WP;
         for (int i = tid * 4; i < words; i += NT * 4) *reinterpret_cast<float4*>(tile + i) = make_float4(0.f, 0.f, 0.f, 0.f);
         __syncthreads();
-        const float* src = img + ((size_t)b * a.G + g) * a.CG * a.H * a.W;
         const int rows = a.CG * NR;
         if (a.vec_in) {
             const int QW = a.W / 4;
@@ -122,6 +171,10 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
                 if ((unsigned)y < (unsigned)a.H) tile[(c * NR + r) * WP + a.P + x] = src[((size_t)c * a.H + y) * a.W + x];
             }
         }
+    } else {
+        xload(0);
+        xstore(tile);
+        xrest(0, tile);
     }
     wstore(wst);
     wrest(0, wst);
@@ -130,7 +183,8 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
     // ---- lane geometry ----
     const int nl = tid % a.NL, ml = tid / a.NL;
     const int hr = ml / a.SEG, w0 = (ml - hr * a.SEG) * kTM;
-    const float* xlane = tile + (hr * S) * WP + w0 * S;        // + (c*NR + i)*WP: 16-byte aligned (WP % 4 == 0)
+    const int xlane_off = (hr * S) * WP + w0 * S;              // + (c*NR + i)*WP: 16-byte aligned (WP % 4 == 0)
+    const float* xlane = tile + xlane_off;
 
     float acc[kTM][kTN];
     int unit[kTM][kTN];
@@ -142,9 +196,13 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
     const int nstage = a.CGP / kCC;
     const float* xch = xlane;
     for (int ch = 0; ch < nstage; ch++) {
-        if (ch + 1 < nstage) wload(ch + 1);
+        if (ch + 1 < nstage) {
+            wload(ch + 1);
+            if constexpr (!RESIDENT) xload(ch + 1);
+        }
         const float* wrow = wst + (ch & 1) * kKC * BNP + kTN * nl;   // walks down the 9*kCC rows of the stage
-        const float* xrow = xch;                                     // walks down the window rows of its channels
+        // walks down the window rows of the stage's channels
+        const float* xrow = RESIDENT ? xch : tile + (ch & 1) * xhalf + xlane_off;
         // The loops over units, channels and window rows stay rolled: one trip is 6 LDS reads and 144
         // arithmetic instructions, and its registers are all the compiler has to keep.
 #pragma unroll 1
@@ -198,6 +256,10 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
         if (ch + 1 < nstage) {
             wstore(wst + ((ch + 1) & 1) * kKC * BNP);
             wrest(ch + 1, wst + ((ch + 1) & 1) * kKC * BNP);
+            if constexpr (!RESIDENT) {
+                xstore(tile + ((ch + 1) & 1) * xhalf);
+                xrest(ch + 1, tile + ((ch + 1) & 1) * xhalf);
+            }
         }
         __syncthreads();
     }
@@ -215,34 +277,55 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
         const int n = n0 + kTN * nl + t;
         if (n >= a.NG) break;
         const float* wn = weight + ((size_t)g * a.NG + n) * K;
-        float wq[kTM][9];
-#pragma unroll
-        for (int e = 0; e < kTM; e++) {
-            const float* wp = wn + unit[e][t] * 9;           // a recorded unit is a real channel: inside the row
-            const f4u q0 = *reinterpret_cast<const f4u*>(wp), q1 = *reinterpret_cast<const f4u*>(wp + 4);
-            wq[e][0] = q0.x; wq[e][1] = q0.y; wq[e][2] = q0.z; wq[e][3] = q0.w;
-            wq[e][4] = q1.x; wq[e][5] = q1.y; wq[e][6] = q1.z; wq[e][7] = q1.w;
-            wq[e][8] = wp[8];
-        }
-        float xq[kTM][9];                                     // all LDS reads first: one wait instead of 72
-#pragma unroll
-        for (int e = 0; e < kTM; e++) {
-            const float* xe = xlane + e * S + unit[e][t] * NR * WP;
-#pragma unroll
-            for (int r = 0; r < 9; r++) xq[e][r] = xe[(r / 3) * WP + r % 3];
-        }
         int ps[kTM];
+        // EB positions at a time: their reads are issued together, then searched (the staged variant has less
+        // room in registers: it also carries the image words of the stage)
+        constexpr int EB = RESIDENT ? kTM : kTM / 2;
 #pragma unroll
-        for (int e = 0; e < kTM; e++) {
-            const float target = acc[e][t];
-            int q = 0;
-            float dq = 0.f;
+        for (int e0 = 0; e0 < kTM; e0 += EB) {
+            float wq[EB][9], xq[EB][9];
 #pragma unroll
-            for (int r = 8; r >= 0; r--) {                    // descending: the lowest match is the one kept
-                const float df = xq[e][r] - wq[e][r];
-                if (__builtin_fabsf(df) == target) { q = r; dq = df; }
+            for (int eb = 0; eb < EB; eb++) {
+                const int e = e0 + eb;
+                const float* wp = wn + unit[e][t] * 9;       // a recorded unit is a real channel: inside the row
+                const f4u q0 = *reinterpret_cast<const f4u*>(wp), q1 = *reinterpret_cast<const f4u*>(wp + 4);
+                wq[eb][0] = q0.x; wq[eb][1] = q0.y; wq[eb][2] = q0.z; wq[eb][3] = q0.w;
+                wq[eb][4] = q1.x; wq[eb][5] = q1.y; wq[eb][6] = q1.z; wq[eb][7] = q1.w;
+                wq[eb][8] = wp[8];
             }
-            ps[e] = target > 0.f ? ((unit[e][t] * 9 + q) | (__float_as_int(dq) & 0x80000000)) : 0;
+#pragma unroll
+            for (int eb = 0; eb < EB; eb++) {
+                const int e = e0 + eb;
+                if constexpr (RESIDENT) {
+                    const float* xe = xlane + e * S + unit[e][t] * NR * WP;
+#pragma unroll
+                    for (int r = 0; r < 9; r++) xq[eb][r] = xe[(r / 3) * WP + r % 3];
+                } else {
+                    // the window of position (h, w0 + e) in the recorded channel; outside the image it reads 0
+                    const unsigned plane = (unsigned)unit[e][t] * (unsigned)(a.H * a.W);
+                    const int yy = h * S - a.P, xx = (w0 + e) * S - a.P;
+#pragma unroll
+                    for (int r = 0; r < 9; r++) {
+                        const int y = yy + r / 3, x = xx + r % 3;
+                        const bool real = (unsigned)y < (unsigned)a.H && (unsigned)x < (unsigned)a.W;
+                        const float v = src[real ? plane + (unsigned)(y * a.W + x) : 0u];
+                        xq[eb][r] = real ? v : 0.f;
+                    }
+                }
+            }
+#pragma unroll
+            for (int eb = 0; eb < EB; eb++) {
+                const int e = e0 + eb;
+                const float target = acc[e][t];
+                int q = 0;
+                float dq = 0.f;
+#pragma unroll
+                for (int r = 8; r >= 0; r--) {                // descending: the lowest match is the one kept
+                    const float df = xq[eb][r] - wq[eb][r];
+                    if (__builtin_fabsf(df) == target) { q = r; dq = df; }
+                }
+                ps[e] = target > 0.f ? ((unit[e][t] * 9 + q) | (__float_as_int(dq) & 0x80000000)) : 0;
+            }
         }
         const size_t at = (((size_t)b * a.G + g) * a.NG + n) * L + (size_t)h * a.WO + w0;
         if (a.vec_out) {
@@ -274,39 +357,61 @@ bool plan(const ConvGeom& q, int G, int CO, ConvFwd& a) {
     a.WP = (wp + 3) / 4 * 4;
     if (a.WP % 32 == 0) a.WP += 4;                     // rows of one lane's window in different banks
     // Outputs per workgroup: at most 64, split evenly over the tiles; more tiles when a workgroup of that
-    // width would have too many lanes (wide images) or too few to carry a weight stage (small images).
+    // width would have too many lanes (wide images).
     const int quads = (a.NG + kTN - 1) / kTN;
-    for (int tiles_n = (quads + 15) / 16; tiles_n <= quads; tiles_n++) {
-        const int NL = (quads + tiles_n - 1) / tiles_n;
-        if (a.SEG * NL > kMaxThreads) continue;
-        const int BN = NL * kTN;
-        // rows per workgroup: the choice that keeps most lanes busy on a CU (LDS limit, 8 waves of this
-        // register footprint, rows computed past the image bottom count as idle); ties take more rows
-        int bestR = 0;
-        double bestScore = -1.0;
-        const int maxR = kMaxThreads / (a.SEG * NL);
-        int forced = g_conv_rows_override;
-        if (forced > maxR) forced = maxR;
-        if (forced > q.HO) forced = q.HO;
-        for (int R = 1; R <= maxR && R <= q.HO; R++) {
-            if (forced > 0 && R != forced) continue;
-            const int NR = (R - 1) * S + 3;
-            const size_t lds = ((size_t)a.CGP * NR * a.WP + 2 * (size_t)kKC * kBNP) * sizeof(float);
-            if (lds > kLdsLimit) break;
-            const int NT = R * a.SEG * NL;
-            const long waves_wg = (NT + 63) / 64;
-            long wgs = (long)(kLdsLimit / lds);
-            if (wgs * waves_wg > 8) wgs = 8 / waves_wg;
-            const int tiles_h = (q.HO + R - 1) / R;
-            const double score = (double)wgs * NT * q.HO / ((double)tiles_h * R);
-            if (score >= bestScore) { bestScore = score; bestR = R; }
+    for (int pass = 0; pass < 2; pass++) {
+        // pass 0: all channels resident in LDS; pass 1: channels staged (needs CG % kCC == 0, so that no
+        // stage holds a channel that does not exist)
+        const bool resident = pass == 0;
+        if (g_conv_staging_override == 1 && !resident) continue;
+        if (g_conv_staging_override == 2 && resident) continue;
+        if (!resident && a.CG % kCC != 0) continue;
+        for (int tiles_n = (quads + 15) / 16; tiles_n <= quads; tiles_n++) {
+            const int NL = (quads + tiles_n - 1) / tiles_n;
+            if (a.SEG * NL > kMaxThreads) continue;
+            const int BN = NL * kTN;
+            // rows per workgroup: the choice that keeps most lanes busy on a CU (LDS limit, 8 waves of this
+            // register footprint, rows computed past the image bottom count as idle); ties take more rows
+            int bestR = 0, bestWords = 0;
+            double bestScore = -1.0;
+            const int maxR = kMaxThreads / (a.SEG * NL);
+            int forced = g_conv_rows_override;
+            if (forced > maxR) forced = maxR;
+            if (forced > q.HO) forced = q.HO;
+            for (int R = 1; R <= maxR && R <= q.HO; R++) {
+                if (forced > 0 && R != forced) continue;
+                const int NR = (R - 1) * S + 3;
+                const int NT = R * a.SEG * NL;
+                int xwords;
+                if (resident) {
+                    xwords = a.CGP * NR * a.WP;
+                } else {
+                    // a lane carries kXRegs image words per stage in registers; what a small workgroup cannot
+                    // carry that way it copies directly, which is slow: only taken when forced
+                    const int stage = kCC * NR * a.WP;
+                    if (stage > kXRegs * NT && forced <= 0) continue;
+                    const int half = stage > kXRegs * NT ? stage : kXRegs * NT;
+                    xwords = 2 * ((half + 3) / 4 * 4);
+                }
+                const size_t lds = ((size_t)xwords + 2 * (size_t)kKC * kBNP) * sizeof(float);
+                if (lds > kLdsLimit) { if (resident) break; else continue; }
+                const long waves_wg = (NT + 63) / 64;
+                long wgs = (long)(kLdsLimit / lds);
+                if (wgs * waves_wg > 8) wgs = 8 / waves_wg;
+                const int tiles_h = (q.HO + R - 1) / R;
+                const double score = (double)wgs * NT * q.HO / ((double)tiles_h * R);
+                if (score >= bestScore) { bestScore = score; bestR = R; bestWords = xwords; }
+            }
+            // below six resident waves per CU this variant does badly: try the other, or leave the layer to
+            // the column kernels
+            if (bestR == 0 || (bestScore < 384.0 && forced <= 0)) continue;
+            a.NL = NL; a.BN = BN; a.tiles_n = (quads + NL - 1) / NL;
+            a.R = bestR; a.NR = (bestR - 1) * S + 3; a.ML = bestR * a.SEG;
+            a.tiles_h = (q.HO + bestR - 1) / bestR;
+            a.resident = resident ? 1 : 0;
+            a.xwords = bestWords;
+            return (long long)q.B * G * a.tiles_h * a.tiles_n < (1LL << 31);
         }
-        // below six resident waves per CU the column kernels, which stream the channels, do better
-        if (bestR == 0 || (bestScore < 384.0 && forced <= 0)) continue;
-        a.NL = NL; a.BN = BN; a.tiles_n = (quads + NL - 1) / NL;
-        a.R = bestR; a.NR = (bestR - 1) * S + 3; a.ML = bestR * a.SEG;
-        a.tiles_h = (q.HO + bestR - 1) / bestR;
-        return (long long)q.B * G * a.tiles_h * a.tiles_n < (1LL << 31);
     }
     return false;
 }
@@ -324,15 +429,16 @@ hipError_t inf_conv_forward(const float* img, const float* weight, float* out, i
     if (!plan(q, G, CO, a)) return hipErrorInvalidValue;   // the API layer asks inf_conv_forward_supported first
     a.vec_in = q.W % 4 == 0 && aligned16(img);
     a.vec_out = aligned16(out) && aligned16(pos);           // WO % 8 == 0 keeps every run of 8 positions aligned
-    const size_t lds = ((size_t)a.CGP * a.NR * a.WP + 2 * (size_t)kKC * kBNP) * sizeof(float);
-    static bool raised[64][2] = {};
-    const int si = q.S - 1;
-    auto kern = q.S == 1 ? inf_conv_forward_kernel<1> : inf_conv_forward_kernel<2>;
-    if (!(device >= 0 && device < 64 && raised[device][si])) {
+    const size_t lds = ((size_t)a.xwords + 2 * (size_t)kKC * kBNP) * sizeof(float);
+    static bool raised[64][4] = {};
+    const int ki = (q.S - 1) * 2 + a.resident;
+    auto kern = q.S == 1 ? (a.resident ? inf_conv_forward_kernel<1, true> : inf_conv_forward_kernel<1, false>)
+                         : (a.resident ? inf_conv_forward_kernel<2, true> : inf_conv_forward_kernel<2, false>);
+    if (!(device >= 0 && device < 64 && raised[device][ki])) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)kLdsLimit);
         if (e != hipSuccess) return e;
-        if (device >= 0 && device < 64) raised[device][si] = true;
+        if (device >= 0 && device < 64) raised[device][ki] = true;
     }
     const unsigned grid = (unsigned)((long long)q.B * G * a.tiles_h * a.tiles_n);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(a.ML * a.NL), lds, stream, img, weight, out, pos, a);

@@ -248,6 +248,12 @@ int ldist_inf_dist_conv_forward(const float* img, const float* weight, int B, in
     return finish(ldist::inf_conv_forward(img, weight, output, pos, q, G, CO, pr.device, (hipStream_t)stream));
 }
 
+int ldist_set_conv_staging_override(int mode) {
+    if (mode < 0 || mode > 2) return LDIST_EINVAL;
+    ldist::g_conv_staging_override = mode;
+    return LDIST_OK;
+}
+
 int ldist_set_conv_rows_override(int rows) {
     if (rows < 0) return LDIST_EINVAL;
     ldist::g_conv_rows_override = rows;

@@ -69,13 +69,15 @@ def test_conv_forward_geometry_query_needs_no_device(lib):
     assert ok(128, 32, 32, 128, 4, 3, 3, 1, 1, 1) == 1      # the benchmark layer
     assert ok(3, 32, 32, 96, 1, 3, 3, 1, 1, 1) == 1         # the CIFAR conv net's first layer
     assert ok(16, 32, 32, 64, 1, 3, 3, 2, 1, 1) == 1        # a stride-2 layer
-    assert ok(96, 32, 32, 96, 1, 3, 3, 1, 1, 1) == 0        # 96 channels in one group: too few rows fit LDS
+    assert ok(96, 32, 32, 96, 1, 3, 3, 1, 1, 1) == 1        # 96 channels in one group: staged four at a time
+    assert ok(96, 32, 32, 192, 1, 3, 3, 2, 1, 1) == 1       # the CIFAR conv net's stride-2 layer
+    assert ok(90, 32, 32, 96, 1, 3, 3, 1, 1, 1) == 0        # too many channels to stay in LDS, and not a multiple of four
     assert ok(4, 28, 28, 8, 1, 3, 3, 1, 1, 1) == 0          # output width not a multiple of 8
     assert ok(4, 16, 16, 8, 1, 5, 5, 1, 2, 1) == 0          # window
     assert ok(4, 16, 16, 8, 1, 3, 3, 1, 2, 2) == 0          # dilation
     assert ok(4, 16, 16, 8, 3, 3, 3, 1, 1, 1) == 0          # channels do not divide into the groups
-    assert ok(4096, 64, 64, 8, 1, 3, 3, 1, 1, 1) == 0       # three image rows of a group exceed LDS
     one = ctypes.c_void_p(16)
     assert lib.ldist_inf_dist_conv_forward(one, one, 1, 4, 28, 28, 8, 1, 3, 3, 1, 1, 1, one, one, None) == -5
     assert lib.ldist_inf_dist_conv_forward(None, one, 1, 4, 32, 32, 8, 1, 3, 3, 1, 1, 1, one, one, None) == -1
     assert lib.ldist_set_conv_rows_override(-1) == -1 and lib.ldist_set_conv_rows_override(0) == 0
+    assert lib.ldist_set_conv_staging_override(3) == -1 and lib.ldist_set_conv_staging_override(0) == 0

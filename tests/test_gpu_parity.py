@@ -40,6 +40,7 @@ def _reset_tile():
     yield
     set_tile(-1)
     pkg._lib.lib().ldist_set_conv_rows_override(0)
+    pkg._lib.lib().ldist_set_conv_staging_override(0)
 
 
 @pytest.mark.parametrize("tile", TILES)
@@ -410,6 +411,43 @@ def test_inf_conv_forward_matches_column_path_bit_exact(case, quant, rows):
     pos = torch.full(eo.shape, -7, device=DEV, dtype=torch.int32)
     cpp.inf_dist_conv_forward(img.to(DEV), w.to(DEV), out, pos, G, 3, s_, p_, 1)
     torch.cuda.synchronize()
+    assert torch.equal(out.cpu(), eo)
+    assert torch.equal(pos.cpu(), ep)
+
+
+STAGED_CASES = [  # B, C, H, W, CO, G, stride, padding: channels per group a multiple of four
+    (2, 8, 16, 16, 24, 2, 1, 1), (2, 128, 32, 32, 128, 4, 1, 1), (2, 96, 32, 32, 96, 1, 1, 1),
+    (2, 96, 32, 32, 192, 1, 2, 1), (1, 192, 16, 16, 192, 1, 1, 1), (2, 8, 17, 17, 12, 1, 2, 0),
+    (1, 8, 8, 64, 40, 1, 1, 1), (2, 4, 6, 6, 8, 1, 1, 2), (3, 12, 9, 16, 10, 1, 1, 1),
+]
+
+
+@pytest.mark.parametrize("rows", [0, 3, 8])
+@pytest.mark.parametrize("quant", [None, 8])
+@pytest.mark.parametrize("case", STAGED_CASES)
+def test_inf_conv_forward_staged_channels_bit_exact(case, quant, rows):
+    """The variant that moves four channels at a time through LDS (many channels per group), forced for
+    every case, against the oracle on torch's unfolded columns."""
+    import torch.nn.functional as F
+    from gpu_common import DEV, cpp, pkg, say
+    B, C, H, W, CO, G, s_, p_ = case
+    say("inf_conv_forward staged", case, "quant", quant, "rows", rows)
+    lib = pkg._lib.lib()
+    assert lib.ldist_set_conv_staging_override(2) == 0 and lib.ldist_set_conv_rows_override(rows) == 0
+    try:
+        if not cpp.inf_dist_conv_forward_supported(C, H, W, CO, G, 3, s_, p_, 1):
+            pytest.skip("left to the column path by the library")
+        img = torch.randn(B, C, H, W, generator=gen(65))
+        w = torch.randn(CO, C // G * 9, generator=gen(66)) * 0.7
+        if quant:
+            img, w = (img * quant).round() / quant, (w * quant).round() / quant
+        eo, ep = oracle.inf_dist_forward(F.unfold(img, 3, 1, p_, s_).contiguous(), w, G)
+        out = torch.full(eo.shape, float("nan"), device=DEV)
+        pos = torch.full(eo.shape, -7, device=DEV, dtype=torch.int32)
+        cpp.inf_dist_conv_forward(img.to(DEV), w.to(DEV), out, pos, G, 3, s_, p_, 1)
+        torch.cuda.synchronize()
+    finally:
+        lib.ldist_set_conv_staging_override(0)
     assert torch.equal(out.cpu(), eo)
     assert torch.equal(pos.cpu(), ep)
 
