@@ -6,7 +6,8 @@ CIFAR-10-shaped 5-layer L_inf-dist MLP 3072 -> 5120 -> 5120 -> 5120 -> 5120 -> 1
 p = inf, batch 512, fp32, forward plus backward (grad_x of every layer and every
 grad_w).  A "step" is one pass of the hot path over one synthetic batch that already
 sits in HBM.  `--workload c0|c2|c3|c4` runs the other BASELINE.json configurations
-with the same output format (they are parity-test cases; the driver's line is c1).
+(`c4i`: configs[4] from the image, `c1t`: configs[1] with the optimizer step) with the
+same output format (they are parity-test cases; the driver's line is c1).
 
 Prints ONE JSON line.  `value` is G dist-ops/s; a dist-op is one (row, output,
 input) triple of one pass (forward, grad-input or grad-weight for the p-norm paths;
@@ -324,8 +325,24 @@ def workload_c4(pkg, torch, dev):
                         "inf_forward_kernel (conv layout, k tracked in the loop)", 2))
 
 
+def workload_c4i(pkg, torch, dev):
+    """configs[4] as a user of the layer runs it: the image goes in and the image gradient comes out; the
+    unfolded tensor and its gradient are never built (forward straight from the image, scatter and fold fused)."""
+    wl = workload_c4(pkg, torch, dev)
+    from_image = dict(wl["step_alt"])["ms_per_step_from_image"]
+    wl.update(step=from_image,
+              step_alt=[("ms_per_step_columns_only_unfold_outside", wl["step"]),
+                        ("ms_per_step_with_torch_unfold_and_fold", dict(wl["step_alt"])["ms_per_step_with_torch_unfold_and_fold"])],
+              name="configs[4] from the image: 3x3 L_inf-dist conv layer, batch 128, 128->128 channels, 32x32, groups 4, "
+                   "forward+backward with patch extraction and its adjoint inside the timed region",
+              kernel=("inf_dist_conv_forward", lambda img_, w_, o_, *_: 2 * o_.numel() * w_.size(1), lambda *a: True,
+                      "inf_conv_forward_kernel (L_inf forward straight from the image, a group's image rows resident "
+                      "in LDS)", 2))
+    return wl
+
+
 WORKLOADS = {"c0": workload_c0, "c1": workload_c1, "c1t": workload_c1t, "c2": workload_c2, "c3": workload_c3,
-             "c4": workload_c4}
+             "c4": workload_c4, "c4i": workload_c4i}
 
 
 def cpu_baseline(wl, target_seconds=12.0):
