@@ -184,8 +184,9 @@ LDIST_API int ldist_inf_dist_conv_forward(const float* img, const float* weight,
 LDIST_API int ldist_set_conv_rows_override(int rows);
 /* Testing and tuning knob, no counterpart in the reference: how ldist_inf_dist_conv_forward keeps the
  * image rows in LDS.  0 (default) = by shape; 1 = only the variant that holds all channels of a group;
- * 2 = only the variant that stages four channels at a time (needs C/G % 4 == 0).  A geometry the forced
- * variant cannot take becomes unsupported.  Process-wide; not thread safe. */
+ * 2 = only the variant that stages four channels at a time (needs C/G % 4 == 0); 3 = neither, so that
+ * every geometry is reported unsupported and callers take the column path (A/B comparisons).  A geometry
+ * the forced variant cannot take becomes unsupported.  Process-wide; not thread safe. */
 LDIST_API int ldist_set_conv_staging_override(int mode);
 
 /* Adjoint of ldist_unfold (what autograd does behind F.unfold): every element of grad_img is written

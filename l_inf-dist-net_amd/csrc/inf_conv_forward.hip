@@ -22,7 +22,7 @@
 namespace ldist {
 
 int g_conv_rows_override = 0;      // > 0: output rows per workgroup forced (tests and tuning)
-int g_conv_staging_override = 0;   // 1: image rows resident in LDS only; 2: staged only; 0: by shape
+int g_conv_staging_override = 0;   // 1: image rows resident in LDS only; 2: staged only; 3: neither; 0: by shape
 
 namespace {
 
@@ -363,6 +363,7 @@ bool plan(const ConvGeom& q, int G, int CO, ConvFwd& a) {
         // pass 0: all channels resident in LDS; pass 1: channels staged (needs CG % kCC == 0, so that no
         // stage holds a channel that does not exist)
         const bool resident = pass == 0;
+        if (g_conv_staging_override == 3) continue;
         if (g_conv_staging_override == 1 && !resident) continue;
         if (g_conv_staging_override == 2 && resident) continue;
         if (!resident && a.CG % kCC != 0) continue;

@@ -249,7 +249,7 @@ int ldist_inf_dist_conv_forward(const float* img, const float* weight, int B, in
 }
 
 int ldist_set_conv_staging_override(int mode) {
-    if (mode < 0 || mode > 2) return LDIST_EINVAL;
+    if (mode < 0 || mode > 3) return LDIST_EINVAL;
     ldist::g_conv_staging_override = mode;
     return LDIST_OK;
 }

@@ -80,4 +80,4 @@ def test_conv_forward_geometry_query_needs_no_device(lib):
     assert lib.ldist_inf_dist_conv_forward(one, one, 1, 4, 28, 28, 8, 1, 3, 3, 1, 1, 1, one, one, None) == -5
     assert lib.ldist_inf_dist_conv_forward(None, one, 1, 4, 32, 32, 8, 1, 3, 3, 1, 1, 1, one, one, None) == -1
     assert lib.ldist_set_conv_rows_override(-1) == -1 and lib.ldist_set_conv_rows_override(0) == 0
-    assert lib.ldist_set_conv_staging_override(3) == -1 and lib.ldist_set_conv_staging_override(0) == 0
+    assert lib.ldist_set_conv_staging_override(4) == -1 and lib.ldist_set_conv_staging_override(0) == 0

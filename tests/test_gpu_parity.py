@@ -517,6 +517,73 @@ def test_conv_layer_image_path_matches_column_path(p):
     torch.testing.assert_close(gwa, layer.weight.grad, rtol=1e-4, atol=5e-5)
 
 
+def test_conv_net_runs_from_the_image_and_matches_the_column_path():
+    """The reference's conv net (3 -> 32 -> 32 -> 64 -> 64 -> 64 channels at width 1) at p = inf: every conv
+    layer is covered by the image kernel (resident first layer, staged wide ones, one stride-2 layer); outputs,
+    input gradient and weight gradients equal those of the same net forced onto the column kernels."""
+    from gpu_common import DEV, cpp, pkg
+    lib = pkg._lib.lib()
+    torch.manual_seed(11)
+    net = pkg.Conv(width=1, input_dim=(3, 32, 32), hidden=64, num_classes=10).to(DEV).train()
+    pkg.set_p_norm(net, float("inf"))
+    for layer in net.conv:
+        assert cpp.inf_dist_conv_forward_supported(layer.in_channels, 32 if layer.in_channels <= 32 else 16,
+                                                   32 if layer.in_channels <= 32 else 16, layer.out_channels, 1, 3,
+                                                   layer.stride, 1, 1)
+    x = torch.rand(4, 3, 32, 32, generator=gen(71)).to(DEV)
+    up = torch.randn(4, 10, generator=gen(72)).to(DEV)
+    results = []
+    for mode in (0, 3):                      # 0: image kernels where they apply; 3: column kernels everywhere
+        assert lib.ldist_set_conv_staging_override(mode) == 0
+        for prm in net.parameters():
+            prm.grad = None
+        for m in net.modules():              # same running means on both passes
+            if isinstance(m, pkg.MeanNorm):
+                m.running_mean.zero_()
+        xi = x.clone().requires_grad_(True)
+        y, _, _ = net(xi)
+        y.backward(up)
+        torch.cuda.synchronize()
+        results.append((y.detach().clone(), xi.grad.clone(), [prm.grad.clone() for prm in net.parameters()]))
+    lib.ldist_set_conv_staging_override(0)
+    (ya, ga, wa), (yb, gb, wb) = results
+    assert torch.equal(ya, yb)                                   # same argmax, same values: bit-identical forward
+    torch.testing.assert_close(ga, gb, rtol=RTOL, atol=ATOL)
+    for a_, b_ in zip(wa, wb):
+        torch.testing.assert_close(a_, b_, rtol=1e-4, atol=5e-5)  # atomics order
+
+
+def test_harness_on_gpu_trains_attacks_and_certifies():
+    """Model(MLP, BoundFinalIdentity): a few training steps at p = 8 lower the loss; PGD stays in its ball; the
+    certified accuracy at eps = 0 equals the clean accuracy and does not grow with eps."""
+    import torch.nn.functional as F
+    from gpu_common import DEV, pkg
+    torch.manual_seed(12)
+    net = pkg.Model(pkg.MLP(depth=3, width=1, input_dim=(1, 8, 8), num_classes=4), pkg.BoundFinalIdentity(),
+                    eps=0.05).to(DEV)
+    pkg.set_p_norm(net, 8.0)
+    x = torch.rand(64, 1, 8, 8, generator=gen(73)).to(DEV)
+    y = torch.randint(0, 4, (64,), generator=gen(74)).to(DEV)
+    opt = pkg.AdamW(net, lr=0.02, weight_decay=0.0)
+    loss_fun = lambda out, worse, t: F.cross_entropy(out, t)
+    first, _ = pkg.train_step(net, loss_fun, opt, x, y)
+    for _ in range(30):
+        last, _ = pkg.train_step(net, loss_fun, opt, x, y)
+    assert last < first
+    net.eval()
+    up_, down_ = torch.ones_like(x[0]), torch.zeros_like(x[0])
+    adv = pkg.AttackPGD(net, 0.05, 0.0125, 5, up_, down_).find(x, y)
+    assert float((adv - x).abs().max()) <= 0.05 + 1e-6 and float(adv.min()) >= 0 and float(adv.max()) <= 1
+    pkg.set_p_norm(net, float("inf"))
+    with torch.no_grad():
+        clean = pkg.cal_acc(net(x), y).mean().item()
+    c0 = pkg.certified_accuracy(net, x, y, 0.0, up_, down_)
+    c1 = pkg.certified_accuracy(net, x, y, 0.02, up_, down_)
+    c2 = pkg.certified_accuracy(net, x, y, 0.2, up_, down_)
+    assert abs(c0 - clean) < 1e-6 and c0 >= c1 >= c2
+    assert pkg.get_p_norm(net) == float("inf") and pkg.get_eps(net) == 0.05
+
+
 def test_error_codes_and_checks():
     from gpu_common import DEV, cpp, pkg
     lib = pkg._lib.lib()

@@ -302,3 +302,78 @@ def test_adamw_constructor_checks_and_closure():
         return torch.tensor(3.0)
 
     assert opt.step(closure).item() == 3.0 and calls == [1]
+
+
+def test_model_wrapper_passes_bounds_only_with_targets():
+    """Reference model/model.py:9-17: without targets the bounds are dropped; with targets and a feature that
+    returns no bounds, the eps-ball around the feature output is what the predictor gets."""
+    pkg = entry.load_package()
+    seen = {}
+
+    class Feature(torch.nn.Module):
+        def forward(self, x, lower=None, upper=None):
+            seen["feature"] = (lower, upper)
+            return x * 2, None, None
+
+    class Predictor(torch.nn.Module):
+        def forward(self, x, lower, upper, targets=None):
+            seen["predictor"] = (lower, upper, targets)
+            return x
+
+    net = pkg.Model(Feature(), Predictor(), eps=0.25)
+    x = torch.ones(2, 3)
+    net(x, lower=x - 1, upper=x + 1)
+    assert seen["feature"] == (None, None) and seen["predictor"] == (None, None, None)
+    t = torch.tensor([0, 1])
+    net(x, lower=x - 1, upper=x + 1, targets=t)
+    lo, up, tt = seen["predictor"]
+    assert torch.equal(lo, x * 2 - 0.25) and torch.equal(up, x * 2 + 0.25) and tt is t
+    pkg.set_eps(net, 0.5)
+    assert pkg.get_eps(net) == 0.5 and pkg.get_eps(torch.nn.Linear(2, 2)) is None
+
+
+def test_pgd_stays_in_the_ball_and_the_range_and_raises_the_loss():
+    """Reference attack.py:15-36 on a plain linear classifier: the result lies within eps of the input and within
+    [down, up], parameters get their requires_grad back, and the cross entropy does not go down."""
+    pkg = entry.load_package()
+    torch.manual_seed(3)
+    net = torch.nn.Linear(12, 4)
+    x = torch.rand(16, 12)
+    y = torch.randint(0, 4, (16,))
+    up, down = torch.ones(12), torch.zeros(12)
+    adv = pkg.AttackPGD(net, eps=0.1, step_size=0.025, num_steps=8, up=up, down=down).find(x, y)
+    assert float((adv - x).abs().max()) <= 0.1 + 1e-6
+    assert float(adv.min()) >= 0.0 and float(adv.max()) <= 1.0
+    assert all(p.requires_grad for p in net.parameters())
+    ce = torch.nn.functional.cross_entropy
+    with torch.no_grad():
+        assert float(ce(net(adv), y)) >= float(ce(net(x), y))
+    fixed = pkg.AttackPGD(net, 0.1, 0.025, 1, up, down, random_start=False).find(x, y)
+    leaf = x.detach().clone().requires_grad_(True)
+    ce(net(leaf), y, reduction="sum").backward()
+    expect = torch.min(torch.max(leaf.detach() + 0.025 * leaf.grad.sign(), down), up)
+    assert torch.allclose(fixed, expect)   # one step without the random start is the signed-gradient step
+
+
+def test_train_step_and_accuracy_helpers():
+    pkg = entry.load_package()
+    torch.manual_seed(4)
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.lin = torch.nn.Linear(6, 3)
+
+        def forward(self, x, targets=None):
+            out = self.lin(x)
+            return out, out - 0.1
+
+    net = Net()
+    opt = torch.optim.SGD(net.parameters(), lr=0.5)
+    x, y = torch.randn(32, 6), torch.randint(0, 3, (32,))
+    loss_fun = lambda out, worse, t: torch.nn.functional.cross_entropy(out, t)
+    first, _ = pkg.train_step(net, loss_fun, opt, x, y)
+    for _ in range(20):
+        last, acc = pkg.train_step(net, loss_fun, opt, x, y)
+    assert last < first and 0.0 <= acc <= 1.0
+    assert pkg.cal_acc(torch.tensor([[0.1, 0.9], [0.8, 0.2]]), torch.tensor([1, 1])).tolist() == [1.0, 0.0]
