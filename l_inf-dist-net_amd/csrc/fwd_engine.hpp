@@ -223,6 +223,8 @@ hipError_t dispatch_forward(const Problem& pr, bool vec4, bool ovec, hipStream_t
             return launch_forward<KERNEL, Geo<128, 80, 8, 5, 2>>(pr, vec4, ovec, stream, args...);
         case TileChoice::M256N32K1:
             return launch_forward<KERNEL, Geo<256, 32, 8, 4, 1>>(pr, vec4, ovec, stream, args...);
+        case TileChoice::M32N32K8:
+            return launch_forward<KERNEL, Geo<32, 32, 4, 4, 8>>(pr, vec4, ovec, stream, args...);
         default:
             return launch_forward<KERNEL, Geo<128, 64, 8, 4, 1>>(pr, vec4, ovec, stream, args...);
     }

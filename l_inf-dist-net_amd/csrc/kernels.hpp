@@ -13,28 +13,32 @@ struct Problem {
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-enum class TileChoice { M128N80K2, M128N64K1, M256N32K1 };
+enum class TileChoice { M128N80K2, M128N64K1, M256N32K1, M32N32K8 };
 
 // Picks the workgroup tiling that leaves the fewest padded (m,n) cells per CU.
 // M128N80K2 (512 lanes, two k-groups) fills a CU with one workgroup and divides
 // 512 x 5120 into exactly 256 tiles; M128N64K1 is the general shape;
 // M256N32K1 serves grouped layers with few outputs per group.
-// -1 = choose by shape; 0, 1, 2 force M128N80K2, M128N64K1, M256N32K1 (tests and tuning).
+// M32N32K8 (512 lanes, eight k-groups of one wave, 4x4 values per lane) is for few rows and outputs with
+// a long reduction (the first fully connected layer behind a conv stack: 128 x 1024 outputs, K = 49152):
+// it makes 80 times more workgroups than the big tiles, at twice their LDS traffic per difference.
+// -1 = choose by shape; 0, 1, 2, 3 force M128N80K2, M128N64K1, M256N32K1, M32N32K8 (tests and tuning).
 extern int g_tile_override;
 extern int g_xcd_remap;  // 1 (default): XCD-aware tile order; 0: plain order (tuning)
 
 inline TileChoice choose_tile(int M, int NG, int G, int num_cu) {
-    if (g_tile_override >= 0 && g_tile_override <= 2) return static_cast<TileChoice>(g_tile_override);
-    struct Cand { TileChoice c; int bm, bn; bool two_groups; };
-    const Cand cands[3] = {{TileChoice::M128N80K2, 128, 80, true},
-                           {TileChoice::M128N64K1, 128, 64, false},
-                           {TileChoice::M256N32K1, 256, 32, false}};
+    if (g_tile_override >= 0 && g_tile_override <= 3) return static_cast<TileChoice>(g_tile_override);
+    struct Cand { TileChoice c; int bm, bn; bool two_groups; double price; };
+    const Cand cands[4] = {{TileChoice::M128N80K2, 128, 80, true, 1.0},
+                           {TileChoice::M128N64K1, 128, 64, false, 1.0},
+                           {TileChoice::M256N32K1, 256, 32, false, 1.0},
+                           {TileChoice::M32N32K8, 32, 32, true, 1.6}};   // a cell of the small tile costs more
     double best = 1e300;
     TileChoice pick = TileChoice::M128N64K1;
     for (const Cand& c : cands) {
         const long tiles = (long)((M + c.bm - 1) / c.bm) * ((NG + c.bn - 1) / c.bn) * G;
         const long rounds = (tiles + num_cu - 1) / num_cu;
-        double cost = (double)rounds * c.bm * c.bn;
+        double cost = (double)rounds * c.bm * c.bn * c.price;
         // a lone single-group workgroup leaves one wave per SIMD: latency shows
         if (!c.two_groups && tiles < 2L * num_cu) cost *= 1.25;
         if (cost < best) { best = cost; pick = c.c; }
