@@ -33,7 +33,8 @@ constexpr int kKC = kCC * 9;      // k values per weight stage
 constexpr int kMaxThreads = 256;
 constexpr int kBNP = 68;          // row length of the weight stage: 64 outputs + 4, a constant so that reads take immediate offsets
 constexpr int kWRegs = 9;         // weight words a lane carries from global to LDS per stage (64 outputs x 36 / 256)
-constexpr int kXRegs = 10;        // image words a lane carries per stage when the channels are staged
+// image words a lane carries per stage when the channels are staged (4 channels x rows held x padded width / lanes)
+__host__ __device__ constexpr int x_regs(int S) { return S == 1 ? 7 : 10; }
 
 struct ConvFwd {
     int B, G, CG, NG, K;         // images, groups, channels and outputs per group, K = 9*CG
@@ -105,6 +106,7 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
     const float* src = img + ((size_t)b * a.G + g) * a.CG * a.H * a.W;   // the group's channels of this image
     // ---- staged: what each lane moves per stage is the same every time, only the channel base advances ----
     const int xhalf = a.xwords / 2;                     // one stage buffer: at least kCC*NR*WP and kXRegs*NT words
+    constexpr int kXRegs = x_regs(S);
     int goff[kXRegs];                                   // element offset inside the stage's kCC channels; -1 = padding
     float xreg[kXRegs];
     if constexpr (!RESIDENT) {
@@ -389,6 +391,7 @@ bool plan(const ConvGeom& q, int G, int CO, ConvFwd& a) {
                 } else {
                     // a lane carries kXRegs image words per stage in registers; what a small workgroup cannot
                     // carry that way it copies directly, which is slow: only taken when forced
+                    const int kXRegs = x_regs(S);
                     const int stage = kCC * NR * a.WP;
                     if (stage > kXRegs * NT && forced <= 0) continue;
                     const int half = stage > kXRegs * NT ? stage : kXRegs * NT;
