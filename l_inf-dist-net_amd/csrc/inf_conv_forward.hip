@@ -154,16 +154,29 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
         __syncthreads();
         const int rows = a.CG * NR;
         if (a.vec_in) {
-            const int QW = a.W / 4;
-            for (int i = tid; i < rows * QW; i += NT) {
-                const int row = i / QW, xq = i - row * QW;
-                const int c = row / NR, r = row - c * NR;
-                const int y = y0 + r;
-                if ((unsigned)y < (unsigned)a.H) {
-                    const float4 v = *reinterpret_cast<const float4*>(src + ((size_t)c * a.H + y) * a.W + 4 * xq);
-                    float* dst = tile + (c * NR + r) * WP + a.P + 4 * xq;
-                    dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+            // four 16-byte loads in flight per lane, then their stores: one at a time, a workgroup would wait out
+            // a memory latency per 4 KB before it can start
+            const int QW = a.W / 4, total = rows * QW;
+            constexpr int UN = 4;
+            for (int i0 = tid; i0 < total; i0 += UN * NT) {
+                float4 v[UN];
+                int at[UN];
+#pragma unroll
+                for (int u = 0; u < UN; u++) {
+                    const int i = i0 + u * NT;
+                    const int row = i / QW, xq = i - row * QW;
+                    const int c = row / NR, r = row - c * NR;
+                    const int y = y0 + r;
+                    const bool real = i < total && (unsigned)y < (unsigned)a.H;
+                    at[u] = real ? (c * NR + r) * WP + a.P + 4 * xq : -1;
+                    v[u] = *reinterpret_cast<const float4*>(src + (real ? ((size_t)c * a.H + y) * a.W + 4 * xq : 0));
                 }
+#pragma unroll
+                for (int u = 0; u < UN; u++)
+                    if (at[u] >= 0) {
+                        float* dst = tile + at[u];
+                        dst[0] = v[u].x; dst[1] = v[u].y; dst[2] = v[u].z; dst[3] = v[u].w;
+                    }
             }
         } else {
             for (int i = tid; i < rows * a.W; i += NT) {
