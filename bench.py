@@ -473,11 +473,11 @@ def main():
             "traffic": None,
         },
     }
-    if args.workload == "c1":
-        # HBM bytes per launch, average over the step's four tiled forward launches, from two
-        # rocprofv3 --pmc runs of this command (profiles/): FETCH_SIZE x 2.0 (copy-probe factor)
-        # + WRITE_SIZE x 1.0
-        out["roofline"]["traffic"] = TRAFFIC_C1_BYTES
+    # HBM bytes per launch of the roofline kernel (c1: average over the step's four tiled forward launches),
+    # from two rocprofv3 --pmc runs of this command (profiles/): FETCH_SIZE x 2.0 (copy-probe factor)
+    # + WRITE_SIZE x 1.0
+    if args.workload in TRAFFIC_BYTES:
+        out["roofline"]["traffic"] = TRAFFIC_BYTES[args.workload]
     for label, alt in wl.get("step_alt", []):
         for _ in range(args.warmup):
             alt()
@@ -493,7 +493,7 @@ def main():
     print(json.dumps(out))
 
 
-TRAFFIC_C1_BYTES = 3.21e8
+TRAFFIC_BYTES = {"c1": 3.20e8, "c4i": 2.15e8}
 
 
 if __name__ == "__main__":

@@ -178,6 +178,19 @@ LDIST_API int ldist_inf_dist_conv_forward_supported(int C, int H, int W, int CO,
 LDIST_API int ldist_inf_dist_conv_forward(const float* img, const float* weight, int B, int C, int H, int W, int CO, int G,
                                 int KH, int KW, int stride, int padding, int dilation, float* output, int32_t* pos,
                                 ldist_stream_t stream);
+/* Interval-bound forward of the convolution-shaped layer straight from the lower and upper images: what
+ * ldist_unfold of both followed by ldist_inf_dist_bound_forward computes (the reference: F.unfold at
+ * model/norm_dist.py:144-145, then inf_dist_bound_forward_cuda), bit for bit, irregular boxes included.
+ *   lower_img, upper_img (B, C, H, W), weight (CO, C/G*KH*KW), output_lower and output_upper (B, CO, HO*WO).
+ * Covers 3x3 windows with dilation 1, stride 1 or 2 and WO % 8 == 0, any number of channels;
+ * ldist_inf_dist_bound_conv_forward_supported returns 1 for such a geometry, 0 otherwise, and
+ * ldist_inf_dist_bound_conv_forward returns LDIST_EUNSUPPORTED for the rest (nothing is enqueued). */
+LDIST_API int ldist_inf_dist_bound_conv_forward_supported(int C, int H, int W, int CO, int G, int KH, int KW, int stride,
+                                                          int padding, int dilation);
+LDIST_API int ldist_inf_dist_bound_conv_forward(const float* lower_img, const float* upper_img, const float* weight,
+                                                int B, int C, int H, int W, int CO, int G, int KH, int KW, int stride,
+                                                int padding, int dilation, float* output_lower, float* output_upper,
+                                                ldist_stream_t stream);
 /* Testing and tuning knob, no counterpart in the reference: output rows per workgroup of
  * ldist_inf_dist_conv_forward; 0 (default) = chosen by shape.  A positive value is clamped to what the
  * geometry allows and also switches off the rule that leaves small or channel-heavy layers, which

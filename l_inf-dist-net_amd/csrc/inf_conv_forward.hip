@@ -17,7 +17,7 @@
 // maximum (subtract + half a v_max3 per difference, three instructions per channel and output); the lowest k
 // inside the recorded channel is found afterwards from nine pixels (LDS when RESIDENT, else the image in
 // global memory) and the channel's nine contiguous weights.
-#include "kernels.hpp"
+#include "conv_image.hpp"
 
 namespace ldist {
 
@@ -26,27 +26,7 @@ int g_conv_staging_override = 0;   // 1: image rows resident in LDS only; 2: sta
 
 namespace {
 
-constexpr int kTM = 8, kTN = 4;   // positions x outputs per lane
-constexpr int kCC = 4;            // channels per weight stage
-constexpr int kTrack = 1;         // channels per recorded unit
-constexpr int kKC = kCC * 9;      // k values per weight stage
-constexpr int kMaxThreads = 256;
-constexpr int kBNP = 68;          // row length of the weight stage: 64 outputs + 4, a constant so that reads take immediate offsets
-constexpr int kWRegs = 9;         // weight words a lane carries from global to LDS per stage (64 outputs x 36 / 256)
-// image words a lane carries per stage when the channels are staged (4 channels x rows held x padded width / lanes)
-__host__ __device__ constexpr int x_regs(int S) { return S == 1 ? 7 : 10; }
-
-struct ConvFwd {
-    int B, G, CG, NG, K;         // images, groups, channels and outputs per group, K = 9*CG
-    int H, W, HO, WO, P;         // image, output positions, padding
-    int R, NR, WP, CGP;          // output rows per workgroup, image rows held, padded row length, CG rounded up to kCC
-    int SEG, ML, NL, BN;         // 8-position segments per output row, lanes along positions / outputs, outputs per
-                                 // workgroup
-    int tiles_h, tiles_n;
-    int vec_in, vec_out;         // 128-bit global loads of image rows / stores of results allowed
-    int resident;                // 1: all channels of the image rows stay in LDS; 0: staged kCC channels at a time
-    int xwords;                  // floats of the image area in LDS
-};
+using namespace convimg;
 
 template <int S, bool RESIDENT>
 __global__ void __launch_bounds__(kMaxThreads, 2)
@@ -353,84 +333,6 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
             for (int e = 0; e < kTM; e++) { out[at + e] = acc[e][t]; pos[at + e] = ps[e]; }
         }
     }
-}
-
-constexpr size_t kLdsLimit = 160 * 1024;
-
-// Fills the launch shape; false when this kernel does not cover the geometry.
-bool plan(const ConvGeom& q, int G, int CO, ConvFwd& a) {
-    if (q.KH != 3 || q.KW != 3 || q.D != 1 || (q.S != 1 && q.S != 2)) return false;
-    if (q.WO % kTM != 0 || G <= 0 || q.C % G != 0 || CO % G != 0) return false;
-    const int S = q.S, NXR = (7 * S + 2) / 4 + 1;
-    a.B = q.B; a.G = G; a.CG = q.C / G; a.NG = CO / G; a.K = a.CG * 9;
-    a.H = q.H; a.W = q.W; a.HO = q.HO; a.WO = q.WO; a.P = q.P;
-    a.CGP = (a.CG + kCC - 1) / kCC * kCC;
-    a.SEG = q.WO / kTM;
-    // the last lane of a row reads NXR*4 words from column (WO-8)*S; the image with its padding is W + 2P wide
-    int wp = (q.WO - kTM) * S + NXR * 4;
-    if (q.W + 2 * q.P > wp) wp = q.W + 2 * q.P;
-    a.WP = (wp + 3) / 4 * 4;
-    if (a.WP % 32 == 0) a.WP += 4;                     // rows of one lane's window in different banks
-    // Outputs per workgroup: at most 64, split evenly over the tiles; more tiles when a workgroup of that
-    // width would have too many lanes (wide images).
-    const int quads = (a.NG + kTN - 1) / kTN;
-    for (int pass = 0; pass < 2; pass++) {
-        // pass 0: all channels resident in LDS; pass 1: channels staged (needs CG % kCC == 0, so that no
-        // stage holds a channel that does not exist)
-        const bool resident = pass == 0;
-        if (g_conv_staging_override == 3) continue;
-        if (g_conv_staging_override == 1 && !resident) continue;
-        if (g_conv_staging_override == 2 && resident) continue;
-        if (!resident && a.CG % kCC != 0) continue;
-        for (int tiles_n = (quads + 15) / 16; tiles_n <= quads; tiles_n++) {
-            const int NL = (quads + tiles_n - 1) / tiles_n;
-            if (a.SEG * NL > kMaxThreads) continue;
-            const int BN = NL * kTN;
-            // rows per workgroup: the choice that keeps most lanes busy on a CU (LDS limit, 8 waves of this
-            // register footprint, rows computed past the image bottom count as idle); ties take more rows
-            int bestR = 0, bestWords = 0;
-            double bestScore = -1.0;
-            const int maxR = kMaxThreads / (a.SEG * NL);
-            int forced = g_conv_rows_override;
-            if (forced > maxR) forced = maxR;
-            if (forced > q.HO) forced = q.HO;
-            for (int R = 1; R <= maxR && R <= q.HO; R++) {
-                if (forced > 0 && R != forced) continue;
-                const int NR = (R - 1) * S + 3;
-                const int NT = R * a.SEG * NL;
-                int xwords;
-                if (resident) {
-                    xwords = a.CGP * NR * a.WP;
-                } else {
-                    // a lane carries kXRegs image words per stage in registers; what a small workgroup cannot
-                    // carry that way it copies directly, which is slow: only taken when forced
-                    const int kXRegs = x_regs(S);
-                    const int stage = kCC * NR * a.WP;
-                    if (stage > kXRegs * NT && forced <= 0) continue;
-                    const int half = stage > kXRegs * NT ? stage : kXRegs * NT;
-                    xwords = 2 * ((half + 3) / 4 * 4);
-                }
-                const size_t lds = ((size_t)xwords + 2 * (size_t)kKC * kBNP) * sizeof(float);
-                if (lds > kLdsLimit) { if (resident) break; else continue; }
-                const long waves_wg = (NT + 63) / 64;
-                long wgs = (long)(kLdsLimit / lds);
-                if (wgs * waves_wg > 8) wgs = 8 / waves_wg;
-                const int tiles_h = (q.HO + R - 1) / R;
-                const double score = (double)wgs * NT * q.HO / ((double)tiles_h * R);
-                if (score >= bestScore) { bestScore = score; bestR = R; bestWords = xwords; }
-            }
-            // below six resident waves per CU this variant does badly: try the other, or leave the layer to
-            // the column kernels
-            if (bestR == 0 || (bestScore < 384.0 && forced <= 0)) continue;
-            a.NL = NL; a.BN = BN; a.tiles_n = (quads + NL - 1) / NL;
-            a.R = bestR; a.NR = (bestR - 1) * S + 3; a.ML = bestR * a.SEG;
-            a.tiles_h = (q.HO + bestR - 1) / bestR;
-            a.resident = resident ? 1 : 0;
-            a.xwords = bestWords;
-            return (long long)q.B * G * a.tiles_h * a.tiles_n < (1LL << 31);
-        }
-    }
-    return false;
 }
 
 }  // namespace

@@ -97,6 +97,10 @@ extern int g_conv_staging_override;
 bool inf_conv_forward_supported(const ConvGeom& q, int G, int CO);
 hipError_t inf_conv_forward(const float* img, const float* weight, float* out, int32_t* pos, const ConvGeom& q, int G,
                             int CO, int device, hipStream_t stream);
+// Interval-bound forward straight from the lower and upper images (same geometries; channels always staged).
+bool bound_conv_forward_supported(const ConvGeom& q, int G, int CO);
+hipError_t bound_conv_forward(const float* lower, const float* upper, const float* weight, float* out_lower,
+                              float* out_upper, const ConvGeom& q, int G, int CO, int device, hipStream_t stream);
 hipError_t inf_backward_input_folded(const float* grad_output, const int32_t* pos, float* grad_img, const ConvGeom& q,
                                      int G, int CO, hipStream_t stream);
 

@@ -248,6 +248,30 @@ int ldist_inf_dist_conv_forward(const float* img, const float* weight, int B, in
     return finish(ldist::inf_conv_forward(img, weight, output, pos, q, G, CO, pr.device, (hipStream_t)stream));
 }
 
+int ldist_inf_dist_bound_conv_forward_supported(int C, int H, int W, int CO, int G, int KH, int KW, int stride,
+                                                int padding, int dilation) {
+    ldist::ConvGeom q{};
+    if (CO <= 0 || G <= 0) return 0;
+    if (conv_geometry(1, C, H, W, KH, KW, stride, padding, dilation, q) != LDIST_OK) return 0;
+    return ldist::bound_conv_forward_supported(q, G, CO) ? 1 : 0;
+}
+
+int ldist_inf_dist_bound_conv_forward(const float* lower_img, const float* upper_img, const float* weight, int B, int C,
+                                      int H, int W, int CO, int G, int KH, int KW, int stride, int padding,
+                                      int dilation, float* output_lower, float* output_upper, ldist_stream_t stream) {
+    ldist::ConvGeom q{};
+    if (!lower_img || !upper_img || !weight || !output_lower || !output_upper || CO <= 0 || G <= 0) return LDIST_EINVAL;
+    if (int rc = conv_geometry(B, C, H, W, KH, KW, stride, padding, dilation, q)) return rc;
+    if (C % G != 0 || CO % G != 0) return LDIST_EINVAL;
+    if ((long long)B * CO * q.HO * q.WO >= (1LL << 31) || (long long)CO * (C / G) * KH * KW >= (1LL << 31))
+        return LDIST_ERANGE;
+    if (!ldist::bound_conv_forward_supported(q, G, CO)) return LDIST_EUNSUPPORTED;
+    ldist::Problem pr{};
+    if (int rc = current_device(pr)) return rc;
+    return finish(ldist::bound_conv_forward(lower_img, upper_img, weight, output_lower, output_upper, q, G, CO,
+                                            pr.device, (hipStream_t)stream));
+}
+
 int ldist_set_conv_staging_override(int mode) {
     if (mode < 0 || mode > 3) return LDIST_EINVAL;
     ldist::g_conv_staging_override = mode;

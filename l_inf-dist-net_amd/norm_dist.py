@@ -292,6 +292,15 @@ class NormDistConv(nn.Module):
                 not (self.kernel_size == 1 and self.stride == 1 and self.padding == 0) and
                 (self.in_channels // self.group) * x.size(3) <= norm_dist_cpp.FOLDED_MAX_ROW_FLOATS)
 
+    def _bound_from_images(self, lower, upper):
+        """True when the interval bounds can be computed straight from the two images (the bound path carries no
+        gradient, as in the reference: it runs in evaluation mode only)."""
+        return (lower.is_cuda and lower.dtype == torch.float32 and upper.dtype == torch.float32 and
+                not (self.kernel_size == 1 and self.stride == 1 and self.padding == 0) and
+                norm_dist_cpp.inf_dist_bound_conv_forward_supported(self.in_channels, lower.size(2), lower.size(3),
+                                                                    self.out_channels, self.group, self.kernel_size,
+                                                                    self.stride, self.padding, self.dilation))
+
     def _shift(self, t):
         if self.normalize is not None:
             t = self.normalize(t)
@@ -311,6 +320,14 @@ class NormDistConv(nn.Module):
         if lower is None or upper is None:
             return y, None, None
         assert math.isinf(self.p) and not self.training
+        if self._bound_from_images(lower, upper):
+            lo = torch.empty(x.size(0), w2d.size(0), out_hw[0] * out_hw[1], device=x.device, dtype=x.dtype)
+            hi = torch.empty_like(lo)
+            with torch.no_grad():
+                norm_dist_cpp.inf_dist_bound_conv_forward(lower.contiguous(), upper.contiguous(), w2d.detach(), lo, hi,
+                                                          self.group, self.kernel_size, self.stride, self.padding,
+                                                          self.dilation)
+            return y, self._shift(lo.view_as(y)), self._shift(hi.view_as(y))
         lo, hi = inf_dist_bound(self._columns(lower), self._columns(upper), w2d, self.group, tag=self.tag)
         return y, self._shift(lo.view_as(y)), self._shift(hi.view_as(y))
 

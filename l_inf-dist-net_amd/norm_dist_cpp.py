@@ -277,3 +277,30 @@ def inf_dist_conv_forward(img, weight, output, pos, G, kernel_size, stride=1, pa
     _expect(output.shape == (B, CO, HO * WO) and pos.shape == output.shape, "output and pos must be (B, CO, HO*WO)")
     _call("ldist_inf_dist_conv_forward", dev, _p(img), _p(weight), B, C, H, W, CO, G, KH, KW, S, P, D, _p(output),
           _p(pos))
+
+
+def inf_dist_bound_conv_forward_supported(C, H, W, CO, G, kernel_size, stride=1, padding=0, dilation=1):
+    """True when inf_dist_bound_conv_forward covers the geometry (3x3, dilation 1, stride 1 or 2, output width a
+    multiple of 8); otherwise unfold both images and call inf_dist_bound_forward."""
+    k = int(kernel_size)
+    return bool(_lib.lib().ldist_inf_dist_bound_conv_forward_supported(int(C), int(H), int(W), int(CO), int(G), k, k,
+                                                                        int(stride), int(padding), int(dilation)))
+
+
+def inf_dist_bound_conv_forward(lower_img, upper_img, weight, output_lower, output_upper, G, kernel_size, stride=1,
+                                padding=0, dilation=1):
+    """Interval bounds of the conv-shaped layer straight from the lower and upper images: equal to
+    inf_dist_bound_forward on F.unfold of both, without building the columns."""
+    for t, n in ((lower_img, "lower_img"), (upper_img, "upper_img"), (weight, "weight"),
+                 (output_lower, "output_lower"), (output_upper, "output_upper")):
+        _check_input(t, n)
+    dev = _same_device(lower_img, upper_img, weight, output_lower, output_upper)
+    _expect(lower_img.shape == upper_img.shape, "lower_img and upper_img must have one shape")
+    B, C, H, W, KH, KW, S, P, D = _conv_args(lower_img, kernel_size, stride, padding, dilation)
+    HO, WO = conv_output_size(H, W, KH, S, P, D)
+    _expect(weight.dim() == 2 and C % G == 0 and weight.size(1) == C // G * KH * KW, "weight must be (CO, C/G*k*k)")
+    CO = weight.size(0)
+    _expect(output_lower.shape == (B, CO, HO * WO) and output_upper.shape == output_lower.shape,
+            "output_lower and output_upper must be (B, CO, HO*WO)")
+    _call("ldist_inf_dist_bound_conv_forward", dev, _p(lower_img), _p(upper_img), _p(weight), B, C, H, W, CO, G, KH, KW,
+          S, P, D, _p(output_lower), _p(output_upper))

@@ -79,5 +79,10 @@ def test_conv_forward_geometry_query_needs_no_device(lib):
     one = ctypes.c_void_p(16)
     assert lib.ldist_inf_dist_conv_forward(one, one, 1, 4, 28, 28, 8, 1, 3, 3, 1, 1, 1, one, one, None) == -5
     assert lib.ldist_inf_dist_conv_forward(None, one, 1, 4, 32, 32, 8, 1, 3, 3, 1, 1, 1, one, one, None) == -1
+    okb = lib.ldist_inf_dist_bound_conv_forward_supported
+    assert okb(128, 32, 32, 128, 4, 3, 3, 1, 1, 1) == 1 and okb(90, 32, 32, 96, 1, 3, 3, 1, 1, 1) == 1   # any channel count
+    assert okb(4, 28, 28, 8, 1, 3, 3, 1, 1, 1) == 0 and okb(4, 16, 16, 8, 1, 5, 5, 1, 2, 1) == 0
+    assert lib.ldist_inf_dist_bound_conv_forward(one, one, one, 1, 4, 28, 28, 8, 1, 3, 3, 1, 1, 1, one, one, None) == -5
+    assert lib.ldist_inf_dist_bound_conv_forward(one, None, one, 1, 4, 32, 32, 8, 1, 3, 3, 1, 1, 1, one, one, None) == -1
     assert lib.ldist_set_conv_rows_override(-1) == -1 and lib.ldist_set_conv_rows_override(0) == 0
     assert lib.ldist_set_conv_staging_override(4) == -1 and lib.ldist_set_conv_staging_override(0) == 0

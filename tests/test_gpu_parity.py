@@ -517,6 +517,50 @@ def test_conv_layer_image_path_matches_column_path(p):
     torch.testing.assert_close(gwa, layer.weight.grad, rtol=1e-4, atol=5e-5)
 
 
+BOUND_IMAGE_CASES = IMPLICIT_CASES + [(2, 96, 32, 32, 96, 1, 1, 1), (1, 192, 16, 16, 192, 1, 1, 1), (2, 96, 32, 32, 192, 1, 2, 1)]
+
+
+@pytest.mark.parametrize("rows", [0, 3])
+@pytest.mark.parametrize("kind", ["regular", "irregular"])
+@pytest.mark.parametrize("case", BOUND_IMAGE_CASES)
+def test_bound_conv_forward_matches_column_path_bit_exact(case, kind, rows):
+    """Interval bounds straight from the lower and upper images against the oracle on torch's unfolded columns,
+    bit for bit: regular boxes (the max3 fast path) and boxes with l > u, NaN and infinities sprinkled in, which
+    send the stages that hold them through the reference's literal predicate."""
+    import torch.nn.functional as F
+    from gpu_common import DEV, cpp, pkg, say
+    B, C, H, W, CO, G, s_, p_ = case
+    say("bound_conv_forward", case, kind, "rows", rows)
+    lib = pkg._lib.lib()
+    assert lib.ldist_set_conv_rows_override(rows) == 0
+    if not cpp.inf_dist_bound_conv_forward_supported(C, H, W, CO, G, 3, s_, p_, 1):
+        assert rows == 0
+        pytest.skip("left to the column path by the library")
+    g = gen(81)
+    centre = torch.randn(B, C, H, W, generator=g)
+    radius = torch.rand(B, C, H, W, generator=g) * 0.3
+    lo_i, up_i = centre - radius, centre + radius
+    w = torch.randn(CO, C // G * 9, generator=g) * 0.7
+    if kind == "irregular":
+        flat_l, flat_u = lo_i.view(-1), up_i.view(-1)
+        n = flat_l.numel()
+        idx = torch.randperm(n, generator=g)[: max(8, n // 500)]
+        flat_l[idx[0::4]], flat_u[idx[0::4]] = flat_u[idx[0::4]].clone(), flat_l[idx[0::4]].clone()   # l > u
+        flat_l[idx[1::4]] = float("nan")
+        flat_u[idx[2::4]] = float("inf")
+        flat_l[idx[3::4]] = -float("inf")
+        w.view(-1)[5] = float("inf")
+    cl = F.unfold(lo_i, 3, 1, p_, s_).contiguous()
+    cu = F.unfold(up_i, 3, 1, p_, s_).contiguous()
+    el, eu = oracle.inf_dist_bound_forward(cl, cu, w, G)
+    ol = torch.full(el.shape, float("nan"), device=DEV)
+    ou = torch.full(el.shape, float("nan"), device=DEV)
+    cpp.inf_dist_bound_conv_forward(lo_i.to(DEV), up_i.to(DEV), w.to(DEV), ol, ou, G, 3, s_, p_, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(torch.nan_to_num(ol.cpu(), nan=-7.0), torch.nan_to_num(el, nan=-7.0))
+    assert torch.equal(torch.nan_to_num(ou.cpu(), nan=-7.0), torch.nan_to_num(eu, nan=-7.0))
+
+
 def test_conv_net_runs_from_the_image_and_matches_the_column_path():
     """The reference's conv net (3 -> 32 -> 32 -> 64 -> 64 -> 64 channels at width 1) at p = inf: every conv
     layer is covered by the image kernel (resident first layer, staged wide ones, one stride-2 layer); outputs,
@@ -551,6 +595,30 @@ def test_conv_net_runs_from_the_image_and_matches_the_column_path():
     torch.testing.assert_close(ga, gb, rtol=RTOL, atol=ATOL)
     for a_, b_ in zip(wa, wb):
         torch.testing.assert_close(a_, b_, rtol=1e-4, atol=5e-5)  # atomics order
+
+
+def test_conv_net_certification_from_the_images_matches_the_column_path():
+    """The conv net in evaluation mode with interval bounds: values and both bounds of the whole net computed
+    through the image kernels are bit-identical to those through unfold + column kernels."""
+    from gpu_common import DEV, pkg
+    lib = pkg._lib.lib()
+    torch.manual_seed(13)
+    net = pkg.Conv(width=1, input_dim=(3, 32, 32), hidden=64, num_classes=10).to(DEV).eval()
+    pkg.set_p_norm(net, float("inf"))
+    x = torch.rand(4, 3, 32, 32, generator=gen(75)).to(DEV)
+    eps = 8.0 / 255
+    lower, upper = (x - eps).clamp(0, 1), (x + eps).clamp(0, 1)
+    results = []
+    for mode in (0, 3):
+        assert lib.ldist_set_conv_staging_override(mode) == 0
+        with torch.no_grad():
+            results.append([t.clone() for t in net(x, lower, upper)])
+    lib.ldist_set_conv_staging_override(0)
+    torch.cuda.synchronize()
+    for a_, b_ in zip(*results):
+        assert torch.equal(a_, b_)
+    y, lo, up = results[0]
+    assert bool((lo <= y).all()) and bool((y <= up).all())
 
 
 def test_harness_on_gpu_trains_attacks_and_certifies():
