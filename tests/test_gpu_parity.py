@@ -561,6 +561,51 @@ def test_bound_conv_forward_matches_column_path_bit_exact(case, kind, rows):
     assert torch.equal(torch.nan_to_num(ou.cpu(), nan=-7.0), torch.nan_to_num(eu, nan=-7.0))
 
 
+def _misaligned(t, dev):
+    """A contiguous copy of t on the device whose first element sits 4 bytes past a 16-byte boundary."""
+    buf = torch.empty(t.numel() + 1, device=dev, dtype=t.dtype)
+    view = buf[1:].view(t.shape)
+    view.copy_(t)
+    assert view.data_ptr() % 16 == 4 and view.is_contiguous()
+    return view
+
+
+def test_conv_image_kernels_with_misaligned_tensors():
+    """Every tensor 4 bytes off a 16-byte boundary: the kernels must take their scalar load and store paths
+    (and the unaligned weight fetch of the argmax search) and give the same bits."""
+    import torch.nn.functional as F
+    from gpu_common import DEV, cpp, pkg
+    B, C, H, W, CO, G = 2, 8, 16, 16, 24, 2
+    g = gen(91)
+    img = torch.randn(B, C, H, W, generator=g)
+    w = torch.randn(CO, C // G * 9, generator=g)
+    cols = F.unfold(img, 3, 1, 1, 1).contiguous()
+    eo, ep = oracle.inf_dist_forward(cols, w, G)
+    out = _misaligned(torch.zeros(eo.shape), DEV)
+    pos = _misaligned(torch.zeros(eo.shape, dtype=torch.int32), DEV)
+    cpp.inf_dist_conv_forward(_misaligned(img, DEV), _misaligned(w, DEV), out, pos, G, 3, 1, 1, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu(), eo) and torch.equal(pos.cpu(), ep)
+    lo_i, up_i = img - 0.1, img + 0.1
+    el, eu = oracle.inf_dist_bound_forward(F.unfold(lo_i, 3, 1, 1, 1).contiguous(), F.unfold(up_i, 3, 1, 1, 1).contiguous(),
+                                           w, G)
+    ol, ou = _misaligned(torch.zeros(el.shape), DEV), _misaligned(torch.zeros(el.shape), DEV)
+    assert pkg._lib.lib().ldist_set_conv_rows_override(4) == 0   # a layer this small is otherwise left to the columns
+    cpp.inf_dist_bound_conv_forward(_misaligned(lo_i, DEV), _misaligned(up_i, DEV), _misaligned(w, DEV), ol, ou, G, 3, 1,
+                                    1, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(ol.cpu(), el) and torch.equal(ou.cpu(), eu)
+    c2 = _misaligned(torch.zeros(cols.shape), DEV)
+    cpp.unfold(_misaligned(img, DEV), c2, 3, 1, 1, 1)
+    gi = _misaligned(torch.zeros(img.shape), DEV)
+    go = torch.randn(eo.shape, generator=g)
+    cpp.inf_dist_backward_input_folded(_misaligned(go, DEV), _misaligned(ep, DEV), gi, G, 3, 1, 1, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(c2.cpu(), cols)
+    expect = F.fold(oracle.inf_dist_backward_input(go, ep, cols.size(1), G).double(), (H, W), 3, 1, 1, 1)
+    torch.testing.assert_close(gi.cpu().double(), expect, rtol=RTOL, atol=1e-5)
+
+
 def test_conv_net_runs_from_the_image_and_matches_the_column_path():
     """The reference's conv net (3 -> 32 -> 32 -> 64 -> 64 -> 64 channels at width 1) at p = inf: every conv
     layer is covered by the image kernel (resident first layer, staged wide ones, one stride-2 layer); outputs,
