@@ -128,9 +128,9 @@ fold_kernel(const float* __restrict__ gcols, float* __restrict__ gimg, ConvGeom 
 // workgroups, each keeping only what lands in its own rows.
 __global__ void __launch_bounds__(256)
 inf_backward_input_folded_kernel(const float* __restrict__ grad_output, const int32_t* __restrict__ pos,
-                                 float* __restrict__ grad_img, ConvGeom q, int G, int NG, int R, int row_tiles,
+                                 float* __restrict__ grad_img, ConvGeom q, int G, int NG, int R, int row_tiles, int vec, int vec_img,
                                  SmallDiv by_khw, SmallDiv by_kw, SmallDiv by_wo) {
-    extern __shared__ float bins[];
+    extern __shared__ __align__(16) float bins[];
     const int CG = q.C / G;
     const int tile = blockIdx.x % row_tiles;
     const int bg = blockIdx.x / row_tiles;          // b * G + g
@@ -138,7 +138,11 @@ inf_backward_input_folded_kernel(const float* __restrict__ grad_output, const in
     const int y0 = tile * R;
     const int rows = min(R, q.H - y0);
     const int nb = CG * rows * q.W;
-    for (int e = threadIdx.x; e < nb; e += 256) bins[e] = 0.f;
+    if (vec_img) {                                    // W % 4 == 0: nb is a multiple of four
+        for (int e = threadIdx.x * 4; e < nb; e += 1024) *reinterpret_cast<float4*>(bins + e) = make_float4(0.f, 0.f, 0.f, 0.f);
+    } else {
+        for (int e = threadIdx.x; e < nb; e += 256) bins[e] = 0.f;
+    }
     __syncthreads();
 
     // output rows h with h*S + i*D - P in [y0, y0 + rows) for some i in [0, KH)
@@ -150,30 +154,60 @@ inf_backward_input_folded_kernel(const float* __restrict__ grad_output, const in
     if (span > 0) {
         const size_t obase = ((size_t)bg * NG) * L + (size_t)h_lo * q.WO;
         const int khw = q.KH * q.KW;
-        // lanes run along the positions of one output channel, channels are shared out over the waves
-        for (int n = threadIdx.x >> 6; n < NG; n += 4)
-        for (int t = threadIdx.x & 63; t < span; t += 64) {
-            const size_t o = obase + (size_t)n * L + t;
-            const int p = pos[o];
+        auto scatter = [&](int p, float gv, int t) {
             const int k = p & 0x7fffffff;
             const int c = by_khw.div(k), r = k - c * khw;
             const int i = by_kw.div(r), j = r - i * q.KW;
             const int th = by_wo.div(t);
             const int h = h_lo + th, w = t - th * q.WO;
             const int y = h * q.S + i * q.D - q.P - y0, x = w * q.S + j * q.D - q.P;
-            if ((unsigned)y < (unsigned)rows && (unsigned)x < (unsigned)q.W && c < CG) {
-                const float gv = grad_output[o];
+            if ((unsigned)y < (unsigned)rows && (unsigned)x < (unsigned)q.W && c < CG)
                 atomicAdd(&bins[(c * rows + y) * q.W + x], p >= 0 ? gv : -gv);
+        };
+        // lanes run along the positions of one output channel, channels are shared out over the waves
+        if (vec) {
+            // four positions per lane and two such groups in flight: one position per trip, the index first and
+            // the gradient after it, left a wave waiting out two memory latencies per 256 bytes
+            const int quads = span / 4;                   // WO % 4 == 0
+            for (int n = threadIdx.x >> 6; n < NG; n += 4) {
+                const int4* pq = reinterpret_cast<const int4*>(pos + obase + (size_t)n * L);
+                const float4* gq = reinterpret_cast<const float4*>(grad_output + obase + (size_t)n * L);
+                for (int t4 = threadIdx.x & 63; t4 < quads; t4 += 128) {
+                    const bool second = t4 + 64 < quads;
+                    const int4 p0 = pq[t4], p1 = pq[second ? t4 + 64 : t4];
+                    const float4 g0 = gq[t4], g1 = gq[second ? t4 + 64 : t4];
+                    scatter(p0.x, g0.x, 4 * t4); scatter(p0.y, g0.y, 4 * t4 + 1);
+                    scatter(p0.z, g0.z, 4 * t4 + 2); scatter(p0.w, g0.w, 4 * t4 + 3);
+                    if (second) {
+                        const int u = 4 * (t4 + 64);
+                        scatter(p1.x, g1.x, u); scatter(p1.y, g1.y, u + 1);
+                        scatter(p1.z, g1.z, u + 2); scatter(p1.w, g1.w, u + 3);
+                    }
+                }
             }
+        } else {
+            for (int n = threadIdx.x >> 6; n < NG; n += 4)
+                for (int t = threadIdx.x & 63; t < span; t += 64) {
+                    const size_t o = obase + (size_t)n * L + t;
+                    scatter(pos[o], grad_output[o], t);
+                }
         }
     }
     __syncthreads();
 
     // bins[c][y][x] -> grad_img[b, g*CG + c, y0 + y, x]: rows of one channel are contiguous in memory
     const int per_c = rows * q.W;
-    for (int e = threadIdx.x; e < nb; e += 256) {
-        const int c = e / per_c, rest = e - c * per_c;
-        grad_img[(((size_t)b * q.C + (size_t)g * CG + c) * q.H + y0) * q.W + rest] = bins[e];
+    if (vec_img) {
+        for (int e = threadIdx.x * 4; e < nb; e += 1024) {
+            const int c = e / per_c, rest = e - c * per_c;
+            *reinterpret_cast<float4*>(grad_img + (((size_t)b * q.C + (size_t)g * CG + c) * q.H + y0) * q.W + rest) =
+                *reinterpret_cast<const float4*>(bins + e);
+        }
+    } else {
+        for (int e = threadIdx.x; e < nb; e += 256) {
+            const int c = e / per_c, rest = e - c * per_c;
+            grad_img[(((size_t)b * q.C + (size_t)g * CG + c) * q.H + y0) * q.W + rest] = bins[e];
+        }
     }
 }
 
@@ -214,14 +248,19 @@ hipError_t fold(const float* gcols, float* gimg, const ConvGeom& q, hipStream_t 
 hipError_t inf_backward_input_folded(const float* grad_output, const int32_t* pos, float* grad_img, const ConvGeom& q,
                                      int G, int CO, hipStream_t stream) {
     const int CG = q.C / G, NG = CO / G;
-    // as many image rows per workgroup as 64 KB of bins hold
-    int R = (int)(16384 / ((long long)CG * q.W));
-    if (R < 1) return hipErrorInvalidValue;          // the API layer screens this out
+    // as many image rows per workgroup as 32 KB of bins hold (four workgroups per CU: their zeroing, scanning
+    // and write-out phases overlap); a single row may take up to 64 KB
+    if ((long long)CG * q.W > 16384) return hipErrorInvalidValue;          // the API layer screens this out
+    int R = (int)(8192 / ((long long)CG * q.W));
+    if (R < 1) R = 1;
     if (R > q.H) R = q.H;
     const int row_tiles = (q.H + R - 1) / R;
     const size_t lds = (size_t)CG * R * q.W * sizeof(float);
+    // 128-bit loads of four neighbouring positions: every run of output rows starts on a multiple of four
+    const int vec = q.WO % 4 == 0 && aligned16(grad_output) && aligned16(pos);
+    const int vec_img = q.W % 4 == 0 && aligned16(grad_img);   // the slab of a channel starts and ends on multiples of four
     hipLaunchKernelGGL(inf_backward_input_folded_kernel, dim3((unsigned)(q.B * G * row_tiles)), dim3(256), lds, stream,
-                       grad_output, pos, grad_img, q, G, NG, R, row_tiles, SmallDiv(q.KH * q.KW), SmallDiv(q.KW),
+                       grad_output, pos, grad_img, q, G, NG, R, row_tiles, vec, vec_img, SmallDiv(q.KH * q.KW), SmallDiv(q.KW),
                        SmallDiv(q.WO));
     return hipGetLastError();
 }

@@ -71,6 +71,52 @@ inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* 
         return;
     }
 
+    // conv layout with HW % 4 == 0, tiles of at least four positions and 16-byte aligned tensors: four
+    // neighbouring positions per lane move with 128-bit loads and stores
+    const bool quad = th_log2 >= 2 && (d.HW & 3) == 0 &&
+                      ((reinterpret_cast<uintptr_t>(grad_output) | reinterpret_cast<uintptr_t>(pos) |
+                        reinterpret_cast<uintptr_t>(grad_input)) & 15u) == 0;
+    if (quad) {
+        float4* b4 = reinterpret_cast<float4*>(bins);
+        for (int e = threadIdx.x; e < nb / 4; e += NT) b4[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+        __syncthreads();
+        const int tq_log2 = th_log2 - 2;                 // quads per tile row
+        const int total_q = d.NG << tq_log2;
+        for (int e = threadIdx.x; e < total_q; e += NT) {
+            const int n = e >> tq_log2, j = (e & ((1 << tq_log2) - 1)) * 4;
+            const int hw = hw0 + j;
+            if (hw < d.HW) {                              // HW % 4 == 0: the whole quad is inside
+                const size_t o = obase + (size_t)n * d.HW + hw;
+                const int4 pv = *reinterpret_cast<const int4*>(pos + o);
+                const float4 gv = *reinterpret_cast<const float4*>(grad_output + o);
+                const int ps[4] = {pv.x, pv.y, pv.z, pv.w};
+                const float gs[4] = {gv.x, gv.y, gv.z, gv.w};
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const int idx = (ps[q] & 0x7fffffff) - k0;
+                    if (idx >= 0 && idx < kc) atomicAdd(&bins[(idx << th_log2) + j + q], ps[q] >= 0 ? gs[q] : -gs[q]);
+                }
+            }
+        }
+        __syncthreads();
+        for (int e = threadIdx.x; e < nb / 4; e += NT) {
+            const int k = e >> tq_log2, j = (e & ((1 << tq_log2) - 1)) * 4;
+            const int hw = hw0 + j;
+            if (hw < d.HW) {
+                float4* dst = reinterpret_cast<float4*>(grad_input + xbase + (size_t)k * d.HW + hw);
+                const float4 v = b4[e];
+                if (OVERWRITE) {
+                    *dst = v;
+                } else if (v.x != 0.f || v.y != 0.f || v.z != 0.f || v.w != 0.f) {
+                    float4 o = *dst;
+                    o.x += v.x; o.y += v.y; o.z += v.z; o.w += v.w;
+                    *dst = o;
+                }
+            }
+        }
+        return;
+    }
+
     for (int e = threadIdx.x; e < nb; e += NT) bins[e] = 0.f;
     __syncthreads();
 
@@ -149,16 +195,33 @@ inf_backward_weight_kernel(const float* __restrict__ grad_output, const int32_t*
             }
         }
     } else {
+        auto add = [&](int p, float gv, int nn) {
+            const int idx = (p & 0x7fffffff) - k0;
+            if (idx >= 0 && idx < kc) atomicAdd(&bins[nn * kc + idx], p < 0 ? gv : -gv);
+        };
+        // HW % 4 == 0 and aligned tensors: four positions per lane with 128-bit loads and two such groups in
+        // flight (one position per trip, the index first and the gradient after it, left a wave waiting out two
+        // memory latencies per 256 bytes)
+        const bool vec_in = (d.HW & 3) == 0 && ((reinterpret_cast<uintptr_t>(grad_output) | reinterpret_cast<uintptr_t>(pos)) & 15u) == 0;
         for (int b = b0; b < b1; b++) {
             const size_t base = (size_t)b * img_stride + first;
-            for (int e = threadIdx.x; e < run; e += 256) {
-                const int nn = e / d.HW;
-                const int p = pos[base + e];
-                const int idx = (p & 0x7fffffff) - k0;
-                if (idx >= 0 && idx < kc) {
-                    const float gv = grad_output[base + e];
-                    atomicAdd(&bins[nn * kc + idx], p < 0 ? gv : -gv);
+            if (vec_in) {
+                const int4* pq = reinterpret_cast<const int4*>(pos + base);
+                const float4* gq = reinterpret_cast<const float4*>(grad_output + base);
+                const int quads = run / 4, hwq = d.HW / 4;
+                for (int q0 = threadIdx.x; q0 < quads; q0 += 512) {
+                    const int q1 = q0 + 256 < quads ? q0 + 256 : q0;
+                    const int4 pa = pq[q0], pb = pq[q1];
+                    const float4 ga = gq[q0], gb = gq[q1];
+                    const int na = q0 / hwq;
+                    add(pa.x, ga.x, na); add(pa.y, ga.y, na); add(pa.z, ga.z, na); add(pa.w, ga.w, na);
+                    if (q1 != q0) {
+                        const int nb_ = q1 / hwq;
+                        add(pb.x, gb.x, nb_); add(pb.y, gb.y, nb_); add(pb.z, gb.z, nb_); add(pb.w, gb.w, nb_);
+                    }
                 }
+            } else {
+                for (int e = threadIdx.x; e < run; e += 256) add(pos[base + e], grad_output[base + e], e / d.HW);
             }
         }
     }
