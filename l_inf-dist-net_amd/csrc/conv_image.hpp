@@ -36,6 +36,7 @@ constexpr size_t kLdsLimit = 160 * 1024;
 inline bool plan(const ConvGeom& q, int G, int CO, ConvFwd& a, int nx = 1) {
     if (q.KH != 3 || q.KW != 3 || q.D != 1 || (q.S != 1 && q.S != 2)) return false;
     if (q.WO % kTM != 0 || G <= 0 || q.C % G != 0 || CO % G != 0) return false;
+    if ((long long)kCC * q.H * q.W >= (1LL << 28)) return false;   // staged loads pack the channel above 28 offset bits
     const int S = q.S, NXR = (7 * S + 2) / 4 + 1;
     a.B = q.B; a.G = G; a.CG = q.C / G; a.NG = CO / G; a.K = a.CG * 9;
     a.H = q.H; a.W = q.W; a.HO = q.HO; a.WO = q.WO; a.P = q.P;

@@ -18,7 +18,7 @@ struct NbDims {
     int B, G, K, NG, HW, M;
 };
 
-constexpr int BKO = 64, RB = 32, LDP = 65;  // tile width, stage depth, padded LDS row
+constexpr int RB = 32;  // stage depth (rows of the reduction per LDS panel)
 
 // WEIGHT = false: grad_input.  WEIGHT = true: grad_weight.
 template <bool WEIGHT, bool CONV>
@@ -40,15 +40,18 @@ struct Views {
 };
 
 // BA = rows of P per workgroup (64, or 32 when 64 would leave the device short of
-// workgroups); a lane owns BA/16 rows x 4 columns.
-template <bool WEIGHT, bool CONV, bool SPLIT, int BA>
+// workgroups), BKO = its columns (64, or 128 when P has so few rows that a 32-row tile is all there
+// is: the wider tile restores sixteen terms per lane and step); a lane owns BA/16 rows x BKO/16 columns.
+template <bool WEIGHT, bool CONV, bool SPLIT, int BA, int BKO>
 __global__ void __launch_bounds__(256)
 norm_backward_kernel(const float* __restrict__ grad_output, const float* __restrict__ input,
                      const float* __restrict__ weight, const float* __restrict__ output, float* __restrict__ grad,
                      float p, NbDims d, int tiles_a, int tiles_k, int r_per_wg) {
+    constexpr int LDP = BKO + 1, LDA = BA + 1;   // padded LDS rows
+    constexpr int CK = BKO / 16;                 // columns per lane
     __shared__ float Os[RB * LDP];  // O[r][k]
-    __shared__ float Cs[RB * LDP];  // c[r][a]     = grad_output
-    __shared__ float Rs[RB * LDP];  // rinv[r][a]  = 1 / output
+    __shared__ float Cs[RB * LDA];  // c[r][a]     = grad_output
+    __shared__ float Rs[RB * LDA];  // rinv[r][a]  = 1 / output
     const int tid = threadIdx.x;
     const int ta = blockIdx.x % tiles_a;
     const int rest = blockIdx.x / tiles_a;
@@ -61,16 +64,16 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
     const int r_begin = blockIdx.y * r_per_wg;
     const int r_end = min(R, r_begin + r_per_wg);
     constexpr int PA = BA / 16;              // rows per lane
-    const int tx = tid & 15, ty = tid >> 4;  // lane's patch: rows a0 + ty*PA.., columns k0 + tx*4..
+    const int tx = tid & 15, ty = tid >> 4;  // lane's patch: rows a0 + ty*PA.., columns k0 + tx, k0 + tx + 16, ...
     const float e = p - 1.0f;
     const int ie = small_int_power(e);
 
-    float q[PA][4], acc[PA][4];
+    float q[PA][CK], acc[PA][CK];
 #pragma unroll
     for (int i = 0; i < PA; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int a = a0 + ty * PA + i, k = k0 + tx * 4 + j;
+        for (int j = 0; j < CK; j++) {
+            const int a = a0 + ty * PA + i, k = k0 + tx + 16 * j;
             acc[i][j] = 0.f;
             q[i][j] = (a < A && k < d.K) ? (WEIGHT ? weight[v.w_at(a, k)] : input[v.x_at(a, k)]) : 0.f;
         }
@@ -105,8 +108,8 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
                     c = grad_output[o];
                     ri = __builtin_amdgcn_rcpf(output[o]);
                 }
-                Cs[rr * LDP + cc] = c;
-                Rs[rr * LDP + cc] = ri;
+                Cs[rr * LDA + cc] = c;
+                Rs[rr * LDA + cc] = ri;
             }
         }
         __syncthreads();
@@ -115,15 +118,15 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
         auto reduce = [&](auto spower) {
 #pragma unroll 2
             for (int rr = 0; rr < RB; rr++) {
-                float o[4], c[PA], ri[PA];
+                float o[CK], c[PA], ri[PA];
 #pragma unroll
-                for (int j = 0; j < 4; j++) o[j] = Os[rr * LDP + tx * 4 + j];
+                for (int j = 0; j < CK; j++) o[j] = Os[rr * LDP + tx + 16 * j];   // neighbouring lanes, neighbouring banks
 #pragma unroll
-                for (int i = 0; i < PA; i++) { c[i] = Cs[rr * LDP + ty * PA + i]; ri[i] = Rs[rr * LDP + ty * PA + i]; }
+                for (int i = 0; i < PA; i++) { c[i] = Cs[rr * LDA + ty * PA + i]; ri[i] = Rs[rr * LDA + ty * PA + i]; }
 #pragma unroll
                 for (int i = 0; i < PA; i++)
 #pragma unroll
-                    for (int j = 0; j < 4; j++) acc[i][j] += c[i] * spower((q[i][j] - o[j]) * ri[i]);
+                    for (int j = 0; j < CK; j++) acc[i][j] += c[i] * spower((q[i][j] - o[j]) * ri[i]);
             }
         };
         switch (ie) {
@@ -140,8 +143,8 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
 #pragma unroll
     for (int i = 0; i < PA; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int a = a0 + ty * PA + i, k = k0 + tx * 4 + j;
+        for (int j = 0; j < CK; j++) {
+            const int a = a0 + ty * PA + i, k = k0 + tx + 16 * j;
             if (a < A && k < d.K) {
                 if (WEIGHT) {
                     float* dst = grad + v.w_at(a, k);
@@ -154,7 +157,7 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
         }
 }
 
-template <bool WEIGHT, int BA>
+template <bool WEIGHT, int BA, int BKO>
 static hipError_t launch_norm_backward_ba(const float* grad_output, const float* input, const float* weight,
                                           const float* output, float* grad, float p, const Problem& pr,
                                           hipStream_t stream) {
@@ -175,7 +178,7 @@ static hipError_t launch_norm_backward_ba(const float* grad_output, const float*
     const dim3 grid((unsigned)tiles, (unsigned)splits);
     const bool conv = pr.HW != 1;
 #define LDIST_LAUNCH(W, C, S)                                                                                      \
-    hipLaunchKernelGGL((norm_backward_kernel<W, C, S, BA>), grid, dim3(256), 0, stream, grad_output, input, weight,    \
+    hipLaunchKernelGGL((norm_backward_kernel<W, C, S, BA, BKO>), grid, dim3(256), 0, stream, grad_output, input, weight,    \
                        output, grad, p, d, tiles_a, tiles_k, r_per_wg)
     if (WEIGHT) {
         if (splits > 1) { if (conv) LDIST_LAUNCH(WEIGHT, true, true); else LDIST_LAUNCH(WEIGHT, false, true); }
@@ -191,12 +194,15 @@ template <bool WEIGHT>
 static hipError_t launch_norm_backward(const float* grad_output, const float* input, const float* weight,
                                        const float* output, float* grad, float p, const Problem& pr,
                                        hipStream_t stream) {
-    // 64-row tiles unless they would give fewer than four workgroups per CU (and the rows allow halving)
+    // 64-row tiles unless they would give fewer than four workgroups per CU (and the rows allow halving);
+    // P with at most 32 rows (grad_weight of a grouped layer with few outputs per group): 32 x 128 tiles
     const int A = WEIGHT ? pr.NG : pr.B * pr.HW;
-    const long tiles64 = (long)((A + 63) / 64) * ((pr.K + BKO - 1) / BKO) * pr.G;
+    if (A <= 32 && pr.K > 64)
+        return launch_norm_backward_ba<WEIGHT, 32, 128>(grad_output, input, weight, output, grad, p, pr, stream);
+    const long tiles64 = (long)((A + 63) / 64) * ((pr.K + 63) / 64) * pr.G;
     if (tiles64 < 4L * pr.num_cu && A > 32)
-        return launch_norm_backward_ba<WEIGHT, 32>(grad_output, input, weight, output, grad, p, pr, stream);
-    return launch_norm_backward_ba<WEIGHT, 64>(grad_output, input, weight, output, grad, p, pr, stream);
+        return launch_norm_backward_ba<WEIGHT, 32, 64>(grad_output, input, weight, output, grad, p, pr, stream);
+    return launch_norm_backward_ba<WEIGHT, 64, 64>(grad_output, input, weight, output, grad, p, pr, stream);
 }
 
 hipError_t norm_backward_input(const float* grad_output, const float* input, const float* weight,
