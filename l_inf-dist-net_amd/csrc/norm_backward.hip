@@ -83,8 +83,20 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
     // along m (= hw) otherwise.  Lanes follow the contiguous axis of each panel.
     constexpr bool O_K_CONTIG = !(WEIGHT && CONV);         // O = w, or x in the fc layout
     constexpr bool C_A_CONTIG = WEIGHT ? !CONV : CONV;     // is `a` the contiguous axis of out/grad_output
+    // grad_weight in the conv layout: every panel element this lane loads belongs to row m = r0 + (tid & 31)
+    // of the reduction, so its image b and position hw are kept up to date from stage to stage instead of
+    // being divided out per element
+    constexpr bool ROW_PER_LANE = WEIGHT && CONV;
+    int mb = 0, mhw = 0;
+    if constexpr (ROW_PER_LANE) {
+        const int m = r_begin + (tid & (RB - 1));
+        mb = m / d.HW;
+        mhw = m - mb * d.HW;
+    }
     for (int r0 = r_begin; r0 < r_end; r0 += RB) {
         __syncthreads();
+        const size_t xrow = ((size_t)(mb * d.G + g) * d.K) * d.HW + mhw;    // ROW_PER_LANE: x[m][0]
+        const size_t orow = ((size_t)(mb * d.G + g) * d.NG) * d.HW + mhw;   // ROW_PER_LANE: out[m][0]
 #pragma unroll
         for (int it = 0; it < RB * BKO / 256; it++) {
             const int id = tid + it * 256;
@@ -92,7 +104,8 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
             const int cc = O_K_CONTIG ? id % BKO : id / RB;
             const int r = r0 + rr, k = k0 + cc;
             float val = 0.f;
-            if (r < r_end && k < d.K) val = WEIGHT ? input[v.x_at(r, k)] : weight[v.w_at(r, k)];
+            if (r < r_end && k < d.K)
+                val = ROW_PER_LANE ? input[xrow + (size_t)k * d.HW] : (WEIGHT ? input[v.x_at(r, k)] : weight[v.w_at(r, k)]);
             Os[rr * LDP + cc] = val;
         }
 #pragma unroll
@@ -104,13 +117,17 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
                 const int r = r0 + rr, a = a0 + cc;
                 float c = 0.f, ri = 0.f;
                 if (r < r_end && a < A) {
-                    const size_t o = WEIGHT ? v.o_at(r, a) : v.o_at(a, r);
+                    const size_t o = ROW_PER_LANE ? orow + (size_t)a * d.HW : (WEIGHT ? v.o_at(r, a) : v.o_at(a, r));
                     c = grad_output[o];
                     ri = __builtin_amdgcn_rcpf(output[o]);
                 }
                 Cs[rr * LDA + cc] = c;
                 Rs[rr * LDA + cc] = ri;
             }
+        }
+        if constexpr (ROW_PER_LANE) {
+            mhw += RB;
+            while (mhw >= d.HW) { mhw -= d.HW; mb++; }
         }
         __syncthreads();
         // spower(u) = sign(u) * |u|^(p-1) for the signed, normalised difference u = (Q - O) * rinv.
