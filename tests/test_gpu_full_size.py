@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import oracle
-from helpers import assert_sum_close, gen
+from helpers import SIGN, assert_sum_close, gen
 
 pytestmark = pytest.mark.gpu
 
@@ -134,3 +134,41 @@ def test_config4_unfolded_conv_layer():
     mx, mw = _scatter_magnitudes(go, ep, 1152, 4)
     assert_sum_close(gx.cpu(), oracle.inf_dist_backward_input(go, ep, 1152, 4), mx)
     assert_sum_close(gw.cpu(), oracle.inf_dist_backward_weight(go, ep, 1152, 4), mw)
+
+
+def test_config4_layer_from_the_image():
+    """Config 4 without the unfolded tensor: forward and interval bounds straight from the images, and the input
+    gradient written as an image, against the oracle on torch's columns (values, indices and bounds bit-exact)."""
+    import torch.nn.functional as F
+    from gpu_common import DEV, cpp, say
+    say("config 4 from the image: 128 x 128 x 32 x 32, 128 outputs, 4 groups")
+    g = gen(8)
+    img = torch.rand(128, 128, 32, 32, generator=g)
+    w = (torch.randn(128, 288, generator=g) / math.sqrt(288)).contiguous()
+    cols = F.unfold(img, 3, padding=1).contiguous()
+    eo, ep = oracle.inf_dist_forward(cols, w, 4)
+    out = torch.empty(128, 128, 1024, device=DEV)
+    pos = torch.empty(128, 128, 1024, device=DEV, dtype=torch.int32)
+    assert cpp.inf_dist_conv_forward_supported(128, 32, 32, 128, 4, 3, 1, 1, 1)
+    cpp.inf_dist_conv_forward(img.to(DEV), w.to(DEV), out, pos, 4, 3, 1, 1, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu(), eo) and torch.equal(pos.cpu(), ep)
+
+    eps = 8.0 / 255
+    lo_i, up_i = (img - eps).clamp(0, 1), (img + eps).clamp(0, 1)
+    el, eu = oracle.inf_dist_bound_forward(F.unfold(lo_i, 3, padding=1).contiguous(),
+                                           F.unfold(up_i, 3, padding=1).contiguous(), w, 4)
+    ol, ou = torch.empty_like(out), torch.empty_like(out)
+    cpp.inf_dist_bound_conv_forward(lo_i.to(DEV), up_i.to(DEV), w.to(DEV), ol, ou, 4, 3, 1, 1, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(ol.cpu(), el) and torch.equal(ou.cpu(), eu)
+    assert bool((el <= eo).all()) and bool((eo <= eu).all())     # the value lies inside its own bounds
+
+    go = torch.randn(128, 128, 1024, generator=g)
+    gimg = torch.empty(128, 128, 32, 32, device=DEV)
+    cpp.inf_dist_backward_input_folded(go.to(DEV), pos, gimg, 4, 3, 1, 1, 1)
+    torch.cuda.synchronize()
+    gcols = oracle.inf_dist_backward_input(go, ep, 1152, 4)
+    expect = F.fold(gcols.double(), (32, 32), 3, padding=1)
+    terms = F.fold(oracle.inf_dist_backward_input(go.abs(), ep & ~SIGN, 1152, 4).double(), (32, 32), 3, padding=1).abs()
+    assert_sum_close(gimg.cpu(), expect, terms)
