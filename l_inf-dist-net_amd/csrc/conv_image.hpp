@@ -59,7 +59,15 @@ inline bool plan(const ConvGeom& q, int G, int CO, ConvFwd& a, int nx = 1) {
         if (g_conv_staging_override == 1 && !resident) continue;
         if (g_conv_staging_override == 2 && resident) continue;
         if (!resident && nx == 1 && a.CG % kCC != 0) continue;
-        for (int tiles_n = (quads + 15) / 16; tiles_n <= quads; tiles_n++) {
+        // Candidates: the fewest output tiles that fit and up to three more (a narrower workgroup may take more
+        // rows, or rows that divide the image evenly); each further tile re-reads the image rows once more,
+        // priced at 3 %.  Past those, more tiles are only tried until something fits at all.
+        const int first_tiles = (quads + 15) / 16;
+        bool have = false;
+        double haveScore = -1.0;
+        ConvFwd pick = a;
+        for (int tiles_n = first_tiles; tiles_n <= quads; tiles_n++) {
+            if (have && tiles_n > first_tiles + 3) break;
             const int NL = (quads + tiles_n - 1) / tiles_n;
             if (a.SEG * NL > kMaxThreads) continue;
             const int BN = NL * kTN;
@@ -99,11 +107,20 @@ inline bool plan(const ConvGeom& q, int G, int CO, ConvFwd& a, int nx = 1) {
             // below six resident waves per CU this variant does badly: try the other, or leave the layer to
             // the column kernels
             if (bestR == 0 || (bestScore < 384.0 && forced <= 0)) continue;
-            a.NL = NL; a.BN = BN; a.tiles_n = (quads + NL - 1) / NL;
-            a.R = bestR; a.NR = (bestR - 1) * S + 3; a.ML = bestR * a.SEG;
-            a.tiles_h = (q.HO + bestR - 1) / bestR;
-            a.resident = resident ? 1 : 0;
-            a.xwords = bestWords;
+            const int real_tiles = (quads + NL - 1) / NL;
+            const double priced = bestScore * (1.0 - 0.03 * (real_tiles - first_tiles));
+            if (have && priced <= haveScore) continue;
+            have = true;
+            haveScore = priced;
+            pick = a;
+            pick.NL = NL; pick.BN = BN; pick.tiles_n = real_tiles;
+            pick.R = bestR; pick.NR = (bestR - 1) * S + 3; pick.ML = bestR * a.SEG;
+            pick.tiles_h = (q.HO + bestR - 1) / bestR;
+            pick.resident = resident ? 1 : 0;
+            pick.xwords = bestWords;
+        }
+        if (have) {
+            a = pick;
             return (long long)q.B * G * a.tiles_h * a.tiles_n < (1LL << 31);
         }
     }
