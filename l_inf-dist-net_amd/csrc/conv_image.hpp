@@ -26,11 +26,16 @@ struct ConvFwd {
     int vec_in, vec_out;         // 128-bit global loads of image rows / stores of results allowed
     int resident;                // 1: all channels of the image rows stay in LDS; 0: staged kCC channels at a time
     int xwords;                  // floats of the image area in LDS
+    int cstride;                 // resident: floats between channels (NR*WP padded to 4 mod 8); staged: unused
 };
 
 constexpr size_t kLdsLimit = 160 * 1024;
 
 // Fills the launch shape; false when this kernel does not cover the geometry.
+// Channel stride of the resident image area: rows stay 16-byte aligned (a multiple of 4) and consecutive
+// channels start 4 banks apart modulo 8, so that channel c begins at bank 4c mod 64.
+inline int channel_stride(int plane) { return plane % 8 == 4 ? plane : plane + (4 - plane % 8 + 8) % 8; }
+
 // nx: images staged side by side (1: the input; 2: lower and upper interval ends, which are always staged and may
 // have any number of channels: that kernel masks the channels a last stage does not have).
 inline bool plan(const ConvGeom& q, int G, int CO, ConvFwd& a, int nx = 1) {
@@ -85,7 +90,7 @@ inline bool plan(const ConvGeom& q, int G, int CO, ConvFwd& a, int nx = 1) {
                 const int NT = R * a.SEG * NL;
                 int xwords;
                 if (resident) {
-                    xwords = a.CGP * NR * a.WP;
+                    xwords = a.CGP * channel_stride(NR * a.WP);
                 } else {
                     // a lane carries kXRegs image words per stage in registers; what a small workgroup cannot
                     // carry that way it copies directly, which is slow: only taken when forced
@@ -118,6 +123,7 @@ inline bool plan(const ConvGeom& q, int G, int CO, ConvFwd& a, int nx = 1) {
             pick.tiles_h = (q.HO + bestR - 1) / bestR;
             pick.resident = resident ? 1 : 0;
             pick.xwords = bestWords;
+            pick.cstride = channel_stride(pick.NR * a.WP);
         }
         if (have) {
             a = pick;

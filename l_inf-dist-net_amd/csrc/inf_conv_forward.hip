@@ -45,6 +45,9 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
     const int h0 = th * a.R, n0 = tn * a.BN;
     const int y0 = h0 * S - a.P;
     const int NR = a.NR, WP = a.WP, K = a.K;
+    // floats between the channels of the image area: resident, padded so that lanes that look into different
+    // channels (the argmax search) spread over the banks; staged, the channels of a stage are packed
+    const int CST = RESIDENT ? a.cstride : NR * WP;
     constexpr int BNP = kBNP;
 
     // ---- weights: global -> registers -> LDS stage, k-major ----
@@ -129,7 +132,7 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
 
     // ---- RESIDENT: image rows -> LDS once, padding as zeros ----
     if constexpr (RESIDENT) {
-        const int words = a.CGP * NR * WP;
+        const int words = a.CGP * CST;
         for (int i = tid * 4; i < words; i += NT * 4) *reinterpret_cast<float4*>(tile + i) = make_float4(0.f, 0.f, 0.f, 0.f);
         __syncthreads();
         const int rows = a.CG * NR;
@@ -148,7 +151,7 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
                     const int c = row / NR, r = row - c * NR;
                     const int y = y0 + r;
                     const bool real = i < total && (unsigned)y < (unsigned)a.H;
-                    at[u] = real ? (c * NR + r) * WP + a.P + 4 * xq : -1;
+                    at[u] = real ? c * CST + r * WP + a.P + 4 * xq : -1;
                     v[u] = *reinterpret_cast<const float4*>(src + (real ? ((size_t)c * a.H + y) * a.W + 4 * xq : 0));
                 }
 #pragma unroll
@@ -163,7 +166,7 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
                 const int row = i / a.W, x = i - row * a.W;
                 const int c = row / NR, r = row - c * NR;
                 const int y = y0 + r;
-                if ((unsigned)y < (unsigned)a.H) tile[(c * NR + r) * WP + a.P + x] = src[((size_t)c * a.H + y) * a.W + x];
+                if ((unsigned)y < (unsigned)a.H) tile[c * CST + r * WP + a.P + x] = src[((size_t)c * a.H + y) * a.W + x];
             }
         }
     } else {
@@ -238,7 +241,7 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
                         for (int t = 0; t < kTN; t++)
                             cm[e][t] = __builtin_fmaxf(cm[e][t], __builtin_fabsf(cur.x[e * S + j] - cur.w[j][t]));
             }
-            xrow += kTrack * NR * WP;
+            xrow += kTrack * CST;
             wrow += 9 * kTrack * BNP;
             const int un = ch * (kCC / kTrack) + u;
 #pragma unroll
@@ -247,7 +250,7 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
                 for (int t = 0; t < kTN; t++)
                     if (cm[e][t] > acc[e][t]) { acc[e][t] = cm[e][t]; unit[e][t] = un; }
         }
-        xch += kCC * NR * WP;
+        xch += kCC * CST;
         if (ch + 1 < nstage) {
             wstore(wst + ((ch + 1) & 1) * kKC * BNP);
             wrest(ch + 1, wst + ((ch + 1) & 1) * kKC * BNP);
@@ -292,7 +295,7 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
             for (int eb = 0; eb < EB; eb++) {
                 const int e = e0 + eb;
                 if constexpr (RESIDENT) {
-                    const float* xe = xlane + e * S + unit[e][t] * NR * WP;
+                    const float* xe = xlane + e * S + unit[e][t] * CST;
 #pragma unroll
                     for (int r = 0; r < 9; r++) xq[eb][r] = xe[(r / 3) * WP + r % 3];
                 } else {
