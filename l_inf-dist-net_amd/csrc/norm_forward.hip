@@ -42,7 +42,7 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
     const int tid = threadIdx.x;
     const int grp = tid / NGRP, t = tid % NGRP;
     const int tx = t % GEO::TX, ty = t / GEO::TX;
-    auto power = [p](float v) {
+    auto power = [&](float v) {   // by reference: the integer-exponent instantiations do not use p
         if constexpr (IP > 0) return pow_int<IP>(v);
         else return pow_pos(v, p);
     };
