@@ -169,8 +169,10 @@ LDIST_API int ldist_unfold(const float* img, int B, int C, int H, int W, int KH,
  * what ldist_unfold followed by ldist_inf_dist_forward computes (the reference: F.unfold at
  * model/norm_dist.py:132, then inf_dist_forward_cuda), bit for bit, reading the image once.
  *   img (B, C, H, W), weight (CO, C/G*KH*KW), output and pos (B, CO, HO*WO).
- * Covers 3x3 windows with dilation 1, stride 1 or 2 and WO % 8 == 0, where a group's channels are few
- * enough for their image rows to stay in LDS or a multiple of four (then they are staged);
+ * Covers 3x3 windows with dilation 1 and stride 1 or 2 (lanes take eight neighbouring positions of a row:
+ * output widths that are multiples of 8 waste none), where a group's channels are few enough for their
+ * image rows to stay in LDS or a multiple of four (then they are staged), and where the layer is large
+ * enough to keep a CU busy;
  * ldist_inf_dist_conv_forward_supported returns 1 for such a geometry, 0 otherwise, and
  * ldist_inf_dist_conv_forward returns LDIST_EUNSUPPORTED for the rest (nothing is enqueued). */
 LDIST_API int ldist_inf_dist_conv_forward_supported(int C, int H, int W, int CO, int G, int KH, int KW, int stride, int padding,
@@ -182,7 +184,7 @@ LDIST_API int ldist_inf_dist_conv_forward(const float* img, const float* weight,
  * ldist_unfold of both followed by ldist_inf_dist_bound_forward computes (the reference: F.unfold at
  * model/norm_dist.py:144-145, then inf_dist_bound_forward_cuda), bit for bit, irregular boxes included.
  *   lower_img, upper_img (B, C, H, W), weight (CO, C/G*KH*KW), output_lower and output_upper (B, CO, HO*WO).
- * Covers 3x3 windows with dilation 1, stride 1 or 2 and WO % 8 == 0, any number of channels;
+ * Covers 3x3 windows with dilation 1 and stride 1 or 2, any number of channels;
  * ldist_inf_dist_bound_conv_forward_supported returns 1 for such a geometry, 0 otherwise, and
  * ldist_inf_dist_bound_conv_forward returns LDIST_EUNSUPPORTED for the rest (nothing is enqueued). */
 LDIST_API int ldist_inf_dist_bound_conv_forward_supported(int C, int H, int W, int CO, int G, int KH, int KW, int stride,

@@ -268,7 +268,8 @@ bound_conv_forward_kernel(const float* __restrict__ lower, const float* __restri
             *reinterpret_cast<float4*>(out_upper + at + 4) = make_float4(up[4][t], up[5][t], up[6][t], up[7][t]);
         } else {
 #pragma unroll
-            for (int e = 0; e < kTM; e++) { out_lower[at + e] = lo[e][t]; out_upper[at + e] = up[e][t]; }
+            for (int e = 0; e < kTM; e++)
+                if (w0 + e < a.WO) { out_lower[at + e] = lo[e][t]; out_upper[at + e] = up[e][t]; }
         }
     }
 }
@@ -285,7 +286,7 @@ hipError_t bound_conv_forward(const float* lower, const float* upper, const floa
     ConvFwd a{};
     if (!plan(q, G, CO, a, 2)) return hipErrorInvalidValue;   // the API layer asks bound_conv_forward_supported first
     a.vec_in = 0;
-    a.vec_out = aligned16(out_lower) && aligned16(out_upper);  // WO % 8 == 0 keeps every run of 8 positions aligned
+    a.vec_out = q.WO % kTM == 0 && aligned16(out_lower) && aligned16(out_upper);   // every run of 8 positions whole and aligned
     const size_t lds = (2 * (size_t)a.xwords + 2 * (size_t)kKC * kBNP) * sizeof(float);
     // The dynamic-LDS limit is raised to what the largest launch so far needed, not to the whole 160 KB: the
     // workgroup-wide vote keeps a little static LDS of its own, and the two must fit together.

@@ -40,15 +40,15 @@ inline int channel_stride(int plane) { return plane % 8 == 4 ? plane : plane + (
 // have any number of channels: that kernel masks the channels a last stage does not have).
 inline bool plan(const ConvGeom& q, int G, int CO, ConvFwd& a, int nx = 1) {
     if (q.KH != 3 || q.KW != 3 || q.D != 1 || (q.S != 1 && q.S != 2)) return false;
-    if (q.WO % kTM != 0 || G <= 0 || q.C % G != 0 || CO % G != 0) return false;
+    if (G <= 0 || q.C % G != 0 || CO % G != 0) return false;
     if ((long long)kCC * q.H * q.W >= (1LL << 28)) return false;   // staged loads pack the channel above 28 offset bits
     const int S = q.S, NXR = (7 * S + 2) / 4 + 1;
     a.B = q.B; a.G = G; a.CG = q.C / G; a.NG = CO / G; a.K = a.CG * 9;
     a.H = q.H; a.W = q.W; a.HO = q.HO; a.WO = q.WO; a.P = q.P;
     a.CGP = (a.CG + kCC - 1) / kCC * kCC;
-    a.SEG = q.WO / kTM;
-    // the last lane of a row reads NXR*4 words from column (WO-8)*S; the image with its padding is W + 2P wide
-    int wp = (q.WO - kTM) * S + NXR * 4;
+    a.SEG = (q.WO + kTM - 1) / kTM;                  // a last segment may reach past the row: those positions are not stored
+    // the last lane of a row reads NXR*4 words from column (SEG-1)*8*S; the image with its padding is W + 2P wide
+    int wp = (a.SEG - 1) * kTM * S + NXR * 4;
     if (q.W + 2 * q.P > wp) wp = q.W + 2 * q.P;
     a.WP = (wp + 3) / 4 * 4;
     if (a.WP % 32 == 0) a.WP += 4;                     // rows of one lane's window in different banks

@@ -333,7 +333,8 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
             *reinterpret_cast<int4*>(pos + at + 4) = make_int4(ps[4], ps[5], ps[6], ps[7]);
         } else {
 #pragma unroll
-            for (int e = 0; e < kTM; e++) { out[at + e] = acc[e][t]; pos[at + e] = ps[e]; }
+            for (int e = 0; e < kTM; e++)
+                if (w0 + e < a.WO) { out[at + e] = acc[e][t]; pos[at + e] = ps[e]; }
         }
     }
 }
@@ -350,7 +351,7 @@ hipError_t inf_conv_forward(const float* img, const float* weight, float* out, i
     ConvFwd a{};
     if (!plan(q, G, CO, a)) return hipErrorInvalidValue;   // the API layer asks inf_conv_forward_supported first
     a.vec_in = q.W % 4 == 0 && aligned16(img);
-    a.vec_out = aligned16(out) && aligned16(pos);           // WO % 8 == 0 keeps every run of 8 positions aligned
+    a.vec_out = q.WO % kTM == 0 && aligned16(out) && aligned16(pos);   // every run of 8 positions whole and aligned
     const size_t lds = ((size_t)a.xwords + 2 * (size_t)kKC * kBNP) * sizeof(float);
     static bool raised[64][4] = {};
     const int ki = (q.S - 1) * 2 + a.resident;

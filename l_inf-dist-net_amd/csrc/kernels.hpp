@@ -90,7 +90,7 @@ struct ConvGeom {
 };
 hipError_t unfold(const float* img, float* cols, const ConvGeom& q, hipStream_t stream);
 hipError_t fold(const float* gcols, float* gimg, const ConvGeom& q, hipStream_t stream);
-// L_inf forward straight from the image (3x3 window, dilation 1, stride 1 or 2, WO % 8 == 0; a group's channels
+// L_inf forward straight from the image (3x3 window, dilation 1, stride 1 or 2; a group's channels
 // either few enough to stay in LDS or a multiple of four); inf_conv_forward_supported tells whether a geometry is covered.
 extern int g_conv_rows_override;
 extern int g_conv_staging_override;

@@ -256,8 +256,9 @@ def inf_dist_backward_input_folded(grad_output, pos, grad_img, G, kernel_size, s
 
 
 def inf_dist_conv_forward_supported(C, H, W, CO, G, kernel_size, stride=1, padding=0, dilation=1):
-    """True when inf_dist_conv_forward covers the geometry (3x3, dilation 1, stride 1 or 2, output width a
-    multiple of 8, a group's image rows fitting LDS); otherwise unfold + inf_dist_forward is the way."""
+    """True when inf_dist_conv_forward covers the geometry (3x3, dilation 1, stride 1 or 2; a group's channels
+    few enough to stay in LDS or a multiple of four; a layer large enough to fill the GPU); otherwise unfold +
+    inf_dist_forward is the way."""
     k = int(kernel_size)
     return bool(_lib.lib().ldist_inf_dist_conv_forward_supported(int(C), int(H), int(W), int(CO), int(G), k, k,
                                                                   int(stride), int(padding), int(dilation)))
@@ -280,8 +281,8 @@ def inf_dist_conv_forward(img, weight, output, pos, G, kernel_size, stride=1, pa
 
 
 def inf_dist_bound_conv_forward_supported(C, H, W, CO, G, kernel_size, stride=1, padding=0, dilation=1):
-    """True when inf_dist_bound_conv_forward covers the geometry (3x3, dilation 1, stride 1 or 2, output width a
-    multiple of 8); otherwise unfold both images and call inf_dist_bound_forward."""
+    """True when inf_dist_bound_conv_forward covers the geometry (3x3, dilation 1, stride 1 or 2, a layer large
+    enough to fill the GPU); otherwise unfold both images and call inf_dist_bound_forward."""
     k = int(kernel_size)
     return bool(_lib.lib().ldist_inf_dist_bound_conv_forward_supported(int(C), int(H), int(W), int(CO), int(G), k, k,
                                                                         int(stride), int(padding), int(dilation)))

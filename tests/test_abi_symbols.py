@@ -72,17 +72,17 @@ def test_conv_forward_geometry_query_needs_no_device(lib):
     assert ok(96, 32, 32, 96, 1, 3, 3, 1, 1, 1) == 1        # 96 channels in one group: staged four at a time
     assert ok(96, 32, 32, 192, 1, 3, 3, 2, 1, 1) == 1       # the CIFAR conv net's stride-2 layer
     assert ok(90, 32, 32, 96, 1, 3, 3, 1, 1, 1) == 0        # too many channels to stay in LDS, and not a multiple of four
-    assert ok(4, 28, 28, 8, 1, 3, 3, 1, 1, 1) == 0          # output width not a multiple of 8
+    assert ok(16, 28, 28, 32, 1, 3, 3, 1, 1, 1) == 1        # output width 28: the last segment of a row is partly idle
     assert ok(4, 16, 16, 8, 1, 5, 5, 1, 2, 1) == 0          # window
     assert ok(4, 16, 16, 8, 1, 3, 3, 1, 2, 2) == 0          # dilation
     assert ok(4, 16, 16, 8, 3, 3, 3, 1, 1, 1) == 0          # channels do not divide into the groups
     one = ctypes.c_void_p(16)
-    assert lib.ldist_inf_dist_conv_forward(one, one, 1, 4, 28, 28, 8, 1, 3, 3, 1, 1, 1, one, one, None) == -5
+    assert lib.ldist_inf_dist_conv_forward(one, one, 1, 4, 28, 28, 8, 1, 5, 5, 1, 2, 1, one, one, None) == -5
     assert lib.ldist_inf_dist_conv_forward(None, one, 1, 4, 32, 32, 8, 1, 3, 3, 1, 1, 1, one, one, None) == -1
     okb = lib.ldist_inf_dist_bound_conv_forward_supported
     assert okb(128, 32, 32, 128, 4, 3, 3, 1, 1, 1) == 1 and okb(90, 32, 32, 96, 1, 3, 3, 1, 1, 1) == 1   # any channel count
-    assert okb(4, 28, 28, 8, 1, 3, 3, 1, 1, 1) == 0 and okb(4, 16, 16, 8, 1, 5, 5, 1, 2, 1) == 0
-    assert lib.ldist_inf_dist_bound_conv_forward(one, one, one, 1, 4, 28, 28, 8, 1, 3, 3, 1, 1, 1, one, one, None) == -5
+    assert okb(16, 28, 28, 32, 1, 3, 3, 1, 1, 1) == 1 and okb(4, 16, 16, 8, 1, 5, 5, 1, 2, 1) == 0
+    assert lib.ldist_inf_dist_bound_conv_forward(one, one, one, 1, 4, 28, 28, 8, 1, 5, 5, 1, 2, 1, one, one, None) == -5
     assert lib.ldist_inf_dist_bound_conv_forward(one, None, one, 1, 4, 32, 32, 8, 1, 3, 3, 1, 1, 1, one, one, None) == -1
     assert lib.ldist_set_conv_rows_override(-1) == -1 and lib.ldist_set_conv_rows_override(0) == 0
     assert lib.ldist_set_conv_staging_override(4) == -1 and lib.ldist_set_conv_staging_override(0) == 0

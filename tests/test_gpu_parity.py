@@ -383,6 +383,9 @@ IMPLICIT_CASES = [  # B, C, H, W, CO, G, stride, padding
     (2, 4, 6, 6, 8, 1, 1, 2),        # padding wider than the window needs
     (1, 8, 8, 64, 40, 1, 1, 1),      # wide rows: eight segments
     (2, 72, 16, 16, 72, 1, 1, 1),    # many channels in one group
+    (2, 16, 28, 28, 32, 1, 1, 1),    # MNIST-sized rows: 28 positions, the fourth segment half idle
+    (2, 8, 13, 13, 16, 2, 1, 0),     # output width 11
+    (2, 8, 21, 21, 12, 1, 2, 1),     # stride 2, output width 11
 ]
 
 
@@ -419,6 +422,7 @@ STAGED_CASES = [  # B, C, H, W, CO, G, stride, padding: channels per group a mul
     (2, 8, 16, 16, 24, 2, 1, 1), (2, 128, 32, 32, 128, 4, 1, 1), (2, 96, 32, 32, 96, 1, 1, 1),
     (2, 96, 32, 32, 192, 1, 2, 1), (1, 192, 16, 16, 192, 1, 1, 1), (2, 8, 17, 17, 12, 1, 2, 0),
     (1, 8, 8, 64, 40, 1, 1, 1), (2, 4, 6, 6, 8, 1, 1, 2), (3, 12, 9, 16, 10, 1, 1, 1),
+    (2, 16, 28, 28, 32, 1, 1, 1), (2, 8, 21, 21, 12, 1, 2, 1),     # output widths 28 and 11: ragged last segment
 ]
 
 
@@ -479,14 +483,13 @@ def test_inf_conv_forward_any_rows_per_workgroup(rows):
 
 def test_inf_conv_forward_refuses_what_it_does_not_cover():
     from gpu_common import DEV, cpp, pkg
-    assert not cpp.inf_dist_conv_forward_supported(4, 28, 28, 8, 1, 3, 1, 1, 1)    # output width 28
     assert not cpp.inf_dist_conv_forward_supported(4, 16, 16, 8, 1, 5, 1, 2, 1)    # 5x5 window
     assert not cpp.inf_dist_conv_forward_supported(4, 16, 16, 8, 1, 3, 1, 2, 2)    # dilation
     img = torch.zeros(1, 4, 28, 28, device=DEV)
-    w = torch.zeros(8, 36, device=DEV)
+    w = torch.zeros(8, 100, device=DEV)
     out = torch.empty(1, 8, 784, device=DEV)
     pos = torch.empty(1, 8, 784, device=DEV, dtype=torch.int32)
-    rc = pkg._lib.lib().ldist_inf_dist_conv_forward(img.data_ptr(), w.data_ptr(), 1, 4, 28, 28, 8, 1, 3, 3, 1, 1, 1,
+    rc = pkg._lib.lib().ldist_inf_dist_conv_forward(img.data_ptr(), w.data_ptr(), 1, 4, 28, 28, 8, 1, 5, 5, 1, 2, 1,
                                                     out.data_ptr(), pos.data_ptr(), None)
     assert rc == -5
 
