@@ -218,6 +218,35 @@ def test_norm_backward(shape, p):
     assert_sum_close(gw.cpu() - 0.125, ew, mw, p, RTOL, ATOL)
 
 
+@pytest.mark.parametrize("p", [2.0, 3.0, 4.0, 8.0])
+@pytest.mark.parametrize("scale", [1e-6, 3e-4, 1.0, 5e3, 1e6, "mixed"])
+def test_norm_backward_at_every_scale(scale, p):
+    """The small integer exponents factor the term as (c * rinv^(p-1)) * (x-w)^(p-1) only while every output of a
+    stage lies within [2^-12, 2^12]; outside (tiny or huge data, or rows of very different magnitude in one stage)
+    the normalised form is used.  Both must meet the tolerance, relative to the magnitude of the summed terms."""
+    from gpu_common import DEV, cpp, say
+    B, CO, CI, G, HW = 70, 96, 130, 1, 1
+    say("norm_backward scale", scale, "p", p)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=23)
+    if scale == "mixed":
+        rows = torch.tensor([1e-5, 1.0, 1e4, 3e-3, 1.0])[torch.arange(B) % 5].view(B, 1, 1)
+        x, w = x * rows, w * 1.0          # some rows tiny, some huge, weights of order one
+    else:
+        x, w = x * scale, w * scale
+    go = torch.randn(B, CO, HW, generator=gen(8))
+    out = oracle.norm_dist_forward(x, w, G, p)
+    ex, mx = oracle.norm_dist_backward_input(go, x, w, out, G, p, with_abs_terms=True)
+    ew, mw = oracle.norm_dist_backward_weight(go, x, w, out, G, p, with_abs_terms=True)
+    gx = torch.full((B, CI, HW), float("nan"), device=DEV)
+    gw = torch.zeros((CO, CI // G), device=DEV)
+    args = (go.to(DEV), x.to(DEV), w.to(DEV), out.to(DEV))
+    cpp.norm_dist_backward_input(*args, gx, G, p)
+    cpp.norm_dist_backward_weight(*args, gw, G, p)
+    torch.cuda.synchronize()
+    assert_sum_close(gx.cpu(), ex, mx, p, RTOL, ATOL)
+    assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
+
+
 @pytest.mark.parametrize("shape", [(512, 5120, 1), (37, 10, 1), (1030, 50, 1), (600, 36, 1), (6, 5, 12), (4, 3, 7),
                                    (16, 8, 1024)])
 def test_mean_shift_kernel(shape):
