@@ -10,6 +10,7 @@ namespace ldist {
 
 constexpr int kMsCols = 32;      // channels per workgroup, L == 1
 constexpr int kMsThreads = 256;
+constexpr int kMsChanThreads = 1024;   // the channel kernel: one workgroup per channel
 
 __device__ __forceinline__ void move_running_mean(float* running_mean, int c, float mean, float momentum) {
     // (1 - momentum) * running + momentum * mean, rounded after each step as two torch ops would
@@ -97,25 +98,45 @@ mean_shift_rows_kernel(const float* __restrict__ x, float* __restrict__ y, float
 }
 
 // L > 1: for a fixed (b, c) the L values are contiguous.  Workgroup = one channel; lanes run along l
-// (128-bit accesses when VEC == 4: L % 4 == 0 and 16-byte aligned bases).
+// (128-bit accesses when VEC == 4: L % 4 == 0 and 16-byte aligned bases).  A channel is one workgroup's work and
+// there are often fewer channels than CUs, so the workgroup is as large as it can be: what limits this kernel is
+// how many loads one CU keeps in flight.
 template <int VEC>
-__global__ void __launch_bounds__(kMsThreads)
+__global__ void __launch_bounds__(kMsChanThreads)
 mean_shift_channel_kernel(const float* __restrict__ x, float* __restrict__ y, float* __restrict__ mean_out,
                           float* __restrict__ running_mean, float momentum, int B, int C, int L) {
-    __shared__ float part[kMsThreads / 64];
+    __shared__ float part[kMsChanThreads / 64];
     __shared__ float mean_s;
     const int c = blockIdx.x;
     const int per_b = L / VEC;                    // vectors per (b, c) run
     const int total = B * per_b;
-    float s = 0.f;
-    for (int i = threadIdx.x; i < total; i += kMsThreads) {
+    // four independent loads in flight per lane: a channel is one workgroup's work, and with one load per trip
+    // the workgroup waits out a memory latency per 4 KB (8 KB with 128-bit loads)
+    constexpr int UN = 4;
+    auto at_of = [&](int i) {
         const int b = i / per_b, q = i - b * per_b;
-        const float* p = x + ((size_t)b * C + c) * L + (size_t)q * VEC;
+        return ((size_t)b * C + c) * L + (size_t)q * VEC;
+    };
+    float s = 0.f;
+    for (int i0 = threadIdx.x; i0 < total; i0 += UN * kMsChanThreads) {
         if constexpr (VEC == 4) {
-            const float4 v = *reinterpret_cast<const float4*>(p);
-            s += (v.x + v.y) + (v.z + v.w);
+            float4 v[UN];
+#pragma unroll
+            for (int u = 0; u < UN; u++) {
+                const int i = i0 + u * kMsChanThreads;
+                v[u] = i < total ? *reinterpret_cast<const float4*>(x + at_of(i)) : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+#pragma unroll
+            for (int u = 0; u < UN; u++) s += (v[u].x + v[u].y) + (v[u].z + v[u].w);
         } else {
-            s += *p;
+            float v[UN];
+#pragma unroll
+            for (int u = 0; u < UN; u++) {
+                const int i = i0 + u * kMsChanThreads;
+                v[u] = i < total ? x[at_of(i)] : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < UN; u++) s += v[u];
         }
     }
 #pragma unroll
@@ -125,7 +146,7 @@ mean_shift_channel_kernel(const float* __restrict__ x, float* __restrict__ y, fl
     if (threadIdx.x == 0) {
         float t = 0.f;
 #pragma unroll
-        for (int q = 0; q < kMsThreads / 64; q++) t += part[q];
+        for (int q = 0; q < kMsChanThreads / 64; q++) t += part[q];
         const float mean = t / ((float)B * (float)L);
         mean_s = mean;
         if (mean_out) mean_out[c] = mean;
@@ -133,15 +154,25 @@ mean_shift_channel_kernel(const float* __restrict__ x, float* __restrict__ y, fl
     }
     __syncthreads();
     const float mean = mean_s;
-    for (int i = threadIdx.x; i < total; i += kMsThreads) {
-        const int b = i / per_b, q = i - b * per_b;
-        const size_t at = ((size_t)b * C + c) * L + (size_t)q * VEC;
+    for (int i0 = threadIdx.x; i0 < total; i0 += UN * kMsChanThreads) {
+        size_t at[UN];
+#pragma unroll
+        for (int u = 0; u < UN; u++) at[u] = at_of(min(i0 + u * kMsChanThreads, total - 1));
         if constexpr (VEC == 4) {
-            float4 v = *reinterpret_cast<const float4*>(x + at);
-            v.x -= mean; v.y -= mean; v.z -= mean; v.w -= mean;
-            *reinterpret_cast<float4*>(y + at) = v;
+            float4 v[UN];
+#pragma unroll
+            for (int u = 0; u < UN; u++) v[u] = *reinterpret_cast<const float4*>(x + at[u]);
+#pragma unroll
+            for (int u = 0; u < UN; u++)
+                if (i0 + u * kMsChanThreads < total)
+                    *reinterpret_cast<float4*>(y + at[u]) = make_float4(v[u].x - mean, v[u].y - mean, v[u].z - mean, v[u].w - mean);
         } else {
-            y[at] = x[at] - mean;
+            float v[UN];
+#pragma unroll
+            for (int u = 0; u < UN; u++) v[u] = x[at[u]];
+#pragma unroll
+            for (int u = 0; u < UN; u++)
+                if (i0 + u * kMsChanThreads < total) y[at[u]] = v[u] - mean;
         }
     }
 }
@@ -157,10 +188,10 @@ hipError_t mean_shift(const float* x, float* y, float* mean_out, float* running_
             hipLaunchKernelGGL(mean_shift_rows_kernel<false>, dim3(grid), dim3(kMsThreads), 0, stream, x, y,
                                mean_out, running_mean, momentum, B, C);
     } else if (L % 4 == 0 && aligned16(x) && aligned16(y)) {
-        hipLaunchKernelGGL(mean_shift_channel_kernel<4>, dim3((unsigned)C), dim3(kMsThreads), 0, stream, x, y,
+        hipLaunchKernelGGL(mean_shift_channel_kernel<4>, dim3((unsigned)C), dim3(kMsChanThreads), 0, stream, x, y,
                            mean_out, running_mean, momentum, B, C, L);
     } else {
-        hipLaunchKernelGGL(mean_shift_channel_kernel<1>, dim3((unsigned)C), dim3(kMsThreads), 0, stream, x, y,
+        hipLaunchKernelGGL(mean_shift_channel_kernel<1>, dim3((unsigned)C), dim3(kMsChanThreads), 0, stream, x, y,
                            mean_out, running_mean, momentum, B, C, L);
     }
     return hipGetLastError();
