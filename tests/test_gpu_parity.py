@@ -219,6 +219,24 @@ def test_norm_backward(shape, p):
 
 
 @pytest.mark.parametrize("p", [2.0, 3.0, 4.0, 8.0])
+@pytest.mark.parametrize("scale", [1e-9, 1e-6, 2e-4, 3e-4, 1.0, 3e3, 5e3, 1e6, 1e15, "mixed"])
+def test_norm_forward_at_every_scale(scale, p):
+    """Small integer p sums raw powers while the running scales of a wave lie within 2^(+-96/p) and takes the
+    normalised path outside (and for the first chunk, and on overflow): every scale, the switch-over points and
+    rows of very different magnitude must give the same relative accuracy."""
+    from gpu_common import gpu_norm_forward, say
+    say("norm_forward scale", scale, "p", p)
+    x, w = make_inputs(70, 96, 260, 1, 1, seed=29)
+    if scale == "mixed":
+        rows = torch.tensor([1e-5, 1.0, 1e4, 3e-3, 1.0])[torch.arange(70) % 5].view(70, 1, 1)
+        x = x * rows
+    else:
+        x, w = x * scale, w * scale
+    out = gpu_norm_forward(x.contiguous(), w.contiguous(), 1, p)
+    torch.testing.assert_close(out, oracle.norm_dist_forward(x.contiguous(), w.contiguous(), 1, p), rtol=RTOL, atol=0)
+
+
+@pytest.mark.parametrize("p", [2.0, 3.0, 4.0, 8.0])
 @pytest.mark.parametrize("scale", [1e-6, 3e-4, 1.0, 5e3, 1e6, "mixed"])
 def test_norm_backward_at_every_scale(scale, p):
     """The small integer exponents factor the term as (c * rinv^(p-1)) * (x-w)^(p-1) only while every output of a
