@@ -20,6 +20,10 @@ struct NbDims {
 
 constexpr int RB = 32;  // stage depth (rows of the reduction per LDS panel)
 
+// Exponents from which the kernels test whether a row of terms can matter before raising them to the power.
+// Below, so many terms matter (normalised differences above 2^(-36/p)) that the test only costs.
+constexpr float kSparseMinP = 64.f;
+
 // WEIGHT = false: grad_input.  WEIGHT = true: grad_weight.
 template <bool WEIGHT, bool CONV>
 struct Views {
@@ -52,7 +56,7 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
     __shared__ float Os[RB * LDP];  // O[r][k]
     __shared__ float Cs[RB * LDA];  // c[r][a]     = grad_output
     __shared__ float Rs[RB * LDA];  // rinv[r][a]  = 1 / output
-    __shared__ float Fs[RB * LDA];  // c * rinv^(p-1), for the small integer exponents (see below)
+    __shared__ float Fs[RB * LDA];  // c * rinv^(p-1) for the small integer exponents, limits for the large ones (see below)
     const int tid = threadIdx.x;
     const int ta = blockIdx.x % tiles_a;
     const int rest = blockIdx.x / tiles_a;
@@ -68,6 +72,8 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
     const int tx = tid & 15, ty = tid >> 4;  // lane's patch: rows a0 + ty*PA.., columns k0 + tx, k0 + tx + 16, ...
     const float e = p - 1.0f;
     const int ie = small_int_power(e);
+    const bool sparse = p >= kSparseMinP;
+    const float cut = __builtin_exp2f(-36.0f / e);   // |u| <= cut  =>  |u|^(p-1) <= 2^-36
 
     float q[PA][CK], acc[PA][CK];
 #pragma unroll
@@ -117,7 +123,7 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
                 const int rr = C_A_CONTIG ? id / BA : id & (RB - 1);
                 const int cc = C_A_CONTIG ? id % BA : id / RB;
                 const int r = r0 + rr, a = a0 + cc;
-                float c = 0.f, ri = 0.f;
+                float c = 0.f, ri = 0.f, lim = 3.0e38f;   // padding never passes the test of the sparse sweep
                 if (r < r_end && a < A) {
                     const size_t o = ROW_PER_LANE ? orow + (size_t)a * d.HW : (WEIGHT ? v.o_at(r, a) : v.o_at(a, r));
                     c = grad_output[o];
@@ -125,11 +131,12 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
                     ri = __builtin_amdgcn_rcpf(out);
                     // the factored form below needs rinv^(p-1) and (Q-O)^(p-1) well inside the float range
                     unsafe |= !(out >= 0x1p-12f && out <= 0x1p12f);
+                    lim = cut * out;
                 }
                 const float r2 = ri * ri, r3 = r2 * ri;
                 Cs[rr * LDA + cc] = c;
                 Rs[rr * LDA + cc] = ri;
-                Fs[rr * LDA + cc] = c * (ie == 1 ? ri : ie == 2 ? r2 : ie == 3 ? r3 : r3 * r3 * ri);
+                Fs[rr * LDA + cc] = sparse ? lim : c * (ie == 1 ? ri : ie == 2 ? r2 : ie == 3 ? r3 : r3 * r3 * ri);
             }
         }
         if constexpr (ROW_PER_LANE) {
@@ -172,6 +179,49 @@ norm_backward_kernel(const float* __restrict__ grad_output, const float* __restr
                     for (int j = 0; j < CK; j++) acc[i][j] += c[i] * spower((q[i][j] - o[j]) * ri[i]);
             }
         };
+        // Large exponents: a normalised difference |u| <= 1 with |u|^(p-1) below 2^-36 adds less to a sum than the
+        // rounding of one term of unit size, and nearly all differences are that small -- while the logarithm and the
+        // exponential are most of a term's cost.  One row of the lane's patch at a time (CK terms that share c and
+        // rinv): when no lane of the wave has |Q - O| above its limit 2^(-36/(p-1)) * output (the Fs panel), the
+        // wave passes over the row.  The four tests of a step are made before the first branch, so that the
+        // branches wait for scalar registers only.
+        auto reduce_sparse = [&]() {
+#pragma unroll 2
+            for (int rr = 0; rr < RB; rr++) {
+                float o[CK], lim[PA], df[PA][CK];
+#pragma unroll
+                for (int j = 0; j < CK; j++) o[j] = Os[rr * LDP + tx + 16 * j];
+#pragma unroll
+                for (int i = 0; i < PA; i++) lim[i] = Fs[rr * LDA + ty * PA + i];
+                unsigned long long hot[PA], any = 0;
+#pragma unroll
+                for (int i = 0; i < PA; i++) {
+                    float top = 0.f;
+#pragma unroll
+                    for (int j = 0; j < CK; j++) {
+                        df[i][j] = q[i][j] - o[j];
+                        top = __builtin_fmaxf(top, __builtin_fabsf(df[i][j]));
+                    }
+                    hot[i] = __builtin_amdgcn_ballot_w64(top > lim[i]);
+                    any |= hot[i];
+                }
+                if (any == 0) continue;
+#pragma unroll
+                for (int i = 0; i < PA; i++) {
+                    if (hot[i] == 0) continue;
+                    const float c = Cs[rr * LDA + ty * PA + i], ri = Rs[rr * LDA + ty * PA + i];
+#pragma unroll
+                    for (int j = 0; j < CK; j++) {
+                        const float u = df[i][j] * ri;
+                        acc[i][j] += c * __builtin_copysignf(pow_pos(__builtin_fabsf(u), e), u);
+                    }
+                }
+            }
+        };
+        if (sparse) {
+            reduce_sparse();
+            continue;
+        }
         if (factored) {
             switch (ie) {
                 case 1: reduce_factored([](float u) { return u; }); break;

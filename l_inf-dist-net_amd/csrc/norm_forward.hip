@@ -4,10 +4,12 @@
 // model/norm_dist_cuda.cu:228-292: mx and the sum are seeded with 1e-10 (:232-233),
 // and whenever a block of k raises mx the sum is rescaled by (mx_old/mx_new)^p
 // (:257-261).  Here the block is a 32-wide chunk.  For p <= 64 a chunk is normally
-// swept once with the scale left by earlier chunks (see the kernel); otherwise
+// swept once with the scale left by earlier chunks (see the kernel); up to p = 128
 // sweep one finds the chunk maximum (sub + half a max3 per element), the rescale
-// runs once per output, sweep two adds (|x-w| / mx)^p.  p = 2, 3, 4, 8 use
-// multiplies only; any other p goes through v_log_f32 / v_exp_f32.
+// runs once per output, sweep two adds (|x-w| / mx)^p; from p = 128 the kernel first
+// finds the maxima over all of k and then takes only the powers that can matter
+// (see MODE 2 in the kernel).  p = 2, 3, 4, 8 use multiplies only; any other p goes
+// through v_log_f32 / v_exp_f32.
 #include "fwd_engine.hpp"
 #include "pow.hpp"
 #include "skinny.hpp"
@@ -18,14 +20,16 @@ namespace ldist {
 // parameter rather than a run-time switch: one kernel holding all five power sweeps next to
 // the maximum sweep pushed the hot loops into scratch.
 //
-// ONE = true (p <= kOneSweepMaxP): a chunk is swept once.  Any scale s gives the same result,
+// MODE 1 (p <= kOneSweepMaxP): a chunk is swept once.  Any scale s gives the same result,
 // out = s * (sum_k (|x-w|/s)^p)^(1/p); the maximum only keeps the powers in range.  So a chunk
 // adds (|x-w| / s)^p with the scale s left by earlier chunks, and only a wave that sees a chunk
 // sum overflow (or turn NaN) goes back over that chunk the long way: find its maximum, move
 // the scale there as the reference does, add the powers again.  The first chunk always takes
-// that road (the scale starts at the reference's seed 1e-10).  ONE = false: every chunk is swept twice
+// that road (the scale starts at the reference's seed 1e-10).  MODE 0: every chunk is swept twice
 // (maximum, then powers), for exponents so large that almost any increase would overflow.
-template <class GEO, bool CONV, int VEC, int IP, bool ONE>
+// MODE 2 (p >= kSparseMinP): two passes over all of k, the second with tests that skip the powers
+// of negligible terms; described where it starts below.
+template <class GEO, bool CONV, int VEC, int IP, int MODE>
 __global__ void __launch_bounds__(GEO::NT, 2)
 norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ weight, float* __restrict__ output,
                     float p, Dims d) {
@@ -59,6 +63,105 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
         for (int j = 0; j < TN; j++) { acc[i][j] = grp == 0 ? 1e-10f : 0.f; rs[i][j] = 1e10f; }
 
     const int nstage = (d.K + KK - 1) / KK;
+    if constexpr (MODE == 2) {
+        // Large p, two passes over all of k.  Pass one finds every output's maximum, which becomes its scale.  In pass
+        // two a normalised difference u below  cut = 2^(-32/p)  has a power below 2^-32, nothing against a sum that
+        // holds the maximum's own 1 -- and nearly all differences are that small, while the logarithm and the
+        // exponential are most of a term's cost.  So pass two only takes the largest u per row of the lane's patch
+        // (a subtraction, a multiplication and half a v_max3 per term), and the powers of a row are taken only when
+        // some lane of the wave has a u above the cut in it.  The rows are tested one by one only after a test of
+        // the whole fragment: every test makes a branch wait for the vector unit.
+        auto all_stages = [&](auto&& body) {
+            st.load(0);
+            st.store(lds);
+            __syncthreads();
+            for (int s = 0; s < nstage; s++) {
+                const float* stage = lds + (s % NBUF) * STAGE;
+                if (s + 1 < nstage) st.load((s + 1) * KK);
+                body(stage + grp * kChunk * GEO::SM, stage + GEO::XS + grp * kChunk * GEO::SN, s);
+                if (NBUF == 1) __syncthreads();
+                if (s + 1 < nstage) st.store(lds + ((s + 1) % NBUF) * STAGE);
+                __syncthreads();
+            }
+        };
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) rs[i][j] = 0.f;   // the maximum, until pass one is over
+        all_stages([&](const float* xp, const float* wp, int) {
+            sweep_chunk<GEO, 1, 2>(xp, wp, tx, ty, [&](const Frag<GEO, 1, 2>& f, int) {
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) {
+                        const float d0 = __builtin_fabsf(f.x[0][0][i] - f.w[0][j]);
+                        const float d1 = __builtin_fabsf(f.x[0][1][i] - f.w[1][j]);
+                        rs[i][j] = __builtin_fmaxf(__builtin_fmaxf(rs[i][j], d0), d1);
+                    }
+            });
+        });
+        // An output that stays on the seed scale 1e-10 has a sum of about 1e-10, not of at least 1: nothing is
+        // negligible against that, so a lane that holds one takes every power (its cut is below every u).
+        float cut = __builtin_exp2f(-32.0f / p);
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                const bool seeded = !(rs[i][j] > 1e-10f);
+                rs[i][j] = seeded ? 1e10f : __builtin_amdgcn_rcpf(rs[i][j]);
+                if (grp == 0) acc[i][j] = 1e-10f * pow_pos(1e-10f * rs[i][j], p);   // the seed, on the final scale
+                if (seeded) cut = -1.f;
+            }
+        // Where most rows do hold a term that counts (moderate p, or differences that crowd below their maximum) the
+        // tests only cost: a wave that took the powers of more than 85 % of a stage's rows sweeps the next seven
+        // stages without tests, then probes again.
+        constexpr int ROWS_PER_STAGE = kChunk / 2 * TM;
+        int taken = 0;   // rows whose powers this wave took in the last tested stage (the same in every lane)
+        all_stages([&](const float* xp, const float* wp, int s) {
+            if (taken * 20 > ROWS_PER_STAGE * 17 && (s & 7) != 0) {
+                sweep_chunk<GEO, 1, 2>(xp, wp, tx, ty, [&](const Frag<GEO, 1, 2>& f, int) {
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int j = 0; j < TN; j++) {
+                            acc[i][j] += pow_pos(__builtin_fabsf(f.x[0][0][i] - f.w[0][j]) * rs[i][j], p);
+                            acc[i][j] += pow_pos(__builtin_fabsf(f.x[0][1][i] - f.w[1][j]) * rs[i][j], p);
+                        }
+                });
+                return;
+            }
+            taken = 0;
+            sweep_chunk<GEO, 1, 2>(xp, wp, tx, ty, [&](const Frag<GEO, 1, 2>& f, int) {
+                float top[TM], all = 0.f;
+#pragma unroll
+                for (int i = 0; i < TM; i++) {
+                    top[i] = 0.f;
+#pragma unroll
+                    for (int j = 0; j < TN; j++) {
+                        const float u0 = __builtin_fabsf(f.x[0][0][i] - f.w[0][j]) * rs[i][j];
+                        const float u1 = __builtin_fabsf(f.x[0][1][i] - f.w[1][j]) * rs[i][j];
+                        top[i] = __builtin_fmaxf(__builtin_fmaxf(top[i], u0), u1);
+                    }
+                    all = __builtin_fmaxf(all, top[i]);
+                }
+                if (__builtin_amdgcn_ballot_w64(all > cut) != 0) {
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+                        if (__builtin_amdgcn_ballot_w64(top[i] > cut) != 0) {
+                            taken++;
+                            // the differences are taken again: kept from the tests they would hold eighty registers
+                            float x0 = f.x[0][0][i], x1 = f.x[0][1][i];
+                            asm volatile("" : "+v"(x0), "+v"(x1));
+#pragma unroll
+                            for (int j = 0; j < TN; j++) {
+                                acc[i][j] += pow_pos(__builtin_fabsf(x0 - f.w[0][j]) * rs[i][j], p);
+                                acc[i][j] += pow_pos(__builtin_fabsf(x1 - f.w[1][j]) * rs[i][j], p);
+                            }
+                        }
+                }
+            });
+        });
+    } else {
     st.load(0);
     st.store(lds);
     __syncthreads();
@@ -86,7 +189,7 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
                     cs[i][j] = 0.f;
                 }
         };
-        if constexpr (ONE) {
+        if constexpr (MODE == 1) {
             bool redo = false;
             if constexpr (IP > 0) {
                 // Small integer p: sum the raw powers |x-w|^p and multiply the chunk sum by rs^p afterwards, which
@@ -187,6 +290,7 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
         if (s + 1 < nstage) st.store(lds + ((s + 1) % NBUF) * STAGE);
         __syncthreads();
     }
+    }
 
     // Merge the k-groups onto the larger scale.
     if constexpr (KS > 1) {
@@ -232,6 +336,10 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
 // do.  Beyond that nearly every new maximum would overflow and the retries would cost more than
 // sweeping every chunk twice.
 constexpr float kOneSweepMaxP = 64.f;
+
+// Exponents from which the forward runs its two passes with tests (MODE 2).  With normally distributed
+// differences over 5120 inputs it overtakes the chunk-by-chunk kernel at p of about 120.
+constexpr float kSparseMinP = 128.f;
 
 // Few outputs per group: two passes over k, first the exact maximum per (row, output),
 // then the sum of (|x-w| / max)^p; lanes split k in both.
@@ -304,11 +412,11 @@ norm_forward_skinny_kernel(const float* __restrict__ input, const float* __restr
 
 template <class GEO, bool CONV, int VEC>
 struct NormForward {
-    template <int IP, bool ONE>
+    template <int IP, int MODE>
     static hipError_t go(unsigned grid, const Dims& d, int device, hipStream_t stream, const float* input,
                          const float* weight, float* output, float p) {
         const size_t lds = Stager<GEO, CONV, VEC, 1>::LDS_BYTES;
-        auto kern = norm_forward_kernel<GEO, CONV, VEC, IP, ONE>;
+        auto kern = norm_forward_kernel<GEO, CONV, VEC, IP, MODE>;
         static bool lds_allowed[64] = {};   // per instantiation of this launcher, i.e. per kernel
         if (hipError_t e = allow_lds(kern, lds, device, lds_allowed); e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(grid), dim3(GEO::NT), lds, stream, input, weight, output, p, d);
@@ -317,13 +425,14 @@ struct NormForward {
     static hipError_t launch(unsigned grid, const Dims& d, int device, hipStream_t stream, const float* input,
                              const float* weight, float* output, float p) {
         switch (small_int_power(p)) {
-            case 2: return go<2, true>(grid, d, device, stream, input, weight, output, p);
-            case 3: return go<3, true>(grid, d, device, stream, input, weight, output, p);
-            case 4: return go<4, true>(grid, d, device, stream, input, weight, output, p);
-            case 8: return go<8, true>(grid, d, device, stream, input, weight, output, p);
+            case 2: return go<2, 1>(grid, d, device, stream, input, weight, output, p);
+            case 3: return go<3, 1>(grid, d, device, stream, input, weight, output, p);
+            case 4: return go<4, 1>(grid, d, device, stream, input, weight, output, p);
+            case 8: return go<8, 1>(grid, d, device, stream, input, weight, output, p);
             default:
-                return p <= kOneSweepMaxP ? go<0, true>(grid, d, device, stream, input, weight, output, p)
-                                          : go<0, false>(grid, d, device, stream, input, weight, output, p);
+                if (p >= kSparseMinP) return go<0, 2>(grid, d, device, stream, input, weight, output, p);
+                return p <= kOneSweepMaxP ? go<0, 1>(grid, d, device, stream, input, weight, output, p)
+                                          : go<0, 0>(grid, d, device, stream, input, weight, output, p);
         }
     }
 };

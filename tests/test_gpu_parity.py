@@ -265,6 +265,49 @@ def test_norm_backward_at_every_scale(scale, p):
     assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
 
 
+@pytest.mark.parametrize("p", [64.0, 100.5, 128.0, 300.0, 1000.0])
+@pytest.mark.parametrize("data", ["normal", "flat", "ties", "tiny", "mixed", "conv", "grouped"])
+def test_norm_large_exponents(data, p):
+    """From p = 64 (backward) and p = 128 (forward) the kernels test whether a row of terms can matter before they
+    take its powers, and pass over rows of negligible terms.  Normal weights: nearly every row is passed over.
+    Flat: differences crowd below the maximum, most rows count (the forward gives up testing).  Ties: many terms
+    equal the maximum exactly.  Tiny: everything below the reference's 1e-10 seed, where nothing is negligible.
+    Mixed: rows of very different magnitude.  All must meet the same tolerance as every other exponent."""
+    from gpu_common import DEV, cpp, gpu_norm_forward, say
+    say("norm large exponent", data, "p", p)
+    B, CO, CI, G, HW = 70, 96, 1100, 1, 1
+    if data == "conv":
+        B, CO, CI, G, HW = 3, 40, 600, 1, 50
+    elif data == "grouped":
+        B, CO, CI, G, HW = 40, 48, 1040, 4, 1
+    g = gen(31)
+    x = torch.randn(B, CI, HW, generator=g)
+    w = torch.randn(CO, CI // G, generator=g)
+    if data == "flat":
+        x, w = torch.rand(B, CI, HW, generator=g), w * 0.01
+    elif data == "ties":
+        x, w = torch.randint(0, 2, (B, CI, HW), generator=g).float(), torch.zeros(CO, CI // G)
+    elif data == "tiny":
+        x, w = x * 1e-12, w * 1e-12
+    elif data == "mixed":
+        x = x * torch.tensor([1e-5, 1.0, 1e4, 3e-3, 1.0])[torch.arange(B) % 5].view(B, 1, 1)
+    x, w = x.contiguous(), w.contiguous()
+    want = oracle.norm_dist_forward(x, w, G, p)
+    out = gpu_norm_forward(x, w, G, p)
+    torch.testing.assert_close(out, want, rtol=RTOL, atol=0)
+    go = torch.randn(B, CO, HW, generator=gen(9))
+    ex, mx = oracle.norm_dist_backward_input(go, x, w, want, G, p, with_abs_terms=True)
+    ew, mw = oracle.norm_dist_backward_weight(go, x, w, want, G, p, with_abs_terms=True)
+    gx = torch.full((B, CI, HW), float("nan"), device=DEV)
+    gw = torch.zeros((CO, CI // G), device=DEV)
+    args = (go.to(DEV), x.to(DEV), w.to(DEV), want.to(DEV))
+    cpp.norm_dist_backward_input(*args, gx, G, p)
+    cpp.norm_dist_backward_weight(*args, gw, G, p)
+    torch.cuda.synchronize()
+    assert_sum_close(gx.cpu(), ex, mx, p, RTOL, ATOL)
+    assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
+
+
 @pytest.mark.parametrize("shape", [(512, 5120, 1), (37, 10, 1), (1030, 50, 1), (600, 36, 1), (6, 5, 12), (4, 3, 7),
                                    (16, 8, 1024)])
 def test_mean_shift_kernel(shape):
