@@ -1,0 +1,139 @@
+"""GPU parity on seeded random problem sizes: every entry point of the distance operators against the CPU oracle.
+
+The hand-picked shapes of test_gpu_parity.py cover the cases the kernels were written for; this file draws sizes
+nobody picked -- prime row counts, reductions shorter than a vector, one output per group, ragged conv layouts --
+with a random forward tile, a random exponent and, for the conv layer, a random image geometry.  Same bars as
+everywhere: L_inf values, indices and bounds bit-exact, everything else rel 1e-5 / abs 1e-6.
+"""
+import random
+
+import pytest
+import torch
+
+import oracle
+from helpers import SIGN, assert_sum_close, gen, make_inputs
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-5, 1e-6
+EXPONENTS = [2.0, 3.0, 4.0, 8.0, 2.5, 16.5, 47.0, 70.0, 150.0, 1000.0]
+
+
+def draw(seed):
+    """B, CO, CI, G, HW, tile, p with B*HW*CO*K bounded so that the oracle takes well under a second."""
+    r = random.Random(seed)
+    G = r.choice([1, 1, 1, 2, 3, 4])
+    NG = r.choice([1, 2, 5, 16, 17, 31, 40, 64, 81, 130])
+    K = r.choice([1, 2, 3, 4, 7, 31, 32, 33, 64, 100, 257, 300, 1100, 2300])
+    HW = r.choice([1, 1, 1, 2, 5, 16, 36, 49])
+    budget = 6_000_000 // (NG * K * HW)
+    B = max(1, min(r.choice([1, 2, 3, 17, 64, 129, 200]), budget))
+    return B, NG * G, K * G, G, HW, r.choice([-1, 0, 1, 2, 3]), r.choice(EXPONENTS)
+
+
+@pytest.fixture(autouse=True)
+def _reset_tile():
+    from gpu_common import set_tile
+    yield
+    set_tile(-1)
+
+
+@pytest.mark.parametrize("seed", range(192))
+def test_random_problem(seed):
+    from gpu_common import DEV, cpp, gpu_bound_forward, gpu_inf_forward, gpu_norm_forward, say, set_tile
+    B, CO, CI, G, HW, tile, p = draw(seed)
+    say("random problem", seed, (B, CO, CI, G, HW), "tile", tile, "p", p)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=1000 + seed, quantize=16 if seed % 3 == 0 else None)
+    set_tile(tile)
+
+    out, pos = gpu_inf_forward(x, w, G)
+    eo, ep = oracle.inf_dist_forward(x, w, G)
+    assert torch.equal(out, eo) and torch.equal(pos, ep)
+
+    lo, up = (x - 0.05).contiguous(), (x + 0.05).contiguous()
+    ol, ou = gpu_bound_forward(lo, up, w, G)
+    el, eu = oracle.inf_dist_bound_forward(lo, up, w, G)
+    assert torch.equal(ol, el) and torch.equal(ou, eu)
+
+    go = torch.randn(B, CO, HW, generator=gen(2000 + seed))
+    gx = torch.full((B, CI, HW), float("nan"), device=DEV)
+    gw = torch.full((CO, CI // G), float("nan"), device=DEV)
+    cpp.inf_dist_backward_input_overwrite(go.to(DEV), ep.to(DEV), gx, G)
+    cpp.inf_dist_backward_weight_overwrite(go.to(DEV), ep.to(DEV), gw, G)
+    torch.cuda.synchronize()
+    # sums of signed terms in another order than the oracle's: the absolute part scales with the sum of |terms|
+    tx = oracle.inf_dist_backward_input(go.abs(), ep & ~SIGN, CI, G).abs()
+    tw = oracle.inf_dist_backward_weight(go.abs(), ep & ~SIGN, CI, G).abs()
+    assert_sum_close(gx.cpu(), oracle.inf_dist_backward_input(go, ep, CI, G), tx, rtol=RTOL, atol=ATOL)
+    assert_sum_close(gw.cpu(), oracle.inf_dist_backward_weight(go, ep, CI, G), tw, rtol=RTOL, atol=ATOL)
+
+    want = oracle.norm_dist_forward(x, w, G, p)
+    torch.testing.assert_close(gpu_norm_forward(x, w, G, p), want, rtol=RTOL, atol=0)
+    ex, mx = oracle.norm_dist_backward_input(go, x, w, want, G, p, with_abs_terms=True)
+    ew, mw = oracle.norm_dist_backward_weight(go, x, w, want, G, p, with_abs_terms=True)
+    gx = torch.full((B, CI, HW), float("nan"), device=DEV)
+    gw = torch.zeros((CO, CI // G), device=DEV)
+    args = (go.to(DEV), x.to(DEV), w.to(DEV), want.to(DEV))
+    cpp.norm_dist_backward_input(*args, gx, G, p)
+    cpp.norm_dist_backward_weight(*args, gw, G, p)
+    torch.cuda.synchronize()
+    assert_sum_close(gx.cpu(), ex, mx, p, RTOL, ATOL)
+    assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
+
+
+def draw_image(seed):
+    """B, C, H, W, CO, G, stride, padding for the 3x3 conv layer taken from the image."""
+    r = random.Random(7000 + seed)
+    G = r.choice([1, 1, 2, 4])
+    CG = r.choice([1, 2, 3, 4, 5, 8, 12, 16])
+    NG = r.choice([1, 3, 4, 8, 12, 20, 32, 48])
+    H, W = r.choice([3, 4, 7, 8, 11, 16, 17, 28, 32]), r.choice([3, 4, 7, 8, 11, 16, 17, 28, 32])
+    stride, padding = r.choice([1, 1, 2]), r.choice([0, 1, 1])
+    B = r.choice([1, 2, 3, 5])
+    return B, CG * G, H, W, NG * G, G, stride, padding
+
+
+@pytest.mark.parametrize("seed", range(96))
+def test_random_conv_layer_from_the_image(seed):
+    """Values, argmax and bounds from the image against the oracle on the unfolded tensor; geometries the image
+    kernels do not take (their query says so) must be refused, and are then checked through the column kernels."""
+    import torch.nn.functional as F
+    from gpu_common import DEV, cpp, gpu_inf_forward, say
+    B, C, H, W, CO, G, stride, padding = draw_image(seed)
+    say("random conv layer", seed, (B, C, H, W, CO, G, stride, padding))
+    img = torch.randn(B, C, H, W, generator=gen(3000 + seed))
+    if seed % 2:
+        img = (img * 8).round() / 8          # ties
+    w = (torch.randn(CO, C // G * 9, generator=gen(4000 + seed)) * 0.7).contiguous()
+    cols = F.unfold(img, 3, 1, padding, stride).contiguous()
+    HO, WO = (H + 2 * padding - 3) // stride + 1, (W + 2 * padding - 3) // stride + 1
+    eo, ep = oracle.inf_dist_forward(cols, w, G)
+    if cpp.inf_dist_conv_forward_supported(C, H, W, CO, G, 3, stride, padding, 1):
+        out = torch.empty(B, CO, HO * WO, device=DEV)
+        pos = torch.empty(B, CO, HO * WO, device=DEV, dtype=torch.int32)
+        cpp.inf_dist_conv_forward(img.to(DEV), w.to(DEV), out, pos, G, 3, stride, padding, 1)
+        torch.cuda.synchronize()
+        out, pos = out.cpu(), pos.cpu()
+    else:
+        out, pos = gpu_inf_forward(cols, w, G)
+    assert torch.equal(out, eo) and torch.equal(pos, ep)
+
+    lo, up = img - 0.03, img + 0.03
+    lc, uc = F.unfold(lo, 3, 1, padding, stride).contiguous(), F.unfold(up, 3, 1, padding, stride).contiguous()
+    el, eu = oracle.inf_dist_bound_forward(lc, uc, w, G)
+    if cpp.inf_dist_bound_conv_forward_supported(C, H, W, CO, G, 3, stride, padding, 1):
+        ol = torch.empty(B, CO, HO * WO, device=DEV)
+        ou = torch.empty_like(ol)
+        cpp.inf_dist_bound_conv_forward(lo.to(DEV), up.to(DEV), w.to(DEV), ol, ou, G, 3, stride, padding, 1)
+        torch.cuda.synchronize()
+        assert torch.equal(ol.cpu(), el) and torch.equal(ou.cpu(), eu)
+
+    go = torch.randn(B, CO, HO * WO, generator=gen(5000 + seed))
+    gcols = oracle.inf_dist_backward_input(go, ep, cols.size(1), G)
+    expect = F.fold(gcols.double(), (H, W), 3, 1, padding, stride)
+    terms = F.fold(oracle.inf_dist_backward_input(go.abs(), ep & ~SIGN, cols.size(1), G).double(), (H, W), 3, 1,
+                   padding, stride).abs()
+    gimg = torch.full(img.shape, float("nan"), device=DEV)
+    cpp.inf_dist_backward_input_folded(go.to(DEV), ep.to(DEV), gimg, G, 3, stride, padding, 1)
+    torch.cuda.synchronize()
+    assert_sum_close(gimg.cpu(), expect, terms, rtol=RTOL, atol=ATOL)
