@@ -137,3 +137,65 @@ def test_random_conv_layer_from_the_image(seed):
     cpp.inf_dist_backward_input_folded(go.to(DEV), ep.to(DEV), gimg, G, 3, stride, padding, 1)
     torch.cuda.synchronize()
     assert_sum_close(gimg.cpu(), expect, terms, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_mean_shift_and_adamw(seed):
+    """The mean shift and the fused AdamW step on sizes nobody picked, against float64 / the oracle."""
+    from gpu_common import DEV, cpp, say
+    r = random.Random(9000 + seed)
+    B, C, L = r.choice([1, 2, 7, 64, 130, 513]), r.choice([1, 3, 10, 33, 96, 500]), r.choice([1, 1, 4, 9, 49, 256])
+    say("random mean shift", seed, (B, C, L))
+    x = torch.randn(B, C, L, generator=gen(9100 + seed)) * 3 + 1.5
+    mean64 = x.double().mean(dim=(0, 2))
+    y, mean_out = torch.full((B, C, L), float("nan"), device=DEV), torch.empty(C, device=DEV)
+    running = torch.linspace(-1, 1, C).to(DEV)
+    cpp.mean_shift(x.to(DEV), y, mean_out, running, 0.25)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(mean_out.cpu().double(), mean64, rtol=1e-6, atol=2e-6)
+    torch.testing.assert_close(y.cpu().double(), x.double() - mean64.view(1, C, 1), rtol=1e-6, atol=4e-6)
+    torch.testing.assert_close(running.cpu().double(), 0.75 * torch.linspace(-1, 1, C).double() + 0.25 * mean64,
+                               rtol=1e-6, atol=2e-6)
+
+    rows, cols = r.choice([1, 2, 10, 77, 300]), r.choice([1, 2, 5, 64, 99, 1000, 3001])
+    p = r.choice([2.0, 8.0, 37.5, 1000.0, float("inf")])
+    say("random adamw", seed, (rows, cols), "p", p)
+    g = gen(9200 + seed)
+    w = torch.randn(rows, cols, generator=g) * 0.5
+    m, v = torch.zeros_like(w), torch.zeros_like(w)
+    wd, md, vd = w.to(DEV), m.to(DEV), v.to(DEV)
+    for step in (1, 2):
+        grad = torch.randn(rows, cols, generator=g)
+        oracle.adamw_lp_step(w, grad, m, v, p, 0.02, (0.9, 0.99), 1e-8, 0.1, step)
+        cpp.adamw_lp_step(wd, grad.to(DEV), md, vd, p, 0.02, 0.9, 0.99, 1e-8, 0.1, step)
+        torch.cuda.synchronize()
+        torch.testing.assert_close(md.cpu(), m, rtol=1e-6, atol=2e-7)
+        torch.testing.assert_close(vd.cpu(), v, rtol=1e-6, atol=1e-9)
+        torch.testing.assert_close(wd.cpu(), w, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_unfold_and_fold(seed):
+    """Patch extraction (bit-equal to F.unfold) and its adjoint on random geometries, dilation included."""
+    import torch.nn.functional as F
+    from gpu_common import DEV, cpp, say
+    r = random.Random(11000 + seed)
+    k, s_, d_ = r.choice([1, 2, 3, 3, 5]), r.choice([1, 1, 2, 3]), r.choice([1, 1, 2])
+    p_ = r.choice([0, 1, 2])
+    span = d_ * (k - 1) + 1
+    H, W = span + r.choice([0, 1, 4, 9, 20]), span + r.choice([0, 2, 3, 11, 25])
+    B, C = r.choice([1, 2, 5]), r.choice([1, 3, 8])
+    say("random unfold/fold", seed, (B, C, H, W, k, s_, p_, d_))
+    img = torch.randn(B, C, H, W, generator=gen(11100 + seed))
+    ref = F.unfold(img, k, d_, p_, s_)
+    cols = torch.full(ref.shape, float("nan"), device=DEV)
+    cpp.unfold(img.to(DEV), cols, k, s_, p_, d_)
+    torch.cuda.synchronize()
+    assert torch.equal(cols.cpu(), ref)
+    gc = torch.randn(ref.shape, generator=gen(11200 + seed))
+    gi = torch.full(img.shape, float("nan"), device=DEV)
+    cpp.fold(gc.to(DEV), gi, k, s_, p_, d_)
+    torch.cuda.synchronize()
+    want = F.fold(gc.double(), (H, W), k, d_, p_, s_)
+    terms = F.fold(gc.double().abs(), (H, W), k, d_, p_, s_)
+    assert_sum_close(gi.cpu(), want, terms, rtol=RTOL, atol=ATOL)
