@@ -80,6 +80,19 @@ LDIST_API int ldist_inf_dist_bound_forward(const float* input_lower, const float
                                  int CO, int CI, int G, int HW, float* output_lower, float* output_upper,
                                  ldist_stream_t stream);
 
+/* Values and interval bounds in one pass over the weights: what ldist_inf_dist_forward (without the index)
+ * and ldist_inf_dist_bound_forward compute for a point `input` and the box [input_lower, input_upper] around it,
+ * bit for bit, followed by the layer's evaluation-mode epilogue.  Replaces the pair of calls certification makes
+ * per layer, norm_dist(...) and inf_dist_bound(...) at model/norm_dist.py:134,144-145 (inf_dist_forward_cuda and
+ * inf_dist_bound_forward_cuda, model/norm_dist.cpp:13-16), and the shifts after them (:146-155).
+ *   mean, bias: (CO) each or NULL; every value v of output channel c leaves as (v - mean[c]) + bias[c], in this
+ *   order, the running-mean shift of MeanNorm in evaluation mode and the layer's bias.
+ * No index is produced: this path carries no gradient (the reference asserts evaluation mode, :142). */
+LDIST_API int ldist_inf_dist_value_bound_forward(const float* input, const float* input_lower, const float* input_upper,
+                                       const float* weight, int B, int CO, int CI, int G, int HW, const float* mean,
+                                       const float* bias, float* output, float* output_lower, float* output_upper,
+                                       ldist_stream_t stream);
+
 /* L_inf backward w.r.t. input.  Replaces inf_dist_backward_input_cuda
  * (model/norm_dist.cpp:17-18, model/inf_dist_cuda.cu:189-196).
  *   grad_input[b, g*K + idx, hw] += (pos >= 0 ? g : -g),  idx = pos & 0x7fffffff

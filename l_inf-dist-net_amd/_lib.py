@@ -20,6 +20,7 @@ _d = ctypes.c_double
 SIGNATURES = {
     "ldist_inf_dist_forward": [_F, _F, _i, _i, _i, _i, _i, _F, _I, _S],
     "ldist_inf_dist_bound_forward": [_F, _F, _F, _i, _i, _i, _i, _i, _F, _F, _S],
+    "ldist_inf_dist_value_bound_forward": [_F, _F, _F, _F, _i, _i, _i, _i, _i, _F, _F, _F, _F, _F, _S],
     "ldist_inf_dist_backward_input": [_F, _I, _i, _i, _i, _i, _i, _F, _S],
     "ldist_inf_dist_backward_weight": [_F, _I, _i, _i, _i, _i, _i, _F, _S],
     "ldist_inf_dist_backward_input_overwrite": [_F, _I, _i, _i, _i, _i, _i, _F, _S],

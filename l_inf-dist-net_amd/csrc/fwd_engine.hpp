@@ -50,19 +50,19 @@ struct Stager {
             else xlk[q].load(in[q], ld_x, rows_x, k0, K, tid);
         }
     }
-    // For the interval kernel (NX == 2: lower, upper): true when some value this lane
+    // For the interval kernels (the last two panels are lower, upper): true when some value this lane
     // just loaded breaks lower <= upper, or is NaN or infinite (weights included).
     __device__ __forceinline__ bool interval_is_irregular() const {
-        static_assert(NX <= 2, "");
         bool bad = false;
-        if constexpr (NX == 2) {
+        if constexpr (NX >= 2) {
             constexpr float INF = __builtin_inff();
+            constexpr int LO = NX - 2, UP = NX - 1;
             if constexpr (CONV) {
 #pragma unroll
                 for (int i = 0; i < XLoadM::N; i++)
 #pragma unroll
                     for (int e = 0; e < VEC; e++) {
-                        const float l = xlm[0].v[i][e], u = xlm[1].v[i][e];
+                        const float l = xlm[LO].v[i][e], u = xlm[UP].v[i][e];
                         bad |= !(l <= u && __builtin_fabsf(l) < INF && __builtin_fabsf(u) < INF);
                     }
             } else {
@@ -70,7 +70,7 @@ struct Stager {
                 for (int i = 0; i < XLoadK::N; i++)
 #pragma unroll
                     for (int e = 0; e < VEC; e++) {
-                        const float l = xlk[0].v[i][e], u = xlk[1].v[i][e];
+                        const float l = xlk[LO].v[i][e], u = xlk[UP].v[i][e];
                         bad |= !(l <= u && __builtin_fabsf(l) < INF && __builtin_fabsf(u) < INF);
                     }
             }

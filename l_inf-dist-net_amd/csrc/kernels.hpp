@@ -60,6 +60,9 @@ inline hipError_t allow_lds(Kern kern, size_t bytes, int device, bool (&done)[64
 
 hipError_t inf_forward(const float* input, const float* weight, float* output, int32_t* pos, const Problem& pr,
                        hipStream_t stream);
+hipError_t value_bound_forward(const float* input, const float* lower, const float* upper, const float* weight,
+                               const float* mean, const float* bias, float* out, float* out_lower, float* out_upper,
+                               const Problem& pr, hipStream_t stream);
 hipError_t bound_forward(const float* lower, const float* upper, const float* weight, float* out_lower,
                          float* out_upper, const Problem& pr, hipStream_t stream);
 hipError_t inf_backward_input(const float* grad_output, const int32_t* pos, float* grad_input, const Problem& pr,

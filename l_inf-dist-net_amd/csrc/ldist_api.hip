@@ -127,6 +127,18 @@ int ldist_inf_dist_bound_forward(const float* input_lower, const float* input_up
                                        (hipStream_t)stream));
 }
 
+int ldist_inf_dist_value_bound_forward(const float* input, const float* input_lower, const float* input_upper,
+                                       const float* weight, int B, int CO, int CI, int G, int HW, const float* mean,
+                                       const float* bias, float* output, float* output_lower, float* output_upper,
+                                       ldist_stream_t stream) {
+    if (!input || !input_lower || !input_upper || !weight || !output || !output_lower || !output_upper)
+        return LDIST_EINVAL;
+    ldist::Problem pr{};
+    if (int rc = check_dims(B, CO, CI, G, HW, pr)) return rc;
+    return finish(ldist::value_bound_forward(input, input_lower, input_upper, weight, mean, bias, output, output_lower,
+                                             output_upper, pr, (hipStream_t)stream));
+}
+
 static int inf_backward_input_impl(const float* grad_output, const int32_t* pos, int B, int CO, int CI, int G,
                                    int HW, float* grad_input, bool overwrite, ldist_stream_t stream) {
     if (!grad_output || !pos || !grad_input) return LDIST_EINVAL;

@@ -120,6 +120,32 @@ def inf_dist_bound_forward(input_lower, input_upper, weight, output_lower, outpu
           _p(output_lower), _p(output_upper))
 
 
+def inf_dist_value_bound_forward(input, input_lower, input_upper, weight, output, output_lower, output_upper, G,
+                                 mean=None, bias=None):
+    """Values and interval bounds in one pass over the weights (no counterpart in model/norm_dist.cpp: the reference
+    calls inf_dist_forward and inf_dist_bound_forward one after the other, model/norm_dist.py:134,144-145), with the
+    evaluation-mode epilogue (v - mean[c]) + bias[c] per output channel when `mean` / `bias` are given (:146-155)."""
+    for t, n in ((input, "input"), (input_lower, "input_lower"), (input_upper, "input_upper"), (weight, "weight"),
+                 (output, "output"), (output_lower, "output_lower"), (output_upper, "output_upper")):
+        _check_input(t, n)
+    tensors = [input, input_lower, input_upper, weight, output, output_lower, output_upper]
+    B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
+    for t, n in ((mean, "mean"), (bias, "bias")):
+        if t is not None:
+            _check_input(t, n)
+            _expect(tuple(t.shape) == (CO,), f"{n} must be (CO,)")
+            tensors.append(t)
+    dev = _same_device(*tensors)
+    _expect(tuple(input_lower.shape) == tuple(input.shape) and tuple(input_upper.shape) == tuple(input.shape),
+            "input_lower and input_upper must match input")
+    _expect(weight.size(0) == CO and weight.size(1) * G == CI, "weight must be (CO, CI/G)")
+    for t in (output, output_lower, output_upper):
+        _expect(tuple(t.shape) == (B, CO, HW), "outputs must be (B, CO, HW)")
+    _call("ldist_inf_dist_value_bound_forward", dev, _p(input), _p(input_lower), _p(input_upper), _p(weight), B, CO, CI,
+          G, HW, _p(mean) if mean is not None else None, _p(bias) if bias is not None else None, _p(output),
+          _p(output_lower), _p(output_upper))
+
+
 def _inf_backward_input(name, grad_output, pos, grad_input, G):
     _check_input(grad_output, "grad_output")
     _check_input(pos, "pos", torch.int32)

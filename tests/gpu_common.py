@@ -42,3 +42,12 @@ def gpu_norm_forward(x, w, G, p):
     cpp.norm_dist_forward(x.to(DEV), w.to(DEV), out, G, p)
     torch.cuda.synchronize()
     return out.cpu()
+
+
+def gpu_value_bound_forward(x, lo, up, w, G, mean=None, bias=None):
+    out = torch.full((x.size(0), w.size(0), x.size(2)), float("nan"), device=DEV)
+    out_l, out_u = torch.full_like(out, float("nan")), torch.full_like(out, float("nan"))
+    cpp.inf_dist_value_bound_forward(x.to(DEV), lo.to(DEV), up.to(DEV), w.to(DEV), out, out_l, out_u, G,
+                                     None if mean is None else mean.to(DEV), None if bias is None else bias.to(DEV))
+    torch.cuda.synchronize()
+    return out.cpu(), out_l.cpu(), out_u.cpu()

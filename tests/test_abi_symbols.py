@@ -62,6 +62,8 @@ def test_argument_checks_need_no_device(lib):
     assert lib.ldist_norm_dist_backward_weight(one, one, one, one, 1, 1, 1, 1, 1, None, 8.0, None) == -1
     assert lib.ldist_inf_dist_bound_forward(one, None, one, 1, 1, 1, 1, 1, one, one, None) == -1
     assert lib.ldist_inf_dist_backward_input_overwrite(one, one, 1, 1, 1, 1, 0, one, None) == -1
+    assert lib.ldist_inf_dist_value_bound_forward(one, one, None, one, 1, 1, 1, 1, 1, None, None, one, one, one, None) == -1
+    assert lib.ldist_inf_dist_value_bound_forward(one, one, one, one, 1, 3, 4, 2, 1, None, None, one, one, one, None) == -1
 
 
 def test_conv_forward_geometry_query_needs_no_device(lib):

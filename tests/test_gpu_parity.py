@@ -138,6 +138,86 @@ def test_inf_backward(shape, overwrite):
     torch.testing.assert_close(gw.cpu(), ew, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("tile", TILES)
+@pytest.mark.parametrize("shape", SHAPES)
+def test_value_bound_forward_bit_exact(shape, tile):
+    """Values and both bounds from the one-pass kernel equal what the value kernel and the bound kernel give (the
+    oracle's), bit for bit; with a mean and a bias every channel leaves as (v - mean) + bias in float32."""
+    from gpu_common import gpu_value_bound_forward, say, set_tile
+    B, CO, CI, G, HW = shape
+    say("value_bound_forward", shape, "tile", tile)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=1 + sum(shape), quantize=8 if tile == 1 else None)
+    lo, up = (x - 8 / 255).clamp(0, 1).contiguous(), (x + 8 / 255).clamp(0, 1).contiguous()
+    ev, _ = oracle.inf_dist_forward(x, w, G)
+    el, eu = oracle.inf_dist_bound_forward(lo, up, w, G)
+    set_tile(tile)
+    ov, ol, ou = gpu_value_bound_forward(x, lo, up, w, G)
+    assert torch.equal(ov, ev) and torch.equal(ol, el) and torch.equal(ou, eu)
+    mean, bias = torch.randn(CO, generator=gen(61)), torch.randn(CO, generator=gen(62))
+    for m_, b_ in ((mean, None), (None, bias), (mean, bias)):
+        ov, ol, ou = gpu_value_bound_forward(x, lo, up, w, G, m_, b_)
+        for got, want in ((ov, ev), (ol, el), (ou, eu)):
+            if m_ is not None:
+                want = want - m_.view(1, CO, 1)
+            if b_ is not None:
+                want = want + b_.view(1, CO, 1)
+            assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("shape", [(33, 100, 77, 1, 1), (130, 70, 260, 1, 1), (2, 64, 64, 2, 64), (40, 10, 300, 1, 1)])
+def test_value_bound_forward_irregular_boxes(shape):
+    """lower > upper, NaN and infinities in the box, the point or the weights: the reference's literal predicate."""
+    from gpu_common import gpu_value_bound_forward
+    B, CO, CI, G, HW = shape
+    x, w = make_inputs(B, CO, CI, G, HW, seed=9)
+    g = gen(4)
+    lo, up = (x - 0.1).contiguous(), (x + 0.1).contiguous()
+    flip = torch.rand(x.shape, generator=g) < 0.05
+    lo2, up2 = torch.where(flip, up, lo).contiguous(), torch.where(flip, lo, up).contiguous()
+    lo2[0, 0, 0] = float("nan")
+    up2[-1, -1, -1] = float("inf")
+    x2 = x.clone()
+    x2[0, 1, 0], x2[-1, 0, -1] = float("nan"), float("-inf")
+    w2 = w.clone()
+    w2[0, 0] = float("-inf")
+    same = lambda a, b: torch.equal(torch.nan_to_num(a, nan=-1.0), torch.nan_to_num(b, nan=-1.0))
+    for (xx, a, b, ww) in ((x2, lo2, up2, w), (x, lo, up, w2)):
+        ov, ol, ou = gpu_value_bound_forward(xx, a, b, ww, G)
+        ev, _ = oracle.inf_dist_forward(xx, ww, G, literal=True)
+        el, eu = oracle.inf_dist_bound_forward(a, b, ww, G)
+        assert same(ov, ev) and same(ol, el) and same(ou, eu)
+
+
+def test_layers_with_few_outputs_certify_through_the_one_pass_kernel():
+    """In evaluation mode without gradients, a layer without a window and with at most 16 outputs per group takes
+    values and bounds from the one-pass kernel, running mean and bias included: same numbers as the separate
+    kernels, bit for bit."""
+    from gpu_common import DEV, pkg
+    torch.manual_seed(3)
+    for bias, mean_normalize, group, hw in ((True, True, 1, 1), (False, True, 2, 1), (True, False, 1, 3), (False, False, 4, 2)):
+        co = 10 * group
+        layer = pkg.NormDistConv(120, co, 1, group=group, p=float("inf"), bias=bias, mean_normalize=mean_normalize).to(DEV)
+        with torch.no_grad():
+            layer.weight.copy_(torch.randn(co, 120 // group, 1, 1))
+            if bias:
+                layer.bias.copy_(torch.randn(co))
+            if mean_normalize:
+                layer.normalize.running_mean.copy_(torch.randn(co))
+        layer.eval()
+        x = torch.rand(37, 120, hw, hw, generator=gen(71)).to(DEV)
+        lo, up = x - 0.02, x + 0.02
+        with torch.no_grad():
+            assert layer._value_and_bounds_in_one_pass(x, lo, up)
+            fused = layer(x, lo, up)
+            layer.FUSED_VALUE_BOUND_MAX_OUTPUTS = 0
+            assert not layer._value_and_bounds_in_one_pass(x, lo, up)
+            separate = layer(x, lo, up)
+        assert all(torch.equal(a, b) for a, b in zip(fused, separate))
+        del layer.FUSED_VALUE_BOUND_MAX_OUTPUTS
+        y, l, u = layer(x.requires_grad_(True), lo, up)      # with gradients enabled: the separate kernels, with autograd
+        assert y.requires_grad and torch.equal(y.detach(), fused[0]) and torch.equal(l, fused[1])
+
+
 PNORM_SHAPES = [s for s in SHAPES if s[1] * s[2] * s[0] * s[4] <= 40_000_000]
 
 

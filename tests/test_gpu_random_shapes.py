@@ -40,7 +40,8 @@ def _reset_tile():
 
 @pytest.mark.parametrize("seed", range(192))
 def test_random_problem(seed):
-    from gpu_common import DEV, cpp, gpu_bound_forward, gpu_inf_forward, gpu_norm_forward, say, set_tile
+    from gpu_common import (DEV, cpp, gpu_bound_forward, gpu_inf_forward, gpu_norm_forward, gpu_value_bound_forward, say,
+                            set_tile)
     B, CO, CI, G, HW, tile, p = draw(seed)
     say("random problem", seed, (B, CO, CI, G, HW), "tile", tile, "p", p)
     x, w = make_inputs(B, CO, CI, G, HW, seed=1000 + seed, quantize=16 if seed % 3 == 0 else None)
@@ -54,6 +55,10 @@ def test_random_problem(seed):
     ol, ou = gpu_bound_forward(lo, up, w, G)
     el, eu = oracle.inf_dist_bound_forward(lo, up, w, G)
     assert torch.equal(ol, el) and torch.equal(ou, eu)
+    mean = torch.randn(CO, generator=gen(2500 + seed))
+    fv, fl, fu = gpu_value_bound_forward(x, lo, up, w, G, mean, None)      # the one-pass kernel with its epilogue
+    shift = mean.view(1, CO, 1)
+    assert torch.equal(fv, eo - shift) and torch.equal(fl, el - shift) and torch.equal(fu, eu - shift)
 
     go = torch.randn(B, CO, HW, generator=gen(2000 + seed))
     gx = torch.full((B, CI, HW), float("nan"), device=DEV)
