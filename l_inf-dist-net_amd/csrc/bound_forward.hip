@@ -126,7 +126,7 @@ bound_forward_kernel(const float* __restrict__ lower, const float* __restrict__ 
 }
 
 // Few outputs per group: lanes split k and apply the reference's literal predicate.
-template <int RW, int NB>
+template <int RW, int NB, bool VEC>
 __global__ void __launch_bounds__(256)
 bound_forward_skinny_kernel(const float* __restrict__ lower, const float* __restrict__ upper,
                             const float* __restrict__ weight, float* __restrict__ out_lower,
@@ -135,32 +135,24 @@ bound_forward_skinny_kernel(const float* __restrict__ lower, const float* __rest
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     SkinnyRows<RW> rows;
     rows.init(d);
-    const int K = d.K, xk = d.HW;
     for (int nb = 0; nb < d.NG; nb += NB) {
         float lo[RW][NB], up[RW][NB];
 #pragma unroll
         for (int r = 0; r < RW; r++)
 #pragma unroll
             for (int j = 0; j < NB; j++) { lo[r][j] = 0.f; up[r][j] = 0.f; }
-        for (int k = tid; k < K; k += 256) {
-            float lv[RW], uv[RW], wv[NB];
-#pragma unroll
-            for (int r = 0; r < RW; r++) {
-                lv[r] = lower[rows.xoff[r] + (size_t)k * xk];
-                uv[r] = upper[rows.xoff[r] + (size_t)k * xk];
-            }
-#pragma unroll
-            for (int j = 0; j < NB; j++) wv[j] = weight[((size_t)rows.g * d.NG + min(nb + j, d.NG - 1)) * K + k];
+        const float* const ins[2] = {lower, upper};
+        skinny_sweep<2, RW, NB, VEC>(ins, weight, rows, d, nb, tid, [&](int, const float (&xv)[2][RW], const float (&wv)[NB]) {
 #pragma unroll
             for (int r = 0; r < RW; r++)
 #pragma unroll
                 for (int j = 0; j < NB; j++) {
-                    const float tl = lv[r] - wv[j], tu = uv[r] - wv[j];
+                    const float tl = xv[0][r] - wv[j], tu = xv[1][r] - wv[j];
                     const float al = __builtin_fabsf(tl), au = __builtin_fabsf(tu);
                     up[r][j] = __builtin_fmaxf(up[r][j], __builtin_fmaxf(al, au));
                     if (!(tl < 0.f && tu > 0.f)) lo[r][j] = __builtin_fmaxf(lo[r][j], __builtin_fminf(al, au));
                 }
-        }
+        });
 #pragma unroll
         for (int r = 0; r < RW; r++)
 #pragma unroll
@@ -201,9 +193,18 @@ hipError_t bound_forward(const float* lower, const float* upper, const float* we
                          float* out_upper, const Problem& pr, hipStream_t stream) {
     if (pr.NG <= kSkinnyMaxNG) {
         const Dims d = make_dims(pr);
-        constexpr int RW = 2;
-        hipLaunchKernelGGL((bound_forward_skinny_kernel<RW, 8>), dim3(skinny_grid(d, RW)), dim3(256), 0, stream, lower,
-                           upper, weight, out_lower, out_upper, d);
+        const bool vec = pr.HW == 1 && pr.K % 4 == 0 && aligned16(lower) && aligned16(upper) && aligned16(weight);
+#define LDIST_LAUNCH_RW(RW, NB, VEC)                                                                                          \
+    hipLaunchKernelGGL((bound_forward_skinny_kernel<RW, NB, VEC>), dim3(skinny_grid(d, RW)), dim3(256), 0, stream, lower, \
+                       upper, weight, out_lower, out_upper, d)
+        // two rows per workgroup share the weight loads; with few rows (up to eight per CU) one each: more workgroups hide more latency
+#define LDIST_LAUNCH_1(NB, VEC) LDIST_LAUNCH_RW(1, NB, VEC)
+#define LDIST_LAUNCH_2(NB, VEC) LDIST_LAUNCH_RW(2, NB, VEC)
+        if ((long)d.M * d.G <= 8L * pr.num_cu) LDIST_SKINNY_DISPATCH(pr.NG, vec, LDIST_LAUNCH_1);
+        else LDIST_SKINNY_DISPATCH(pr.NG, vec, LDIST_LAUNCH_2);
+#undef LDIST_LAUNCH_1
+#undef LDIST_LAUNCH_2
+#undef LDIST_LAUNCH_RW
         return hipGetLastError();
     }
     return dispatch_forward<BoundForward>(pr, can_vec4(pr, lower, upper, weight),

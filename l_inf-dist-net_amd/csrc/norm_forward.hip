@@ -343,7 +343,7 @@ constexpr float kSparseMinP = 128.f;
 
 // Few outputs per group: two passes over k, first the exact maximum per (row, output),
 // then the sum of (|x-w| / max)^p; lanes split k in both.
-template <int RW, int NB>
+template <int RW, int NB, bool VEC>
 __global__ void __launch_bounds__(256)
 norm_forward_skinny_kernel(const float* __restrict__ input, const float* __restrict__ weight,
                            float* __restrict__ output, float p, Dims d) {
@@ -352,7 +352,6 @@ norm_forward_skinny_kernel(const float* __restrict__ input, const float* __restr
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     SkinnyRows<RW> rows;
     rows.init(d);
-    const int K = d.K, xk = d.HW;
     for (int nb = 0; nb < d.NG; nb += NB) {
         float acc[RW][NB], rmx[RW][NB];
         // pass 0: maximum; pass 1: power sum
@@ -361,21 +360,17 @@ norm_forward_skinny_kernel(const float* __restrict__ input, const float* __restr
             for (int r = 0; r < RW; r++)
 #pragma unroll
                 for (int j = 0; j < NB; j++) acc[r][j] = 0.f;
-            for (int k = tid; k < K; k += 256) {
-                float xv[RW], wv[NB];
-#pragma unroll
-                for (int r = 0; r < RW; r++) xv[r] = input[rows.xoff[r] + (size_t)k * xk];
-#pragma unroll
-                for (int j = 0; j < NB; j++) wv[j] = weight[((size_t)rows.g * d.NG + min(nb + j, d.NG - 1)) * K + k];
+            const float* const ins[1] = {input};
+            skinny_sweep<1, RW, NB, VEC>(ins, weight, rows, d, nb, tid, [&](int, const float (&xv)[1][RW], const float (&wv)[NB]) {
 #pragma unroll
                 for (int r = 0; r < RW; r++)
 #pragma unroll
                     for (int j = 0; j < NB; j++) {
-                        const float a = __builtin_fabsf(xv[r] - wv[j]);
+                        const float a = __builtin_fabsf(xv[0][r] - wv[j]);
                         if (pass == 0) acc[r][j] = __builtin_fmaxf(acc[r][j], a);
                         else acc[r][j] += pow_pos(a * rmx[r][j], p);
                     }
-            }
+            });
 #pragma unroll
             for (int r = 0; r < RW; r++)
 #pragma unroll
@@ -442,9 +437,18 @@ hipError_t norm_forward(const float* input, const float* weight, float* output, 
                         hipStream_t stream) {
     if (pr.NG <= kSkinnyMaxNG) {
         const Dims d = make_dims(pr);
-        constexpr int RW = 2;
-        hipLaunchKernelGGL((norm_forward_skinny_kernel<RW, 8>), dim3(skinny_grid(d, RW)), dim3(256), 0, stream, input,
-                           weight, output, p, d);
+        const bool vec = pr.HW == 1 && pr.K % 4 == 0 && aligned16(input) && aligned16(weight);
+#define LDIST_LAUNCH_RW(RW, NB, VEC)                                                                                        \
+    hipLaunchKernelGGL((norm_forward_skinny_kernel<RW, NB, VEC>), dim3(skinny_grid(d, RW)), dim3(256), 0, stream, input, \
+                       weight, output, p, d)
+        // two rows per workgroup share the weight loads; with few rows (up to eight per CU) one each: more workgroups hide more latency
+#define LDIST_LAUNCH_1(NB, VEC) LDIST_LAUNCH_RW(1, NB, VEC)
+#define LDIST_LAUNCH_2(NB, VEC) LDIST_LAUNCH_RW(2, NB, VEC)
+        if ((long)d.M * d.G <= 8L * pr.num_cu) LDIST_SKINNY_DISPATCH(pr.NG, vec, LDIST_LAUNCH_1);
+        else LDIST_SKINNY_DISPATCH(pr.NG, vec, LDIST_LAUNCH_2);
+#undef LDIST_LAUNCH_1
+#undef LDIST_LAUNCH_2
+#undef LDIST_LAUNCH_RW
         return hipGetLastError();
     }
     return dispatch_forward<NormForward>(pr, can_vec4(pr, input, weight), can_vec4_out(pr, output), stream, input,

@@ -28,6 +28,65 @@ struct SkinnyRows {
     }
 };
 
+// One walk over k for the lane: f(k, x[NX][RW], w[NB]) for every k of the lane, ascending; NX input tensors of
+// one shape (the point, or the lower and upper ends of a box, or all three).
+// VEC (fc layout, K % 4 == 0, 16-byte aligned tensors): a lane takes four consecutive k per trip with
+// 128-bit loads -- a quarter of the load instructions, in kernels that wait for memory.  Outputs past
+// the group's last one repeat it (their results are never written).
+template <int NX, int RW, int NB, bool VEC, class F>
+__device__ __forceinline__ void skinny_sweep(const float* const (&input)[NX], const float* __restrict__ weight,
+                                             const SkinnyRows<RW>& rows, const Dims& d, int nb, int tid, F&& f) {
+    const int K = d.K;
+    const float* wrow[NB];
+#pragma unroll
+    for (int j = 0; j < NB; j++) wrow[j] = weight + ((size_t)rows.g * d.NG + min(nb + j, d.NG - 1)) * K;
+    if constexpr (VEC) {
+        for (int k = tid * 4; k < K; k += 1024) {
+            float4 xq[NX][RW], wq[NB];
+#pragma unroll
+            for (int q = 0; q < NX; q++)
+#pragma unroll
+                for (int r = 0; r < RW; r++) xq[q][r] = *reinterpret_cast<const float4*>(input[q] + rows.xoff[r] + k);
+#pragma unroll
+            for (int j = 0; j < NB; j++) wq[j] = *reinterpret_cast<const float4*>(wrow[j] + k);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                float xv[NX][RW], wv[NB];
+#pragma unroll
+                for (int q = 0; q < NX; q++)
+#pragma unroll
+                    for (int r = 0; r < RW; r++)
+                        xv[q][r] = e == 0 ? xq[q][r].x : e == 1 ? xq[q][r].y : e == 2 ? xq[q][r].z : xq[q][r].w;
+#pragma unroll
+                for (int j = 0; j < NB; j++) wv[j] = e == 0 ? wq[j].x : e == 1 ? wq[j].y : e == 2 ? wq[j].z : wq[j].w;
+                f(k + e, xv, wv);
+            }
+        }
+    } else {
+        const int xk = d.HW;
+        for (int k = tid; k < K; k += 256) {
+            float xv[NX][RW], wv[NB];
+#pragma unroll
+            for (int q = 0; q < NX; q++)
+#pragma unroll
+                for (int r = 0; r < RW; r++) xv[q][r] = input[q][rows.xoff[r] + (size_t)k * xk];
+#pragma unroll
+            for (int j = 0; j < NB; j++) wv[j] = wrow[j][k];
+            f(k, xv, wv);
+        }
+    }
+}
+
+// Calls LAUNCH(NB, VEC) with the smallest NB in {4, 8, 12, 16} that holds all outputs of a group in one
+// pass over k (the 10-way head: 12).  vec: see skinny_sweep.
+#define LDIST_SKINNY_DISPATCH(ng, vec, LAUNCH)                                     \
+    do {                                                                           \
+        if ((ng) <= 4) { if (vec) LAUNCH(4, true); else LAUNCH(4, false); }        \
+        else if ((ng) <= 8) { if (vec) LAUNCH(8, true); else LAUNCH(8, false); }   \
+        else if ((ng) <= 12) { if (vec) LAUNCH(12, true); else LAUNCH(12, false); } \
+        else { if (vec) LAUNCH(16, true); else LAUNCH(16, false); }                \
+    } while (0)
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) v = __builtin_fmaxf(v, __shfl_xor(v, off, 64));

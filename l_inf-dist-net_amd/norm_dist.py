@@ -309,7 +309,7 @@ class NormDistConv(nn.Module):
         return t
 
     # Outputs per group up to which the one-pass kernel for values and bounds beats the two separate kernels (the
-    # head of the 5120-wide net at batch 1024: 65 us against 39 + 57 us and six elementwise shifts).  For wide layers
+    # head of the 5120-wide net at batch 1024: 31 us against 24 + 28 us and six elementwise shifts).  For wide layers
     # it is slower: one pass holds three accumulator sets and cannot pair the values in one v_max3 (4.6 ms against
     # 1.25 + 2.67 ms on 1024 x 5120 -> 5120).
     FUSED_VALUE_BOUND_MAX_OUTPUTS = 16
