@@ -160,9 +160,15 @@ __global__ void __launch_bounds__(256)
 inf_backward_weight_kernel(const float* __restrict__ grad_output, const int32_t* __restrict__ pos,
                            float* __restrict__ grad_weight, BwdDims d, int NB, int KC, int n_blocks, int b_per_wg) {
     extern __shared__ float bins[];
-    const int nblk = blockIdx.x % n_blocks;
+    // Neighbouring blocks of outputs read neighbouring few-byte pieces of the same memory lines (in the fc layout a
+    // block's grad_output / pos entries of one image are NB * 4 bytes).  Workgroups go to the eight XCDs in turn, each
+    // with its own L2, so XCD x takes the x-th eighth of the blocks: neighbours then share the lines in one L2
+    // instead of fetching them eight times.  n_blocks is rounded up to a multiple of eight by the launcher.
+    const int id = blockIdx.x % n_blocks;
     const int g = blockIdx.x / n_blocks;
+    const int nblk = (id % 8) * (n_blocks / 8) + id / 8;
     const int n0 = nblk * NB;
+    if (n0 >= d.NG) return;
     const int nb = min(NB, d.NG - n0);
     const int k0 = blockIdx.y * KC;
     const int kc = min(KC, d.K - k0);
@@ -183,15 +189,26 @@ inf_backward_weight_kernel(const float* __restrict__ grad_output, const int32_t*
     const size_t first = ((size_t)g * d.NG + n0) * d.HW;
     if (d.HW == 1) {
         // several images per pass: element i -> (image i / nb, output i % nb)
+        // index and gradient of four elements are fetched together: one after the other (the gradient only once the
+        // index says it is wanted) a wave waited out two memory latencies per element
         const int total = (b1 - b0) * nb;
-        for (int i = threadIdx.x; i < total; i += 256) {
-            const int bb = i / nb, nn = i - bb * nb;
-            const size_t o = (size_t)(b0 + bb) * img_stride + first + nn;
-            const int p = pos[o];
-            const int idx = (p & 0x7fffffff) - k0;
-            if (idx >= 0 && idx < kc) {
-                const float gv = grad_output[o];
-                atomicAdd(&bins[nn * kc + idx], p < 0 ? gv : -gv);
+        for (int i0 = threadIdx.x; i0 < total; i0 += 1024) {
+            int p[4], nn[4];
+            float gv[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int i = i0 + 256 * u < total ? i0 + 256 * u : i0;   // past the end: the first one again, not added
+                const int bb = i / nb;
+                nn[u] = i - bb * nb;
+                const size_t o = (size_t)(b0 + bb) * img_stride + first + nn[u];
+                p[u] = pos[o];
+                gv[u] = grad_output[o];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int idx = (p[u] & 0x7fffffff) - k0;
+                if ((u == 0 || i0 + 256 * u < total) && idx >= 0 && idx < kc)
+                    atomicAdd(&bins[nn[u] * kc + idx], p[u] < 0 ? gv[u] : -gv[u]);
             }
         }
     } else {
@@ -300,7 +317,7 @@ hipError_t inf_backward_weight(const float* grad_output, const int32_t* pos, flo
     // grad_output/pos columns for every channel range costs more than the smaller row block.
     const int KC = min(pr.K, kBinFloats);
     const int NB = max(1, min(min(pr.NG, 8), kBinFloats / KC));
-    const int n_blocks = (pr.NG + NB - 1) / NB;
+    const int n_blocks = ((pr.NG + NB - 1) / NB + 7) / 8 * 8;   // a multiple of eight: see the kernel's block order
     const int k_ranges = (pr.K + KC - 1) / KC;
     const long slabs = (long)pr.G * n_blocks * k_ranges;
     // split the images over workgroups only when the slabs alone cannot fill the device
