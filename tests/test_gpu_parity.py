@@ -779,6 +779,57 @@ def test_conv_image_kernels_with_misaligned_tensors():
     torch.testing.assert_close(gi.cpu().double(), expect, rtol=RTOL, atol=1e-5)
 
 
+@pytest.mark.parametrize("shape", [(40, 10, 320, 1, 1), (9, 16, 64, 2, 1), (70, 96, 260, 1, 1), (3, 12, 40, 1, 8)])
+def test_column_kernels_with_misaligned_tensors(shape):
+    """Every tensor 4 bytes off a 16-byte boundary: the tiled and the few-output kernels must leave their 128-bit
+    load and store paths and give the same results as on aligned tensors."""
+    from gpu_common import DEV, cpp
+    B, CO, CI, G, HW = shape
+    x, w = make_inputs(B, CO, CI, G, HW, seed=17 + sum(shape))
+    lo, up = (x - 0.04).contiguous(), (x + 0.04).contiguous()
+    eo, ep = oracle.inf_dist_forward(x, w, G)
+    el, eu = oracle.inf_dist_bound_forward(lo, up, w, G)
+    mis = lambda t: _misaligned(t, DEV)
+    blank = lambda dtype=torch.float32: _misaligned(torch.zeros(B, CO, HW, dtype=dtype), DEV)
+    xd, wd, ld, ud = mis(x), mis(w), mis(lo), mis(up)
+    out, pos = blank(), blank(torch.int32)
+    cpp.inf_dist_forward(xd, wd, out, pos, G)
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu(), eo) and torch.equal(pos.cpu(), ep)
+    ol, ou = blank(), blank()
+    cpp.inf_dist_bound_forward(ld, ud, wd, ol, ou, G)
+    torch.cuda.synchronize()
+    assert torch.equal(ol.cpu(), el) and torch.equal(ou.cpu(), eu)
+    ov, ol, ou = blank(), blank(), blank()
+    cpp.inf_dist_value_bound_forward(xd, ld, ud, wd, ov, ol, ou, G, mis(torch.zeros(CO)), None)
+    torch.cuda.synchronize()
+    assert torch.equal(ov.cpu(), eo) and torch.equal(ol.cpu(), el) and torch.equal(ou.cpu(), eu)
+    for p in (8.0, 150.0):
+        on = blank()
+        cpp.norm_dist_forward(xd, wd, on, G, p)
+        torch.cuda.synchronize()
+        want = oracle.norm_dist_forward(x, w, G, p)
+        torch.testing.assert_close(on.cpu(), want, rtol=RTOL, atol=0)
+        go = torch.randn(B, CO, HW, generator=gen(19))
+        ex, mx = oracle.norm_dist_backward_input(go, x, w, want, G, p, with_abs_terms=True)
+        ew, mw = oracle.norm_dist_backward_weight(go, x, w, want, G, p, with_abs_terms=True)
+        gx, gw = mis(torch.zeros_like(x)), mis(torch.zeros_like(w))
+        cpp.norm_dist_backward_input(mis(go), xd, wd, mis(want), gx, G, p)
+        cpp.norm_dist_backward_weight(mis(go), xd, wd, mis(want), gw, G, p)
+        torch.cuda.synchronize()
+        assert_sum_close(gx.cpu(), ex, mx, p, RTOL, ATOL)
+        assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
+    go = torch.randn(B, CO, HW, generator=gen(20))
+    gx, gw = mis(torch.zeros_like(x)), mis(torch.zeros_like(w))
+    cpp.inf_dist_backward_input_overwrite(mis(go), mis(ep), gx, G)
+    cpp.inf_dist_backward_weight_overwrite(mis(go), mis(ep), gw, G)
+    torch.cuda.synchronize()
+    tx = oracle.inf_dist_backward_input(go.abs(), ep & ~SIGN, CI, G).abs()
+    tw = oracle.inf_dist_backward_weight(go.abs(), ep & ~SIGN, CI, G).abs()
+    assert_sum_close(gx.cpu(), oracle.inf_dist_backward_input(go, ep, CI, G), tx, rtol=RTOL, atol=ATOL)
+    assert_sum_close(gw.cpu(), oracle.inf_dist_backward_weight(go, ep, CI, G), tw, rtol=RTOL, atol=ATOL)
+
+
 def test_conv_net_runs_from_the_image_and_matches_the_column_path():
     """The reference's conv net (3 -> 32 -> 32 -> 64 -> 64 -> 64 channels at width 1) at p = inf: every conv
     layer is covered by the image kernel (resident first layer, staged wide ones, one stride-2 layer); outputs,
