@@ -158,7 +158,7 @@ bound_forward_skinny_kernel(const float* __restrict__ lower, const float* __rest
 #pragma unroll
             for (int j = 0; j < NB; j++) {
                 const float l = wave_max(lo[r][j]), u = wave_max(up[r][j]);
-                if (lane == 0) { sl[wave][r * NB + j] = l; su[wave][r * NB + j] = u; }
+                if (lane == 63) { sl[wave][r * NB + j] = l; su[wave][r * NB + j] = u; }
             }
         __syncthreads();
         if (tid < RW * NB) {

@@ -363,9 +363,8 @@ inf_forward_skinny_kernel(const float* __restrict__ input, const float* __restri
             for (int j = 0; j < NB; j++) {
                 float v = best[r][j];
                 int p = bp[r][j];
-#pragma unroll
-                for (int off = 32; off >= 1; off >>= 1) take_better(v, p, __shfl_xor(v, off, 64), __shfl_xor(p, off, 64));
-                if (lane == 0) { sv[wave][r * NB + j] = v; sp[wave][r * NB + j] = p; }
+                wave_best(v, p);
+                if (lane == 63) { sv[wave][r * NB + j] = v; sp[wave][r * NB + j] = p; }
             }
         __syncthreads();
         if (tid < RW * NB) {

@@ -376,7 +376,7 @@ norm_forward_skinny_kernel(const float* __restrict__ input, const float* __restr
 #pragma unroll
                 for (int j = 0; j < NB; j++) {
                     const float v = pass == 0 ? wave_max(acc[r][j]) : wave_sum(acc[r][j]);
-                    if (lane == 0) red[wave][r * NB + j] = v;
+                    if (lane == 63) red[wave][r * NB + j] = v;
                 }
             __syncthreads();
             if (tid < RW * NB) {

@@ -195,7 +195,7 @@ value_bound_forward_skinny_kernel(const float* __restrict__ input, const float* 
 #pragma unroll
             for (int j = 0; j < NB; j++) {
                 const float v = wave_max(val[r][j]), l = wave_max(lo[r][j]), u = wave_max(up[r][j]);
-                if (lane == 0) { sv[wave][r * NB + j] = v; sl[wave][r * NB + j] = l; su[wave][r * NB + j] = u; }
+                if (lane == 63) { sv[wave][r * NB + j] = v; sl[wave][r * NB + j] = l; su[wave][r * NB + j] = u; }
             }
         __syncthreads();
         if (tid < RW * NB) {
