@@ -163,10 +163,11 @@ inf_backward_weight_kernel(const float* __restrict__ grad_output, const int32_t*
     // Neighbouring blocks of outputs read neighbouring few-byte pieces of the same memory lines (in the fc layout a
     // block's grad_output / pos entries of one image are NB * 4 bytes).  Workgroups go to the eight XCDs in turn, each
     // with its own L2, so XCD x takes the x-th eighth of the blocks: neighbours then share the lines in one L2
-    // instead of fetching them eight times.  n_blocks is rounded up to a multiple of eight by the launcher.
+    // instead of fetching them eight times.  Where that matters (many blocks) the launcher rounds n_blocks up to a
+    // multiple of eight; otherwise the blocks keep their order.
     const int id = blockIdx.x % n_blocks;
     const int g = blockIdx.x / n_blocks;
-    const int nblk = (id % 8) * (n_blocks / 8) + id / 8;
+    const int nblk = (n_blocks & 7) == 0 ? (id % 8) * (n_blocks / 8) + id / 8 : id;
     const int n0 = nblk * NB;
     if (n0 >= d.NG) return;
     const int nb = min(NB, d.NG - n0);
@@ -317,9 +318,11 @@ hipError_t inf_backward_weight(const float* grad_output, const int32_t* pos, flo
     // grad_output/pos columns for every channel range costs more than the smaller row block.
     const int KC = min(pr.K, kBinFloats);
     const int NB = max(1, min(min(pr.NG, 8), kBinFloats / KC));
-    const int n_blocks = ((pr.NG + NB - 1) / NB + 7) / 8 * 8;   // a multiple of eight: see the kernel's block order
+    const int real_blocks = (pr.NG + NB - 1) / NB;
+    // many blocks: a multiple of eight, for the kernel's XCD-aware block order (the extra workgroups leave at once)
+    const int n_blocks = real_blocks >= 64 ? (real_blocks + 7) / 8 * 8 : real_blocks;
     const int k_ranges = (pr.K + KC - 1) / KC;
-    const long slabs = (long)pr.G * n_blocks * k_ranges;
+    const long slabs = (long)pr.G * real_blocks * k_ranges;
     // split the images over workgroups only when the slabs alone cannot fill the device
     int splits = 1;
     if (slabs < 2L * pr.num_cu) {
