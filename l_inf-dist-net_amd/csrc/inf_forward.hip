@@ -42,12 +42,12 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
     const float* const ins[1] = {input};
     st.init(ins, weight, d, m0, n0, g, tid);
 
-    float acc[TM][TN];
+    float acc[TM][TN], cm[TM][TN];   // running maximum before / after the current chunk
     int cidx[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++) { acc[i][j] = 0.f; cidx[i][j] = 0; }
+        for (int j = 0; j < TN; j++) { acc[i][j] = 0.f; cm[i][j] = 0.f; cidx[i][j] = 0; }
 
     const int nstage = (K + KK - 1) / KK;
     st.load(0);
@@ -56,11 +56,6 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
     for (int s = 0; s < nstage; s++) {
         const float* stage = lds + (s % NBUF) * STAGE;
         if (s + 1 < nstage) st.load((s + 1) * KK);
-        float cm[TM][TN];
-#pragma unroll
-        for (int i = 0; i < TM; i++)
-#pragma unroll
-            for (int j = 0; j < TN; j++) cm[i][j] = 0.f;
         const float* xp = stage + grp * kChunk * GEO::SM;
         const float* wp = stage + GEO::XS + grp * kChunk * GEO::SN;
         const int c = s * KS + grp;
@@ -92,7 +87,9 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int j = 0; j < TN; j++) {
-                    if (cm[i][j] > acc[i][j]) { acc[i][j] = cm[i][j]; cidx[i][j] = c; }
+                    // cm is never reset: it is the running maximum, so it grew iff this chunk raised it
+                    if (cm[i][j] > acc[i][j]) cidx[i][j] = c;
+                    acc[i][j] = cm[i][j];
                 }
         }
         if (NBUF == 1) __syncthreads();  // everyone is done reading the only buffer
