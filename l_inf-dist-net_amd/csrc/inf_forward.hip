@@ -42,7 +42,7 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
     const float* const ins[1] = {input};
     st.init(ins, weight, d, m0, n0, g, tid);
 
-    float acc[TM][TN], cm[TM][TN];   // running maximum before / after the current chunk
+    float acc[TM][TN], cm[TM][TN];   // running maxima; the stages alternate between them
     int cidx[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; i++)
@@ -53,7 +53,11 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
     st.load(0);
     st.store(lds);
     __syncthreads();
-    for (int s = 0; s < nstage; s++) {
+    // One stage: a k-group sweeps its chunk of the resident panels.  prev holds the running
+    // maximum before the chunk and is left alone; cur continues from it, so the chunk raised the
+    // maximum iff cur > prev afterwards.  The two arrays swap roles from stage to stage, which
+    // saves copying cur back (EXACT keeps everything in prev).
+    auto run_stage = [&](float (&prev)[TM][TN], float (&cur)[TM][TN], int s) {
         const float* stage = lds + (s % NBUF) * STAGE;
         if (s + 1 < nstage) st.load((s + 1) * KK);
         const float* xp = stage + grp * kChunk * GEO::SM;
@@ -68,11 +72,15 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
                     for (int j = 0; j < TN; j++) {
                         const float d0 = __builtin_fabsf(f.x[0][0][i] - f.w[0][j]);
                         const float d1 = __builtin_fabsf(f.x[0][1][i] - f.w[1][j]);
-                        if (d0 > acc[i][j]) { acc[i][j] = d0; cidx[i][j] = k0; }
-                        if (d1 > acc[i][j]) { acc[i][j] = d1; cidx[i][j] = k0 + 1; }
+                        if (d0 > prev[i][j]) { prev[i][j] = d0; cidx[i][j] = k0; }
+                        if (d1 > prev[i][j]) { prev[i][j] = d1; cidx[i][j] = k0 + 1; }
                     }
             });
         } else {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) cur[i][j] = prev[i][j];
             sweep_chunk<GEO, 1, 2>(xp, wp, tx, ty, [&](const Frag<GEO, 1, 2>& f, int) {
 #pragma unroll
                 for (int i = 0; i < TM; i++)
@@ -80,21 +88,33 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
                     for (int j = 0; j < TN; j++) {
                         const float d0 = __builtin_fabsf(f.x[0][0][i] - f.w[0][j]);
                         const float d1 = __builtin_fabsf(f.x[0][1][i] - f.w[1][j]);
-                        cm[i][j] = __builtin_fmaxf(__builtin_fmaxf(cm[i][j], d0), d1);
+                        cur[i][j] = __builtin_fmaxf(__builtin_fmaxf(cur[i][j], d0), d1);
                     }
             });
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
-                for (int j = 0; j < TN; j++) {
-                    // cm is never reset: it is the running maximum, so it grew iff this chunk raised it
-                    if (cm[i][j] > acc[i][j]) cidx[i][j] = c;
-                    acc[i][j] = cm[i][j];
-                }
+                for (int j = 0; j < TN; j++)
+                    if (cur[i][j] > prev[i][j]) cidx[i][j] = c;
         }
         if (NBUF == 1) __syncthreads();  // everyone is done reading the only buffer
         if (s + 1 < nstage) st.store(lds + ((s + 1) % NBUF) * STAGE);
         __syncthreads();
+    };
+    if constexpr (EXACT) {
+        for (int s = 0; s < nstage; s++) run_stage(acc, acc, s);
+    } else {
+        for (int s = 0; s < nstage; s += 2) {
+            run_stage(acc, cm, s);
+            if (s + 1 < nstage) {
+                run_stage(cm, acc, s + 1);
+            } else {
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) acc[i][j] = cm[i][j];
+            }
+        }
     }
 
     // Epilogue, independent of the lane patch: the tile's (value, chunk or k) pairs are parked in
