@@ -399,10 +399,12 @@ def cpu_formula_baseline(wl, target_seconds=5.0):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    # The GPU's clock takes some tens of milliseconds of load to settle: with 5 warm-up steps the
-    # first timed steps of a 2 ms workload still run about 5 % slow.  The defaults cover that.
+    # The GPU's clock takes some tens of milliseconds of load to settle (--settle-ms covers that
+    # for any --warmup); the defaults below are long enough for a stable mean.
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--settle-ms", type=float, default=150.0,
+                    help="untimed set-up: run the workload this long before the warm-up steps so the clock settles")
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c1")
     ap.add_argument("--p", type=float, default=None,
                     help="exponent for --workload c2 (default 8, the configuration; the reference anneals it to 1000)")
@@ -432,6 +434,17 @@ def main():
     kname, flops_of, accept, kdesc, flops_per_op = wl["kernel"]
 
     with KernelTimer(pkg.norm_dist_cpp, torch, kname, flops_of, accept) as kt:
+        # Set-up, before the warm-up proper: keep the GPU under this load until its clock has settled
+        # (after an idle period the first tens of milliseconds run 5-10 % slow), whatever --warmup says.
+        if args.settle_ms > 0:
+            step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            step()
+            torch.cuda.synchronize()
+            one = max(time.perf_counter() - t0, 1e-5)
+            for _ in range(min(5000, int(args.settle_ms * 1e-3 / one) + 1)):   # back to back, no gaps
+                step()
         for _ in range(args.warmup):
             step()
         torch.cuda.synchronize()
