@@ -165,8 +165,12 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
         struct Slot { float4 x, w; int kb; };
         auto issue = [&](int it, Slot& sl) {
             if (it >= NIT) return;                       // the last trip has nothing left to prefetch
-            const int o = it * NGQ + gq;
-            const int ml = o / BN, nl = o - ml * BN;
+            // outputs are walked column by column (all rows of one weight row, then the next): the
+            // 128 touches of a weight row's chunk lines then fall close together in time and partly
+            // hit in the vector cache (short rows most: K = 784 is 25 lines per row)
+            const int q = it * NGQ + gq;
+            const int nl = q / BM, ml = q - nl * BM;
+            const int o = ml * BN + nl;
             const unsigned m = min(m0 + ml, d.M - 1), n = min(n0 + nl, d.NG - 1);
             const int kb = cand_c[o] * kChunk;
             // a lane whose 16 bytes lie past the end of the row reads the chunk's first 16 instead (masked
@@ -177,7 +181,8 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
             sl.w = *reinterpret_cast<const float4*>(wg + (n * (unsigned)K + off));
         };
         auto finish = [&](int it, const Slot& sl) {
-            const int o = it * NGQ + gq;
+            const int qo = it * NGQ + gq;
+            const int o = (qo % BM) * BN + qo / BM;
             const float target = cand_v[o];
             const float d0 = sl.x.x - sl.w.x, d1 = sl.x.y - sl.w.y, d2 = sl.x.z - sl.w.z, d3 = sl.x.w - sl.w.w;
             int q = -1;
