@@ -162,17 +162,10 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
         const float* wg = weight + (size_t)g * d.NG * K;
         // element offsets fit 32 bits: the entry point rejects tensors of 2^31 elements or more
         const unsigned ldx = (unsigned)d.G * K;
-        // Order of the walk over the tile's outputs.  Short rows (at most 64 chunk lines): column by
-        // column, so the BM touches of one weight row's lines fall close together and mostly hit in
-        // the vector cache (K = 784: a quarter less time in this loop).  Long rows have more lines
-        // than touches; there the column walk only spreads the x lines out (13 % more bytes fetched,
-        // same time), so they are walked row by row.
-        const bool by_column = K <= 64 * kChunk;
-        auto walk = [&](int q) { return by_column ? (q % BM) * BN + q / BM : q; };
         struct Slot { float4 x, w; int kb; };
         auto issue = [&](int it, Slot& sl) {
             if (it >= NIT) return;                       // the last trip has nothing left to prefetch
-            const int o = walk(it * NGQ + gq);
+            const int o = it * NGQ + gq;
             const int ml = o / BN, nl = o - ml * BN;
             const unsigned m = min(m0 + ml, d.M - 1), n = min(n0 + nl, d.NG - 1);
             const int kb = cand_c[o] * kChunk;
@@ -184,7 +177,7 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
             sl.w = *reinterpret_cast<const float4*>(wg + (n * (unsigned)K + off));
         };
         auto finish = [&](int it, const Slot& sl) {
-            const int o = walk(it * NGQ + gq);
+            const int o = it * NGQ + gq;
             const float target = cand_v[o];
             const float d0 = sl.x.x - sl.w.x, d1 = sl.x.y - sl.w.y, d2 = sl.x.z - sl.w.z, d3 = sl.x.w - sl.w.w;
             int q = -1;
