@@ -122,7 +122,16 @@ def workload_c0(pkg, torch, dev):
         pkg.norm_dist(x[:rows].contiguous(), w, 1, INF, use_custom_cuda_func=False)
         return rows * 784 * 5120
 
-    return dict(step=step, ops=512 * 784 * 5120, images=512, full_rows=512, cpu=cpu, formula=formula,
+    def check(oracle, stack_check):
+        rep = stack_check.Report()
+        step()
+        torch.cuda.synchronize()
+        ev, ep = oracle.inf_dist_forward(x, w, 1)
+        rep.equal("values", out.cpu(), ev)
+        rep.equal("argmax index and sign", pos.cpu(), ep)
+        return rep
+
+    return dict(step=step, ops=512 * 784 * 5120, images=512, full_rows=512, cpu=cpu, formula=formula, check=check,
                 name="configs[0]: single L_inf-dist fc layer forward, 512 x 784 -> 5120, values + argmax",
                 kernel=("inf_dist_forward", lambda x_, w_, *_: 2 * mnk(x_, w_), lambda *a: True,
                         "inf_forward_kernel (tiled L_inf forward)", 2))
@@ -178,12 +187,19 @@ def mlp_workload(pkg, torch, dev, p):
         out.backward(upstream[:rows].reshape(rows, -1, 1))
         return stack_ops(rows) * (1 if math.isinf(p) else 3)
 
-    return step, cpu, formula
+    def check(oracle, stack_check):
+        # one training step of the whole stack, every layer repeated by the oracle on what the GPU really fed it:
+        # p = inf on the full batch; p-norm (slow on the CPU) on 16 batch rows and 32 weight rows per layer
+        if math.isinf(p):
+            return stack_check.check_training_step(model, x, upstream, p, dev)
+        return stack_check.check_training_step(model, x, upstream, p, dev, rows=slice(100, 116), weight_rows=slice(64, 96))
+
+    return step, cpu, formula, check
 
 
 def workload_c1(pkg, torch, dev):
-    step, cpu, formula = mlp_workload(pkg, torch, dev, INF)
-    return dict(step=step, ops=stack_ops(512), images=512, full_rows=512, cpu=cpu, formula=formula,
+    step, cpu, formula, check = mlp_workload(pkg, torch, dev, INF)
+    return dict(step=step, ops=stack_ops(512), images=512, full_rows=512, cpu=cpu, formula=formula, check=check,
                 name="configs[1]: 5-layer L_inf-dist MLP 3072-5120-5120-5120-5120-10, p=inf, batch 512, "
                      "forward+backward (all grad_x and grad_w), mean shift in training mode",
                 kernel=("inf_dist_forward", lambda x_, w_, *_: 2 * mnk(x_, w_),
@@ -219,8 +235,8 @@ C2_P = 8.0   # --p moves it along the reference's annealing schedule (8 ... 1000
 
 
 def workload_c2(pkg, torch, dev):
-    step, cpu, formula = mlp_workload(pkg, torch, dev, C2_P)
-    return dict(step=step, ops=3 * stack_ops(512), images=512, full_rows=512, cpu=cpu, formula=formula,
+    step, cpu, formula, check = mlp_workload(pkg, torch, dev, C2_P)
+    return dict(step=step, ops=3 * stack_ops(512), images=512, full_rows=512, cpu=cpu, formula=formula, check=check,
                 name=f"configs[2]: the same MLP at p={C2_P:g}, forward+backward (3 dist-op passes per layer)",
                 kernel=("norm_dist_backward_input", lambda go, x_, w_, *_: 7 * mnk(x_, w_),
                         lambda go, x_, w_, *_: w_.size(0) > 16, "norm_backward_kernel (grad_input)", 7))
@@ -261,7 +277,24 @@ def workload_c3(pkg, torch, dev):
             h, l, u = ((t - m.view(1, -1, 1)).contiguous() for t in (out, ol, ou))
         return 2 * stack_ops(rows)
 
-    return dict(step=step, ops=2 * stack_ops(1024), images=1024, full_rows=1024, cpu=cpu, formula=formula,
+    def check(oracle, stack_check, rows=64):
+        # evaluation mode: rows are independent and the shift by the running mean is one exact subtraction, so the
+        # oracle's free-running pass must reproduce values, both bounds and the certified margins bit for bit
+        rep = stack_check.Report()
+        with torch.no_grad():
+            y, l, u = model(xd[:rows], lod[:rows], upd[:rows])
+            _, res = final(y, l, u, targets[:rows])
+        torch.cuda.synchronize()
+        biases = [None] * 4 + [model.fc_last.bias.detach().cpu()]
+        ey, el, eu, er = stack_check.oracle_certification(ws, means, biases, x[:rows], lo[:rows], up[:rows],
+                                                          targets[:rows].cpu())
+        rep.equal("values", y.cpu(), ey)
+        rep.equal("lower bounds", l.cpu(), el)
+        rep.equal("upper bounds", u.cpu(), eu)
+        rep.equal("certified margins", res.cpu(), er)
+        return rep
+
+    return dict(step=step, ops=2 * stack_ops(1024), images=1024, full_rows=1024, cpu=cpu, formula=formula, check=check,
                 name="configs[3]: interval-bound certification forward through the MLP, batch 1024, eps=8/255: "
                      "value path + lower/upper bounds + certified margins (bound-ops and dist-ops both counted)",
                 kernel=("inf_dist_bound_forward", lambda l_, u_, w_, *_: 6 * mnk(l_, w_),
@@ -319,7 +352,36 @@ def workload_c4(pkg, torch, dev):
         y = pkg.norm_dist(F.unfold(xi, 3, padding=1), wd, 4, INF)
         y.backward(god)
 
-    return dict(step=step, ops=128 * 1024 * 128 * 288, images=128, full_rows=128, cpu=cpu, formula=formula,
+    def check(oracle, stack_check, rows=4):
+        # the first images of the batch (rows are independent; grad_weight of a batch subset is a valid problem),
+        # through the column kernels and through the layer that works on the image
+        rep = stack_check.Report()
+        xs, gs = cols[:rows].contiguous(), go[:rows].contiguous()
+        ev, ep = oracle.inf_dist_forward(xs, w, 4)
+        mag = ep & 0x7FFFFFFF
+        egx, mgx = oracle.inf_dist_backward_input(gs, ep, 1152, 4), oracle.inf_dist_backward_input(gs.abs(), mag, 1152, 4)
+        egw, mgw = oracle.inf_dist_backward_weight(gs, ep, 1152, 4), -oracle.inf_dist_backward_weight(gs.abs(), mag, 1152, 4)
+        xs_d = xs.to(dev).requires_grad_(True)
+        w_d = w.to(dev).requires_grad_(True)
+        y = pkg.norm_dist(xs_d, w_d, 4, INF)
+        y.backward(gs.to(dev))
+        rep.equal("columns: values", y.detach().cpu(), ev)
+        rep.ratio("columns: grad_input", stack_check.sum_ratio(xs_d.grad.cpu(), egx, mgx), xs_d.grad.cpu(), egx)
+        rep.ratio("columns: grad_weight", stack_check.sum_ratio(w_d.grad.cpu(), egw, mgw), w_d.grad.cpu(), egw)
+        layer.weight.grad = None
+        xi = imgd[:rows].detach().requires_grad_(True)
+        yi, _, _ = layer(xi)
+        yi.backward(god4[:rows])
+        rep.equal("image: values", yi.detach().cpu().reshape(rows, 128, 1024), ev)
+        egi = F.fold(egx.double(), (32, 32), 3, padding=1)
+        mgi = F.fold(mgx.double(), (32, 32), 3, padding=1)
+        rep.ratio("image: grad_image", stack_check.sum_ratio(xi.grad.cpu(), egi, mgi), xi.grad.cpu(), egi)
+        rep.ratio("image: grad_weight", stack_check.sum_ratio(layer.weight.grad.cpu().reshape(128, 288), egw, mgw),
+                  layer.weight.grad.cpu().reshape(128, 288), egw)
+        layer.weight.grad = None
+        return rep
+
+    return dict(step=step, ops=128 * 1024 * 128 * 288, images=128, full_rows=128, cpu=cpu, formula=formula, check=check,
                 step_alt=[("ms_per_step_from_image", step_from_image),
                           ("ms_per_step_with_torch_unfold_and_fold", step_torch_unfold)],
                 name="configs[4]: unfolded 3x3 L_inf-dist conv layer, batch 128, 128->128 channels, 32x32, groups 4, "
@@ -409,6 +471,8 @@ def main():
     ap.add_argument("--p", type=float, default=None,
                     help="exponent for --workload c2 (default 8, the configuration; the reference anneals it to 1000)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-parity", action="store_true",
+                    help="skip the comparison with the CPU oracle that runs before the timed region (profiler runs)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run three plain 256 MiB device copies, the known-size kernel that "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -432,6 +496,19 @@ def main():
     wl = WORKLOADS[args.workload](pkg, torch, dev)
     step = wl["step"]
     kname, flops_of, accept, kdesc, flops_per_op = wl["kernel"]
+
+    # Parity first, in this process, on this workload's own tensors: a wrong result must not be timed.
+    parity = {"checked": False, "note": "skipped (--no-parity)"}
+    if not args.no_parity:
+        import oracle
+        from oracle import stack_check
+        t0 = time.perf_counter()
+        rep = wl["check"](oracle, stack_check)
+        parity = rep.as_json()
+        parity["seconds"] = round(time.perf_counter() - t0, 1)
+        if not rep.ok:
+            print(json.dumps({"parity": parity}))
+            sys.exit("bench.py: the GPU results differ from the CPU oracle; nothing was timed")
 
     with KernelTimer(pkg.norm_dist_cpp, torch, kname, flops_of, accept) as kt:
         # Set-up, before the warm-up proper: keep the GPU under this load until its clock has settled
@@ -474,6 +551,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_ms": args.settle_ms,
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True,
         "scaling": "weak",
@@ -483,6 +561,7 @@ def main():
         "config": {"workload": wl["name"], "dist_ops_per_step": ops},
         "img_per_s": round(wl["images"] / (ms_per_step * 1e-3), 1),
         "pct_fp32_valu_peak": round(100 * value * 1e9 * flops_per_op / (FP32_PEAK_TFLOPS * 1e12), 2),
+        "parity": parity,
         "roofline": {
             "bound": "mfma",
             "kernel": kdesc + " -- VALU only: a max / power-sum reduction has no multiply-accumulate for MFMA; "
@@ -498,11 +577,11 @@ def main():
             "traffic": None,
         },
     }
-    # HBM bytes per launch of the roofline kernel (c1: average over the step's four tiled forward launches),
-    # from two rocprofv3 --pmc runs of this command (profiles/): FETCH_SIZE x 2.0 (copy-probe factor)
-    # + WRITE_SIZE x 1.0
-    if args.workload in TRAFFIC_BYTES:
-        out["roofline"]["traffic"] = TRAFFIC_BYTES[args.workload]
+    # HBM bytes per launch of the roofline kernel (c1: average over the step's four tiled forward launches), from
+    # two rocprofv3 --pmc runs of this command: FETCH_SIZE and WRITE_SIZE, each scaled by what the counter reads for
+    # a plain copy of known size.  The figure is read from the counter summary kept under profiles/, which names
+    # the kernel it was measured on; null when there is no summary for this workload's kernel.
+    out["roofline"]["traffic"], out["roofline"]["traffic_source"] = profile_traffic(args.workload)
     for label, alt in wl.get("step_alt", []):
         for _ in range(args.warmup):
             alt()
@@ -518,7 +597,20 @@ def main():
     print(json.dumps(out))
 
 
-TRAFFIC_BYTES = {"c1": 3.20e8, "c4i": 2.15e8}
+TRAFFIC_PROFILES = {"c1": "inf_forward_c1_mlp.md", "c1t": "inf_forward_c1_mlp.md", "c4": "inf_forward_c4_columns.md",
+                    "c4i": "inf_conv_forward_c4_from_image.md"}
+
+
+def profile_traffic(workload):
+    """(bytes per launch, source file) from the line 'traffic_bytes_per_launch: <number>' of the workload's
+    counter summary under profiles/, or (None, None)."""
+    import re
+    name = TRAFFIC_PROFILES.get(workload)
+    path = os.path.join(ROOT, "profiles", name) if name else None
+    if not path or not os.path.exists(path):
+        return None, None
+    m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", open(path).read(), re.M)
+    return (float(m.group(1)), "profiles/" + name) if m else (None, None)
 
 
 if __name__ == "__main__":

@@ -94,6 +94,115 @@ def test_config2_pnorm_layer_rows_and_invariants():
     assert_sum_close(gw.cpu(), ew, mw, p)
 
 
+@pytest.mark.parametrize("ci", [3072, 5120])
+def test_config2_backward_at_the_full_batch(ci):
+    """Both p-norm gradients on the GPU at batch 512 (the launches the benchmark makes: 64-row tiles for
+    grad_input, the reduction over all 512 rows for grad_weight), compared with the oracle on 16 rows of
+    grad_input (rows are independent) and 32 rows of grad_weight over all 512 images (each weight row is an
+    independent reduction).  Reference: model/norm_dist_cuda.cu:299-425."""
+    from gpu_common import DEV, cpp, gpu_norm_forward, say
+    say("config 2 layer backward at batch 512:", ci, "-> 5120, p = 8")
+    p = 8.0
+    x, w = _layer(512, ci, 5120, seed=40 + ci)
+    x = ((x - 0.47) / 0.2009).contiguous()
+    out = gpu_norm_forward(x, w, 1, p)
+    go = torch.randn(512, 5120, 1, generator=gen(41))
+    gx = torch.empty(512, ci, 1, device=DEV)
+    gw = torch.zeros(5120, ci, device=DEV)
+    args = (go.to(DEV), x.to(DEV), w.to(DEV), out.to(DEV))
+    cpp.norm_dist_backward_input(*args, gx, 1, p)
+    cpp.norm_dist_backward_weight(*args, gw, 1, p)
+    torch.cuda.synchronize()
+    gx, gw = gx.cpu(), gw.cpu()
+    for rows in (slice(100, 116), slice(496, 512)):
+        ex, mx = oracle.norm_dist_backward_input(go[rows].contiguous(), x[rows].contiguous(), w, out[rows].contiguous(), 1, p,
+                                                 with_abs_terms=True)
+        say("  grad_input rows", rows.start, "worst err/bound", round(assert_sum_close(gx[rows], ex, mx, p), 3))
+    for n0 in (0, 2077, 5088):
+        cols = slice(n0, n0 + 32)
+        ew, mw = oracle.norm_dist_backward_weight(go[:, cols].contiguous(), x, w[cols].contiguous(),
+                                                  out[:, cols].contiguous(), 1, p, with_abs_terms=True)
+        say("  grad_weight rows", n0, "worst err/bound", round(assert_sum_close(gw[cols], ew, mw, p), 3))
+    # whole-tensor invariant (Euler: the norm is homogeneous of degree one in (x, w)):
+    # sum x*grad_x + sum w*grad_w = sum g*out
+    lhs = float((x.double().squeeze(-1) * gx.double().squeeze(-1)).sum() + (w.double() * gw.double()).sum())
+    rhs = float((go.double() * out.double()).sum())
+    scale = float((go.double() * out.double()).abs().sum())
+    assert abs(lhs - rhs) <= 1e-5 * scale, (lhs, rhs, scale)
+
+
+def _bench_mlp(p, train, batch):
+    """The benchmark's own net, weights and inputs (bench.py: configs 1-3)."""
+    import bench
+    from gpu_common import DEV, pkg
+    g = torch.Generator().manual_seed(0)
+    img = torch.rand(batch, 3, 32, 32, generator=g)
+    ws = bench.stack_weights(g)
+    model = bench.build_mlp(pkg, ws, DEV, p, train=train)
+    return bench, model, img, ws, g
+
+
+def test_config1_whole_stack_training_step():
+    """The whole 5-layer net of config 1 (training-mode mean shift, head as the benchmark builds it), one forward +
+    backward on the GPU; every layer repeated by the oracle on what the GPU fed it (values bit-exact, both scatter
+    gradients within the float32-sum tolerance), and the oracle's own free-running stack against the last output.
+    Reference: model/mlp.py:17-23, model/norm_dist.py:85-96."""
+    from gpu_common import DEV, say
+    from oracle import stack_check
+    say("config 1: whole stack, batch 512, p = inf")
+    bench, model, img, ws, g = _bench_mlp(float("inf"), True, 512)
+    upstream = torch.randn(512, 10, generator=g)
+    rep = stack_check.check_training_step(model, bench.normalise(img), upstream, float("inf"), DEV)
+    say("  ", rep.as_json())
+    for what, d in rep.details.items():
+        say("   worst element of", what, d)
+    assert rep.ok, rep.failures
+    assert rep.exact == 5 and rep.toleranced >= 15
+
+
+def test_config2_whole_stack_training_step():
+    """Config 2 (p = 8) through the whole net: every layer's forward on 16 batch rows, grad_input on the same rows and
+    32 weight rows of grad_weight over the whole batch against the oracle, on the tensors the GPU really fed the layer."""
+    from gpu_common import DEV, say
+    from oracle import stack_check
+    say("config 2: whole stack, batch 512, p = 8")
+    bench, model, img, ws, g = _bench_mlp(8.0, True, 512)
+    upstream = torch.randn(512, 10, generator=g)
+    rep = stack_check.check_training_step(model, bench.normalise(img), upstream, 8.0, DEV, rows=slice(100, 116),
+                                          weight_rows=slice(64, 96))
+    say("  ", rep.as_json())
+    assert rep.ok, rep.failures
+
+
+def test_config3_whole_certification_pass_with_margins():
+    """Config 3 end to end: values, lower and upper bounds through the five layers in evaluation mode (running means
+    subtracted) and the certified margins of BoundFinalIdentity, bit for bit against the oracle's own pass
+    (rows are independent in evaluation mode: 96 of the 1024 rows).  Reference: model/bound_module.py:95-103."""
+    from gpu_common import DEV, pkg, say
+    from oracle import stack_check
+    say("config 3: whole certification pass, batch 1024 (96 rows compared)")
+    bench, model, img, ws, g = _bench_mlp(float("inf"), False, 1024)
+    means = [torch.randn(o, generator=g) * 0.1 for o in bench.LAYERS[1:]]
+    with torch.no_grad():
+        for layer, m in zip(list(model.fc) + [model.fc_last], means):
+            layer.normalize.running_mean.copy_(m)
+        model.fc_last.bias.copy_(torch.randn(10, generator=g) * 0.05)
+    targets = torch.randint(0, 10, (1024,), generator=g)
+    x, lo, up = (bench.normalise(t) for t in (img, (img - bench.EPS).clamp(0, 1), (img + bench.EPS).clamp(0, 1)))
+    with torch.no_grad():
+        y, l, u = model(x.to(DEV), lo.to(DEV), up.to(DEV))
+        _, res = pkg.BoundFinalIdentity()(y, l, u, targets.to(DEV))
+    torch.cuda.synchronize()
+    rows = slice(400, 496)
+    biases = [None] * 4 + [model.fc_last.bias.detach().cpu()]
+    ey, el, eu, er = stack_check.oracle_certification(ws, means, biases, x[rows], lo[rows], up[rows], targets[rows])
+    assert torch.equal(y.cpu()[rows], ey) and torch.equal(l.cpu()[rows], el) and torch.equal(u.cpu()[rows], eu)
+    assert torch.equal(res.cpu()[rows], er)
+    # on the whole batch: the value lies inside its bounds and the target's margin is zero
+    assert bool((l <= y).all()) and bool((y <= u).all())
+    assert bool((res.cpu().gather(1, targets.view(-1, 1)) == 0).all())
+
+
 def test_config3_bound_layer():
     from gpu_common import gpu_bound_forward, gpu_inf_forward, say
     say("config 3 layer: 1024 x 5120 -> 5120 bounds")

@@ -377,3 +377,74 @@ def test_train_step_and_accuracy_helpers():
         last, acc = pkg.train_step(net, loss_fun, opt, x, y)
     assert last < first and 0.0 <= acc <= 1.0
     assert pkg.cal_acc(torch.tensor([[0.1, 0.9], [0.8, 0.2]]), torch.tensor([1, 1])).tolist() == [1.0, 0.0]
+
+
+@pytest.mark.parametrize("p", [float("inf"), 8.0])
+def test_stack_checker_passes_on_a_correct_net_and_catches_a_wrong_one(fake_native, p):
+    """The whole-stack checker (oracle/stack_check.py) on a small MLP on the CPU, native calls faked by the oracle:
+    it must accept the correct net, and must notice a layer whose gradient routing or values were tampered with."""
+    from oracle import stack_check
+    torch.manual_seed(5)
+    model = pkg.MLP(depth=3, width=1, input_dim=24, num_classes=10, head_mean_normalize=True)
+    import l_inf_dist_net_amd.mlp as mlp_mod
+    pkg.set_p_norm(model, p)
+    model.train()
+    x = torch.rand(12, 24, generator=gen(1))
+    up = torch.randn(12, 10, generator=gen(2))
+    rep = stack_check.check_training_step(model, x, up, p, torch.device("cpu"))
+    assert rep.ok, rep.failures
+    assert rep.toleranced >= 9 and (rep.exact == 3 if math.isinf(p) else rep.exact == 0)
+
+    # a wrong operator: values off by one ulp-sized factor in one layer
+    good = cpp.inf_dist_forward if math.isinf(p) else cpp.norm_dist_forward
+
+    def off_values(*a):
+        good(*a)
+        a[2].mul_(1.0 + 3e-5)
+    name = "inf_dist_forward" if math.isinf(p) else "norm_dist_forward"
+    setattr(cpp, name, off_values)
+    try:
+        bad = stack_check.check_training_step(model, x, up, p, torch.device("cpu"))
+    finally:
+        setattr(cpp, name, good)
+    assert not bad.ok and any("values" in f for f in bad.failures)
+
+    # a wrong gradient: grad_weight scaled
+    wname = "inf_dist_backward_weight_overwrite" if math.isinf(p) else "norm_dist_backward_weight"
+    good_w = getattr(cpp, wname)
+
+    def off_grad(*a):
+        good_w(*a)
+        (a[2] if math.isinf(p) else a[4]).mul_(1.001)
+    setattr(cpp, wname, off_grad)
+    try:
+        bad = stack_check.check_training_step(model, x, up, p, torch.device("cpu"))
+    finally:
+        setattr(cpp, wname, good_w)
+    assert not bad.ok and any("grad_weight" in f for f in bad.failures)
+
+
+def test_oracle_certification_matches_the_modules(fake_native):
+    """oracle_certification (the free-running evaluation pass with margins) against the package's own MLP +
+    BoundFinalIdentity driven by the faked native calls: same arithmetic, bit for bit."""
+    from oracle import stack_check
+    torch.manual_seed(6)
+    model = pkg.MLP(depth=3, width=1, input_dim=24, num_classes=10, head_mean_normalize=True)
+    pkg.set_p_norm(model, float("inf"))
+    model.eval()
+    layers = list(model.fc) + [model.fc_last]
+    with torch.no_grad():
+        for layer in layers:
+            layer.normalize.running_mean.copy_(torch.randn(layer.out_channels) * 0.1)
+        model.fc_last.bias.copy_(torch.randn(10) * 0.1)
+    x = torch.rand(9, 24, generator=gen(3))
+    lo, up = (x - 0.03).clamp(0, 1), (x + 0.03).clamp(0, 1)
+    targets = torch.randint(0, 10, (9,), generator=gen(4))
+    with torch.no_grad():
+        y, l, u = model(x, lo, up)
+        _, res = pkg.BoundFinalIdentity()(y, l, u, targets)
+    ws = [ly.weight.detach().reshape(ly.weight.size(0), -1).contiguous() for ly in layers]
+    means = [ly.normalize.running_mean.clone() for ly in layers]
+    biases = [None, None, model.fc_last.bias.detach()]
+    ey, el, eu, er = stack_check.oracle_certification(ws, means, biases, x, lo, up, targets)
+    assert torch.equal(y, ey) and torch.equal(l, el) and torch.equal(u, eu) and torch.equal(res, er)
