@@ -55,7 +55,9 @@ LDIST_API int ldist_last_hip_error(void);
 /* Testing and tuning knob, no counterpart in the reference: forces the workgroup
  * tiling of the three forward kernels.  -1 = choose by shape (default), 0 = 128x80
  * tile with two k-groups, 1 = 128x64, 2 = 256x32, 3 = 32x32 with eight k-groups.
- * Process-wide; not thread safe. */
+ * 0..3 also keep the L_inf forward of an unfolded-conv layout on the tiled kernels
+ * where it would otherwise take the kernel that holds a tile's whole reduction axis
+ * in LDS (K up to 320).  Process-wide; not thread safe. */
 LDIST_API int ldist_set_tile_override(int choice);
 /* Tuning knob, no counterpart in the reference: 1 (default) orders the tiles of
  * the forward kernels so that each of the 8 XCDs works on one contiguous run of

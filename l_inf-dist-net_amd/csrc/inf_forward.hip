@@ -417,6 +417,9 @@ hipError_t inf_forward(const float* input, const float* weight, float* output, i
 #undef LDIST_LAUNCH_RW
         return hipGetLastError();
     }
+    // unfolded-conv layout with a short reduction: the kernel that keeps the whole K of a tile in LDS
+    if (g_tile_override < 0 && inf_forward_shortk_applicable(pr, input, output, pos))
+        return inf_forward_shortk(input, weight, output, pos, pr, stream);
     return dispatch_forward<InfForward>(pr, can_vec4(pr, input, weight), can_vec4_out(pr, output, pos), stream, input,
                                         weight, output, pos);
 }

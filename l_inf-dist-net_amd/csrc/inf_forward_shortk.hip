@@ -1,5 +1,5 @@
 // L_inf distance forward with argmax for the unfolded-conv layout (HW > 1) when the reduction is short:
-// the whole K of a 32-row x 32-output tile stays in LDS.  Same results, bit for bit, as inf_forward.hip;
+// the whole K of a 64-row x 32-output tile stays in LDS.  Same results, bit for bit, as inf_forward.hip;
 // semantics of the reference kernel model/inf_dist_cuda.cu:10-68.
 //
 // In this layout a recorded 32-wide chunk cannot be read again cheaply at the end (k has stride HW in the
@@ -10,72 +10,111 @@
 // loop ends, the lowest k inside the recorded window is then found from LDS: eight differences per output,
 // once per output instead of once per output and stage.
 //
-// Workgroup: 256 lanes = four waves that split K in four contiguous ranges (a range is a whole number of
-// windows); a wave covers the whole 32 x 32 tile with a 4 x 4 register patch per lane.  The four partial
-// results meet in LDS in ascending order of k ("strictly larger wins"), which keeps the lowest k on ties.
-// LDS: X[k][32 rows] and W[k][32 outputs] (k-major), plus 6 KB for the merge.  The input is row-contiguous in
-// memory and goes in with 128-bit stores.  The weights are read along k with coalesced 32-bit loads, four
-// neighbouring outputs per lane, and stored as one 128-bit word whose place in row k is XORed with k % 8
-// (in units of four outputs): the 64 lanes of a store, which differ in k, then cover all banks instead of
-// four.  K = 288 (a 3x3 window over 32 channels) takes 78 KB: two workgroups per CU, whose load and compute
-// phases overlap each other.
+// Workgroup: 512 lanes = eight waves, one workgroup per CU, which walks every grid-th tile.  Waves
+// 0..3 take the upper 32 rows of the tile, waves 4..7 the lower 32; the four waves of a half split K in four
+// contiguous ranges (a range is a whole number of windows) and each covers its 32 x 32 half tile with a 4 x 4
+// register patch per lane.  Every wave parks its (value, window) pairs in a slab of its own; after one barrier
+// the lane that finishes an output reads the four pairs in ascending order of k ("strictly larger wins",
+// which keeps the lowest k on ties).
+// LDS: X[k][64 rows] and W[k][32 outputs] (k-major), plus 40 KB of slabs; K = 288 (a 3x3 window over 32
+// channels) takes 148 KB.  The weight panel is loaded once per run of tiles that share it.  The input panel
+// of the next tile is loaded into registers before the current tile's arithmetic and written to LDS after
+// its epilogue, so the loads wait behind a whole tile of arithmetic.  The input is row-contiguous in memory
+// and goes in with 128-bit stores.  The weights are read along k with coalesced 32-bit loads, four
+// neighbouring outputs per lane, and stored as one 128-bit word whose place in row k is XORed with k % 8 (in
+// units of four outputs): the 64 lanes of a store, which differ in k, then cover all banks instead of four.
 #include "fwd_engine.hpp"
 
 namespace ldist {
 
 namespace shortk {
-constexpr int BM = 32, BN = 32, NT = 256, NGROUP = 4, WIN = 8;
+constexpr int BM = 64, BN = 32, NT = 512, NGROUP = 4, WIN = 8;
 constexpr int KQ = NGROUP * WIN;                  // K is padded to a multiple of this
-constexpr int MAX_KP_TWO_PER_CU = 288;            // (2*Kp*32 + 1024)*4 + 2048 bytes <= 80 KB
+constexpr int XROWS = NT / (BM / 4);              // k rows of the input panel that one pass of the workgroup loads
+constexpr int MAXPASS = 10;                       // padded K / 32 the kernel is built for: K <= 320
+static_assert(XROWS == KQ, "one pass loads one padding quantum of k");
 // float offset inside row k of W of the group of four outputs nq (0..7)
 __device__ __forceinline__ constexpr int wslot(int k, int nq) { return ((nq ^ (k & 7)) << 2); }
 inline int padded_k(int K) { return (K + KQ - 1) / KQ * KQ; }
-inline size_t lds_bytes(int Kp) { return ((size_t)2 * Kp * BM + BM * BN) * sizeof(float) + BM * BN * sizeof(uint16_t); }
+// panels, four value slabs (float) and four window slabs (one byte per output: at most 40 windows)
+inline size_t lds_bytes(int Kp) { return ((size_t)Kp * (BM + BN) + NGROUP * BM * BN) * sizeof(float) + NGROUP * BM * BN; }
+// Place of (output n, row m) in the merge area: row-contiguous like the output tensor, with m XORed by a
+// constant of n's group of four, so that the 64 lanes of a wave (8 groups of outputs x 8 groups of rows, 16 bytes
+// each) spread over all banks when they park their patch, instead of over eight 16-byte slots.
+__device__ __forceinline__ constexpr int cslot(int n, int m) {
+    return n * BM + (m ^ ((((n >> 2) & 7) << 2) | (((n >> 2) & 1) << 5)));
+}
+// Byte offset of (output n, row m) in a window slab: four neighbouring rows share a 32-bit word, words are laid
+// out rows-of-four major with n XORed by two bits of the row group, which spreads a wave's 64 word stores (and
+// the finishing lanes' byte reads) over the banks.
+__device__ __forceinline__ constexpr int bslot(int n, int m) { return (((m >> 2) * BN + (n ^ ((m >> 3) & 3))) << 2) | (m & 3); }
 }  // namespace shortk
 
+// Kp = padded K.  Kp / 32 is the number of windows per k range and also the number of passes in which the
+// workgroup loads an input panel; NP >= Kp / 32 is how many of them the kernel is built for (the loads are
+// issued as one straight run: no branch between them, so nothing waits until the panel is written).
+template <int NP>
 __global__ void __launch_bounds__(shortk::NT, 2)
 inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restrict__ weight,
-                          float* __restrict__ output, int32_t* __restrict__ pos, Dims d, int Kp) {
+                          float* __restrict__ output, int32_t* __restrict__ pos, Dims d, int Kp, int tiles_total) {
     using namespace shortk;
+    const int npass = Kp / KQ, nwin = npass, Kg = Kp / NGROUP;
     extern __shared__ __align__(16) float lds[];
     float* X = lds;                         // [Kp][BM]
     float* W = lds + (size_t)Kp * BM;       // [Kp][BN]
-    float* cand_v = W + (size_t)Kp * BN;    // [BN][BM]: the row index is innermost, like the output tensor
-    uint16_t* cand_w = reinterpret_cast<uint16_t*>(cand_v + BM * BN);
+    float* slab_v = W + (size_t)Kp * BN;    // [NGROUP][BN][BM] values per k range, see cslot(); slab 0 then holds the
+    int* out_p = reinterpret_cast<int*>(slab_v + BM * BN);      // finished values and slab 1 (as integers) the finished pos
+    unsigned char* slab_w = reinterpret_cast<unsigned char*>(slab_v + NGROUP * BM * BN);   // [NGROUP][..] windows, see bslot()
 
     const int tid = threadIdx.x;
-    int id = blockIdx.x;
-    const int tm = id % d.tiles_m;
-    id /= d.tiles_m;
-    const int tn = id % d.tiles_n, g = id / d.tiles_n;
-    const int m0 = tm * BM, n0 = tn * BN;
     const int K = d.K, HW = d.HW;
+    // Workgroup w takes tiles w, w + grid, w + 2 grid, ...: at any time the workgroups then read neighbouring
+    // pieces of the input (with a contiguous run per workgroup they would all sit at the same offset inside
+    // their images, i.e. on the same few memory channels).  Tiles are ordered rows first, so the weight panel
+    // changes only when a workgroup's walk crosses into the next output tile or group.
+    const int t_begin = blockIdx.x, t_step = gridDim.x, t_end = tiles_total;
+    if (t_begin >= t_end) return;           // the whole workgroup leaves together
 
-    // ---- global -> LDS, the whole reduction axis at once -------------------------------------------
-    {
-        // input: a lane keeps its four rows (consecutive positions of one image: HW % 4 == 0) and walks k
-        const int mq = tid % (BM / 4), kx = tid / (BM / 4);
-        const int m = m0 + mq * 4;
-        const bool row_ok = m < d.M;
-        const int b = row_ok ? m / HW : 0, hw = row_ok ? m % HW : 0;
-        const float* xin = input + ((size_t)(b * d.G + g) * K) * HW + hw;
-        // weights: lanes run along k (coalesced 32-bit loads), a lane takes four neighbouring outputs
-        const int npass = Kp / (NT / (BM / 4));   // = Kp / 32 for both panels
-        constexpr int BATCH = 3;
-#pragma unroll 1
-        for (int p0 = 0; p0 < npass; p0 += BATCH) {
-            float4 xv[BATCH], wv[BATCH];
+    // input panel: a lane keeps its four rows (consecutive positions of one image: HW % 4 == 0) and walks k
+    const int lmq = tid % (BM / 4), lkx = tid / (BM / 4);
+    float4 park[NP];
+    // Loads never branch per lane: a lane outside the tensor (rows past M, k past K in the last pass) reads a clamped,
+    // valid address and its value is replaced by 0 when the panel is written.
+    auto x_base = [&](int t) {
+        const int tm = t % d.tiles_m, g = (t / d.tiles_m) / d.tiles_n;
+        const int m = min(tm * BM + lmq * 4, d.M - 4);
+        const int b = m / HW, hw = m % HW;
+        return input + ((size_t)(b * d.G + g) * K) * HW + hw;
+    };
+    auto issue_x = [&](int t) {
+        const float* xin = x_base(t);
 #pragma unroll
-            for (int e = 0; e < BATCH; e++) {
-                const int p = p0 + e;
-                xv[e] = make_float4(0.f, 0.f, 0.f, 0.f);
-                wv[e] = xv[e];
-                if (p < npass) {
-                    const int k = kx + p * (NT / (BM / 4));
-                    if (row_ok && k < K) xv[e] = *reinterpret_cast<const float4*>(xin + (size_t)k * HW);
-                    const int wid = tid + p * NT;            // < Kp * 8
-                    const int kw = wid % Kp, nq = wid / Kp;
-                    const int n = n0 + nq * 4;
+        for (int p = 0; p < NP; p++)   // passes beyond Kp / 32 read row K - 1 again and are dropped
+            park[p] = *reinterpret_cast<const float4*>(xin + (size_t)min(lkx + p * XROWS, K - 1) * HW);
+    };
+    auto store_x = [&](int t) {
+        const bool row_ok = (t % d.tiles_m) * BM + lmq * 4 < d.M;
+#pragma unroll
+        for (int p = 0; p < NP; p++)
+            if (p < npass) {
+                const bool ok = row_ok && lkx + p * XROWS < K;
+                *reinterpret_cast<float4*>(X + (lkx + p * XROWS) * BM + lmq * 4) =
+                    ok ? park[p] : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+    };
+    // weight panel of (group g, output tile tn): lanes run along k, a lane takes four neighbouring outputs
+    auto load_w = [&](int g, int tn) {
+        const int n0 = tn * BN;
+        const int items = Kp * (BN / 4);
+#pragma unroll 1
+        for (int i0 = tid; i0 < items; i0 += 2 * NT) {
+            float4 wv[2];
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                const int i = i0 + e * NT;
+                wv[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (i < items) {
+                    const int kw = i % Kp, n = n0 + (i / Kp) * 4;
                     if (kw < K) {
                         const float* wr = weight + ((size_t)g * d.NG + n) * K + kw;
                         if (n + 0 < d.NG) wv[e].x = wr[0];
@@ -86,166 +125,197 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
                 }
             }
 #pragma unroll
-            for (int e = 0; e < BATCH; e++) {
-                const int p = p0 + e;
-                if (p < npass) {
-                    const int k = kx + p * (NT / (BM / 4));
-                    *reinterpret_cast<float4*>(X + k * BM + mq * 4) = xv[e];
-                    const int wid = tid + p * NT;
-                    const int kw = wid % Kp, nq = wid / Kp;
-                    *reinterpret_cast<float4*>(W + kw * BN + wslot(kw, nq)) = wv[e];
+            for (int e = 0; e < 2; e++) {
+                const int i = i0 + e * NT;
+                if (i < items) {
+                    const int kw = i % Kp;
+                    *reinterpret_cast<float4*>(W + kw * BN + wslot(kw, i / Kp)) = wv[e];
                 }
             }
         }
-    }
-    __syncthreads();
+    };
 
-    // ---- the reduction: wave q takes k in [q*Kg, (q+1)*Kg) -----------------------------------------
-    const int lane = tid & 63, grp = tid >> 6;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int half = wave / NGROUP, grp = wave % NGROUP;
     const int tx = lane % 8, ty = lane / 8;
-    const int Kg = Kp / NGROUP, nwin = Kg / WIN;
-    float accA[4][4], accB[4][4];
-    int widx[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) { accA[i][j] = 0.f; accB[i][j] = 0.f; widx[i][j] = 0; }
-
-    // Operand addresses: row kb + e of a window (kb a multiple of 8) keeps the lane's four outputs at group tx ^ e,
-    // so eight lane constants, added to a pointer that moves by a window at a time, serve the whole loop.
-    const float* xp = X + (size_t)grp * Kg * BM + ty * 4;
-    const float* wp = W + (size_t)grp * Kg * BN;
-    int woff[WIN];
+    int woff[WIN];   // row kb + e of a window (kb % 8 == 0) keeps the lane's four outputs at group tx ^ e
 #pragma unroll
     for (int e = 0; e < WIN; e++) woff[e] = e * BN + ((tx ^ e) << 2);
-    float4 xa[2], wa[2], xb[2], wb[2];
-    auto fetch = [&](float4 (&xf)[2], float4 (&wf)[2], int kk) {   // rows kk, kk + 1 of the current window
-#pragma unroll
-        for (int e = 0; e < 2; e++) {
-            xf[e] = *reinterpret_cast<const float4*>(xp + (kk + e) * BM);
-            wf[e] = *reinterpret_cast<const float4*>(wp + woff[kk + e]);
+
+    // Tile -> global, from slabs 0 and 1: a lane stores four neighbouring rows of one output with 128-bit stores.
+    // A tile's results go out at the start of the next tile, after that tile's input panel has been written to
+    // LDS: the wait for the parked loads (the counter also covers stores) then never waits for stores just issued.
+    auto flush = [&](int t) {
+        const int tm = t % d.tiles_m, wkey = t / d.tiles_m;
+        const int tn = wkey % d.tiles_n, g = wkey / d.tiles_n;
+        const int nl = tid / (BM / 4), mq = tid % (BM / 4);
+        const int o = cslot(nl, mq * 4);
+        const int m = tm * BM + mq * 4, n = tn * BN + nl;
+        if (m < d.M && n < d.NG) {                     // HW % 4 == 0: the four rows lie inside the tensor and one image
+            const int b = m / HW, hw = m % HW;
+            const size_t at = ((size_t)(b * d.G + g) * d.NG + n) * HW + hw;
+            *reinterpret_cast<float4*>(output + at) = *reinterpret_cast<const float4*>(slab_v + o);
+            *reinterpret_cast<int4*>(pos + at) = *reinterpret_cast<const int4*>(out_p + o);
         }
     };
-    // One window: cur continues the running maximum from prev (prev is left alone), so the window raised the
-    // maximum iff cur > prev afterwards.  The arrays swap roles from window to window: nothing is copied.
-    // Four pairs of k; the next pair's operands are fetched while the current pair is reduced, the first pair
-    // of the next window during the last reduction (after the last window that reads rows which belong to the
-    // next range or lie just behind the panel, inside the allocation; they are never used).
-    auto window = [&](const float (&prev)[4][4], float (&cur)[4][4], int wid) {
-        auto reduce = [&](const float4 (&xf)[2], const float4 (&wf)[2], const float (&from)[4][4]) {
-            const float x0[4] = {xf[0].x, xf[0].y, xf[0].z, xf[0].w}, x1[4] = {xf[1].x, xf[1].y, xf[1].z, xf[1].w};
-            const float w0[4] = {wf[0].x, wf[0].y, wf[0].z, wf[0].w}, w1[4] = {wf[1].x, wf[1].y, wf[1].z, wf[1].w};
+
+    int w_loaded = -1;
+    issue_x(t_begin);
+#pragma unroll 1
+    for (int t = t_begin; t < t_end; t += t_step) {
+        const int wkey = t / d.tiles_m;
+        if (wkey != w_loaded) {   // every lane of the previous tile is past its epilogue
+            load_w(wkey / d.tiles_n, wkey % d.tiles_n);
+            w_loaded = wkey;
+        }
+        store_x(t);
+        __syncthreads();
+        if (t > t_begin) {
+            flush(t - t_step);
+            __syncthreads();      // the slabs are read before any wave of this tile parks its patch there
+        }
+        if (t + t_step < t_end) issue_x(t + t_step);   // the next tile's panel, parked in registers until this tile is done
+
+        // ---- the reduction: the wave takes rows half*32.. of the tile and k in [grp*Kg, (grp+1)*Kg) --------
+        float accA[4][4], accB[4][4];
+        int widx[4][4];
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) { accA[i][j] = 0.f; accB[i][j] = 0.f; widx[i][j] = 0; }
+        const float* xp = X + (size_t)grp * Kg * BM + half * 32 + ty * 4;
+        const float* wp = W + (size_t)grp * Kg * BN;
+        float4 xa[2], wa[2], xb[2], wb[2];
+        auto fetch = [&](float4 (&xf)[2], float4 (&wf)[2], int kk) {   // rows kk, kk + 1 of the current window
+#pragma unroll
+            for (int e = 0; e < 2; e++) {
+                xf[e] = *reinterpret_cast<const float4*>(xp + (kk + e) * BM);
+                wf[e] = *reinterpret_cast<const float4*>(wp + woff[kk + e]);
+            }
+        };
+        // One window: cur continues the running maximum from prev (prev is left alone), so the window raised the
+        // maximum iff cur > prev afterwards.  The arrays swap roles from window to window: nothing is copied.
+        // Four pairs of k; the next pair's operands are fetched while the current pair is reduced, the first pair
+        // of the next window during the last reduction (after the last window that reads rows of the next range
+        // or just behind the panel, inside the allocation; they are never used).
+        auto window = [&](const float (&prev)[4][4], float (&cur)[4][4], int wid) {
+            auto reduce = [&](const float4 (&xf)[2], const float4 (&wf)[2], const float (&from)[4][4]) {
+                const float x0[4] = {xf[0].x, xf[0].y, xf[0].z, xf[0].w}, x1[4] = {xf[1].x, xf[1].y, xf[1].z, xf[1].w};
+                const float w0[4] = {wf[0].x, wf[0].y, wf[0].z, wf[0].w}, w1[4] = {wf[1].x, wf[1].y, wf[1].z, wf[1].w};
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        cur[i][j] = __builtin_fmaxf(__builtin_fmaxf(from[i][j], __builtin_fabsf(x0[i] - w0[j])),
+                                                    __builtin_fabsf(x1[i] - w1[j]));
+            };
+            fetch(xb, wb, 2);
+            __builtin_amdgcn_sched_barrier(0);
+            reduce(xa, wa, prev);
+            fetch(xa, wa, 4);
+            __builtin_amdgcn_sched_barrier(0);
+            reduce(xb, wb, cur);
+            fetch(xb, wb, 6);
+            __builtin_amdgcn_sched_barrier(0);
+            reduce(xa, wa, cur);
+            xp += WIN * BM;
+            wp += WIN * BN;
+            fetch(xa, wa, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            reduce(xb, wb, cur);
 #pragma unroll
             for (int i = 0; i < 4; i++)
 #pragma unroll
                 for (int j = 0; j < 4; j++)
-                    cur[i][j] = __builtin_fmaxf(__builtin_fmaxf(from[i][j], __builtin_fabsf(x0[i] - w0[j])),
-                                                __builtin_fabsf(x1[i] - w1[j]));
+                    if (cur[i][j] > prev[i][j]) widx[i][j] = wid;
         };
-        fetch(xb, wb, 2);
-        __builtin_amdgcn_sched_barrier(0);
-        reduce(xa, wa, prev);
-        fetch(xa, wa, 4);
-        __builtin_amdgcn_sched_barrier(0);
-        reduce(xb, wb, cur);
-        fetch(xb, wb, 6);
-        __builtin_amdgcn_sched_barrier(0);
-        reduce(xa, wa, cur);
-        xp += WIN * BM;
-        wp += WIN * BN;
         fetch(xa, wa, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        reduce(xb, wb, cur);
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-                if (cur[i][j] > prev[i][j]) widx[i][j] = wid;
-    };
-    fetch(xa, wa, 0);
-    const int wid0 = grp * nwin;
 #pragma unroll 1
-    for (int w = 0; w < nwin; w += 2) {
-        window(accA, accB, wid0 + w);
-        if (w + 1 < nwin) {
-            window(accB, accA, wid0 + w + 1);
-        } else {
+        for (int w = 0; w < nwin; w += 2) {
+            window(accA, accB, w);
+            if (w + 1 < nwin) {
+                window(accB, accA, w + 1);
+            } else {
 #pragma unroll
-            for (int i = 0; i < 4; i++)
+                for (int i = 0; i < 4; i++)
 #pragma unroll
-                for (int j = 0; j < 4; j++) accA[i][j] = accB[i][j];
+                    for (int j = 0; j < 4; j++) accA[i][j] = accB[i][j];
+            }
         }
-    }
 
-    // ---- the four k ranges meet in LDS, ascending k: a later range wins only with a strictly larger value
-#pragma unroll 1
-    for (int turn = 0; turn < NGROUP; turn++) {
-        if (grp == turn) {
+        // ---- every wave parks its patch in the slab of its k range: values as 128-bit words of four rows, windows
+        // (counted inside the range: they fit a byte) as one word of four rows
+        {
+            float* sv = slab_v + grp * (BM * BN);
+            unsigned* sw = reinterpret_cast<unsigned*>(slab_w + grp * (BM * BN));
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const int o = (tx * 4 + j) * BM + ty * 4;
-                float4 v = make_float4(accA[0][j], accA[1][j], accA[2][j], accA[3][j]);
-                int wsel[4] = {widx[0][j], widx[1][j], widx[2][j], widx[3][j]};
-                if (turn > 0) {
-                    const float4 old = *reinterpret_cast<const float4*>(cand_v + o);
-                    const ushort4 ow = *reinterpret_cast<const ushort4*>(cand_w + o);
-                    if (!(v.x > old.x)) { v.x = old.x; wsel[0] = ow.x; }
-                    if (!(v.y > old.y)) { v.y = old.y; wsel[1] = ow.y; }
-                    if (!(v.z > old.z)) { v.z = old.z; wsel[2] = ow.z; }
-                    if (!(v.w > old.w)) { v.w = old.w; wsel[3] = ow.w; }
-                }
-                *reinterpret_cast<float4*>(cand_v + o) = v;
-                *reinterpret_cast<ushort4*>(cand_w + o) =
-                    make_ushort4((unsigned short)wsel[0], (unsigned short)wsel[1], (unsigned short)wsel[2], (unsigned short)wsel[3]);
+                const int n = tx * 4 + j, m = half * 32 + ty * 4;
+                *reinterpret_cast<float4*>(sv + cslot(n, m)) = make_float4(accA[0][j], accA[1][j], accA[2][j], accA[3][j]);
+                sw[bslot(n, m) >> 2] = (unsigned)widx[0][j] | ((unsigned)widx[1][j] << 8) | ((unsigned)widx[2][j] << 16) |
+                                       ((unsigned)widx[3][j] << 24);
             }
         }
         __syncthreads();
-    }
 
-    // ---- lowest k inside the recorded window, from the panels; a lane takes four neighbouring rows of one output
-    {
-        const int nl = tid / (BM / 4), mq = tid % (BM / 4);
-        const int o = nl * BM + mq * 4;
-        const float4 v4 = *reinterpret_cast<const float4*>(cand_v + o);
-        const ushort4 w4 = *reinterpret_cast<const ushort4*>(cand_w + o);
-        const float vs[4] = {v4.x, v4.y, v4.z, v4.w};
-        const int ws[4] = {w4.x, w4.y, w4.z, w4.w};
-        int ps[4];
+        // ---- an output is finished by one lane: the four ranges in ascending k (a later range wins only with a
+        // strictly larger value), then the lowest k inside the winner's window, from the panels.  Every lane reads a
+        // different window, i.e. other rows of the panels, so lanes must differ in the column they read or they meet
+        // in one bank: lane l of a wave takes row l of the tile and, in round r, output (l + r) % 32 -- 64 different
+        // columns of X and 32 of W.
+        {
+            const int ml = lane;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int kb = ws[i] * WIN;
-            const float* xr = X + kb * BM + mq * 4 + i;
-            const float* wr = W + kb * BN + (nl & 3);
-            float xv[WIN], wv[WIN];
+            for (int rr = 0; rr < BN / (NT / 64); rr++) {
+                const int nl = (lane + wave * (BN / (NT / 64)) + rr) % BN;
+                const int o = cslot(nl, ml), ob = bslot(nl, ml);
+                float v = slab_v[o];
+                int wsel = slab_w[ob];
 #pragma unroll
-            for (int e = 0; e < WIN; e++) { xv[e] = xr[e * BM]; wv[e] = wr[e * BN + wslot(e, nl >> 2)]; }   // kb % 8 == 0
-            int p = 0;
+                for (int q = 1; q < NGROUP; q++) {
+                    const float vq = slab_v[q * (BM * BN) + o];
+                    const int wq = slab_w[q * (BM * BN) + ob] + q * nwin;
+                    if (vq > v) { v = vq; wsel = wq; }
+                }
+                const int kb = wsel * WIN;
+                const float* xr = X + kb * BM + ml;
+                const float* wr = W + kb * BN + (nl & 3);
+                float xv[WIN], wv[WIN];
 #pragma unroll
-            for (int e = WIN - 1; e >= 0; e--) {   // descending: the lowest match is written last
-                const float df = xv[e] - wv[e];
-                if (__builtin_fabsf(df) == vs[i]) p = (kb + e) | (__float_as_int(df) & 0x80000000);
+                for (int e = 0; e < WIN; e++) { xv[e] = xr[e * BM]; wv[e] = wr[e * BN + wslot(e, nl >> 2)]; }   // kb % 8 == 0
+                int p = 0;
+#pragma unroll
+                for (int e = WIN - 1; e >= 0; e--) {   // descending: the lowest match is written last
+                    const float df = xv[e] - wv[e];
+                    if (__builtin_fabsf(df) == v) p = (kb + e) | (__float_as_int(df) & 0x80000000);
+                }
+                slab_v[o] = v;                         // slabs 0 and 1 now carry the tile's results; nobody else reads
+                out_p[o] = v > 0.f ? p : 0;            // these two words.  v == 0: the reference leaves pos = 0
             }
-            ps[i] = vs[i] > 0.f ? p : 0;           // nothing exceeded the initial 0: the reference leaves pos = 0
         }
-        const int m = m0 + mq * 4, n = n0 + nl;
-        if (m < d.M && n < d.NG) {                 // HW % 4 == 0: the four rows lie inside the tensor and one image
-            const int b = m / HW, hw = m % HW;
-            const size_t at = ((size_t)(b * d.G + g) * d.NG + n) * HW + hw;
-            *reinterpret_cast<float4*>(output + at) = v4;
-            *reinterpret_cast<int4*>(pos + at) = make_int4(ps[0], ps[1], ps[2], ps[3]);
-        }
+        __syncthreads();   // the panels are free for the next tile; its results wait in the merge area
     }
+    flush(t_begin + (t_end - 1 - t_begin) / t_step * t_step);
 }
 
 // Whether the kernel above serves the problem: conv layout with rows in aligned groups of four, and a K whose
-// panels leave room for two workgroups per CU (`any_k`: for one as well -- tests and tuning).
-bool inf_forward_shortk_applicable(const Problem& pr, const void* input, const void* output, const void* pos, bool any_k) {
+// panels fit LDS.
+bool inf_forward_shortk_applicable(const Problem& pr, const void* input, const void* output, const void* pos) {
     if (pr.HW == 1 || pr.HW % 4 != 0) return false;
     if (!aligned16(input) || !aligned16(output) || !aligned16(pos)) return false;
     const int Kp = shortk::padded_k(pr.K);
-    if (Kp / shortk::WIN > 65535) return false;                         // window ids are parked as 16-bit
-    if (shortk::lds_bytes(Kp) > 160 * 1024) return false;
-    return any_k || Kp <= shortk::MAX_KP_TWO_PER_CU;
+    return Kp / shortk::XROWS <= shortk::MAXPASS && Kp / (shortk::NGROUP * shortk::WIN) <= 255 &&
+           shortk::lds_bytes(Kp) <= 160 * 1024;
+}
+
+template <int NP>
+static hipError_t launch_shortk(unsigned grid, size_t lds, int device, hipStream_t stream, const float* input,
+                                const float* weight, float* output, int32_t* pos, const Dims& d, int Kp, int tiles) {
+    static bool lds_allowed[64] = {};
+    if (hipError_t e = allow_lds(inf_forward_shortk_kernel<NP>, 160 * 1024, device, lds_allowed); e != hipSuccess) return e;
+    hipLaunchKernelGGL(inf_forward_shortk_kernel<NP>, dim3(grid), dim3(shortk::NT), lds, stream, input, weight, output,
+                       pos, d, Kp, tiles);
+    return hipGetLastError();
 }
 
 hipError_t inf_forward_shortk(const float* input, const float* weight, float* output, int32_t* pos, const Problem& pr,
@@ -255,12 +325,18 @@ hipError_t inf_forward_shortk(const float* input, const float* weight, float* ou
     d.tiles_n = (d.NG + shortk::BN - 1) / shortk::BN;
     const int Kp = shortk::padded_k(pr.K);
     const size_t lds = shortk::lds_bytes(Kp);
-    static bool lds_allowed[64] = {};
-    if (hipError_t e = allow_lds(inf_forward_shortk_kernel, 160 * 1024, pr.device, lds_allowed); e != hipSuccess) return e;
-    const unsigned grid = (unsigned)d.tiles_m * d.tiles_n * d.G;
-    hipLaunchKernelGGL(inf_forward_shortk_kernel, dim3(grid), dim3(shortk::NT), lds, stream, input, weight, output, pos,
-                       d, Kp);
-    return hipGetLastError();
+    // one workgroup per CU
+    const long tiles = (long)d.tiles_m * d.tiles_n * d.G;
+    const unsigned grid = (unsigned)(tiles < pr.num_cu ? tiles : pr.num_cu);
+    const int np = Kp / shortk::KQ;
+#define LDIST_SHORTK(NP) \
+    return launch_shortk<NP>(grid, lds, pr.device, stream, input, weight, output, pos, d, Kp, (int)tiles)
+    if (np <= 2) LDIST_SHORTK(2);
+    if (np <= 4) LDIST_SHORTK(4);
+    if (np <= 6) LDIST_SHORTK(6);
+    if (np <= 9) LDIST_SHORTK(9);
+    LDIST_SHORTK(shortk::MAXPASS);
+#undef LDIST_SHORTK
 }
 
 }  // namespace ldist

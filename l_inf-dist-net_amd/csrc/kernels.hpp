@@ -22,7 +22,8 @@ enum class TileChoice { M128N80K2, M128N64K1, M256N32K1, M32N32K8 };
 // M32N32K8 (512 lanes, eight k-groups of one wave, 4x4 values per lane) is for few rows and outputs with
 // a long reduction (the first fully connected layer behind a conv stack: 128 x 1024 outputs, K = 49152):
 // it makes 80 times more workgroups than the big tiles, at twice their LDS traffic per difference.
-// -1 = choose by shape; 0, 1, 2, 3 force M128N80K2, M128N64K1, M256N32K1, M32N32K8 (tests and tuning).
+// -1 = choose by shape; 0, 1, 2, 3 force M128N80K2, M128N64K1, M256N32K1, M32N32K8 (tests and tuning), which also
+// keeps the L_inf forward of the unfolded-conv layout on the tiled kernels instead of the short-reduction kernel.
 extern int g_tile_override;
 extern int g_xcd_remap;  // 1 (default): XCD-aware tile order; 0: plain order (tuning)
 
@@ -60,6 +61,9 @@ inline hipError_t allow_lds(Kern kern, size_t bytes, int device, bool (&done)[64
 
 hipError_t inf_forward(const float* input, const float* weight, float* output, int32_t* pos, const Problem& pr,
                        hipStream_t stream);
+bool inf_forward_shortk_applicable(const Problem& pr, const void* input, const void* output, const void* pos);
+hipError_t inf_forward_shortk(const float* input, const float* weight, float* output, int32_t* pos, const Problem& pr,
+                              hipStream_t stream);
 hipError_t value_bound_forward(const float* input, const float* lower, const float* upper, const float* weight,
                                const float* mean, const float* bias, float* out, float* out_lower, float* out_upper,
                                const Problem& pr, hipStream_t stream);

@@ -58,6 +58,66 @@ def test_inf_forward_bit_exact(shape, tile, quant):
     assert torch.equal(pos, ep)
 
 
+# B, CO, CI, G, HW -- unfolded-conv layouts for the kernel that keeps a tile's whole reduction axis in LDS
+SHORTK_SHAPES = [
+    (2, 64, 64, 2, 64),       # K = 32: one window per k range
+    (4, 128, 1152, 4, 100),   # the 3x3 conv layer over 32 channels per group (K = 288); rows end inside a tile
+    (3, 40, 27, 1, 36),       # K = 27 (three channels): padded k, outputs end inside a tile (40 = 32 + 8)
+    (2, 20, 100, 1, 16),      # K not a multiple of 8, one output tile with a tail, a single partial row tile
+    (1, 70, 200, 2, 1024),    # 35 outputs per group, a whole 32 x 32 image
+    (5, 33, 9, 1, 4),         # tiny: one group of four rows per image
+    (2, 32, 320, 1, 32),      # K = 320: the longest reduction the kernel takes
+    (70, 64, 96, 2, 64),      # more tiles than CUs: 140 row tiles x 2 groups, runs of tiles that change group
+]
+
+
+@pytest.mark.parametrize("quant", [None, 8])
+@pytest.mark.parametrize("shape", SHORTK_SHAPES)
+def test_inf_forward_short_reduction_kernel_bit_exact(shape, quant):
+    """Values and indices of the LDS-resident short-K kernel (the default for these shapes) against the oracle, with
+    quantised inputs for ties inside and across windows and k ranges; the same shapes through the tiled kernel
+    (override 1) must agree as well."""
+    from gpu_common import gpu_inf_forward, say, set_tile
+    B, CO, CI, G, HW = shape
+    say("inf_forward short-K", shape, "quant", quant)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=7 + sum(shape), quantize=quant)
+    eo, ep = oracle.inf_dist_forward(x, w, G)
+    set_tile(-1)
+    out, pos = gpu_inf_forward(x, w, G)
+    assert torch.equal(out, eo)
+    assert torch.equal(pos, ep)
+    set_tile(1)
+    out, pos = gpu_inf_forward(x, w, G)
+    assert torch.equal(out, eo) and torch.equal(pos, ep)
+
+
+def test_inf_forward_short_reduction_kernel_specials():
+    """NaN never wins, infinities do, an all-equal row gives (0, 0), and the sign bit follows x - w < 0, in the
+    conv layout through the short-K kernel (reference model/inf_dist_cuda.cu:36-43)."""
+    from gpu_common import gpu_inf_forward, set_tile
+    nan, inf = float("nan"), float("inf")
+    g = gen(77)
+    x = torch.rand(2, 24, 8, generator=g)
+    w = torch.randn(20, 24, generator=g) * 0.2
+    x[0, 3, 1] = nan
+    x[0, :, 2] = nan
+    x[1, 5, 0] = inf
+    x[1, 7, 4] = -inf
+    x[1, 9, 4] = inf          # two infinite differences in one row: the lower k wins
+    x[0, :, 5] = 0.25
+    w[2, :] = 0.25            # row 5 of image 0 equals weight row 2 everywhere: value 0, pos 0
+    x[1, :, 6] = 0.0
+    w[4, :] = 0.0
+    w[4, 11] = 0.5            # only k = 11 differs, x - w < 0
+    set_tile(-1)
+    out, pos = gpu_inf_forward(x, w, 1)
+    eo, ep = oracle.inf_dist_forward(x, w, 1, literal=True)
+    assert torch.equal(out, eo) and torch.equal(pos, ep)
+    assert out[0, 2, 5].item() == 0.0 and pos[0, 2, 5].item() == 0
+    assert pos[1, 4, 6].item() == (11 | SIGN)
+    assert pos[1, 0, 4].item() == (7 | SIGN) and out[1, 0, 4].item() == inf
+
+
 def test_inf_forward_known_answers_and_specials():
     from gpu_common import gpu_inf_forward
     nan, inf = float("nan"), float("inf")
