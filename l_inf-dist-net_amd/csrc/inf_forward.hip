@@ -124,21 +124,55 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
     auto slot = [](int ml, int nl) { return CONV ? nl * BM + ml : ml * BN + nl; };
     float* cand_v = lds;
     int* cand_c = reinterpret_cast<int*>(lds) + BM * BN;
+    // A lane's patch comes in runs of four along the contiguous axis of the parking area (four neighbouring
+    // columns in the fc layout, four neighbouring rows in the conv layout): those go through 128-bit LDS accesses,
+    // the fifth column of a 5-wide patch singly.
+    auto merge4 = [&](int o, float (&v)[4], int (&c)[4], bool compare) {
+        if (compare) {   // larger value wins; equal values keep the lower chunk (or k)
+            const float4 ov = *reinterpret_cast<const float4*>(cand_v + o);
+            const int4 oc = *reinterpret_cast<const int4*>(cand_c + o);
+            const float pv[4] = {ov.x, ov.y, ov.z, ov.w};
+            const int pc[4] = {oc.x, oc.y, oc.z, oc.w};
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (!(v[e] > pv[e] || (v[e] == pv[e] && c[e] < pc[e]))) { v[e] = pv[e]; c[e] = pc[e]; }
+        }
+        *reinterpret_cast<float4*>(cand_v + o) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<int4*>(cand_c + o) = make_int4(c[0], c[1], c[2], c[3]);
+    };
 #pragma unroll 1
     for (int turn = 0; turn < KS; turn++) {
         if (grp == turn) {
+            if constexpr (!CONV) {
 #pragma unroll
-            for (int i = 0; i < TM; i++)
+                for (int i = 0; i < TM; i++) {
 #pragma unroll
-                for (int j = 0; j < TN; j++) {
-                    const int o = slot(GEO::row(ty, i), GEO::col(tx, j));
-                    bool take = true;
-                    if (turn > 0) {   // larger value wins; equal values keep the lower chunk (or k)
-                        const float v = cand_v[o];
-                        take = acc[i][j] > v || (acc[i][j] == v && cidx[i][j] < cand_c[o]);
+                    for (int q = 0; q < TN / 4; q++) {
+                        float v[4] = {acc[i][4 * q], acc[i][4 * q + 1], acc[i][4 * q + 2], acc[i][4 * q + 3]};
+                        int c[4] = {cidx[i][4 * q], cidx[i][4 * q + 1], cidx[i][4 * q + 2], cidx[i][4 * q + 3]};
+                        merge4(slot(GEO::row(ty, i), GEO::col(tx, 4 * q)), v, c, turn > 0);
                     }
-                    if (take) { cand_v[o] = acc[i][j]; cand_c[o] = cidx[i][j]; }
+#pragma unroll
+                    for (int j = TN / 4 * 4; j < TN; j++) {
+                        const int o = slot(GEO::row(ty, i), GEO::col(tx, j));
+                        bool take = true;
+                        if (turn > 0) {
+                            const float v = cand_v[o];
+                            take = acc[i][j] > v || (acc[i][j] == v && cidx[i][j] < cand_c[o]);
+                        }
+                        if (take) { cand_v[o] = acc[i][j]; cand_c[o] = cidx[i][j]; }
+                    }
                 }
+            } else {
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int r = 0; r < TM / 4; r++) {
+                        float v[4] = {acc[4 * r][j], acc[4 * r + 1][j], acc[4 * r + 2][j], acc[4 * r + 3][j]};
+                        int c[4] = {cidx[4 * r][j], cidx[4 * r + 1][j], cidx[4 * r + 2][j], cidx[4 * r + 3][j]};
+                        merge4(slot(GEO::row(ty, 4 * r), GEO::col(tx, j)), v, c, turn > 0);
+                    }
+            }
         }
         __syncthreads();
     }
