@@ -81,7 +81,7 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int j = 0; j < TN; j++) cur[i][j] = prev[i][j];
-            sweep_chunk<GEO, 1, 2>(xp, wp, tx, ty, [&](const Frag<GEO, 1, 2>& f, int) {
+            sweep_chunk<GEO, 1, 2, true>(xp, wp, tx, ty, [&](const Frag<GEO, 1, 2>& f, int) {
 #pragma unroll
                 for (int i = 0; i < TM; i++)
 #pragma unroll
