@@ -597,19 +597,24 @@ def main():
     print(json.dumps(out))
 
 
-TRAFFIC_PROFILES = {"c1": "inf_forward_c1_mlp.md", "c1t": "inf_forward_c1_mlp.md", "c4": "inf_forward_c4_columns.md",
-                    "c4i": "inf_conv_forward_c4_from_image.md"}
+# workload -> (counter summary under profiles/, the roofline kernel's name in it)
+TRAFFIC_PROFILES = {"c1": ("counters_c1_mlp_inf.md", "inf_forward_kernel"), "c1t": ("counters_c1_mlp_inf.md", "inf_forward_kernel"),
+                    "c0": ("counters_c0_fc_layer.md", "inf_forward_kernel"),
+                    "c2": ("counters_c2_mlp_p8.md", "norm_backward_kernel"),
+                    "c3": ("counters_c3_certification.md", "bound_forward_kernel"),
+                    "c4": ("counters_c4_conv_columns.md", "inf_forward_shortk_kernel"),
+                    "c4i": ("counters_c4_conv_from_image.md", "inf_conv_forward_kernel")}
 
 
 def profile_traffic(workload):
-    """(bytes per launch, source file) from the line 'traffic_bytes_per_launch: <number>' of the workload's
-    counter summary under profiles/, or (None, None)."""
+    """(bytes per launch, source file) from the line 'traffic_bytes_per_launch[<kernel>]: <number>' of the
+    workload's counter summary under profiles/, or (None, None)."""
     import re
-    name = TRAFFIC_PROFILES.get(workload)
+    name, kernel = TRAFFIC_PROFILES.get(workload, (None, None))
     path = os.path.join(ROOT, "profiles", name) if name else None
     if not path or not os.path.exists(path):
         return None, None
-    m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", open(path).read(), re.M)
+    m = re.search(r"^traffic_bytes_per_launch\[" + re.escape(kernel) + r"\]:\s*([0-9.eE+]+)", open(path).read(), re.M)
     return (float(m.group(1)), "profiles/" + name) if m else (None, None)
 
 

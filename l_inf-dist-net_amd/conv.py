@@ -10,27 +10,32 @@ from .norm_dist import NormDist, NormDistConv
 net_width = 32
 
 
+def _negated(triple):
+    """(-y, -upper, -lower): the net's outputs are negated distances, which exchanges the two bounds."""
+    y, lo, up = triple
+    return [None if t is None else -t for t in (y, up, lo)]
+
+
 class Conv(nn.Module):
+    # (out channels as a multiple of the base width, stride) of the five 3x3 layers
+    PLAN = ((1, 1), (1, 1), (2, 2), (2, 1), (2, 1))
+
     def __init__(self, width, input_dim, hidden=512, num_classes=10):
         super().__init__()
-        pixels = input_dim[1] * input_dim[2]
-        width *= net_width
-        layers = [NormDistConv(input_dim[0], width, 3, bias=False, mean_normalize=True, padding=1),
-                  NormDistConv(width, width, 3, bias=False, mean_normalize=True, padding=1)]
-        pixels //= 4
-        width *= 2
-        layers += [NormDistConv(width // 2, width, 3, bias=False, padding=1, stride=2, mean_normalize=True),
-                   NormDistConv(width, width, 3, bias=False, padding=1, mean_normalize=True),
-                   NormDistConv(width, width, 3, bias=False, padding=1, mean_normalize=True)]
+        base = width * net_width
+        channels, height, wide = input_dim
+        layers, c_in = [], channels
+        for mult, stride in self.PLAN:
+            layers.append(NormDistConv(c_in, mult * base, 3, stride=stride, padding=1, bias=False, mean_normalize=True))
+            c_in = mult * base
+            height, wide = (height + stride - 1) // stride, (wide + stride - 1) // stride
         self.conv = nn.ModuleList(layers)
-        self.fc = NormDist(pixels * width, hidden, bias=False, mean_normalize=True)
+        self.fc = NormDist(height * wide * c_in, hidden, bias=False, mean_normalize=True)
         self.fc_last = NormDist(hidden, num_classes, bias=True, mean_normalize=False)
 
     def forward(self, x, lower=None, upper=None):
-        paras = (x, lower, upper)
+        triple = (x, lower, upper)
         for layer in self.conv:
-            paras = layer(*paras)
-        paras = [None if y is None else y.view(y.size(0), -1) for y in paras]
-        paras = self.fc(*paras)
-        y, lo, up = self.fc_last(*paras)
-        return [None if t is None else -t for t in (y, up, lo)]
+            triple = layer(*triple)
+        flat = [None if t is None else t.flatten(1) for t in triple]
+        return _negated(self.fc_last(*self.fc(*flat)))

@@ -290,15 +290,18 @@ hipError_t bound_conv_forward(const float* lower, const float* upper, const floa
     const size_t lds = (2 * (size_t)a.xwords + 2 * (size_t)kKC * kBNP) * sizeof(float);
     // The dynamic-LDS limit is raised to what the largest launch so far needed, not to the whole 160 KB: the
     // workgroup-wide vote keeps a little static LDS of its own, and the two must fit together.
-    static size_t raised[64][2] = {};
+    static std::atomic<size_t> raised[64][2] = {};   // callers may come from several threads
     const int ki = q.S - 1;
     auto kern = q.S == 1 ? bound_conv_forward_kernel<1> : bound_conv_forward_kernel<2>;
     const int di = device >= 0 && device < 64 ? device : 0;
-    if (lds > raised[di][ki] || di != device) {
+    if (lds > raised[di][ki].load(std::memory_order_acquire) || di != device) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)lds);
         if (e != hipSuccess) return e;
-        if (di == device) raised[di][ki] = lds;
+        if (di == device) {   // keep the largest: another thread may have raised it further meanwhile
+            size_t seen = raised[di][ki].load(std::memory_order_relaxed);
+            while (seen < lds && !raised[di][ki].compare_exchange_weak(seen, lds, std::memory_order_release)) {}
+        }
     }
     const unsigned grid = (unsigned)((long long)q.B * G * a.tiles_h * a.tiles_n);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(a.ML * a.NL), lds, stream, lower, upper, weight, out_lower, out_upper, a);

@@ -181,7 +181,7 @@ struct BoundForward {
                              const float* upper, const float* weight, float* out_lower, float* out_upper) {
         const size_t lds = Stager<GEO, CONV, VEC, 2>::LDS_BYTES;
         auto kern = bound_forward_kernel<GEO, CONV, VEC>;
-        static bool lds_allowed[64] = {};   // per instantiation of this launcher, i.e. per kernel
+        static LdsRecord lds_allowed = {};   // per instantiation of this launcher, i.e. per kernel
         if (hipError_t e = allow_lds(kern, lds, device, lds_allowed); e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(grid), dim3(GEO::NT), lds, stream, lower, upper, weight, out_lower, out_upper,
                            d);

@@ -353,15 +353,15 @@ hipError_t inf_conv_forward(const float* img, const float* weight, float* out, i
     a.vec_in = q.W % 4 == 0 && aligned16(img);
     a.vec_out = q.WO % kTM == 0 && aligned16(out) && aligned16(pos);   // every run of 8 positions whole and aligned
     const size_t lds = ((size_t)a.xwords + 2 * (size_t)kKC * kBNP) * sizeof(float);
-    static bool raised[64][4] = {};
+    static std::atomic<bool> raised[64][4] = {};   // callers may come from several threads
     const int ki = (q.S - 1) * 2 + a.resident;
     auto kern = q.S == 1 ? (a.resident ? inf_conv_forward_kernel<1, true> : inf_conv_forward_kernel<1, false>)
                          : (a.resident ? inf_conv_forward_kernel<2, true> : inf_conv_forward_kernel<2, false>);
-    if (!(device >= 0 && device < 64 && raised[device][ki])) {
+    if (!(device >= 0 && device < 64 && raised[device][ki].load(std::memory_order_acquire))) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)kLdsLimit);
         if (e != hipSuccess) return e;
-        if (device >= 0 && device < 64) raised[device][ki] = true;
+        if (device >= 0 && device < 64) raised[device][ki].store(true, std::memory_order_release);
     }
     const unsigned grid = (unsigned)((long long)q.B * G * a.tiles_h * a.tiles_n);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(a.ML * a.NL), lds, stream, img, weight, out, pos, a);

@@ -179,13 +179,17 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
 
     if constexpr (!EXACT && !CONV && VEC == 4) {
         // fc layout: a recorded chunk is 128 contiguous, 16-byte aligned bytes of the x row and of
-        // the w row.  Eight neighbouring lanes take one output: each loads 16 bytes of both rows,
-        // so a wave's load instruction touches 8 whole lines instead of 64 partial ones (a lane
+        // the w row.  Four neighbouring lanes take one output: each loads 32 bytes of both rows,
+        // so a wave's load instruction touches 16 whole lines instead of 64 partial ones (a lane
         // that walks its own outputs alone is bound by the tag look-ups of the vector cache, not
         // by bytes).  The lowest matching k is the match of the lowest lane that has one: a ballot
-        // tells every lane whether a lower lane of its eight matched.  Rows and columns past the
+        // tells every lane whether a lower lane of its four matched.  Rows and columns past the
         // edge of the tensor read a clamped, valid address and are never stored.
-        constexpr int LPO = kChunk / 4;             // lanes per output
+        // The walk is as much a matter of vector instructions as of bytes (about fifty per output and lane group
+        // with eight lanes of 16 bytes each; four lanes of 32 bytes need 30 per output), so the row and column
+        // of the next output and their offsets are carried along instead of divided and multiplied out.
+        constexpr int VPL = 2;                      // 16-byte vectors per lane and operand
+        constexpr int LPO = kChunk / (4 * VPL);     // lanes per output
         constexpr int NGQ = GEO::NT / LPO;          // outputs in flight per trip of the workgroup
         constexpr int NIT = BM * BN / NGQ;          // trips
         constexpr int DEPTH = 4;                    // outputs per lane group whose loads are issued together
@@ -196,34 +200,47 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
         const float* wg = weight + (size_t)g * d.NG * K;
         // element offsets fit 32 bits: the entry point rejects tensors of 2^31 elements or more
         const unsigned ldx = (unsigned)d.G * K;
-        struct Slot { float4 x, w; int kb; };
-        auto issue = [&](int it, Slot& sl) {
+        // output gq of trip 0, then NGQ further per trip: tile row, tile column and the element offsets of both rows
+        int ml = gq / BN, nl = gq % BN;
+        unsigned xrow = (unsigned)(m0 + ml) * ldx, wrow = (unsigned)(n0 + nl) * (unsigned)K;
+        const unsigned xrow_last = (unsigned)(d.M - 1) * ldx, wrow_last = (unsigned)(d.NG - 1) * (unsigned)K;
+        const unsigned wstep = (unsigned)(NGQ % BN) * (unsigned)K, wwrap = (unsigned)BN * (unsigned)K;
+        struct Slot { float4 x[VPL], w[VPL]; int kb, o; };
+        auto issue = [&](int it, Slot& sl) {             // called with it = 0, 1, 2, ... in this order
             if (it >= NIT) return;                       // the last trip has nothing left to prefetch
-            const int o = it * NGQ + gq;
-            const int ml = o / BN, nl = o - ml * BN;
-            const unsigned m = min(m0 + ml, d.M - 1), n = min(n0 + nl, d.NG - 1);
+            const int o = ml * BN + nl;
             const int kb = cand_c[o] * kChunk;
-            // a lane whose 16 bytes lie past the end of the row reads the chunk's first 16 instead (masked
+            // a lane whose bytes lie past the end of the row reads the chunk's first ones instead (masked
             // below); the offset must never go negative, it is added as an unsigned 32-bit quantity
-            const unsigned off = kb + 4 * sub < K ? kb + 4 * sub : kb;
             sl.kb = kb;
-            sl.x = *reinterpret_cast<const float4*>(xg + (m * ldx + off));
-            sl.w = *reinterpret_cast<const float4*>(wg + (n * (unsigned)K + off));
+            sl.o = o;
+            const unsigned xo = min(xrow, xrow_last), wo = min(wrow, wrow_last);
+#pragma unroll
+            for (int v = 0; v < VPL; v++) {
+                const int kv = kb + 4 * (VPL * sub + v);
+                const unsigned off = kv < K ? kv : kb;
+                sl.x[v] = *reinterpret_cast<const float4*>(xg + (xo + off));
+                sl.w[v] = *reinterpret_cast<const float4*>(wg + (wo + off));
+            }
+            ml += NGQ / BN; xrow += (NGQ / BN) * ldx;
+            nl += NGQ % BN; wrow += wstep;
+            if (nl >= BN) { nl -= BN; wrow -= wwrap; ml += 1; xrow += ldx; }
         };
-        auto finish = [&](int it, const Slot& sl) {
-            const int o = it * NGQ + gq;
+        auto finish = [&](const Slot& sl) {
+            const int o = sl.o;
             const float target = cand_v[o];
-            const float d0 = sl.x.x - sl.w.x, d1 = sl.x.y - sl.w.y, d2 = sl.x.z - sl.w.z, d3 = sl.x.w - sl.w.w;
-            int q = -1;
-            float df = 0.f;
-            if (__builtin_fabsf(d3) == target) { q = 3; df = d3; }   // descending: the lowest match is kept
-            if (__builtin_fabsf(d2) == target) { q = 2; df = d2; }
-            if (__builtin_fabsf(d1) == target) { q = 1; df = d1; }
-            if (__builtin_fabsf(d0) == target) { q = 0; df = d0; }
-            const int k = sl.kb + 4 * sub + q;
-            const bool hit = q >= 0 && sl.kb + 4 * sub < K && target > 0.f;
+            int found = -1;                              // element index inside the lane's 4 * VPL, sign in bit 31
+#pragma unroll
+            for (int v = VPL - 1; v >= 0; v--) {         // descending: the lowest match is kept
+                const float dd[4] = {sl.x[v].x - sl.w[v].x, sl.x[v].y - sl.w[v].y, sl.x[v].z - sl.w[v].z, sl.x[v].w - sl.w[v].w};
+                const bool inside = sl.kb + 4 * (VPL * sub + v) < K;
+#pragma unroll
+                for (int e = 3; e >= 0; e--)
+                    if (__builtin_fabsf(dd[e]) == target && inside) found = (4 * v + e) | (__float_as_int(dd[e]) & 0x80000000);
+            }
+            const bool hit = found != -1 && target > 0.f;
             const unsigned mine = (unsigned)(__builtin_amdgcn_ballot_w64(hit) >> shift) & ((1u << LPO) - 1);
-            if (hit && (mine & ((1u << sub) - 1)) == 0) cand_c[o] = k | (__float_as_int(df) & 0x80000000);
+            if (hit && (mine & ((1u << sub) - 1)) == 0) cand_c[o] = found + sl.kb + 4 * VPL * sub;   // adds to the low bits only
             if (sub == 0 && mine == 0) cand_c[o] = 0;
         };
         Slot sa[DEPTH], sb[DEPTH];
@@ -234,11 +251,11 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
 #pragma unroll
             for (int e = 0; e < DEPTH; e++) issue(it + DEPTH + e, sb[e]);
 #pragma unroll
-            for (int e = 0; e < DEPTH; e++) finish(it + e, sa[e]);
+            for (int e = 0; e < DEPTH; e++) finish(sa[e]);
 #pragma unroll
             for (int e = 0; e < DEPTH; e++) issue(it + 2 * DEPTH + e, sa[e]);
 #pragma unroll
-            for (int e = 0; e < DEPTH; e++) finish(it + DEPTH + e, sb[e]);
+            for (int e = 0; e < DEPTH; e++) finish(sb[e]);
         }
     } else {
         // Other layouts: every lane takes outputs tid, tid + NT, ... of the tile on its own.
@@ -324,7 +341,7 @@ struct InfForward {
         constexpr size_t pipe = Stager<GEO, CONV, VEC, 1>::LDS_BYTES;
         const size_t lds = park > pipe ? park : pipe;
         auto kern = inf_forward_kernel<GEO, CONV, VEC, EXACT>;
-        static bool lds_allowed[64] = {};   // per instantiation of this launcher, i.e. per kernel
+        static LdsRecord lds_allowed = {};   // per instantiation of this launcher, i.e. per kernel
         if (hipError_t e = allow_lds(kern, lds, device, lds_allowed); e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(grid), dim3(GEO::NT), lds, stream, input, weight, output, pos, d);
         return hipGetLastError();

@@ -311,7 +311,7 @@ bool inf_forward_shortk_applicable(const Problem& pr, const void* input, const v
 template <int NP>
 static hipError_t launch_shortk(unsigned grid, size_t lds, int device, hipStream_t stream, const float* input,
                                 const float* weight, float* output, int32_t* pos, const Dims& d, int Kp, int tiles) {
-    static bool lds_allowed[64] = {};
+    static LdsRecord lds_allowed = {};
     if (hipError_t e = allow_lds(inf_forward_shortk_kernel<NP>, 160 * 1024, device, lds_allowed); e != hipSuccess) return e;
     hipLaunchKernelGGL(inf_forward_shortk_kernel<NP>, dim3(grid), dim3(shortk::NT), lds, stream, input, weight, output,
                        pos, d, Kp, tiles);

@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace ldist {
 
 struct Problem {
@@ -50,12 +52,15 @@ inline TileChoice choose_tile(int M, int NG, int G, int num_cu) {
 // Sets the dynamic-LDS limit of a kernel once per device.  `done` is the caller's record for that one
 // kernel (a function-local static of the launcher instantiated per kernel): kernels share their
 // function-pointer type, so a record kept here per type would be shared between them.
+// The entry points may be called from several threads at once (a forward thread and autograd's backward thread):
+// the record is atomic, and two threads that both find it unset both set the attribute, which is harmless.
+using LdsRecord = std::atomic<bool>[64];
 template <class Kern>
-inline hipError_t allow_lds(Kern kern, size_t bytes, int device, bool (&done)[64]) {
-    if (device >= 0 && device < 64 && done[device]) return hipSuccess;
+inline hipError_t allow_lds(Kern kern, size_t bytes, int device, LdsRecord& done) {
+    if (device >= 0 && device < 64 && done[device].load(std::memory_order_acquire)) return hipSuccess;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    if (e == hipSuccess && device >= 0 && device < 64) done[device] = true;
+    if (e == hipSuccess && device >= 0 && device < 64) done[device].store(true, std::memory_order_release);
     return e;
 }
 

@@ -3,6 +3,7 @@
 // device memory or synchronises; every call only enqueues work on `stream`.
 #include "../../include/ldist.h"
 
+#include <atomic>
 #include <cmath>
 #include <string>
 
@@ -17,30 +18,24 @@ namespace {
 
 thread_local int g_last_hip_error = 0;
 
-struct DeviceInfo {
-    int num_cu = 0;
-    bool is_gfx950 = false;
-    bool known = false;
-};
-
-// Compute-unit count and architecture of the current device (looked up once per device).
+// Compute-unit count and architecture of the current device, looked up once per device and kept in one atomic word
+// per device (0 = not looked up yet, else num_cu << 1 | is_gfx950): callers may come from several threads.
 int current_device(ldist::Problem& pr) {
-    static DeviceInfo info[64];
+    static std::atomic<int> info[64] = {};
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return LDIST_ELAUNCH; }
-    DeviceInfo local;
-    DeviceInfo& di = (dev >= 0 && dev < 64) ? info[dev] : local;
-    if (!di.known) {
+    int word = (dev >= 0 && dev < 64) ? info[dev].load(std::memory_order_acquire) : 0;
+    if (word == 0) {
         hipDeviceProp_t prop;
         e = hipGetDeviceProperties(&prop, dev);
         if (e != hipSuccess) { g_last_hip_error = (int)e; return LDIST_ELAUNCH; }
-        di.num_cu = prop.multiProcessorCount;
-        di.is_gfx950 = std::string(prop.gcnArchName).rfind("gfx950", 0) == 0;
-        di.known = true;
+        const int num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+        word = (num_cu << 1) | (std::string(prop.gcnArchName).rfind("gfx950", 0) == 0 ? 1 : 0);
+        if (dev >= 0 && dev < 64) info[dev].store(word, std::memory_order_release);
     }
-    if (!di.is_gfx950) return LDIST_EDEVICE;
-    pr.num_cu = di.num_cu > 0 ? di.num_cu : 256;
+    if (!(word & 1)) return LDIST_EDEVICE;
+    pr.num_cu = word >> 1;
     pr.device = dev;
     return LDIST_OK;
 }

@@ -412,7 +412,7 @@ struct NormForward {
                          const float* weight, float* output, float p) {
         const size_t lds = Stager<GEO, CONV, VEC, 1>::LDS_BYTES;
         auto kern = norm_forward_kernel<GEO, CONV, VEC, IP, MODE>;
-        static bool lds_allowed[64] = {};   // per instantiation of this launcher, i.e. per kernel
+        static LdsRecord lds_allowed = {};   // per instantiation of this launcher, i.e. per kernel
         if (hipError_t e = allow_lds(kern, lds, device, lds_allowed); e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(grid), dim3(GEO::NT), lds, stream, input, weight, output, p, d);
         return hipGetLastError();

@@ -228,7 +228,7 @@ struct ValueBoundForward {
                              const float* bias, float* out, float* out_lower, float* out_upper) {
         const size_t lds = Stager<GEO, CONV, VEC, 3>::LDS_BYTES;
         auto kern = value_bound_forward_kernel<GEO, CONV, VEC>;
-        static bool lds_allowed[64] = {};   // per instantiation of this launcher, i.e. per kernel
+        static LdsRecord lds_allowed = {};   // per instantiation of this launcher, i.e. per kernel
         if (hipError_t e = allow_lds(kern, lds, device, lds_allowed); e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(grid), dim3(GEO::NT), lds, stream, input, lower, upper, weight, mean, bias, out,
                            out_lower, out_upper, d);

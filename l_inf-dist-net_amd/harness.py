@@ -1,10 +1,13 @@
-"""Thin end-to-end harness around the distance-neuron operators: the model wrapper, a training step, the PGD
-attack and the certified-accuracy evaluation of the reference, for one batch at a time (the reference's loops
-over a data loader, its logging and its schedules are not part of this package).
+"""Thin end-to-end harness around the distance-neuron operators, one batch at a time: a wrapper that routes an
+input (and, for certification, its interval) through a feature net and a head, one optimisation step, a
+projected-gradient attack, and the certified-accuracy evaluation.  The reference's loops over a data loader,
+its logging and its schedules are not part of this package.
 
-Reference: model/model.py:3-29 (Model, set_eps, get_eps), attack.py:4-36 (AttackPGD), main.py:60-105 (train),
-main.py:166-194 (certified_test).
+Same public names, signatures and results as the reference's model/model.py:3-29 (Model, set_eps, get_eps),
+attack.py:4-36 (AttackPGD), main.py:60-105 (train) and main.py:166-194 (certified_test).
 """
+import contextlib
+
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
@@ -12,98 +15,113 @@ import torch.nn.functional as F
 from .norm_dist import get_p_norm, set_p_norm
 
 
+def _box(x, lo, hi):
+    """x clipped elementwise into [lo, hi] (tensors or numbers that broadcast)."""
+    return torch.minimum(torch.maximum(x, torch.as_tensor(lo, dtype=x.dtype, device=x.device)),
+                         torch.as_tensor(hi, dtype=x.dtype, device=x.device))
+
+
 class Model(nn.Module):
-    """feature (a dist net returning (y, lower, upper)) followed by predictor (a head taking them plus targets)."""
+    """`feature` maps (x, lower, upper) to such a triple; `predictor` turns the triple (and the targets) into the
+    outputs.  Bounds only travel when targets are given; if the feature net produced none (or there is no feature
+    net), the head gets the eps-ball around the features."""
 
     def __init__(self, feature, predictor, eps):
         super().__init__()
-        self.feature = feature
-        self.predictor = predictor
-        self.eps = eps
+        self.feature, self.predictor, self.eps = feature, predictor, eps
 
     def forward(self, x, lower=None, upper=None, targets=None):
-        if targets is None:
-            lower = upper = None
+        certify = targets is not None
+        triple = (x, lower if certify else None, upper if certify else None)
         if self.feature is not None:
-            x, lower, upper = self.feature(x, lower=lower, upper=upper)
-        if targets is not None and (lower is None or upper is None):
-            lower = x - self.eps
-            upper = x + self.eps
-        return self.predictor(x, lower, upper, targets=targets)
+            triple = self.feature(triple[0], lower=triple[1], upper=triple[2])
+        feat, lo, hi = triple
+        if certify and (lo is None or hi is None):
+            lo, hi = feat - self.eps, feat + self.eps
+        return self.predictor(feat, lo, hi, targets=targets)
+
+
+def _wrappers(model):
+    return (m for m in model.modules() if isinstance(m, Model))
 
 
 def set_eps(model, eps):
-    for m in model.modules():
-        if isinstance(m, Model):
-            m.eps = eps
+    for wrapper in _wrappers(model):
+        wrapper.eps = eps
 
 
 def get_eps(model):
-    for m in model.modules():
-        if isinstance(m, Model):
-            return m.eps
-    return None
+    return next((wrapper.eps for wrapper in _wrappers(model)), None)
 
 
 def cal_acc(outputs, targets):
-    return (outputs.max(dim=1)[1] == targets).float()
+    return outputs.argmax(dim=1).eq(targets).float()
 
 
 def train_step(net, loss_fun, optimizer, inputs, targets):
-    """One optimisation step as the reference's training loop makes it; returns (loss, accuracy) of the batch.
-    net(inputs, targets=targets) gives (outputs, worse_outputs); loss_fun takes them and the targets."""
+    """One optimisation step; returns (loss, accuracy) of the batch.  net(inputs, targets=targets) gives
+    (outputs, worse_outputs); loss_fun takes them and the targets."""
     net.train()
     outputs, worse_outputs = net(inputs, targets=targets)
     loss = loss_fun(outputs, worse_outputs, targets)
     optimizer.zero_grad()
     loss.backward()
     optimizer.step()
-    with torch.no_grad():
-        return loss.item(), cal_acc(outputs, targets).mean().item()
+    return loss.item(), cal_acc(outputs.detach(), targets).mean().item()
+
+
+@contextlib.contextmanager
+def _frozen(net):
+    """Parameters take no gradient inside the block; their flags come back afterwards."""
+    flags = {p: p.requires_grad for p in net.parameters()}
+    net.requires_grad_(False)
+    try:
+        yield
+    finally:
+        for p, flag in flags.items():
+            p.requires_grad_(flag)
 
 
 class AttackPGD:
-    """Projected gradient ascent on the cross entropy inside the eps-ball (L_inf) around the inputs, clipped to
-    the data range [down, up]."""
+    """Signed-gradient ascent on the summed cross entropy, projected after every step onto the L_inf ball of
+    radius eps around the inputs and onto the data range [down, up].  random_start: a clipped Gaussian offset
+    (std eps/4, at most eps/2) first."""
 
     def __init__(self, net, eps, step_size, num_steps, up, down, random_start=True):
         self.net, self.eps, self.step_size, self.num_steps = net, eps, step_size, num_steps
         self.up, self.down, self.rand = up, down, random_start
 
+    def _project(self, x, centre=None):
+        if centre is not None:
+            x = _box(x, centre - self.eps, centre + self.eps)
+        return _box(x, self.down, self.up)
+
     def find(self, inputs, targets):
-        saved = [p.requires_grad for p in self.net.parameters()]
-        self.net.requires_grad_(False)
-        x = inputs.detach()
+        start = inputs.detach()
         if self.rand:
-            noise = torch.zeros_like(x).normal_(0, self.eps / 4)
-            x = x + torch.clamp(noise, -self.eps / 2, self.eps / 2)
-            x = torch.min(torch.max(x, self.down), self.up)
-        for _ in range(self.num_steps):
-            x.requires_grad_()
-            loss = F.cross_entropy(self.net(x), targets, reduction="sum")
-            loss.backward()
-            x = torch.add(x.detach(), torch.sign(x.grad.detach()), alpha=self.step_size)
-            x = torch.min(torch.max(x, inputs - self.eps), inputs + self.eps)
-            x = torch.min(torch.max(x, self.down), self.up)
-        for p, r in zip(self.net.parameters(), saved):
-            p.requires_grad_(r)
-        return x
+            offset = torch.empty_like(start).normal_(0, self.eps / 4).clamp_(-self.eps / 2, self.eps / 2)
+            start = self._project(start + offset)
+        adv = start
+        with _frozen(self.net):
+            for _ in range(self.num_steps):
+                adv = adv.detach().requires_grad_(True)
+                F.cross_entropy(self.net(adv), targets, reduction="sum").backward()
+                adv = self._project(adv.detach() + self.step_size * adv.grad.sign(), centre=inputs)
+        return adv.detach()
 
 
 @torch.no_grad()
 def certified_accuracy(net, inputs, targets, eps, up, down):
     """Fraction of the batch whose prediction is certified for every perturbation of L_inf size eps: the interval
     bounds go through the net at p = inf, and the worst-case margins must still favour the label."""
-    save_p, save_eps = get_p_norm(net), get_eps(net)
+    keep = (get_p_norm(net), get_eps(net), net.training)
     set_eps(net, eps)
     set_p_norm(net, float("inf"))
-    was_training = net.training
     net.eval()
-    lower = torch.max(inputs - eps, down)
-    upper = torch.min(inputs + eps, up)
-    worst = net(inputs, lower=lower, upper=upper, targets=targets)[1]
-    res = cal_acc(worst, targets).mean().item()
-    set_p_norm(net, save_p)
-    set_eps(net, save_eps)
-    net.train(was_training)
-    return res
+    try:
+        worst = net(inputs, lower=_box(inputs - eps, down, up), upper=_box(inputs + eps, down, up), targets=targets)[1]
+        return cal_acc(worst, targets).mean().item()
+    finally:
+        set_p_norm(net, keep[0])
+        set_eps(net, keep[1])
+        net.train(keep[2])

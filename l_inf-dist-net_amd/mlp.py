@@ -26,11 +26,11 @@ class MLP(nn.Module):
         self.fc_last = NormDist(dim, num_classes, bias=True, mean_normalize=head_mean_normalize)
 
     def forward(self, x, lower=None, upper=None):
-        paras = [None if y is None else y.view(y.size(0), -1) for y in (x, lower, upper)]
-        for layer in self.fc:
-            paras = layer(*paras)
-        y, lo, up = self.fc_last(*paras)
-        return [None if t is None else -t for t in (y, up, lo)]
+        triple = [None if t is None else t.flatten(1) for t in (x, lower, upper)]
+        for layer in (*self.fc, self.fc_last):
+            triple = layer(*triple)
+        y, lo, up = triple
+        return [None if t is None else -t for t in (y, up, lo)]   # negated distances: the bounds change places
 
 
 class BoundFinalIdentity(nn.Module):
@@ -39,6 +39,6 @@ class BoundFinalIdentity(nn.Module):
     def forward(self, x, lower=None, upper=None, targets=None):
         if lower is None or upper is None or targets is None:
             return x
-        res = upper - torch.gather(lower, dim=1, index=targets.unsqueeze(-1))
-        res = res.scatter(dim=1, index=targets.unsqueeze(-1), value=0)
-        return x, res
+        at = targets.view(-1, 1)
+        margins = upper - lower.gather(1, at)          # every class's upper bound against the label's lower bound
+        return x, margins.scatter(1, at, 0.0)

@@ -280,7 +280,7 @@ class NormDistConv(nn.Module):
     def _columns(self, t):
         """(B, C*k*k, L) patches of t; a 1x1 window needs no unfold (which launches one kernel per image)."""
         if self.kernel_size == 1 and self.stride == 1 and self.padding == 0:
-            return t.reshape(t.size(0), t.size(1), -1)
+            return t.reshape(t.size(0), t.size(1), -1).contiguous()   # F.unfold always hands over a contiguous tensor
         if t.is_cuda and t.dtype == torch.float32:
             return _Unfold.apply(t, self.kernel_size, self.dilation, self.padding, self.stride)
         return F.unfold(t, self.kernel_size, self.dilation, self.padding, self.stride)
