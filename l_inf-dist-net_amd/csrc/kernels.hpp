@@ -83,6 +83,16 @@ hipError_t norm_forward(const float* input, const float* weight, float* output, 
 hipError_t norm_backward_input(const float* grad_output, const float* input, const float* weight,
                                const float* output, float* grad_input, float p, const Problem& pr,
                                hipStream_t stream);
+bool norm_backward_input_tiled_applicable(const Problem& pr, float p, const void* grad_output, const void* input,
+                                          const void* weight, const void* output, const void* grad_input);
+hipError_t norm_backward_input_tiled(const float* grad_output, const float* input, const float* weight,
+                                     const float* output, float* grad_input, float p, const Problem& pr,
+                                     hipStream_t stream);
+bool norm_backward_weight_tiled_applicable(const Problem& pr, float p, const void* grad_output, const void* input,
+                                           const void* weight, const void* output, const void* grad_weight);
+hipError_t norm_backward_weight_tiled(const float* grad_output, const float* input, const float* weight,
+                                      const float* output, float* grad_weight, float p, const Problem& pr,
+                                      hipStream_t stream);
 hipError_t norm_backward_weight(const float* grad_output, const float* input, const float* weight,
                                 const float* output, float* grad_weight, float p, const Problem& pr,
                                 hipStream_t stream);

@@ -312,12 +312,16 @@ static hipError_t launch_norm_backward(const float* grad_output, const float* in
 hipError_t norm_backward_input(const float* grad_output, const float* input, const float* weight,
                                const float* output, float* grad_input, float p, const Problem& pr,
                                hipStream_t stream) {
+    if (norm_backward_input_tiled_applicable(pr, p, grad_output, input, weight, output, grad_input))
+        return norm_backward_input_tiled(grad_output, input, weight, output, grad_input, p, pr, stream);
     return launch_norm_backward<false>(grad_output, input, weight, output, grad_input, p, pr, stream);
 }
 
 hipError_t norm_backward_weight(const float* grad_output, const float* input, const float* weight,
                                 const float* output, float* grad_weight, float p, const Problem& pr,
                                 hipStream_t stream) {
+    if (norm_backward_weight_tiled_applicable(pr, p, grad_output, input, weight, output, grad_weight))
+        return norm_backward_weight_tiled(grad_output, input, weight, output, grad_weight, p, pr, stream);
     return launch_norm_backward<true>(grad_output, input, weight, output, grad_weight, p, pr, stream);
 }
 

@@ -358,6 +358,112 @@ def test_norm_backward(shape, p):
     assert_sum_close(gw.cpu() - 0.125, ew, mw, p, RTOL, ATOL)
 
 
+# B, CO, CI, G, HW -- shapes the register-tiled grad_input kernel can take (K % 4 == 0; NG % 4 == 0 or HW % 4 == 0)
+TILED_BACKWARD_SHAPES = [
+    (130, 72, 260, 1, 1),     # fc: row tail, column tails of the 80- and 64-wide tiles, reduction shorter than two stages
+    (64, 96, 96, 3, 1),       # groups, one stage of exactly 32 outputs per group
+    (200, 300, 164, 1, 1),    # several stages with a ragged last one (300 = 4 * 64 + 44), K = 164: a tile's last group of four
+    (2, 64, 64, 2, 64),       # conv layout
+    (3, 40, 36, 1, 100),      # conv layout: rows end inside a tile (300 rows), images change inside a tile
+    (4, 128, 1152, 4, 100),   # the grouped 3x3 conv layer shape at a small image
+]
+
+
+@pytest.mark.parametrize("tile", [0, 1])
+@pytest.mark.parametrize("p", [8.0, 2.0, 3.0, 4.0])
+@pytest.mark.parametrize("shape", TILED_BACKWARD_SHAPES)
+def test_norm_backward_input_register_tiled(shape, p, tile):
+    """grad_input of the multiply-only exponents on the register-tiled kernel (forced with the tile override:
+    0 = 128 x 80 tiles, 1 = 128 x 64; by itself it only takes large layers) against the oracle, and against the
+    64 x 64 kernel it replaces there (override 2), with the same tolerance."""
+    from gpu_common import DEV, cpp, say, set_tile
+    B, CO, CI, G, HW = shape
+    say("norm_backward_input tiled", shape, "p", p, "tile", tile)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=16 + sum(shape))
+    go = torch.randn(B, CO, HW, generator=gen(17))
+    out = oracle.norm_dist_forward(x, w, G, p)
+    ex, mx = oracle.norm_dist_backward_input(go, x, w, out, G, p, with_abs_terms=True)
+    args = (go.to(DEV), x.to(DEV), w.to(DEV), out.to(DEV))
+    for choice in (tile, 2):
+        set_tile(choice)
+        gx = torch.full((B, CI, HW), float("nan"), device=DEV)
+        cpp.norm_dist_backward_input(*args, gx, G, p)
+        torch.cuda.synchronize()
+        assert_sum_close(gx.cpu(), ex, mx, p, RTOL, ATOL)
+
+
+@pytest.mark.parametrize("tile", [0, 1])
+@pytest.mark.parametrize("p", [8.0, 2.0, 3.0, 4.0])
+@pytest.mark.parametrize("shape", [sh for sh in TILED_BACKWARD_SHAPES if sh[4] == 1] + [(515, 140, 100, 1, 1), (70, 200, 132, 1, 1)])
+def test_norm_backward_weight_register_tiled(shape, p, tile):
+    """grad_weight of the multiply-only exponents in the fc layout on the register-tiled kernel (forced with the
+    tile override) against the oracle; the kernel adds onto the buffer it is given (reference contract)."""
+    from gpu_common import DEV, cpp, say, set_tile
+    B, CO, CI, G, HW = shape
+    say("norm_backward_weight tiled", shape, "p", p, "tile", tile)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=26 + sum(shape))
+    go = torch.randn(B, CO, HW, generator=gen(27))
+    out = oracle.norm_dist_forward(x, w, G, p)
+    ew, mw = oracle.norm_dist_backward_weight(go, x, w, out, G, p, with_abs_terms=True)
+    args = (go.to(DEV), x.to(DEV), w.to(DEV), out.to(DEV))
+    for choice in (tile, 2):
+        set_tile(choice)
+        gw = torch.full((CO, CI // G), 0.125, device=DEV)
+        cpp.norm_dist_backward_weight(*args, gw, G, p)
+        torch.cuda.synchronize()
+        assert_sum_close(gw.cpu() - 0.125, ew, mw, p, RTOL, ATOL)
+
+
+@pytest.mark.parametrize("p", [2.0, 4.0, 8.0])
+@pytest.mark.parametrize("scale", [1e-6, 1.0, 1e6, "mixed"])
+def test_norm_backward_weight_register_tiled_at_every_scale(scale, p):
+    from gpu_common import DEV, cpp, say, set_tile
+    B, CO, CI, G, HW = 200, 72, 132, 1, 1
+    say("norm_backward_weight tiled scale", scale, "p", p)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=43)
+    if scale == "mixed":
+        x = x * torch.tensor([1e-5, 1.0, 1e4, 3e-3, 1.0])[torch.arange(B) % 5].view(B, 1, 1)
+    else:
+        x, w = x * scale, w * scale
+    x, w = x.contiguous(), w.contiguous()
+    go = torch.randn(B, CO, HW, generator=gen(28))
+    out = oracle.norm_dist_forward(x, w, G, p)
+    ew, mw = oracle.norm_dist_backward_weight(go, x, w, out, G, p, with_abs_terms=True)
+    set_tile(0)
+    gw = torch.zeros((CO, CI // G), device=DEV)
+    cpp.norm_dist_backward_weight(go.to(DEV), x.to(DEV), w.to(DEV), out.to(DEV), gw, G, p)
+    torch.cuda.synchronize()
+    assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
+
+
+@pytest.mark.parametrize("p", [2.0, 3.0, 4.0, 8.0])
+@pytest.mark.parametrize("scale", [1e-6, 3e-4, 1.0, 5e3, 1e6, "mixed", "one tiny row"])
+def test_norm_backward_input_register_tiled_at_every_scale(scale, p):
+    """The tiled kernel takes powers of raw differences only while every output of a stage lies within [2^-12, 2^12];
+    a stage that holds one outside goes the normalised way.  Tiny and huge data, rows of very different magnitude
+    in one stage, and a single tiny row among ordinary ones (so that some stages switch and others do not)."""
+    from gpu_common import DEV, cpp, say, set_tile
+    B, CO, CI, G, HW = 70, 200, 132, 1, 1
+    say("norm_backward_input tiled scale", scale, "p", p)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=33)
+    if scale == "mixed":
+        x = x * torch.tensor([1e-5, 1.0, 1e4, 3e-3, 1.0])[torch.arange(B) % 5].view(B, 1, 1)
+    elif scale == "one tiny row":
+        x[17] *= 1e-7
+        w[100:] *= 1e-7          # only the outputs of the later stages are tiny for that row
+    else:
+        x, w = x * scale, w * scale
+    x, w = x.contiguous(), w.contiguous()
+    go = torch.randn(B, CO, HW, generator=gen(18))
+    out = oracle.norm_dist_forward(x, w, G, p)
+    ex, mx = oracle.norm_dist_backward_input(go, x, w, out, G, p, with_abs_terms=True)
+    set_tile(0)
+    gx = torch.full((B, CI, HW), float("nan"), device=DEV)
+    cpp.norm_dist_backward_input(go.to(DEV), x.to(DEV), w.to(DEV), out.to(DEV), gx, G, p)
+    torch.cuda.synchronize()
+    assert_sum_close(gx.cpu(), ex, mx, p, RTOL, ATOL)
+
+
 @pytest.mark.parametrize("p", [2.0, 3.0, 4.0, 8.0])
 @pytest.mark.parametrize("scale", [1e-9, 1e-6, 2e-4, 3e-4, 1.0, 3e3, 5e3, 1e6, 1e15, "mixed"])
 def test_norm_forward_at_every_scale(scale, p):
