@@ -20,7 +20,9 @@ namespace ldist {
 // EXACT = true: track k itself (subtract, compare, two selects = 4 instructions per
 // element, no re-read).  That pays in the conv layout with short K, where the re-read is a
 // strided gather that costs more than the whole reduction.
-template <class GEO, bool CONV, int VEC, bool EXACT>
+// HALF (fc layout with vector loads, short reductions): the chunk is recorded in halves of 16, which halves what the
+// search after the loop reads per output, for one more compare, select and copy per output and chunk in the loop.
+template <class GEO, bool CONV, int VEC, bool EXACT, bool HALF = false>
 __global__ void __launch_bounds__(GEO::NT, 2)
 inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ weight, float* __restrict__ output,
                    int32_t* __restrict__ pos, Dims d) {
@@ -81,7 +83,7 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int j = 0; j < TN; j++) cur[i][j] = prev[i][j];
-            sweep_chunk<GEO, 1, 2, true>(xp, wp, tx, ty, [&](const Frag<GEO, 1, 2>& f, int) {
+            auto body = [&](const Frag<GEO, 1, 2>& f, int) {
 #pragma unroll
                 for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -90,12 +92,25 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
                         const float d1 = __builtin_fabsf(f.x[0][1][i] - f.w[1][j]);
                         cur[i][j] = __builtin_fmaxf(__builtin_fmaxf(cur[i][j], d0), d1);
                     }
-            });
+            };
+            if constexpr (HALF) {
+                sweep_chunk<GEO, 1, 2, true>(xp, wp, tx, ty, body, [&]() {   // after the first 16 k: record, move prev up
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int j = 0; j < TN; j++) {
+                            if (cur[i][j] > prev[i][j]) cidx[i][j] = 2 * c;
+                            prev[i][j] = cur[i][j];
+                        }
+                });
+            } else {
+                sweep_chunk<GEO, 1, 2, true>(xp, wp, tx, ty, body);
+            }
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int j = 0; j < TN; j++)
-                    if (cur[i][j] > prev[i][j]) cidx[i][j] = c;
+                    if (cur[i][j] > prev[i][j]) cidx[i][j] = HALF ? 2 * c + 1 : c;
         }
         if (NBUF == 1) __syncthreads();  // everyone is done reading the only buffer
         if (s + 1 < nstage) st.store(lds + ((s + 1) % NBUF) * STAGE);
@@ -188,11 +203,12 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
         // The walk is as much a matter of vector instructions as of bytes (about fifty per output and lane group
         // with eight lanes of 16 bytes each; four lanes of 32 bytes need 30 per output), so the row and column
         // of the next output and their offsets are carried along instead of divided and multiplied out.
+        constexpr int RUN = HALF ? kChunk / 2 : kChunk;   // k values a recorded index stands for
         constexpr int VPL = 2;                      // 16-byte vectors per lane and operand
-        constexpr int LPO = kChunk / (4 * VPL);     // lanes per output
+        constexpr int LPO = RUN / (4 * VPL);        // lanes per output
         constexpr int NGQ = GEO::NT / LPO;          // outputs in flight per trip of the workgroup
         constexpr int NIT = BM * BN / NGQ;          // trips
-        constexpr int DEPTH = 4;                    // outputs per lane group whose loads are issued together
+        constexpr int DEPTH = NIT % 8 == 0 ? 4 : NIT % 4 == 0 ? 2 : 1;   // outputs per lane group whose loads are issued together
         static_assert(BM * BN % NGQ == 0 && NIT % (2 * DEPTH) == 0, "whole batches");
         const int sub = tid % LPO, gq = tid / LPO;
         const int shift = (tid & 63) - sub;         // bit of this lane group's first lane in a ballot
@@ -209,7 +225,7 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
         auto issue = [&](int it, Slot& sl) {             // called with it = 0, 1, 2, ... in this order
             if (it >= NIT) return;                       // the last trip has nothing left to prefetch
             const int o = ml * BN + nl;
-            const int kb = cand_c[o] * kChunk;
+            const int kb = cand_c[o] * RUN;
             // a lane whose bytes lie past the end of the row reads the chunk's first ones instead (masked
             // below); the offset must never go negative, it is added as an unsigned 32-bit quantity
             sl.kb = kb;
@@ -330,17 +346,21 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
 
 // Above this K the chunk re-read is cheaper than tracking k in the loop (conv layout).
 constexpr int kExactMaxK = 1024;
+// Up to this K the fc kernel records halves of a chunk: the loop runs about 10 % longer for it, the search after the
+// loop (whose cost hardly depends on K) takes half as long.  Measured on 512 x K -> 5120: K = 784 120 against 128 us,
+// K = 2048 a loss.
+constexpr int kHalfMaxK = 1024;
 
 template <class GEO, bool CONV, int VEC>
 struct InfForward {
-    template <bool EXACT>
+    template <bool EXACT, bool HALF = false>
     static hipError_t go(unsigned grid, const Dims& d, int device, hipStream_t stream, const float* input,
                          const float* weight, float* output, int32_t* pos) {
         // pipeline buffers, or the tile's (value, chunk) parking area of the epilogue if larger
         constexpr size_t park = (size_t)GEO::BM * GEO::BN * 2 * sizeof(float);
         constexpr size_t pipe = Stager<GEO, CONV, VEC, 1>::LDS_BYTES;
         const size_t lds = park > pipe ? park : pipe;
-        auto kern = inf_forward_kernel<GEO, CONV, VEC, EXACT>;
+        auto kern = inf_forward_kernel<GEO, CONV, VEC, EXACT, HALF>;
         static LdsRecord lds_allowed = {};   // per instantiation of this launcher, i.e. per kernel
         if (hipError_t e = allow_lds(kern, lds, device, lds_allowed); e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(grid), dim3(GEO::NT), lds, stream, input, weight, output, pos, d);
@@ -350,6 +370,9 @@ struct InfForward {
                              const float* weight, float* output, int32_t* pos) {
         if constexpr (CONV) {
             if (d.K <= kExactMaxK) return go<true>(grid, d, device, stream, input, weight, output, pos);
+        }
+        if constexpr (!CONV && VEC == 4) {
+            if (d.K <= kHalfMaxK) return go<false, true>(grid, d, device, stream, input, weight, output, pos);
         }
         return go<false>(grid, d, device, stream, input, weight, output, pos);
     }

@@ -19,6 +19,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace ldist {
 
 constexpr int kChunk = 32;  // k values between two "did the maximum move" checks
@@ -186,8 +188,11 @@ __device__ __forceinline__ void read_frag(Frag<GEO, NX, KP>& f, const LaneAddr<G
 // above the arithmetic and spills the accumulators.  Without the scheduling
 // barriers it sinks each fetch down to its first use, which puts the LDS
 // latency back on the critical path.
-template <class GEO, int NX, int KP, bool BYTE_ADDR = false, class F>
-__device__ __forceinline__ void sweep_chunk(const float* xp, const float* wp, int tx, int ty, F&& f) {
+struct NoMid { __device__ __forceinline__ void operator()() const {} };
+
+// mid() runs once, between rows 15 and 16 of the chunk (after the trip that reduces rows 12..15).
+template <class GEO, int NX, int KP, bool BYTE_ADDR = false, class F, class MID = NoMid>
+__device__ __forceinline__ void sweep_chunk(const float* xp, const float* wp, int tx, int ty, F&& f, MID&& mid = MID()) {
     static_assert(KP == 1 || KP == 2, "a trip must stay inside one aligned run of four rows");
     constexpr int XSTRIDE = GEO::XS;
     // LDS instructions of one fragment read: 128-bit reads of x and w, plus the fifth column
@@ -222,6 +227,8 @@ __device__ __forceinline__ void sweep_chunk(const float* xp, const float* wp, in
             __builtin_amdgcn_sched_barrier(0);
             f(b, kk + KP);
             cur = nxt;
+            if constexpr (!std::is_same<typename std::decay<MID>::type, NoMid>::value)
+                if (kk == kChunk / 2 - 2 * KP) mid();
         }
     } else {
         LanePtr<GEO> cur, nxt;
@@ -242,6 +249,8 @@ __device__ __forceinline__ void sweep_chunk(const float* xp, const float* wp, in
             __builtin_amdgcn_sched_barrier(0);
             f(b, kk + KP);
             cur = nxt;
+            if constexpr (!std::is_same<typename std::decay<MID>::type, NoMid>::value)
+                if (kk == kChunk / 2 - 2 * KP) mid();
         }
     }
 }
