@@ -3,10 +3,10 @@
 // that no power can overflow for any p.  Semantics follow the reference kernel
 // model/norm_dist_cuda.cu:228-292: mx and the sum are seeded with 1e-10 (:232-233),
 // and whenever a block of k raises mx the sum is rescaled by (mx_old/mx_new)^p
-// (:257-261).  Here the block is a 32-wide chunk.  For p <= 64 a chunk is normally
-// swept once with the scale left by earlier chunks (see the kernel); up to p = 128
-// sweep one finds the chunk maximum (sub + half a max3 per element), the rescale
-// runs once per output, sweep two adds (|x-w| / mx)^p; from p = 128 the kernel first
+// (:257-261).  Here the block is a 32-wide chunk.  Below p = 128 a chunk is normally
+// swept once with the scale left by earlier chunks (see the kernel; a chunk that
+// overflows is swept again the reference's way: maximum, rescale, powers);
+// from p = 128 the kernel first
 // finds the maxima over all of k and then takes only the powers that can matter
 // (see MODE 2 in the kernel).  p = 2, 3, 4, 8 use multiplies only; any other p goes
 // through v_log_f32 / v_exp_f32.
@@ -332,10 +332,11 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
 }
 
 // Largest exponent for the one-sweep kernel.  A chunk goes back the long way once it exceeds the
-// scale by 10^(30/p): a factor of 70 at p = 16, still 2.9 at p = 64, which later chunks rarely
-// do.  Beyond that nearly every new maximum would overflow and the retries would cost more than
-// sweeping every chunk twice.
-constexpr float kOneSweepMaxP = 64.f;
+// scale by 10^(30/p): a factor of 70 at p = 16, 2.9 at p = 64, still 1.7 at p = 128, which later chunks
+// (the scale is the maximum of all chunks before) rarely do: on 512 x 5120 -> 5120 one sweep takes 3.08 ms
+// for any p from 37 to 127, against 3.4 ms for sweeping every chunk twice.  A general-p term is a logarithm
+// and an exponential, and 13.4 G of them in 3.08 ms is 89 % of what the transcendental unit issues.
+constexpr float kOneSweepMaxP = 127.99f;
 
 // Exponents from which the forward runs its two passes with tests (MODE 2).  With normally distributed
 // differences over 5120 inputs it overtakes the chunk-by-chunk kernel at p of about 120.
