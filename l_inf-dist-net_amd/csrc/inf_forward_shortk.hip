@@ -21,8 +21,9 @@
 // of the next tile is loaded into registers before the current tile's arithmetic and written to LDS after
 // its epilogue, so the loads wait behind a whole tile of arithmetic.  The input is row-contiguous in memory
 // and goes in with 128-bit stores.  The weights are read along k with coalesced 32-bit loads, four
-// neighbouring outputs per lane, and stored as one 128-bit word whose place in row k is XORed with k % 8 (in
-// units of four outputs): the 64 lanes of a store, which differ in k, then cover all banks instead of four.
+// neighbouring outputs per lane, and stored as one 128-bit word (the lanes of such a store differ in k and
+// meet in few banks; it happens once per run of tiles, and plain rows let every later read of the panel use
+// one address register and constant offsets).
 #include "fwd_engine.hpp"
 
 namespace ldist {
@@ -33,8 +34,6 @@ constexpr int KQ = NGROUP * WIN;                  // K is padded to a multiple o
 constexpr int XROWS = NT / (BM / 4);              // k rows of the input panel that one pass of the workgroup loads
 constexpr int MAXPASS = 10;                       // padded K / 32 the kernel is built for: K <= 320
 static_assert(XROWS == KQ, "one pass loads one padding quantum of k");
-// float offset inside row k of W of the group of four outputs nq (0..7)
-__device__ __forceinline__ constexpr int wslot(int k, int nq) { return ((nq ^ (k & 7)) << 2); }
 inline int padded_k(int K) { return (K + KQ - 1) / KQ * KQ; }
 // panels, four value slabs (float) and four window slabs (one byte per output: at most 40 windows)
 inline size_t lds_bytes(int Kp) { return ((size_t)Kp * (BM + BN) + NGROUP * BM * BN) * sizeof(float) + NGROUP * BM * BN; }
@@ -129,7 +128,7 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
                 const int i = i0 + e * NT;
                 if (i < items) {
                     const int kw = i % Kp;
-                    *reinterpret_cast<float4*>(W + kw * BN + wslot(kw, i / Kp)) = wv[e];
+                    *reinterpret_cast<float4*>(W + kw * BN + (i / Kp) * 4) = wv[e];
                 }
             }
         }
@@ -138,13 +137,11 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
     const int lane = tid & 63, wave = tid >> 6;
     const int half = wave / NGROUP, grp = wave % NGROUP;
     const int tx = lane % 8, ty = lane / 8;
-    int woff[WIN];   // row kb + e of a window (kb % 8 == 0) keeps the lane's four outputs at group tx ^ e
-#pragma unroll
-    for (int e = 0; e < WIN; e++) woff[e] = e * BN + ((tx ^ e) << 2);
 
     // Tile -> global, from slabs 0 and 1: a lane stores four neighbouring rows of one output with 128-bit stores.
     // A tile's results go out at the start of the next tile, after that tile's input panel has been written to
-    // LDS: the wait for the parked loads (the counter also covers stores) then never waits for stores just issued.
+    // LDS and the loads of the panel after it are on their way: the wait for parked loads (the counter also covers
+    // stores) then only ever waits for loads that are older than the stores.
     auto flush = [&](int t) {
         const int tm = t % d.tiles_m, wkey = t / d.tiles_m;
         const int tn = wkey % d.tiles_n, g = wkey / d.tiles_n;
@@ -170,11 +167,17 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
         }
         store_x(t);
         __syncthreads();
+        // The next tile's panel, parked in registers until this tile is done.  The loads go out before the stores of
+        // the flush: behind them they would first wait until the stores have read the registers they share.
+        // The load unit takes some thirty clocks per load of a wave, and a wave that issues loads does nothing else: the
+        // upper half's waves issue theirs here, the lower half's waves in the middle of their reduction, so that on
+        // every SIMD one of its two waves computes while the other queues loads.
+        const bool more = t + t_step < t_end;
+        if (more && half == 0) issue_x(t + t_step);
         if (t > t_begin) {
             flush(t - t_step);
             __syncthreads();      // the slabs are read before any wave of this tile parks its patch there
         }
-        if (t + t_step < t_end) issue_x(t + t_step);   // the next tile's panel, parked in registers until this tile is done
 
         // ---- the reduction: the wave takes rows half*32.. of the tile and k in [grp*Kg, (grp+1)*Kg) --------
         float accA[4][4], accB[4][4];
@@ -184,13 +187,13 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
 #pragma unroll
             for (int j = 0; j < 4; j++) { accA[i][j] = 0.f; accB[i][j] = 0.f; widx[i][j] = 0; }
         const float* xp = X + (size_t)grp * Kg * BM + half * 32 + ty * 4;
-        const float* wp = W + (size_t)grp * Kg * BN;
+        const float* wp = W + (size_t)grp * Kg * BN + tx * 4;
         float4 xa[2], wa[2], xb[2], wb[2];
         auto fetch = [&](float4 (&xf)[2], float4 (&wf)[2], int kk) {   // rows kk, kk + 1 of the current window
 #pragma unroll
             for (int e = 0; e < 2; e++) {
                 xf[e] = *reinterpret_cast<const float4*>(xp + (kk + e) * BM);
-                wf[e] = *reinterpret_cast<const float4*>(wp + woff[kk + e]);
+                wf[e] = *reinterpret_cast<const float4*>(wp + (kk + e) * BN);
             }
         };
         // One window: cur continues the running maximum from prev (prev is left alone), so the window raised the
@@ -230,8 +233,10 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
                     if (cur[i][j] > prev[i][j]) widx[i][j] = wid;
         };
         fetch(xa, wa, 0);
+        const int w_issue = (nwin / 2) & ~1;
 #pragma unroll 1
         for (int w = 0; w < nwin; w += 2) {
+            if (more && half == 1 && w == w_issue) issue_x(t + t_step);
             window(accA, accB, w);
             if (w + 1 < nwin) {
                 window(accB, accA, w + 1);
@@ -264,33 +269,64 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
         // in one bank: lane l of a wave takes row l of the tile and, in round r, output (l + r) % 32 -- 64 different
         // columns of X and 32 of W.
         {
+            constexpr int ROUNDS = BN / (NT / 64);
             const int ml = lane;
+            int o[ROUNDS], kb[ROUNDS], pfound[ROUNDS];
+            float v[ROUNDS];
+            // all slab reads first, then all panel reads, then all writes: a write to the merge area between two
+            // rounds would order the next round's reads behind it
+            float vq[ROUNDS][NGROUP];
+            int wq[ROUNDS][NGROUP];
 #pragma unroll
-            for (int rr = 0; rr < BN / (NT / 64); rr++) {
-                const int nl = (lane + wave * (BN / (NT / 64)) + rr) % BN;
-                const int o = cslot(nl, ml), ob = bslot(nl, ml);
-                float v = slab_v[o];
-                int wsel = slab_w[ob];
+            for (int rr = 0; rr < ROUNDS; rr++) {
+                const int nl = (lane + wave * ROUNDS + rr) % BN;
+                const int ob = bslot(nl, ml);
+                o[rr] = cslot(nl, ml);
+#pragma unroll
+                for (int q = 0; q < NGROUP; q++) {
+                    vq[rr][q] = slab_v[q * (BM * BN) + o[rr]];
+                    wq[rr][q] = slab_w[q * (BM * BN) + ob];
+                }
+            }
+            // The values exist here, whatever the comparisons below say: otherwise the compiler moves each read behind
+            // the comparison that needs it, and the reads wait for one another.
+#pragma unroll
+            for (int rr = 0; rr < ROUNDS; rr++)
+                asm volatile("" : "+v"(vq[rr][0]), "+v"(vq[rr][1]), "+v"(vq[rr][2]), "+v"(vq[rr][3]), "+v"(wq[rr][0]),
+                             "+v"(wq[rr][1]), "+v"(wq[rr][2]), "+v"(wq[rr][3]));
+            static_assert(NGROUP == 4, "the statement above names four ranges");
+#pragma unroll
+            for (int rr = 0; rr < ROUNDS; rr++) {
+                v[rr] = vq[rr][0];
+                int wsel = wq[rr][0];
 #pragma unroll
                 for (int q = 1; q < NGROUP; q++) {
-                    const float vq = slab_v[q * (BM * BN) + o];
-                    const int wq = slab_w[q * (BM * BN) + ob] + q * nwin;
-                    if (vq > v) { v = vq; wsel = wq; }
+                    const bool gt = vq[rr][q] > v[rr];
+                    v[rr] = gt ? vq[rr][q] : v[rr];
+                    wsel = gt ? wq[rr][q] + q * nwin : wsel;
                 }
-                const int kb = wsel * WIN;
-                const float* xr = X + kb * BM + ml;
-                const float* wr = W + kb * BN + (nl & 3);
+                kb[rr] = wsel * WIN;
+            }
+#pragma unroll
+            for (int rr = 0; rr < ROUNDS; rr++) {
+                const int nl = (lane + wave * ROUNDS + rr) % BN;
+                const float* xr = X + kb[rr] * BM + ml;
+                const float* wr = W + kb[rr] * BN + nl;
                 float xv[WIN], wv[WIN];
 #pragma unroll
-                for (int e = 0; e < WIN; e++) { xv[e] = xr[e * BM]; wv[e] = wr[e * BN + wslot(e, nl >> 2)]; }   // kb % 8 == 0
+                for (int e = 0; e < WIN; e++) { xv[e] = xr[e * BM]; wv[e] = wr[e * BN]; }
                 int p = 0;
 #pragma unroll
                 for (int e = WIN - 1; e >= 0; e--) {   // descending: the lowest match is written last
                     const float df = xv[e] - wv[e];
-                    if (__builtin_fabsf(df) == v) p = (kb + e) | (__float_as_int(df) & 0x80000000);
+                    if (__builtin_fabsf(df) == v[rr]) p = (kb[rr] + e) | (__float_as_int(df) & 0x80000000);
                 }
-                slab_v[o] = v;                         // slabs 0 and 1 now carry the tile's results; nobody else reads
-                out_p[o] = v > 0.f ? p : 0;            // these two words.  v == 0: the reference leaves pos = 0
+                pfound[rr] = v[rr] > 0.f ? p : 0;      // v == 0: the reference leaves pos = 0
+            }
+#pragma unroll
+            for (int rr = 0; rr < ROUNDS; rr++) {      // slabs 0 and 1 now carry the tile's results; nobody else
+                slab_v[o[rr]] = v[rr];                 // reads these two words
+                out_p[o[rr]] = pfound[rr];
             }
         }
         __syncthreads();   // the panels are free for the next tile; its results wait in the merge area
