@@ -6,7 +6,8 @@ CIFAR-10-shaped 5-layer L_inf-dist MLP 3072 -> 5120 -> 5120 -> 5120 -> 5120 -> 1
 p = inf, batch 512, fp32, forward plus backward (grad_x of every layer and every
 grad_w).  A "step" is one pass of the hot path over one synthetic batch that already
 sits in HBM.  `--workload c0|c2|c3|c4` runs the other BASELINE.json configurations
-(`c4i`: configs[4] from the image, `c1t`: configs[1] with the optimizer step) with the
+(`c4i`: configs[4] from the image, `c4p`: the same layer at finite p from the image, `c1t`: configs[1] with the
+optimizer step) with the
 same output format (they are parity-test cases; the driver's line is c1).
 
 Prints ONE JSON line.  `value` is G dist-ops/s; a dist-op is one (row, output,
@@ -387,7 +388,7 @@ def workload_c4(pkg, torch, dev):
                 name="configs[4]: unfolded 3x3 L_inf-dist conv layer, batch 128, 128->128 channels, 32x32, groups 4, "
                      "forward+backward (unfold outside the timed region)",
                 kernel=("inf_dist_forward", lambda x_, w_, *_: 2 * mnk(x_, w_), lambda *a: True,
-                        "inf_forward_kernel (conv layout, k tracked in the loop)", 2))
+                        "inf_forward_shortk_kernel (conv layout, the whole reduction of a tile resident in LDS)", 2))
 
 
 def workload_c4i(pkg, torch, dev):
@@ -406,8 +407,94 @@ def workload_c4i(pkg, torch, dev):
     return wl
 
 
+C4_P = 8.0   # --p moves it, as for c2
+
+
+def workload_c4p(pkg, torch, dev):
+    """configs[4]'s layer in the p-norm phase of training (the reference's conv recipe spends most epochs at finite
+    p): the image goes in and the image gradient comes out, straight from the image."""
+    import torch.nn.functional as F
+    p = C4_P
+    g = torch.Generator().manual_seed(0)
+    img = torch.rand(128, 128, 32, 32, generator=g)
+    w = (torch.randn(128, 32, 3, 3, generator=g) / math.sqrt(288)).reshape(128, 288).contiguous()
+    go = torch.randn(128, 128, 1024, generator=g)
+    imgd, god4 = img.to(dev), go.to(dev).view(128, 128, 32, 32)
+    layer = pkg.NormDistConv(128, 128, 3, padding=1, group=4, p=p, bias=False, mean_normalize=False).to(dev)
+    with torch.no_grad():
+        layer.weight.copy_(w.view_as(layer.weight))
+    cpp = pkg.norm_dist_cpp
+
+    def step():
+        layer.weight.grad = None
+        xi = imgd.detach().requires_grad_(True)
+        y, _, _ = layer(xi)
+        y.backward(god4)
+
+    def step_columns():
+        # the same layer through the native unfold, the column kernels and the native fold
+        keep = cpp.norm_dist_conv_supported
+        cpp.norm_dist_conv_supported = lambda *a, **k: False
+        try:
+            step()
+        finally:
+            cpp.norm_dist_conv_supported = keep
+
+    wd = w.to(dev).requires_grad_(True)
+
+    def step_torch_unfold():
+        # through torch's unfold and autograd's fold, as the reference's layer does it
+        wd.grad = None
+        xi = imgd.detach().requires_grad_(True)
+        y = pkg.norm_dist(F.unfold(xi, 3, padding=1), wd, 4, p)
+        y.backward(god4.view(128, 128, 1024))
+
+    def cpu(oracle, rows):
+        xs, gs = F.unfold(img[:rows], 3, padding=1).contiguous(), go[:rows].contiguous()
+        out = oracle.norm_dist_forward(xs, w, 4, p)
+        oracle.norm_dist_backward_input(gs, xs, w, out, 4, p)
+        oracle.norm_dist_backward_weight(gs, xs, w, out, 4, p)
+        return 3 * rows * 1024 * 128 * 288
+
+    def formula(rows):
+        xs = F.unfold(img[:rows], 3, padding=1).requires_grad_(True)
+        wr = w.clone().requires_grad_(True)
+        pkg.norm_dist(xs, wr, 4, p, use_custom_cuda_func=False).backward(go[:rows])
+        return 3 * rows * 1024 * 128 * 288
+
+    def check(oracle, stack_check, rows=4):
+        rep = stack_check.Report()
+        xs, gs = F.unfold(img[:rows], 3, padding=1).contiguous(), go[:rows].contiguous()
+        ev = oracle.norm_dist_forward(xs, w, 4, p)
+        egx, mgx = oracle.norm_dist_backward_input(gs, xs, w, ev, 4, p, with_abs_terms=True)
+        egw, mgw = oracle.norm_dist_backward_weight(gs, xs, w, ev, 4, p, with_abs_terms=True)
+        layer.weight.grad = None
+        xi = imgd[:rows].detach().requires_grad_(True)
+        yi, _, _ = layer(xi)
+        yi.backward(god4[:rows])
+        torch.cuda.synchronize()
+        got = yi.detach().cpu().reshape(rows, 128, 1024)
+        rep.ratio("image: values", stack_check.close_ratio(got, ev), got, ev)
+        egi = F.fold(egx.double(), (32, 32), 3, padding=1)
+        mgi = F.fold(mgx.double(), (32, 32), 3, padding=1)
+        rep.ratio("image: grad_image", stack_check.sum_ratio(xi.grad.cpu(), egi, mgi, p=p), xi.grad.cpu(), egi)
+        gw = layer.weight.grad.cpu().reshape(128, 288)
+        rep.ratio("image: grad_weight", stack_check.sum_ratio(gw, egw, mgw, p=p, n_terms=torch.full_like(egw, rows * 1024)), gw, egw)
+        layer.weight.grad = None
+        return rep
+
+    return dict(step=step, ops=3 * 128 * 1024 * 128 * 288, images=128, full_rows=128, cpu=cpu, formula=formula,
+                check=check,
+                step_alt=[("ms_per_step_native_unfold_columns_fold", step_columns),
+                          ("ms_per_step_with_torch_unfold_and_fold", step_torch_unfold)],
+                name=f"configs[4]'s layer at p={p:g} from the image: 3x3 p-norm dist conv layer, batch 128, 128->128 "
+                     "channels, 32x32, groups 4, forward+backward (3 dist-op passes), no unfolded tensor",
+                kernel=("norm_dist_conv_backward_input", lambda go_, img_, w_, o_, *_: 7 * o_.numel() * w_.size(1),
+                        lambda *a: True, "norm_backward_kernel (grad_input added onto the image)", 7))
+
+
 WORKLOADS = {"c0": workload_c0, "c1": workload_c1, "c1t": workload_c1t, "c2": workload_c2, "c3": workload_c3,
-             "c4": workload_c4, "c4i": workload_c4i}
+             "c4": workload_c4, "c4i": workload_c4i, "c4p": workload_c4p}
 
 
 def cpu_baseline(wl, target_seconds=12.0):
@@ -469,7 +556,8 @@ def main():
                     help="untimed set-up: run the workload this long before the warm-up steps so the clock settles")
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c1")
     ap.add_argument("--p", type=float, default=None,
-                    help="exponent for --workload c2 (default 8, the configuration; the reference anneals it to 1000)")
+                    help="exponent for --workload c2 or c4p (default 8, the configuration; the reference anneals it "
+                         "to 1000)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-parity", action="store_true",
                     help="skip the comparison with the CPU oracle that runs before the timed region (profiler runs)")
@@ -489,10 +577,10 @@ def main():
     torch.cuda.set_device(dev)
 
     if args.p is not None:
-        if args.workload != "c2" or not (args.p > 1 and math.isfinite(args.p)):
-            sys.exit("--p applies to --workload c2 and must be a finite exponent above 1")
-        global C2_P
-        C2_P = args.p
+        if args.workload not in ("c2", "c4p") or not (args.p > 1 and math.isfinite(args.p)):
+            sys.exit("--p applies to --workload c2 or c4p and must be a finite exponent above 1")
+        global C2_P, C4_P
+        C2_P = C4_P = args.p
     wl = WORKLOADS[args.workload](pkg, torch, dev)
     step = wl["step"]
     kname, flops_of, accept, kdesc, flops_per_op = wl["kernel"]

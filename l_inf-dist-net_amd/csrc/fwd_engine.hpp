@@ -9,9 +9,11 @@
 namespace ldist {
 
 // Global -> register -> LDS staging of one pipeline stage: NX input panels
-// (x, or lower and upper) followed by the weight panel.
-template <class GEO, bool CONV, int VEC, int NX>
+// (x, or lower and upper) followed by the weight panel.  IMG: the input is the image of a convolution-shaped
+// layer and the panel is gathered from it (set `win` before init); the output keeps the conv layout.
+template <class GEO, bool CONV, int VEC, int NX, bool IMG = false>
 struct Stager {
+    static_assert(!IMG || CONV, "an image has positions");
     static constexpr int STAGE = NX * GEO::XS + GEO::WS;  // floats per stage
     // Two LDS buffers (one barrier per stage) when that still lets a CU hold two waves
     // per SIMD, i.e. one 512-lane or two 256-lane workgroups in 160 KB; else one buffer.
@@ -23,6 +25,10 @@ struct Stager {
     WLoad wl;
     XLoadK xlk[NX];
     XLoadM xlm[NX];
+    using XLoadI = RowsImg<GEO::BM, GEO::SM, GEO::NT, GEO::KK>;
+    XLoadI xli[IMG ? NX : 1];
+    ImgWin win;
+    int grp_;
     int off_m[XLoadM::N];
     const float* wbase;
     const float* in[NX];
@@ -40,13 +46,20 @@ struct Stager {
 #pragma unroll
         for (int q = 0; q < NX; q++)
             in[q] = CONV ? input[q] : input[q] + ((size_t)m0 * d.G + g) * K;  // fc: row m is image b
-        if constexpr (CONV) XLoadM::offsets(off_m, m0, d.M, d.HW, d.G, g, K, tid);
+        grp_ = g;
+        if constexpr (IMG) {
+#pragma unroll
+            for (int q = 0; q < NX; q++) xli[q].init(win, m0, d.M, tid);
+        } else if constexpr (CONV) {
+            XLoadM::offsets(off_m, m0, d.M, d.HW, d.G, g, K, tid);
+        }
     }
     __device__ __forceinline__ void load(int k0) {
         wl.load(wbase, K, rows_w, k0, K, tid);
 #pragma unroll
         for (int q = 0; q < NX; q++) {
-            if constexpr (CONV) xlm[q].load(in[q], off_m, kstride, k0, K, tid);
+            if constexpr (IMG) xli[q].load(in[q], win, grp_, k0, K, tid);
+            else if constexpr (CONV) xlm[q].load(in[q], off_m, kstride, k0, K, tid);
             else xlk[q].load(in[q], ld_x, rows_x, k0, K, tid);
         }
     }
@@ -84,7 +97,8 @@ struct Stager {
     __device__ __forceinline__ void store(float* stage) const {
 #pragma unroll
         for (int q = 0; q < NX; q++) {
-            if constexpr (CONV) xlm[q].store(stage + q * GEO::XS, tid);
+            if constexpr (IMG) xli[q].store(stage + q * GEO::XS, tid);
+            else if constexpr (CONV) xlm[q].store(stage + q * GEO::XS, tid);
             else xlk[q].store(stage + q * GEO::XS, tid);
         }
         wl.store(stage + NX * GEO::XS, tid);

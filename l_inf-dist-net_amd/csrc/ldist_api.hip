@@ -279,6 +279,62 @@ int ldist_inf_dist_bound_conv_forward(const float* lower_img, const float* upper
                                             pr.device, (hipStream_t)stream));
 }
 
+int ldist_norm_dist_conv_supported(int C, int H, int W, int CO, int G, int KH, int KW, int stride, int padding,
+                                   int dilation) {
+    ldist::ConvGeom q{};
+    if (CO <= 0 || G <= 0) return 0;
+    if (conv_geometry(1, C, H, W, KH, KW, stride, padding, dilation, q) != LDIST_OK) return 0;
+    return ldist::norm_conv_supported(q, G, CO) ? 1 : 0;
+}
+
+namespace {
+// Shared argument checks of the three p-norm entry points that read the image.
+int norm_conv_prepare(int B, int C, int H, int W, int CO, int G, int KH, int KW, int stride, int padding, int dilation,
+                      float p, ldist::ConvGeom& q, ldist::Problem& pr) {
+    if (CO <= 0 || G <= 0 || !valid_p(p)) return LDIST_EINVAL;
+    if (int rc = conv_geometry(B, C, H, W, KH, KW, stride, padding, dilation, q)) return rc;
+    if (C % G != 0 || CO % G != 0) return LDIST_EINVAL;
+    if ((long long)B * CO * q.HO * q.WO >= (1LL << 31) || (long long)CO * (C / G) * KH * KW >= (1LL << 31))
+        return LDIST_ERANGE;
+    if (!ldist::norm_conv_supported(q, G, CO)) return LDIST_EUNSUPPORTED;
+    return current_device(pr);
+}
+}  // namespace
+
+int ldist_norm_dist_conv_forward(const float* img, const float* weight, int B, int C, int H, int W, int CO, int G, int KH,
+                                 int KW, int stride, int padding, int dilation, float* output, float p,
+                                 ldist_stream_t stream) {
+    ldist::ConvGeom q{};
+    ldist::Problem pr{};
+    if (!img || !weight || !output) return LDIST_EINVAL;
+    if (int rc = norm_conv_prepare(B, C, H, W, CO, G, KH, KW, stride, padding, dilation, p, q, pr)) return rc;
+    return finish(ldist::norm_conv_forward(img, weight, output, p, q, G, CO, pr.num_cu, pr.device, (hipStream_t)stream));
+}
+
+int ldist_norm_dist_conv_backward_input(const float* grad_output, const float* img, const float* weight,
+                                        const float* output, int B, int C, int H, int W, int CO, int G, int KH, int KW,
+                                        int stride, int padding, int dilation, float* grad_img, float p,
+                                        ldist_stream_t stream) {
+    ldist::ConvGeom q{};
+    ldist::Problem pr{};
+    if (!grad_output || !img || !weight || !output || !grad_img) return LDIST_EINVAL;
+    if (int rc = norm_conv_prepare(B, C, H, W, CO, G, KH, KW, stride, padding, dilation, p, q, pr)) return rc;
+    return finish(ldist::norm_conv_backward_input(grad_output, img, weight, output, grad_img, p, q, G, CO, pr.num_cu,
+                                                  pr.device, (hipStream_t)stream));
+}
+
+int ldist_norm_dist_conv_backward_weight(const float* grad_output, const float* img, const float* weight,
+                                         const float* output, int B, int C, int H, int W, int CO, int G, int KH, int KW,
+                                         int stride, int padding, int dilation, float* grad_weight, float p,
+                                         ldist_stream_t stream) {
+    ldist::ConvGeom q{};
+    ldist::Problem pr{};
+    if (!grad_output || !img || !weight || !output || !grad_weight) return LDIST_EINVAL;
+    if (int rc = norm_conv_prepare(B, C, H, W, CO, G, KH, KW, stride, padding, dilation, p, q, pr)) return rc;
+    return finish(ldist::norm_conv_backward_weight(grad_output, img, weight, output, grad_weight, p, q, G, CO, pr.num_cu,
+                                                   pr.device, (hipStream_t)stream));
+}
+
 int ldist_set_conv_staging_override(int mode) {
     if (mode < 0 || mode > 3) return LDIST_EINVAL;
     ldist::g_conv_staging_override = mode;

@@ -21,6 +21,8 @@
 
 #include <type_traits>
 
+#include "conv_window.hpp"
+
 namespace ldist {
 
 constexpr int kChunk = 32;  // k values between two "did the maximum move" checks
@@ -378,6 +380,42 @@ struct RowsM {
             } else {
                 off_m[i] = -1;
             }
+        }
+    }
+};
+
+// The input panel of the convolution-shaped layer gathered from the image (see conv_window.hpp): same panel as
+// RowsM would load from the unfolded tensor.  A lane keeps one row of the tile, i.e. one window, and walks k.
+template <int ROWS, int LD, int NT, int KK>
+struct RowsImg {
+    static constexpr int TOTAL = KK * ROWS;
+    static constexpr int N = TOTAL / NT;
+    static constexpr int KSTEP = NT / ROWS;
+    static_assert(NT % ROWS == 0 && TOTAL % NT == 0, "lane keeps its row across iterations");
+    float v[N];
+    WinRow row;
+    bool row_ok;
+
+    __device__ __forceinline__ void init(const ImgWin& q, int m0, int M, int tid) {
+        const int m = m0 + tid % ROWS;
+        row_ok = m < M;
+        row.set(q, row_ok ? m : 0);
+    }
+    __device__ __forceinline__ void load(const float* __restrict__ img, const ImgWin& q, int g, int k0, int K, int tid) {
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const int k = k0 + tid / ROWS + i * KSTEP;
+            size_t off;
+            const bool ok = win_tap(q, row, g, k < K ? k : 0, off) && row_ok && k < K;
+            v[i] = ok ? img[off] : 0.f;
+        }
+    }
+    __device__ __forceinline__ void store(float* __restrict__ panel, int tid) const {
+        const int mq = tid % ROWS;
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const int kk = tid / ROWS + i * KSTEP;
+            panel[kk * LD + (mq ^ swz(kk))] = v[i];
         }
     }
 };

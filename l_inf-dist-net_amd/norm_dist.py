@@ -138,6 +138,35 @@ class _ConvInfDist(torch.autograd.Function):
         return grad_img, grad_w, None, None, None, None, None
 
 
+class _ConvNormDist(torch.autograd.Function):
+    """The p-norm layer (finite p) on an image, forward and both gradients from the image itself: neither the
+    unfolded input nor the gradient of the columns exists.  Same results as unfold + DistF to float rounding."""
+
+    @staticmethod
+    def forward(ctx, img, weight, group, p, kernel_size, dilation, padding, stride):
+        img = img.contiguous()
+        weight = weight.contiguous()
+        ho, wo = norm_dist_cpp.conv_output_size(img.size(2), img.size(3), kernel_size, stride, padding, dilation)
+        y = torch.empty(img.size(0), weight.size(0), ho * wo, device=img.device, dtype=img.dtype)
+        norm_dist_cpp.norm_dist_conv_forward(img, weight, y, group, p, kernel_size, stride, padding, dilation)
+        ctx.save_for_backward(img, weight, y)
+        ctx.group, ctx.p, ctx.window = group, p, (kernel_size, stride, padding, dilation)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        img, weight, y = ctx.saved_tensors
+        g = grad_output.contiguous()
+        grad_img = grad_w = None
+        if ctx.needs_input_grad[0]:
+            grad_img = torch.empty_like(img)   # the call writes every element
+            norm_dist_cpp.norm_dist_conv_backward_input(g, img, weight, y, grad_img, ctx.group, ctx.p, *ctx.window)
+        if ctx.needs_input_grad[1]:
+            grad_w = torch.zeros_like(weight)  # this kernel adds onto the buffer
+            norm_dist_cpp.norm_dist_conv_backward_weight(g, img, weight, y, grad_w, ctx.group, ctx.p, *ctx.window)
+        return grad_img, grad_w, None, None, None, None, None, None
+
+
 def _pairwise_difference(inp, weight, group):
     """(B, G, CO/G, CI/G, HW) tensor of input minus weight, by broadcasting."""
     b, _, hw = inp.shape
@@ -292,6 +321,15 @@ class NormDistConv(nn.Module):
                 not (self.kernel_size == 1 and self.stride == 1 and self.padding == 0) and
                 (self.in_channels // self.group) * x.size(3) <= norm_dist_cpp.FOLDED_MAX_ROW_FLOATS)
 
+    def _norm_from_image(self, x):
+        """True when the p-norm layer runs from the image (finite p, float32 on the GPU, a geometry the image
+        kernels cover)."""
+        return (not math.isinf(self.p) and self.p > 1 and x.is_cuda and x.dtype == torch.float32 and
+                self.weight.dtype == torch.float32 and
+                norm_dist_cpp.norm_dist_conv_supported(self.in_channels, x.size(2), x.size(3), self.out_channels,
+                                                       self.group, self.kernel_size, self.stride, self.padding,
+                                                       self.dilation))
+
     def _bound_from_images(self, lower, upper):
         """True when the interval bounds can be computed straight from the two images (the bound path carries no
         gradient, as in the reference: it runs in evaluation mode only)."""
@@ -338,6 +376,9 @@ class NormDistConv(nn.Module):
             return y.view(shape), lo.view(shape), hi.view(shape)
         if self._fused_inf_conv(x):
             y = _ConvInfDist.apply(x, w2d, self.group, self.kernel_size, self.dilation, self.padding, self.stride)
+        elif self._norm_from_image(x):
+            y = _ConvNormDist.apply(x, w2d, self.group, self.p, self.kernel_size, self.dilation, self.padding,
+                                    self.stride)
         else:
             y = norm_dist(self._columns(x), w2d, self.group, p=self.p, tag=self.tag)
         y = self._shift(y.view(x.size(0), -1, *out_hw))  # in training mode only y moves the running mean

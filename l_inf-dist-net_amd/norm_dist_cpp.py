@@ -306,6 +306,63 @@ def inf_dist_conv_forward(img, weight, output, pos, G, kernel_size, stride=1, pa
           _p(pos))
 
 
+def norm_dist_conv_supported(C, H, W, CO, G, kernel_size, stride=1, padding=0, dilation=1):
+    """True when the three norm_dist_conv_* calls cover the geometry (3x3 windows, more than one output position,
+    more than 16 outputs per group); otherwise unfold + the column calls are the way."""
+    k = int(kernel_size)
+    return bool(_lib.lib().ldist_norm_dist_conv_supported(int(C), int(H), int(W), int(CO), int(G), k, k, int(stride),
+                                                           int(padding), int(dilation)))
+
+
+def _norm_conv_args(img, weight, output, G, kernel_size, stride, padding, dilation):
+    B, C, H, W, KH, KW, S, P, D = _conv_args(img, kernel_size, stride, padding, dilation)
+    HO, WO = conv_output_size(H, W, KH, S, P, D)
+    _expect(weight.dim() == 2 and C % G == 0 and weight.size(1) == C // G * KH * KW, "weight must be (CO, C/G*k*k)")
+    CO = weight.size(0)
+    _expect(output.shape == (B, CO, HO * WO), "output must be (B, CO, HO*WO)")
+    return B, C, H, W, CO, G, KH, KW, S, P, D
+
+
+def norm_dist_conv_forward(img, weight, output, G, p, kernel_size, stride=1, padding=0, dilation=1):
+    """p-norm forward of the conv-shaped layer straight from the image: output (B, CO, HO*WO) equal to
+    norm_dist_forward on F.unfold(img, ...), without building the columns."""
+    for t, n in ((img, "img"), (weight, "weight"), (output, "output")):
+        _check_input(t, n)
+    dev = _same_device(img, weight, output)
+    args = _norm_conv_args(img, weight, output, G, kernel_size, stride, padding, dilation)
+    _call("ldist_norm_dist_conv_forward", dev, _p(img), _p(weight), *args, _p(output), float(p))
+
+
+def norm_dist_conv_backward_input(grad_output, img, weight, output, grad_img, G, p, kernel_size, stride=1, padding=0,
+                                  dilation=1):
+    """Gradient of the p-norm conv-shaped layer with respect to the image: norm_dist_backward_input on the columns
+    followed by fold, without either tensor of columns.  Every element of grad_img is written."""
+    for t, n in ((grad_output, "grad_output"), (img, "img"), (weight, "weight"), (output, "output"),
+                 (grad_img, "grad_img")):
+        _check_input(t, n)
+    dev = _same_device(grad_output, img, weight, output, grad_img)
+    args = _norm_conv_args(img, weight, output, G, kernel_size, stride, padding, dilation)
+    _expect(grad_output.shape == output.shape and grad_img.shape == img.shape,
+            "grad_output must match output and grad_img the image")
+    _call("ldist_norm_dist_conv_backward_input", dev, _p(grad_output), _p(img), _p(weight), _p(output), *args,
+          _p(grad_img), float(p))
+
+
+def norm_dist_conv_backward_weight(grad_output, img, weight, output, grad_weight, G, p, kernel_size, stride=1,
+                                   padding=0, dilation=1):
+    """Gradient of the p-norm conv-shaped layer with respect to the weight, reading the image instead of the
+    columns.  Added onto grad_weight, like norm_dist_backward_weight."""
+    for t, n in ((grad_output, "grad_output"), (img, "img"), (weight, "weight"), (output, "output"),
+                 (grad_weight, "grad_weight")):
+        _check_input(t, n)
+    dev = _same_device(grad_output, img, weight, output, grad_weight)
+    args = _norm_conv_args(img, weight, output, G, kernel_size, stride, padding, dilation)
+    _expect(grad_output.shape == output.shape and grad_weight.shape == weight.shape,
+            "grad_output must match output and grad_weight the weight")
+    _call("ldist_norm_dist_conv_backward_weight", dev, _p(grad_output), _p(img), _p(weight), _p(output), *args,
+          _p(grad_weight), float(p))
+
+
 def inf_dist_bound_conv_forward_supported(C, H, W, CO, G, kernel_size, stride=1, padding=0, dilation=1):
     """True when inf_dist_bound_conv_forward covers the geometry (3x3, dilation 1, stride 1 or 2, a layer large
     enough to fill the GPU); otherwise unfold both images and call inf_dist_bound_forward."""

@@ -1104,3 +1104,139 @@ def test_error_codes_and_checks():
         cpp.inf_dist_forward(x, torch.zeros(6, 4, device=DEV).t(), out, pos, 1)  # weight not contiguous
     with pytest.raises(RuntimeError):
         cpp.norm_dist_forward(x, w, out, 1, 0.5)
+
+
+NORM_IMAGE_CASES = [  # B, C, H, W, CO, G, stride, padding, dilation
+    (2, 3, 32, 32, 20, 1, 1, 1, 1),      # first layer of the CIFAR net: 3 channels, K = 27 (not a multiple of 4)
+    (1, 16, 32, 32, 96, 1, 1, 1, 1),
+    (2, 128, 32, 32, 128, 4, 1, 1, 1),   # the benchmark layer at a small batch
+    (1, 8, 8, 64, 40, 1, 1, 1, 1),       # wide rows
+    (2, 72, 16, 16, 72, 1, 1, 1, 1),     # many channels in one group
+    (2, 16, 28, 28, 32, 1, 1, 1, 1),     # MNIST-sized rows
+    (2, 8, 16, 16, 24, 1, 2, 1, 1),      # stride 2
+    (2, 5, 17, 17, 20, 1, 2, 0, 1),      # stride 2 without padding, odd image, odd channel count
+    (2, 4, 6, 6, 24, 1, 1, 2, 1),        # padding wider than the window needs
+    (2, 6, 12, 12, 20, 1, 1, 2, 2),      # dilation 2
+    (2, 8, 16, 16, 40, 2, 1, 1, 1),      # two groups of 20 outputs
+    (3, 8, 9, 7, 18, 1, 1, 1, 1),        # 63 positions per image: rows of a tile cross image borders, HW % 4 != 0
+]
+
+
+def _norm_image_problem(case, seed):
+    import torch.nn.functional as F
+    B, C, H, W, CO, G, s_, p_, d_ = case
+    g = gen(seed)
+    img = torch.rand(B, C, H, W, generator=g)
+    w = torch.randn(CO, C // G * 9, generator=g) / (C // G * 9) ** 0.5
+    cols = F.unfold(img, 3, d_, p_, s_).contiguous()
+    go = torch.randn(B, CO, cols.size(2), generator=g)
+    return img, w, cols, go
+
+
+@pytest.mark.parametrize("p", [8.0, 3.0, 5.5, 100.0])
+@pytest.mark.parametrize("case", NORM_IMAGE_CASES)
+def test_norm_conv_forward_from_the_image(case, p):
+    """p-norm forward straight from the image against the oracle on torch's unfolded columns (rel 1e-5), and
+    against this library's column kernel on the same columns bit for bit (the same arithmetic in the same order:
+    only the loads differ)."""
+    from gpu_common import DEV, cpp, say
+    B, C, H, W, CO, G, s_, p_, d_ = case
+    say("norm_conv_forward", case, "p", p)
+    assert cpp.norm_dist_conv_supported(C, H, W, CO, G, 3, s_, p_, d_)
+    img, w, cols, _ = _norm_image_problem(case, 91)
+    want = oracle.norm_dist_forward(cols, w, G, p)
+    out = torch.full(want.shape, float("nan"), device=DEV)
+    cpp.norm_dist_conv_forward(img.to(DEV), w.to(DEV), out, G, p, 3, s_, p_, d_)
+    from_cols = torch.full(want.shape, float("nan"), device=DEV)
+    cpp.norm_dist_forward(cols.to(DEV), w.to(DEV), from_cols, G, p)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out.cpu(), want, rtol=RTOL, atol=ATOL)
+    assert torch.equal(out, from_cols)
+
+
+@pytest.mark.parametrize("p", [8.0, 3.0, 5.5, 100.0])
+@pytest.mark.parametrize("case", NORM_IMAGE_CASES)
+def test_norm_conv_backward_from_the_image(case, p):
+    """Both p-norm gradients straight from the image: grad_weight against the oracle on the unfolded columns,
+    grad_img against the oracle's gradient of the columns folded back in float64 (rel 1e-5 / abs 1e-6 relative to
+    the magnitude of the summed terms).  grad_img starts as NaN (the call writes every element), grad_weight at
+    0.125 (the call adds)."""
+    import torch.nn.functional as F
+    from gpu_common import DEV, cpp, say
+    B, C, H, W, CO, G, s_, p_, d_ = case
+    say("norm_conv_backward", case, "p", p)
+    img, w, cols, go = _norm_image_problem(case, 92)
+    out = oracle.norm_dist_forward(cols, w, G, p)
+    ex, mx = oracle.norm_dist_backward_input(go, cols, w, out, G, p, with_abs_terms=True)
+    ew, mw = oracle.norm_dist_backward_weight(go, cols, w, out, G, p, with_abs_terms=True)
+    fold = lambda t: F.fold(t.double(), (H, W), 3, d_, p_, s_)
+    gi = torch.full((B, C, H, W), float("nan"), device=DEV)
+    gw = torch.full((CO, C // G * 9), 0.125, device=DEV)
+    args = (go.to(DEV), img.to(DEV), w.to(DEV), out.to(DEV))
+    cpp.norm_dist_conv_backward_input(*args, gi, G, p, 3, s_, p_, d_)
+    cpp.norm_dist_conv_backward_weight(*args, gw, G, p, 3, s_, p_, d_)
+    torch.cuda.synchronize()
+    assert_sum_close(gi.cpu(), fold(ex), fold(mx), p, RTOL, ATOL)
+    assert_sum_close(gw.cpu() - 0.125, ew, mw, p, RTOL, ATOL)
+
+
+def test_norm_conv_unsupported_geometries_are_refused():
+    """Windows other than 3x3, a single output position and layers with at most 16 outputs per group are left to
+    the column kernels: the query says so and the entry point enqueues nothing."""
+    from gpu_common import DEV, cpp, pkg
+    assert not cpp.norm_dist_conv_supported(8, 16, 16, 32, 1, 5, 1, 2, 1)
+    assert not cpp.norm_dist_conv_supported(8, 3, 3, 32, 1, 3, 1, 0, 1)
+    assert not cpp.norm_dist_conv_supported(8, 16, 16, 16, 1, 3, 1, 1, 1)
+    assert cpp.norm_dist_conv_supported(8, 16, 16, 40, 2, 3, 1, 1, 1)        # 20 per group: covered
+    img = torch.rand(1, 8, 16, 16, device=DEV)
+    w = torch.randn(16, 72, device=DEV)
+    out = torch.full((1, 16, 256), 7.0, device=DEV)
+    with pytest.raises(RuntimeError):
+        cpp.norm_dist_conv_forward(img, w, out, 1, 8.0, 3, 1, 1, 1)
+    torch.cuda.synchronize()
+    assert bool((out == 7.0).all())
+    del pkg
+
+
+@pytest.mark.parametrize("p", [8.0, 20.0])
+def test_norm_dist_conv_layer_runs_from_the_image_without_columns(p):
+    """NormDistConv at finite p: same output and gradients as the layer forced through unfold + columns, and the
+    peak of allocated memory stays below the size of the unfolded input (which therefore was never built)."""
+    from gpu_common import DEV, cpp, pkg, say
+    say("norm_dist_conv_layer", p)
+    torch.manual_seed(5)
+    layer = pkg.NormDistConv(128, 128, 3, padding=1, group=4, p=p, bias=True, mean_normalize=False).to(DEV)
+    x = torch.rand(8, 128, 32, 32, device=DEV)
+    go = torch.randn(8, 128, 32, 32, device=DEV)
+
+    def run(force_columns):
+        layer.zero_grad(set_to_none=True)
+        xi = x.clone().requires_grad_(True)
+        keep = cpp.norm_dist_conv_supported
+        if force_columns:
+            cpp.norm_dist_conv_supported = lambda *a, **k: False
+        try:
+            torch.cuda.synchronize()
+            torch.cuda.reset_peak_memory_stats()
+            base = torch.cuda.memory_allocated()
+            y, _, _ = layer(xi)
+            y.backward(go)
+            torch.cuda.synchronize()
+            peak = torch.cuda.max_memory_allocated() - base
+        finally:
+            cpp.norm_dist_conv_supported = keep
+        return y.detach(), xi.grad, layer.weight.grad.clone(), peak
+
+    layer.train()
+    y1, gx1, gw1, peak_img = run(False)
+    y0, gx0, gw0, peak_cols = run(True)
+    cols_bytes = 8 * 128 * 9 * 1024 * 4
+    assert peak_img < cols_bytes <= peak_cols
+    torch.testing.assert_close(y1, y0, rtol=RTOL, atol=ATOL)
+    # Two float32 sums in different orders.  grad_weight adds 8192 terms of either sign per element, split over
+    # workgroups that add their parts atomically in either path; the kernels' own accuracy is what the two tests
+    # above check against the oracle.  A wrong tap or sign would be off by the gradient itself.  (No mean shift in
+    # this layer: it centres the incoming gradient, and the terms of the -10 centre taps, all of one sign and of
+    # ratio 1, then cancel to nothing, which leaves only rounding noise to compare.)
+    for a, b in ((gx1, gx0), (gw1, gw0)):
+        assert float((a - b).abs().max()) <= 1e-3 * float(b.abs().max())
