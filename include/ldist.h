@@ -213,15 +213,16 @@ LDIST_API int ldist_inf_dist_bound_conv_forward(const float* lower_img, const fl
  * norm_dist_backward_input_cuda and norm_dist_backward_weight_cuda (model/norm_dist.cpp:5-12,
  * model/norm_dist_cuda.cu:228-459) and the fold that autograd runs behind F.unfold:
  *   img (B, C, H, W), weight (CO, C/G*KH*KW), output and grad_output (B, CO, HO*WO), p > 1 finite.
- * Same values as the column entry points on ldist_unfold(img) to float rounding (forward and grad_weight: the same
- * arithmetic in the same order; grad_img: a pixel adds up to KH*KW partial sums in no fixed order).
+ * Same values as the column entry points on ldist_unfold(img) to float rounding (forward with more than 16 outputs
+ * per group and grad_weight: the same arithmetic in the same order; grad_img: a pixel adds up to KH*KW partial sums
+ * in no fixed order).
  *   forward:          output is written.
  *   backward_input:   grad_img (B, C, H, W) is written whole; it may be uninitialised on entry.
  *   backward_weight:  grad_weight (CO, C/G*KH*KW) is added to and must hold zeros (or the values to accumulate
  *                     onto) on entry, as with ldist_norm_dist_backward_weight.
- * Covers 3x3 windows of any stride, padding and dilation with more than one output position and more than 16
- * outputs per group; ldist_norm_dist_conv_supported returns 1 for such a geometry, 0 otherwise, and the three
- * entry points return LDIST_EUNSUPPORTED for the rest (nothing is enqueued). */
+ * Covers 3x3 windows of any stride, padding and dilation with more than one output position;
+ * ldist_norm_dist_conv_supported returns 1 for such a geometry, 0 otherwise, and the three entry points return
+ * LDIST_EUNSUPPORTED for the rest (nothing is enqueued). */
 LDIST_API int ldist_norm_dist_conv_supported(int C, int H, int W, int CO, int G, int KH, int KW, int stride, int padding,
                                              int dilation);
 LDIST_API int ldist_norm_dist_conv_forward(const float* img, const float* weight, int B, int C, int H, int W, int CO, int G,

@@ -114,8 +114,8 @@ hipError_t unfold(const float* img, float* cols, const ConvGeom& q, hipStream_t 
 hipError_t fold(const float* gcols, float* gimg, const ConvGeom& q, hipStream_t stream);
 // L_inf forward straight from the image (3x3 window, dilation 1, stride 1 or 2; a group's channels
 // either few enough to stay in LDS or a multiple of four); inf_conv_forward_supported tells whether a geometry is covered.
-// p-norm layer of convolution shape straight from the image (norm_conv.hip): 3x3 windows, more than 16 outputs per
-// group; norm_conv_supported tells whether a geometry is covered.
+// p-norm layer of convolution shape straight from the image (norm_conv.hip): 3x3 windows, more than one output
+// position; norm_conv_supported tells whether a geometry is covered.
 bool norm_conv_supported(const ConvGeom& q, int G, int CO);
 hipError_t norm_conv_forward(const float* img, const float* weight, float* output, float p, const ConvGeom& q, int G,
                              int CO, int num_cu, int device, hipStream_t stream);

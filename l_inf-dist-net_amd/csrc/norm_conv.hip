@@ -13,7 +13,6 @@
 // read nine times over, from L2.
 #include "norm_backward_kernel.hpp"
 #include "norm_forward_kernel.hpp"
-#include "skinny.hpp"
 
 namespace ldist {
 
@@ -45,13 +44,12 @@ __global__ void __launch_bounds__(256) zero_fill_kernel(float* __restrict__ p, s
 
 }  // namespace
 
-// 3x3 windows (any stride, padding, dilation), more than one output position, and more outputs per group than the
-// kernels for skinny layers take (those have no image form).
+// 3x3 windows (any stride, padding, dilation) with more than one output position.  Layers with few outputs per
+// group, for which the column entry point has a kernel of its own, run on the tiled kernel here.
 bool norm_conv_supported(const ConvGeom& q, int G, int CO) {
     if (q.KH != 3 || q.KW != 3) return false;
     if (G <= 0 || q.C % G != 0 || CO % G != 0) return false;
-    if ((long long)q.HO * q.WO <= 1) return false;
-    return CO / G > kSkinnyMaxNG;
+    return (long long)q.HO * q.WO > 1;
 }
 
 hipError_t norm_conv_forward(const float* img, const float* weight, float* output, float p, const ConvGeom& q, int G,

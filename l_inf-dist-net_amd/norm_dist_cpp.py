@@ -307,8 +307,8 @@ def inf_dist_conv_forward(img, weight, output, pos, G, kernel_size, stride=1, pa
 
 
 def norm_dist_conv_supported(C, H, W, CO, G, kernel_size, stride=1, padding=0, dilation=1):
-    """True when the three norm_dist_conv_* calls cover the geometry (3x3 windows, more than one output position,
-    more than 16 outputs per group); otherwise unfold + the column calls are the way."""
+    """True when the three norm_dist_conv_* calls cover the geometry (3x3 windows, more than one output position);
+    otherwise unfold + the column calls are the way."""
     k = int(kernel_size)
     return bool(_lib.lib().ldist_norm_dist_conv_supported(int(C), int(H), int(W), int(CO), int(G), k, k, int(stride),
                                                            int(padding), int(dilation)))

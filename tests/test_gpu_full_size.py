@@ -281,3 +281,46 @@ def test_config4_layer_from_the_image():
     expect = F.fold(gcols.double(), (32, 32), 3, padding=1)
     terms = F.fold(oracle.inf_dist_backward_input(go.abs(), ep & ~SIGN, 1152, 4).double(), (32, 32), 3, padding=1).abs()
     assert_sum_close(gimg.cpu(), expect, terms)
+
+
+def test_config4_layer_at_p8_from_the_image():
+    """Config 4's layer in the p-norm phase, straight from the image at the full batch of 128.  The forward is
+    checked on every image against this library's column kernel (bit for bit: the same arithmetic) and on the first
+    four against the oracle; the gradients are taken for a grad_output that is zero outside the first four images, so
+    that grad_weight of the full-size launch equals the oracle's on those four (rows are independent) and grad_img
+    must be exactly zero everywhere else."""
+    import torch.nn.functional as F
+    from gpu_common import DEV, cpp, say
+    say("config 4 at p = 8 from the image: 128 x 128 x 32 x 32, 128 outputs, 4 groups")
+    p, rows = 8.0, 4
+    g = gen(9)
+    img = torch.rand(128, 128, 32, 32, generator=g)
+    w = (torch.randn(128, 288, generator=g) / math.sqrt(288)).contiguous()
+    assert cpp.norm_dist_conv_supported(128, 32, 32, 128, 4, 3, 1, 1, 1)
+    imgd, wd = img.to(DEV), w.to(DEV)
+    out = torch.empty(128, 128, 1024, device=DEV)
+    cpp.norm_dist_conv_forward(imgd, wd, out, 4, p, 3, 1, 1, 1)
+    cols_d = torch.empty(128, 1152, 1024, device=DEV)
+    cpp.unfold(imgd, cols_d, 3, 1, 1, 1)
+    from_cols = torch.empty_like(out)
+    cpp.norm_dist_forward(cols_d, wd, from_cols, 4, p)
+    torch.cuda.synchronize()
+    assert torch.equal(out, from_cols)
+    del cols_d, from_cols
+    cols = F.unfold(img[:rows], 3, padding=1).contiguous()
+    ev = oracle.norm_dist_forward(cols, w, 4, p)
+    torch.testing.assert_close(out[:rows].cpu(), ev, rtol=1e-5, atol=1e-6)
+
+    go = torch.zeros(128, 128, 1024)
+    go[:rows] = torch.randn(rows, 128, 1024, generator=g)
+    gimg = torch.full((128, 128, 32, 32), float("nan"), device=DEV)
+    gw = torch.zeros(128, 288, device=DEV)
+    cpp.norm_dist_conv_backward_input(go.to(DEV), imgd, wd, out, gimg, 4, p, 3, 1, 1, 1)
+    cpp.norm_dist_conv_backward_weight(go.to(DEV), imgd, wd, out, gw, 4, p, 3, 1, 1, 1)
+    torch.cuda.synchronize()
+    ex, mx = oracle.norm_dist_backward_input(go[:rows].contiguous(), cols, w, ev, 4, p, with_abs_terms=True)
+    ew, mw = oracle.norm_dist_backward_weight(go[:rows].contiguous(), cols, w, ev, 4, p, with_abs_terms=True)
+    fold = lambda t: F.fold(t.double(), (32, 32), 3, padding=1)
+    assert_sum_close(gimg[:rows].cpu(), fold(ex), fold(mx), p)
+    assert bool((gimg[rows:] == 0).all())
+    assert_sum_close(gw.cpu(), ew, mw, p)
