@@ -240,7 +240,13 @@ def workload_c2(pkg, torch, dev):
     return dict(step=step, ops=3 * stack_ops(512), images=512, full_rows=512, cpu=cpu, formula=formula, check=check,
                 name=f"configs[2]: the same MLP at p={C2_P:g}, forward+backward (3 dist-op passes per layer)",
                 kernel=("norm_dist_backward_input", lambda go, x_, w_, *_: 7 * mnk(x_, w_),
-                        lambda go, x_, w_, *_: w_.size(0) > 16, "norm_backward_kernel (grad_input)", 7))
+                        lambda go, x_, w_, *_: w_.size(0) > 16,
+                        "norm_backward_input_tiled_kernel (grad_input, register-tiled)", 7)
+                if C2_P in (2.0, 3.0, 4.0, 8.0) else
+                       ("norm_dist_backward", lambda go, x_, w_, *_: 2 * 7 * mnk(x_, w_),
+                        lambda go, x_, w_, *_: w_.size(0) > 16,
+                        "norm_backward_fused_kernel (both gradients from one evaluation of every term; the flops are "
+                        "those of the two sums as the reference computes them)", 7))
 
 
 def workload_c3(pkg, torch, dev):

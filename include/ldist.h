@@ -57,7 +57,9 @@ LDIST_API int ldist_last_hip_error(void);
  * tile with two k-groups, 1 = 128x64, 2 = 256x32, 3 = 32x32 with eight k-groups.
  * 0..3 also keep the L_inf forward of an unfolded-conv layout on the tiled kernels
  * where it would otherwise take the kernel that holds a tile's whole reduction axis
- * in LDS (K up to 320).  Process-wide; not thread safe. */
+ * in LDS (K up to 320), and 0 / 1 force the register-tiled p-norm backward kernels
+ * (128x80 / 128x64 tiles), the one-pass kernel of ldist_norm_dist_backward included,
+ * 2 / 3 keep them off.  Process-wide; not thread safe. */
 LDIST_API int ldist_set_tile_override(int choice);
 /* Tuning knob, no counterpart in the reference: 1 (default) orders the tiles of
  * the forward kernels so that each of the 8 XCDs works on one contiguous run of
@@ -133,6 +135,19 @@ LDIST_API int ldist_norm_dist_backward_input(const float* grad_output, const flo
 LDIST_API int ldist_norm_dist_backward_weight(const float* grad_output, const float* input, const float* weight,
                                     const float* output, int B, int CO, int CI, int G, int HW, float* grad_weight,
                                     float p, ldist_stream_t stream);
+
+/* Both p-norm gradients in one call: what ldist_norm_dist_backward_input followed by
+ * ldist_norm_dist_backward_weight computes (the reference's norm_dist_backward_input_cuda and
+ * norm_dist_backward_weight_cuda, model/norm_dist.cpp:9-12, which its autograd function calls one after the other,
+ * model/norm_dist.py:41-46).  No single counterpart in the reference.  Every term
+ *   g[m,n] * (|x-w| / output[m,n])^(p-1) * sign(x-w)
+ * belongs to both sums; for fully connected layers large enough to fill the device one kernel evaluates it once
+ * and adds it to both (grad_weight then collects one addend per tile of 128 rows with float atomics, in no fixed
+ * order); other shapes run the two separate kernels.  grad_input is written whole and may be uninitialised;
+ * grad_weight is added to and must hold zeros (or the values to accumulate onto) on entry. */
+LDIST_API int ldist_norm_dist_backward(const float* grad_output, const float* input, const float* weight,
+                                       const float* output, int B, int CO, int CI, int G, int HW, float* grad_input,
+                                       float* grad_weight, float p, ldist_stream_t stream);
 
 /* The two scatter backward passes again, but writing EVERY element of the
  * gradient (zeros where nothing lands) so the caller can pass uninitialised

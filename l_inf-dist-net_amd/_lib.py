@@ -28,6 +28,7 @@ SIGNATURES = {
     "ldist_norm_dist_forward": [_F, _F, _i, _i, _i, _i, _i, _F, _f, _S],
     "ldist_norm_dist_backward_input": [_F, _F, _F, _F, _i, _i, _i, _i, _i, _F, _f, _S],
     "ldist_norm_dist_backward_weight": [_F, _F, _F, _F, _i, _i, _i, _i, _i, _F, _f, _S],
+    "ldist_norm_dist_backward": [_F, _F, _F, _F, _i, _i, _i, _i, _i, _F, _F, _f, _S],
     "ldist_mean_shift": [_F, _i, _i, _i, _F, _F, _F, _f, _S],
     "ldist_unfold": [_F, _i, _i, _i, _i, _i, _i, _i, _i, _i, _F, _S],
     "ldist_inf_dist_conv_forward_supported": [_i, _i, _i, _i, _i, _i, _i, _i, _i, _i],

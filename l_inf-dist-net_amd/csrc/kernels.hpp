@@ -114,6 +114,12 @@ hipError_t unfold(const float* img, float* cols, const ConvGeom& q, hipStream_t 
 hipError_t fold(const float* gcols, float* gimg, const ConvGeom& q, hipStream_t stream);
 // L_inf forward straight from the image (3x3 window, dilation 1, stride 1 or 2; a group's channels
 // either few enough to stay in LDS or a multiple of four); inf_conv_forward_supported tells whether a geometry is covered.
+// Both p-norm gradients in one pass over the terms (norm_backward_fused.hip; the fc layout).
+bool norm_backward_fused_applicable(const Problem& pr, float p, const void* grad_output, const void* input,
+                                    const void* weight, const void* output, const void* grad_input,
+                                    const void* grad_weight);
+hipError_t norm_backward_fused(const float* grad_output, const float* input, const float* weight, const float* output,
+                               float* grad_input, float* grad_weight, float p, const Problem& pr, hipStream_t stream);
 // p-norm layer of convolution shape straight from the image (norm_conv.hip): 3x3 windows, more than one output
 // position; norm_conv_supported tells whether a geometry is covered.
 bool norm_conv_supported(const ConvGeom& q, int G, int CO);

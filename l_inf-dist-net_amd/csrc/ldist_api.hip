@@ -198,6 +198,22 @@ int ldist_norm_dist_backward_weight(const float* grad_output, const float* input
                                               (hipStream_t)stream));
 }
 
+int ldist_norm_dist_backward(const float* grad_output, const float* input, const float* weight, const float* output,
+                             int B, int CO, int CI, int G, int HW, float* grad_input, float* grad_weight, float p,
+                             ldist_stream_t stream) {
+    if (!grad_output || !input || !weight || !output || !grad_input || !grad_weight || !valid_p(p)) return LDIST_EINVAL;
+    ldist::Problem pr{};
+    if (int rc = check_dims(B, CO, CI, G, HW, pr)) return rc;
+    if (ldist::norm_backward_fused_applicable(pr, p, grad_output, input, weight, output, grad_input, grad_weight))
+        return finish(ldist::norm_backward_fused(grad_output, input, weight, output, grad_input, grad_weight, p, pr,
+                                                 (hipStream_t)stream));
+    if (hipError_t e = ldist::norm_backward_input(grad_output, input, weight, output, grad_input, p, pr, (hipStream_t)stream);
+        e != hipSuccess)
+        return finish(e);
+    return finish(ldist::norm_backward_weight(grad_output, input, weight, output, grad_weight, p, pr,
+                                              (hipStream_t)stream));
+}
+
 int ldist_mean_shift(const float* x, int B, int C, int L, float* y, float* mean_out, float* running_mean,
                      float momentum, ldist_stream_t stream) {
     if (!x || !y || B <= 0 || C <= 0 || L <= 0 || !(momentum >= 0.0f && momentum <= 1.0f)) return LDIST_EINVAL;

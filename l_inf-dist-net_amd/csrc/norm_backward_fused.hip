@@ -1,0 +1,257 @@
+// Both p-norm gradients of a fully connected layer in one pass over the terms, for exponents that need the
+// transcendental unit (reference model/norm_dist_cuda.cu:294-425 computes the gradients in two kernels that each
+// evaluate every term):
+//   t[m,n,k]          = g[m,n] * (|x[m,k] - w[n,k]| / out[m,n])^(p-1) * sign(x - w)
+//   grad_input [m,k]  = sum_n t[m,n,k]          grad_weight[n,k] += -sum_m t[m,n,k]
+// For a general p the term is a logarithm and an exponential (v_log_f32, v_exp_f32: a quarter of the rate of
+// the other instructions), and that is what bounds either gradient; sharing the term between the two sums takes
+// 4.2 ms on 512 x 5120 -> 5120 at p = 20.5 where the two separate kernels take 3.7 + 3.1 ms.  (For p = 2, 3, 4, 8
+// a term is a handful of multiplications, the additions below weigh as much as the term itself, and the two
+// register-tiled kernels of norm_backward_tiled.hip stay faster: 3.35 ms against 4.65 ms.)
+//
+// The kernel has the shape of the register-tiled grad_input kernel: a workgroup owns 128 rows m x BN inputs k and
+// walks the outputs n; a lane keeps an 8 x TN patch of x and of the grad_input sums.  For grad_weight the lane
+// also adds, per output n, its eight rows' terms of each of its TN columns (one more fused multiply-add per term),
+// the sixteen lanes that share those columns (one DPP row: the lane index runs along m first here) add their
+// partial sums with four row shifts, and the row's last lane adds the total of the tile's 128 rows onto
+// grad_weight[n,k] with a float atomic.  grad_weight therefore collects one addend per tile of 128 rows, in no fixed
+// order, and must be zero-filled (or hold the values to accumulate onto) by the caller, as with the separate call.
+// The power is taken of the normalised difference (x - w) / out, which never leaves the float range.
+#include "fwd_engine.hpp"
+#include "pow.hpp"
+
+namespace ldist {
+
+namespace {
+
+// Sum over the 16 lanes of a DPP row; the total arrives in the row's last lane (the others hold prefix sums).
+__device__ __forceinline__ float row_total(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x111, 0xf, 0xf, true));  // row_shr:1
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x112, 0xf, 0xf, true));  // row_shr:2
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x114, 0xf, 0xf, true));  // row_shr:4
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x118, 0xf, 0xf, true));  // row_shr:8
+    return v;
+}
+
+template <int COLS, int LD, int NT, int KK>
+struct WeightRows {   // P[rr][col] = weight[n0 + rr][k0 + col], 128-bit loads along k
+    static constexpr int PER_ROW = COLS / 4;
+    static constexpr int TOTAL = KK * PER_ROW;
+    static constexpr int N = (TOTAL + NT - 1) / NT;
+    float4 v[N];
+    __device__ __forceinline__ void load(const float* __restrict__ base, int stride, int n0, int R, int k0, int K, int tid) {
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const int id = tid + i * NT;
+            const int rr = id / PER_ROW, cq = id % PER_ROW;
+            const int n = n0 + rr, k = k0 + cq * 4;
+            v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if ((TOTAL % NT == 0 || id < TOTAL) && n < R && k < K) v[i] = *reinterpret_cast<const float4*>(base + (size_t)n * stride + k);
+        }
+    }
+    __device__ __forceinline__ void store(float* __restrict__ panel, int tid) const {
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const int id = tid + i * NT;
+            if (TOTAL % NT != 0 && id >= TOTAL) continue;
+            const int rr = id / PER_ROW, cq = id % PER_ROW;
+            *reinterpret_cast<float4*>(panel + rr * LD + ((cq * 4) ^ swz(rr))) = v[i];
+        }
+    }
+};
+
+}  // namespace
+
+template <class GEO>
+__global__ void __launch_bounds__(GEO::NT, 2)
+norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* __restrict__ input,
+                           const float* __restrict__ weight, const float* __restrict__ output,
+                           float* __restrict__ grad_input, float* __restrict__ grad_weight, float e, Dims d) {
+    constexpr int BM = GEO::BM, BN = GEO::BN, TM = GEO::TM, TN = GEO::TN, KS = GEO::KS, KK = GEO::KK;
+    constexpr int NGRP = GEO::NGRP, NT = GEO::NT, XS = GEO::XS, WS = GEO::WS;
+    constexpr int STAGE = 2 * XS + WS;     // [F or g][1/out][w]
+    static_assert(GEO::TY == 16, "the lanes that share a column fill one DPP row");
+    using RowLoad = RowsK<BM, GEO::SM, NT, KK, 4>;   // outputs are contiguous in g and out
+    using ColLoad = WeightRows<BN, GEO::SN, NT, KK>;
+    static_assert((KS - 1) * TM * TN * NGRP <= STAGE, "merge area fits in the panels");
+    extern __shared__ __align__(16) float lds[];
+
+    int tm, tk, g;
+    tile_of_block(d, tm, tk, g);
+    const int m0 = tm * BM, k0 = tk * BN;
+    const int tid = threadIdx.x;
+    const int grp = tid / NGRP, t = tid % NGRP;
+    const int ty = t % GEO::TY, tx = t / GEO::TY;    // m first: the 16 lanes of a column group are neighbours
+    const int K = d.K, NG = d.NG;
+
+    // sign(u) * |u|^(p-1); u == 0 gives 0 either way
+    auto spower = [e](float u) { return __builtin_copysignf(pow_pos(__builtin_fabsf(u), e), u); };
+
+    // the lane's patch of x, and where its columns' sums go in grad_weight (row n = 0 of group g)
+    float q[TM][TN], acc[TM][TN];
+    int wcol[TN];
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int k = k0 + GEO::col(tx, j);
+        wcol[j] = k < K ? k : -1;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+        const int m = m0 + GEO::row(ty, i);
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            acc[i][j] = 0.f;
+            q[i][j] = (m < d.M && wcol[j] >= 0) ? input[((size_t)m * d.G + g) * K + wcol[j]] : 0.f;
+        }
+    }
+    float* const gw_group = grad_weight + (size_t)g * NG * K;
+    // Adds the lane's column sums of output n (already summed over its rows) over the 16 lanes of the row and
+    // onto grad_weight; the sign: d/dw of |x - w| is minus d/dx.
+    auto add_weight_row = [&](int n, const float (&s)[TN]) {
+        float tot[TN];
+#pragma unroll
+        for (int j = 0; j < TN; j++) tot[j] = row_total(s[j]);
+        if (ty == GEO::TY - 1 && n < NG) {
+            float* row = gw_group + (size_t)n * K;
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                if (wcol[j] >= 0) atomicAdd(row + wcol[j], -tot[j]);
+        }
+    };
+
+    // ---- staging: g and out (rows m, reduction n) and the weights of the stage's outputs ----
+    RowLoad gk, ok_;
+    ColLoad wl;
+    const float* gbase = grad_output + ((size_t)m0 * d.G + g) * NG;
+    const float* obase = output + ((size_t)m0 * d.G + g) * NG;
+    const float* wbase = weight + (size_t)g * NG * K;
+    auto load = [&](int n_first) {
+        wl.load(wbase, K, n_first, NG, k0, K, tid);
+        gk.load(gbase, d.G * NG, d.M - m0, n_first, NG, tid);
+        ok_.load(obase, d.G * NG, d.M - m0, n_first, NG, tid);
+    };
+    // Turns the parked out values into what the panel holds: 1/out, and 0 where nothing was loaded (padding loads g
+    // and out as 0; a real 0 output gives inf like the reference), so that padding multiplies by 0, not by infinity.
+    auto convert = [&]() {
+#pragma unroll
+        for (int i = 0; i < RowLoad::N; i++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const bool present = ok_.v[i][c] != 0.f || gk.v[i][c] != 0.f;
+                ok_.v[i][c] = present ? __builtin_amdgcn_rcpf(ok_.v[i][c]) : 0.f;
+            }
+    };
+    auto store = [&]() {
+        gk.store(lds, tid);
+        ok_.store(lds + XS, tid);
+        wl.store(lds + 2 * XS, tid);
+    };
+
+    const int nstage = (NG + KK - 1) / KK;
+    load(0);
+    convert();
+    store();
+    __syncthreads();
+    for (int s = 0; s < nstage; s++) {
+        if (s + 1 < nstage) load((s + 1) * KK);
+        const float* fp = lds + grp * kChunk * GEO::SM;
+        const float* wp = lds + 2 * XS + grp * kChunk * GEO::SN;
+        const int n_chunk = s * KK + grp * kChunk;
+        // No operand prefetch: a second fragment in flight does not fit next to the patch, the sums and the weight
+        // row's partial sums (it spills, and measured 15 % slower); the LDS latency of a row hides behind the forty
+        // logarithms and exponentials of the other wave on the SIMD.
+        sweep_chunk_plain<GEO, 2>(fp, wp, tx, ty, [&](const Frag<GEO, 2, 1>& f, int kk) {
+            float sum[TN];
+#pragma unroll
+            for (int j = 0; j < TN; j++) sum[j] = 0.f;
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    const float sp = spower((q[i][j] - f.w[0][j]) * f.x[1][0][i]);
+                    acc[i][j] = __builtin_fmaf(f.x[0][0][i], sp, acc[i][j]);   // two fused multiply-adds, not a
+                    sum[j] = __builtin_fmaf(f.x[0][0][i], sp, sum[j]);         // shared product and two additions
+                }
+            add_weight_row(n_chunk + kk, sum);
+        });
+        __syncthreads();   // everyone is done reading the panels
+        if (s + 1 < nstage) {
+            convert();
+            store();
+        }
+        __syncthreads();
+    }
+
+    // ---- the k-groups add their grad_input sums through LDS, the first one writes the tile ----
+    float* part = lds;
+#pragma unroll 1
+    for (int turn = KS - 1; turn >= 1; turn--) {
+        if (grp == turn) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) part[(i * TN + j) * NGRP + t] = acc[i][j];
+        }
+        __syncthreads();
+        if (grp == 0) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) acc[i][j] += part[(i * TN + j) * NGRP + t];
+        }
+        __syncthreads();
+    }
+    if (grp == 0) {
+        Dims od = d;
+        od.NG = K;   // the result has the input's shape: K columns per group
+        store_patch<GEO, false>(grad_input, acc, od, m0, k0, g, tx, ty, d.ovec != 0);
+    }
+}
+
+template <class GEO>
+static hipError_t launch_fused(const Problem& pr, hipStream_t stream, const float* grad_output, const float* input,
+                               const float* weight, const float* output, float* grad_input, float* grad_weight, float p) {
+    Dims d = make_dims(pr);
+    d.ovec = 1;   // the result has the input's shape: K % 4 == 0, aligned
+    d.tiles_m = (d.M + GEO::BM - 1) / GEO::BM;
+    d.tiles_n = (d.K + GEO::BN - 1) / GEO::BN;
+    const unsigned grid = (unsigned)d.tiles_m * d.tiles_n * d.G;
+    constexpr size_t lds = (size_t)(2 * GEO::XS + GEO::WS) * sizeof(float);
+    auto kern = norm_backward_fused_kernel<GEO>;
+    static LdsRecord lds_allowed = {};
+    if (hipError_t e = allow_lds(kern, lds, pr.device, lds_allowed); e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(GEO::NT), lds, stream, grad_output, input, weight, output, grad_input,
+                       grad_weight, p - 1.0f, d);
+    return hipGetLastError();
+}
+
+// Whether the one-pass kernel takes the problem: an exponent that is not multiply-only, the fc layout, every panel
+// loadable with 128-bit loads, and a shape that fills the device with 128-row tiles (the rest stays with the two
+// separate kernels).
+bool norm_backward_fused_applicable(const Problem& pr, float p, const void* grad_output, const void* input,
+                                    const void* weight, const void* output, const void* grad_input,
+                                    const void* grad_weight) {
+    const int ie = small_int_power(p - 1.0f);
+    if (ie == 1 || ie == 2 || ie == 3 || ie == 7) return false;
+    if (pr.HW != 1 || pr.K % 4 != 0 || pr.NG % 4 != 0) return false;
+    if (!(aligned16(grad_output) && aligned16(input) && aligned16(weight) && aligned16(output) && aligned16(grad_input) &&
+          aligned16(grad_weight)))
+        return false;
+    if (g_tile_override == 0 || g_tile_override == 1) return true;   // tests and tuning: forced on (128 x 80, 128 x 64)
+    if (g_tile_override >= 2) return false;                          // forced off
+    const long M = (long)pr.B * pr.HW;
+    const long t80 = ((M + 127) / 128) * ((pr.K + 79) / 80) * pr.G, t64 = ((M + 127) / 128) * ((pr.K + 63) / 64) * pr.G;
+    return (t80 > t64 ? t80 : t64) * 10 >= 7L * pr.num_cu && pr.NG >= 256;
+}
+
+hipError_t norm_backward_fused(const float* grad_output, const float* input, const float* weight, const float* output,
+                               float* grad_input, float* grad_weight, float p, const Problem& pr, hipStream_t stream) {
+    const long rows = (long)pr.B * pr.HW;
+    const long t80 = ((rows + 127) / 128) * ((pr.K + 79) / 80) * pr.G, t64 = ((rows + 127) / 128) * ((pr.K + 63) / 64) * pr.G;
+    const double c80 = (double)((t80 + pr.num_cu - 1) / pr.num_cu) * 80, c64 = (double)((t64 + pr.num_cu - 1) / pr.num_cu) * 64 * 1.1;
+    const bool wide = g_tile_override == 0 || (g_tile_override != 1 && c80 <= c64);
+    return wide ? launch_fused<Geo<128, 80, 8, 5, 2>>(pr, stream, grad_output, input, weight, output, grad_input, grad_weight, p)
+                : launch_fused<Geo<128, 64, 8, 4, 2>>(pr, stream, grad_output, input, weight, output, grad_input, grad_weight, p);
+}
+
+}  // namespace ldist

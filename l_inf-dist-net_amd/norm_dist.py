@@ -22,6 +22,8 @@ import torch.nn.functional as F
 from . import norm_dist_cpp
 
 _INF = float("inf")
+# exponents whose powers are a few multiplications: the two separate gradient kernels are the faster way there
+_MULTIPLY_ONLY_P = (2.0, 3.0, 4.0, 8.0)
 
 
 def _out_shape(x, weight):
@@ -67,10 +69,14 @@ class DistF(torch.autograd.Function):
                 norm_dist_cpp.inf_dist_backward_weight_overwrite(g, argmax, gw, ctx.group)
         else:
             x, weight, y = ctx.saved_tensors
-            if want_x:
+            if want_x and want_w and ctx.p not in _MULTIPLY_ONLY_P:
+                # every term belongs to both sums: one call, which evaluates it once where one kernel can serve both
+                gx, gw = torch.empty_like(x), torch.zeros_like(weight)
+                norm_dist_cpp.norm_dist_backward(g, x, weight, y, gx, gw, ctx.group, ctx.p)
+            elif want_x:
                 gx = torch.empty_like(x)
                 norm_dist_cpp.norm_dist_backward_input(g, x, weight, y, gx, ctx.group, ctx.p)
-            if want_w:
+            elif want_w:
                 gw = torch.zeros_like(weight)  # this kernel adds onto the buffer
                 norm_dist_cpp.norm_dist_backward_weight(g, x, weight, y, gw, ctx.group, ctx.p)
         return gx, gw, None, None, None

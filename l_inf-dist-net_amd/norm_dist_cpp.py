@@ -92,6 +92,23 @@ def norm_dist_backward_weight(grad_output, input, weight, output, grad_weight, G
           HW, _p(grad_weight), float(p))
 
 
+def norm_dist_backward(grad_output, input, weight, output, grad_input, grad_weight, G, p):
+    """Both gradients in one call (the reference's two backward calls, model/norm_dist.cpp:30-52, with every term
+    evaluated once where one kernel can serve both).  grad_input is written whole; grad_weight is accumulated onto."""
+    for t, n in ((grad_output, "grad_output"), (input, "input"), (weight, "weight"), (output, "output"),
+                 (grad_input, "grad_input"), (grad_weight, "grad_weight")):
+        _check_input(t, n)
+    dev = _same_device(grad_output, input, weight, output, grad_input, grad_weight)
+    B, CO, CI, HW = grad_output.size(0), output.size(1), input.size(1), input.size(2)
+    _expect(weight.size(0) == CO and weight.size(1) * G == CI, "weight must be (CO, CI/G)")
+    _expect(tuple(output.shape) == (B, CO, HW) and tuple(grad_output.shape) == (B, CO, HW),
+            "output and grad_output must be (B, CO, HW)")
+    _expect(tuple(grad_input.shape) == tuple(input.shape), "grad_input must match input")
+    _expect(tuple(grad_weight.shape) == tuple(weight.shape) and input.size(0) == B, "grad_weight must match weight")
+    _call("ldist_norm_dist_backward", dev, _p(grad_output), _p(input), _p(weight), _p(output), B, CO, CI, G, HW,
+          _p(grad_input), _p(grad_weight), float(p))
+
+
 def inf_dist_forward(input, weight, output, pos, G):
     """model/norm_dist.cpp:54-62."""
     for t, n in ((input, "input"), (weight, "weight"), (output, "output")):

@@ -1235,3 +1235,62 @@ def test_norm_dist_conv_layer_runs_from_the_image_without_columns(p):
     # ratio 1, then cancel to nothing, which leaves only rounding noise to compare.)
     for a, b in ((gx1, gx0), (gw1, gw0)):
         assert float((a - b).abs().max()) <= 1e-3 * float(b.abs().max())
+
+
+FUSED_BACKWARD_SHAPES = [sh for sh in TILED_BACKWARD_SHAPES if sh[4] == 1] + [(515, 140, 100, 1, 1), (70, 200, 132, 1, 1)]
+
+
+@pytest.mark.parametrize("tile", [0, 1])
+@pytest.mark.parametrize("p", [5.0, 5.5, 9.0, 20.0, 100.0, 8.0])
+@pytest.mark.parametrize("shape", FUSED_BACKWARD_SHAPES)
+def test_norm_backward_both_gradients_in_one_pass(shape, p, tile):
+    """norm_dist_backward against the oracle.  For exponents that need the transcendental unit it runs the kernel
+    that evaluates every term once for both gradients (forced with the tile override; by itself it only takes
+    large layers); p = 8 is multiply-only and runs the two separate kernels through the same call.  grad_weight is
+    added onto the buffer (0.125 here) like the separate call's.  Override 2 switches the one-pass kernel off."""
+    from gpu_common import DEV, cpp, say, set_tile
+    B, CO, CI, G, HW = shape
+    say("norm_backward fused", shape, "p", p, "tile", tile)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=36 + sum(shape))
+    go = torch.randn(B, CO, HW, generator=gen(37))
+    out = oracle.norm_dist_forward(x, w, G, p)
+    ex, mx = oracle.norm_dist_backward_input(go, x, w, out, G, p, with_abs_terms=True)
+    ew, mw = oracle.norm_dist_backward_weight(go, x, w, out, G, p, with_abs_terms=True)
+    args = (go.to(DEV), x.to(DEV), w.to(DEV), out.to(DEV))
+    for choice in (tile, 2):
+        set_tile(choice)
+        gx = torch.full((B, CI, HW), float("nan"), device=DEV)
+        gw = torch.full((CO, CI // G), 0.125, device=DEV)
+        cpp.norm_dist_backward(*args, gx, gw, G, p)
+        torch.cuda.synchronize()
+        assert_sum_close(gx.cpu(), ex, mx, p, RTOL, ATOL)
+        assert_sum_close(gw.cpu() - 0.125, ew, mw, p, RTOL, ATOL)
+
+
+@pytest.mark.parametrize("p", [2.5, 20.0, 300.0])
+@pytest.mark.parametrize("scale", [1e-6, 3e-4, 1.0, 5e3, 1e6, "mixed", "one tiny row"])
+def test_norm_backward_both_gradients_at_every_scale(scale, p):
+    """The one-pass kernel on inputs of every magnitude: the power is taken of the normalised difference, so
+    nothing may overflow or vanish with the scale of the data."""
+    from gpu_common import DEV, cpp, say, set_tile
+    B, CO, CI, G, HW = 200, 72, 132, 1, 1
+    say("norm_backward fused scale", scale, "p", p)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=44)
+    if scale == "mixed":
+        x = x * torch.tensor([1e-5, 1.0, 1e4, 3e-3, 1.0])[torch.arange(B) % 5].view(B, 1, 1)
+    elif scale == "one tiny row":
+        x[7] *= 1e-7
+    else:
+        x, w = x * scale, w * scale
+    x, w = x.contiguous(), w.contiguous()
+    go = torch.randn(B, CO, HW, generator=gen(38))
+    out = oracle.norm_dist_forward(x, w, G, p)
+    ex, mx = oracle.norm_dist_backward_input(go, x, w, out, G, p, with_abs_terms=True)
+    ew, mw = oracle.norm_dist_backward_weight(go, x, w, out, G, p, with_abs_terms=True)
+    set_tile(0)
+    gx = torch.full((B, CI, HW), float("nan"), device=DEV)
+    gw = torch.zeros((CO, CI // G), device=DEV)
+    cpp.norm_dist_backward(go.to(DEV), x.to(DEV), w.to(DEV), out.to(DEV), gx, gw, G, p)
+    torch.cuda.synchronize()
+    assert_sum_close(gx.cpu(), ex, mx, p, RTOL, ATOL)
+    assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
