@@ -141,9 +141,10 @@ LDIST_API int ldist_norm_dist_backward_weight(const float* grad_output, const fl
  * norm_dist_backward_weight_cuda, model/norm_dist.cpp:9-12, which its autograd function calls one after the other,
  * model/norm_dist.py:41-46).  No single counterpart in the reference.  Every term
  *   g[m,n] * (|x-w| / output[m,n])^(p-1) * sign(x-w)
- * belongs to both sums; for fully connected layers large enough to fill the device one kernel evaluates it once
- * and adds it to both (grad_weight then collects one addend per tile of 128 rows with float atomics, in no fixed
- * order); other shapes run the two separate kernels.  grad_input is written whole and may be uninitialised;
+ * belongs to both sums.  One kernel evaluates it once and adds it to both for fully connected layers large enough to
+ * fill the device when p needs the transcendental unit (p - 1 not 1, 2, 3 or 7; grad_weight then collects one addend
+ * per tile of 128 rows with float atomics, in no fixed order), and for the unfolded-conv layout (HW > 1) with up to
+ * about 140 outputs per group (one addend per workgroup); other shapes run the two separate kernels.  grad_input is written whole and may be uninitialised;
  * grad_weight is added to and must hold zeros (or the values to accumulate onto) on entry. */
 LDIST_API int ldist_norm_dist_backward(const float* grad_output, const float* input, const float* weight,
                                        const float* output, int B, int CO, int CI, int G, int HW, float* grad_input,
@@ -251,6 +252,15 @@ LDIST_API int ldist_norm_dist_conv_backward_weight(const float* grad_output, con
                                                    const float* output, int B, int C, int H, int W, int CO, int G, int KH,
                                                    int KW, int stride, int padding, int dilation, float* grad_weight,
                                                    float p, ldist_stream_t stream);
+/* Both gradients of the layer above in one call: what ldist_norm_dist_conv_backward_input followed by
+ * ldist_norm_dist_conv_backward_weight computes, with the same contracts for grad_img (written whole) and
+ * grad_weight (added to).  Where a group's outputs are few enough for its weights to stay in LDS (up to about 140
+ * outputs per group) one kernel evaluates every term once and adds it to both sums, and every pixel of grad_img is
+ * written by one workgroup (no atomics: grad_img does not depend on scheduling); other layers run the two kernels. */
+LDIST_API int ldist_norm_dist_conv_backward(const float* grad_output, const float* img, const float* weight,
+                                            const float* output, int B, int C, int H, int W, int CO, int G, int KH, int KW,
+                                            int stride, int padding, int dilation, float* grad_img, float* grad_weight,
+                                            float p, ldist_stream_t stream);
 /* Testing and tuning knob, no counterpart in the reference: output rows per workgroup of
  * ldist_inf_dist_conv_forward; 0 (default) = chosen by shape.  A positive value is clamped to what the
  * geometry allows and also switches off the rule that leaves small or channel-heavy layers, which

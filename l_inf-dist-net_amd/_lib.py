@@ -39,6 +39,7 @@ SIGNATURES = {
     "ldist_norm_dist_conv_forward": [_F, _F, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _F, _f, _S],
     "ldist_norm_dist_conv_backward_input": [_F, _F, _F, _F, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _F, _f, _S],
     "ldist_norm_dist_conv_backward_weight": [_F, _F, _F, _F, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _F, _f, _S],
+    "ldist_norm_dist_conv_backward": [_F, _F, _F, _F, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _F, _F, _f, _S],
     "ldist_fold": [_F, _i, _i, _i, _i, _i, _i, _i, _i, _i, _F, _S],
     "ldist_inf_dist_backward_input_folded": [_F, _I, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _F, _S],
     "ldist_adamw_lp_step": [_F, _F, _F, _F, _i, _i, _d, _d, _d, _d, _d, _d, _i, _S],

@@ -120,6 +120,16 @@ bool norm_backward_fused_applicable(const Problem& pr, float p, const void* grad
                                     const void* grad_weight);
 hipError_t norm_backward_fused(const float* grad_output, const float* input, const float* weight, const float* output,
                                float* grad_input, float* grad_weight, float p, const Problem& pr, hipStream_t stream);
+// Both p-norm gradients of a convolution-shaped layer in one pass (norm_conv_backward.hip), from the unfolded
+// input or from the image.
+bool norm_conv_backward_fused_applicable(const Problem& pr);
+bool norm_conv_backward_fused_image_applicable(const ConvGeom& q, int G, int CO, int num_cu);
+hipError_t norm_conv_backward_fused_columns(const float* grad_output, const float* input, const float* weight,
+                                            const float* output, float* grad_input, float* grad_weight, float p,
+                                            const Problem& pr, hipStream_t stream);
+hipError_t norm_conv_backward_fused_image(const float* grad_output, const float* img, const float* weight,
+                                          const float* output, float* grad_img, float* grad_weight, float p,
+                                          const ConvGeom& q, int G, int CO, int num_cu, int device, hipStream_t stream);
 // p-norm layer of convolution shape straight from the image (norm_conv.hip): 3x3 windows, more than one output
 // position; norm_conv_supported tells whether a geometry is covered.
 bool norm_conv_supported(const ConvGeom& q, int G, int CO);

@@ -207,6 +207,9 @@ int ldist_norm_dist_backward(const float* grad_output, const float* input, const
     if (ldist::norm_backward_fused_applicable(pr, p, grad_output, input, weight, output, grad_input, grad_weight))
         return finish(ldist::norm_backward_fused(grad_output, input, weight, output, grad_input, grad_weight, p, pr,
                                                  (hipStream_t)stream));
+    if (ldist::norm_conv_backward_fused_applicable(pr))
+        return finish(ldist::norm_conv_backward_fused_columns(grad_output, input, weight, output, grad_input, grad_weight,
+                                                              p, pr, (hipStream_t)stream));
     if (hipError_t e = ldist::norm_backward_input(grad_output, input, weight, output, grad_input, p, pr, (hipStream_t)stream);
         e != hipSuccess)
         return finish(e);
@@ -347,6 +350,24 @@ int ldist_norm_dist_conv_backward_weight(const float* grad_output, const float* 
     ldist::Problem pr{};
     if (!grad_output || !img || !weight || !output || !grad_weight) return LDIST_EINVAL;
     if (int rc = norm_conv_prepare(B, C, H, W, CO, G, KH, KW, stride, padding, dilation, p, q, pr)) return rc;
+    return finish(ldist::norm_conv_backward_weight(grad_output, img, weight, output, grad_weight, p, q, G, CO, pr.num_cu,
+                                                   pr.device, (hipStream_t)stream));
+}
+
+int ldist_norm_dist_conv_backward(const float* grad_output, const float* img, const float* weight, const float* output,
+                                  int B, int C, int H, int W, int CO, int G, int KH, int KW, int stride, int padding,
+                                  int dilation, float* grad_img, float* grad_weight, float p, ldist_stream_t stream) {
+    ldist::ConvGeom q{};
+    ldist::Problem pr{};
+    if (!grad_output || !img || !weight || !output || !grad_img || !grad_weight) return LDIST_EINVAL;
+    if (int rc = norm_conv_prepare(B, C, H, W, CO, G, KH, KW, stride, padding, dilation, p, q, pr)) return rc;
+    if (ldist::norm_conv_backward_fused_image_applicable(q, G, CO, pr.num_cu))
+        return finish(ldist::norm_conv_backward_fused_image(grad_output, img, weight, output, grad_img, grad_weight, p, q,
+                                                            G, CO, pr.num_cu, pr.device, (hipStream_t)stream));
+    if (hipError_t e = ldist::norm_conv_backward_input(grad_output, img, weight, output, grad_img, p, q, G, CO, pr.num_cu,
+                                                       pr.device, (hipStream_t)stream);
+        e != hipSuccess)
+        return finish(e);
     return finish(ldist::norm_conv_backward_weight(grad_output, img, weight, output, grad_weight, p, q, G, CO, pr.num_cu,
                                                    pr.device, (hipStream_t)stream));
 }

@@ -1,0 +1,368 @@
+// Both p-norm gradients of a convolution-shaped layer in one pass over the terms (reference
+// model/norm_dist_cuda.cu:294-425 computes them in two kernels that each evaluate every term, on the unfolded
+// input of model/norm_dist.py:132):
+//   t[m,n,k]          = g[m,n] * (|x[m,k] - w[n,k]| / out[m,n])^(p-1) * sign(x - w)
+//   grad_input [m,k]  = sum_n t[m,n,k]          grad_weight[n,k] += -sum_m t[m,n,k]
+// with m = (image, output position), n the outputs of one group, k = (channel, tap) of the group's window.
+//
+// A layer of this shape has few outputs per group and very many rows, so a workgroup keeps the weights of its
+// columns k for ALL outputs of the group in LDS, next to a tile of grad_weight sums of the same shape, and walks
+// tiles of 64 rows.  Per tile it stages g and 1/out (NG x 64 each), and every lane reduces a 4 x 4 patch of
+// (row, column) over n: a term is evaluated once, added to the lane's grad_input sum and to the column's partial sum
+// over the lane's four rows; the sixteen lanes that share the columns (one DPP row) add those with four row shifts
+// and the row's last lane, the only one that ever touches these four words, adds the total onto the LDS tile of
+// grad_weight.  After its last tile the workgroup adds the LDS tile onto grad_weight with float atomics (one
+// addend per workgroup and element).
+//
+// grad_input.  From the unfolded tensor (IMG = false) a tile is 64 columns wide and every element is written once.
+// From the image (IMG = true, 3x3 windows) a pixel collects up to nine columns.  Float atomics for that, in memory
+// or in LDS, cost as much as the arithmetic (151 M of them for 128 images of 128 x 32 x 32: 1.2 -> 2.0 ms), so the
+// work is cut such that every pixel has one owner: a tile is 63 columns wide, i.e. seven whole channels, a
+// workgroup takes whole images, and it keeps the image rows of its seven channel planes that its windows are
+// still adding to in LDS (a ring of rows: a tile of 64 positions covers a few output rows, and everything above
+// the next tile's first window is final).  A tile's sums go there in nine rounds, one per tap, with a barrier
+// between them: inside a round the (position, channel) pairs, and therefore the pixels, are all different, so
+// plain read-add-write is safe.  Final rows are written to memory with plain stores and their ring rows cleared:
+// grad_img needs no zero fill, and the result does not depend on the order in which workgroups run.
+//
+// IE = p - 1 for the multiply-only exponents (1, 2, 3, 7): the power is taken of the raw difference and the
+// coefficient g / out^(p-1) is staged instead of g, unless a tile holds an output outside [2^-12, 2^12], which then
+// takes the normalised difference like IE = 0 (any p > 1, through v_log_f32 / v_exp_f32).
+#include "conv_window.hpp"
+#include "kernels.hpp"
+#include "pow.hpp"
+
+#include <algorithm>
+
+namespace ldist {
+
+namespace {
+
+constexpr int TR = 64;              // rows of a tile
+constexpr int TCP = 64;             // columns a tile has lanes for
+constexpr int WLD = TCP + 4;        // row length of the weight and grad_weight tiles (rows 16-byte aligned)
+constexpr int kPlanes = 7;          // IMG: channels per tile (63 columns)
+constexpr size_t kMaxLds = 159 * 1024;   // all of LDS less the kernel's own static words
+
+__device__ __forceinline__ float row_total16(float v) {   // sum over a DPP row; the total arrives in its last lane
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x111, 0xf, 0xf, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x112, 0xf, 0xf, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x114, 0xf, 0xf, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x118, 0xf, 0xf, true));
+    return v;
+}
+
+struct ConvBwd {
+    int B, G, K, NG, HW, M;          // the unfolded problem: K = 9 channels per group (image) or CI / G
+    int tiles_k;                     // column tiles per group
+    int units, units_per_wg;         // what a workgroup walks: tiles of 64 rows (columns), whole images (image)
+    int ring_rows;                   // IMG: image rows per channel plane held in LDS, a power of two
+};
+
+inline size_t lds_bytes(int NG, size_t plane_floats) {
+    return ((size_t)2 * NG * WLD + (size_t)2 * NG * TR + plane_floats) * sizeof(float);
+}
+
+}  // namespace
+
+template <bool IMG, int IE>
+__global__ void __launch_bounds__(256)
+norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __restrict__ input,
+                          const float* __restrict__ weight, const float* __restrict__ output,
+                          float* __restrict__ grad_input, float* __restrict__ grad_weight, float e, ConvBwd d,
+                          ImgWin win) {
+    constexpr int TC = IMG ? 9 * kPlanes : TCP;   // columns per tile
+    extern __shared__ __align__(16) float lds[];
+    const int NG = d.NG, K = d.K;
+    float* Ws = lds;                     // [NG][WLD]  w[n][k0 + c]
+    float* Gw = Ws + NG * WLD;           // [NG][WLD]  sums for grad_weight[n][k0 + c]
+    float* Cs = Gw + NG * WLD;           // [NG][TR]   g, or g / out^IE
+    float* Rs = Cs + NG * TR;            // [NG][TR]   1 / out
+    float* Fp = Rs + NG * TR;            // IMG: [kPlanes][ring_rows][W] gradient of the image rows still being added to
+    const int tid = threadIdx.x;
+    const int ty = tid & 15, tx = tid >> 4;   // rows first: the 16 lanes of a column group form a DPP row
+    const int tk = blockIdx.x % d.tiles_k, g = blockIdx.x / d.tiles_k;
+    const int k0 = tk * TC;
+    const int u_begin = blockIdx.y * d.units_per_wg, u_end = min(d.units, u_begin + d.units_per_wg);
+
+    auto spower = [&](float u) {   // sign(u) * |u|^(p-1); by reference: the integer-exponent instantiations do not use e
+        if constexpr (IE == 0) return __builtin_copysignf(pow_pos(__builtin_fabsf(u), e), u);   // u == 0: 0 either way
+        else if constexpr (IE == 1) return u;
+        else if constexpr (IE == 2) return u * __builtin_fabsf(u);
+        else return pow_int<IE>(u);
+    };
+
+    for (int i = tid; i < NG * TCP; i += 256) {
+        const int n = i / TCP, c = i % TCP;
+        Ws[n * WLD + c] = (c < TC && k0 + c < K) ? weight[((size_t)g * NG + n) * K + k0 + c] : 0.f;
+        Gw[n * WLD + c] = 0.f;
+    }
+    // the lane's four columns: whether they exist, and for the image their channel plane and tap
+    bool col_ok[4];
+    int col_plane[4], col_tap[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int c = tx * 4 + j;
+        col_ok[j] = c < TC && k0 + c < K;
+        col_plane[j] = c / 9;
+        col_tap[j] = c - col_plane[j] * 9;
+    }
+
+    // One tile: rows first_row .. first_row + 63 of the unfolded matrix, of which `rows` exist (IMG: rows of image b
+    // from position pos0).  Leaves the grad_input sums of the lane's patch in acc.
+    auto tile = [&](int first_row, int rows, int b, int pos0, float (&acc)[4][4], WinRow (&wrow)[4], size_t (&xoff)[4]) {
+        float q[4][4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int r = min(ty * 4 + i, rows - 1);
+            if constexpr (IMG) {
+                const int pos = pos0 + r, ho = pos / win.WO;
+                wrow[i].b = b;
+                wrow[i].h0 = ho * win.S - win.P;
+                wrow[i].w0 = (pos - ho * win.WO) * win.S - win.P;
+            } else {
+                const int m = first_row + r, bi = m / d.HW;
+                xoff[i] = ((size_t)(bi * d.G + g) * K) * d.HW + (m - bi * d.HW);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int k = k0 + tx * 4 + j;
+                acc[i][j] = 0.f;
+                bool ok = ty * 4 + i < rows && col_ok[j];
+                size_t off;
+                if constexpr (IMG) ok = win_tap(win, wrow[i], g, ok ? k : 0, off) && ok;
+                else off = xoff[i] + (size_t)k * d.HW;
+                q[i][j] = ok ? input[off] : 0.f;
+            }
+        // g and out of the tile's rows for every output of the group; rows are contiguous in memory
+        bool unsafe = IE == 0;
+        for (int i = tid; i < NG * TR; i += 256) {
+            const int n = i / TR, r = i % TR;
+            float c = 0.f, ri = 0.f;
+            if (r < rows) {
+                size_t o;
+                if constexpr (IMG) {
+                    o = ((size_t)(b * d.G + g) * NG + n) * d.HW + pos0 + r;
+                } else {
+                    const int m = first_row + r, bi = m / d.HW;
+                    o = ((size_t)(bi * d.G + g) * NG + n) * d.HW + (m - bi * d.HW);
+                }
+                c = grad_output[o];
+                const float out = output[o];
+                ri = __builtin_amdgcn_rcpf(out);
+                unsafe |= !(out >= 0x1p-12f && out <= 0x1p12f);   // the factored form needs out^(p-1) inside the float range
+            }
+            Cs[i] = c;
+            Rs[i] = ri;
+        }
+        const bool factored = !__syncthreads_or(unsafe);   // also: the panels are written
+        if (IE > 0 && factored) {
+            for (int i = tid; i < NG * TR; i += 256) Cs[i] *= pow_int<(IE > 0 ? IE : 1)>(Rs[i]);   // each lane its own elements
+            __syncthreads();
+        }
+        auto reduce = [&](auto term) {   // term(x - w, 1/out): the power that g (or g / out^IE) multiplies
+            for (int n = 0; n < NG; n++) {
+                const float4 c4 = *reinterpret_cast<const float4*>(Cs + n * TR + ty * 4);
+                const float4 r4 = *reinterpret_cast<const float4*>(Rs + n * TR + ty * 4);
+                const float4 w4 = *reinterpret_cast<const float4*>(Ws + n * WLD + tx * 4);
+                const float cv[4] = {c4.x, c4.y, c4.z, c4.w}, rv[4] = {r4.x, r4.y, r4.z, r4.w}, wv[4] = {w4.x, w4.y, w4.z, w4.w};
+                float s[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const float sp = term(q[i][j] - wv[j], rv[i]);
+                        acc[i][j] = __builtin_fmaf(cv[i], sp, acc[i][j]);   // two fused multiply-adds, not a shared
+                        s[j] = __builtin_fmaf(cv[i], sp, s[j]);             // product and two additions
+                    }
+                float tot[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) tot[j] = row_total16(s[j]);
+                if (ty == 15) {   // d/dw of |x - w| is minus d/dx
+                    float4* gp = reinterpret_cast<float4*>(Gw + n * WLD + tx * 4);
+                    float4 v = *gp;
+                    v.x -= tot[0]; v.y -= tot[1]; v.z -= tot[2]; v.w -= tot[3];
+                    *gp = v;
+                }
+            }
+        };
+        if (IE > 0 && factored) reduce([&](float df, float) { return spower(df); });
+        else reduce([&](float df, float ri) { return spower(df * ri); });
+    };
+
+    float acc[4][4];
+    WinRow wrow[4];
+    size_t xoff[4];
+    if constexpr (IMG) {
+        const int H = win.H, W = win.W, R = d.ring_rows, first_ch = tk * kPlanes;
+        const int planes = min(kPlanes, win.CG - first_ch);
+        for (int b = u_begin; b < u_end; b++) {
+            float* dst = grad_input + ((size_t)b * win.C + g * win.CG + first_ch) * H * W;
+            // Writes image rows h_from .. h_to - 1 of the planes to memory and clears their ring rows.  Rows more than
+            // a ring away from h_from have never been touched (the windows reach less far): they are zero.
+            auto flush_rows = [&](int h_from, int h_to) {
+                const int nrow = h_to - h_from;
+                for (int i = tid; i < planes * nrow * W; i += 256) {
+                    const int w = i % W, rest = i / W, hr = rest % nrow, c = rest / nrow, h = h_from + hr;
+                    float v = 0.f;
+                    if (hr < R) {
+                        float* cell = Fp + (c * R + (h & (R - 1))) * W + w;
+                        v = *cell;
+                        *cell = 0.f;
+                    }
+                    dst[(c * H + h) * W + w] = v;
+                }
+            };
+            for (int i = tid; i < kPlanes * R * W; i += 256) Fp[i] = 0.f;   // the first tile's barriers come before its use
+            int flushed = 0;   // image rows below this one are in memory
+            for (int pos0 = 0; pos0 < d.HW; pos0 += TR) {
+                const int rows = min(TR, d.HW - pos0);
+                tile(0, rows, b, pos0, acc, wrow, xoff);
+                // rows above this tile's first window are final (the last tile's rounds ended with a barrier)
+                const int h_lo = min(H, max(flushed, (pos0 / win.WO) * win.S - win.P));
+                if (h_lo > flushed) flush_rows(flushed, h_lo);
+                flushed = h_lo;
+                __syncthreads();   // ring rows cleared above may be this tile's; every lane is done with the panels
+                // the tile's sums join the planes: nine rounds, one per tap (see the top of the file)
+                for (int tap = 0; tap < 9; tap++) {
+                    const int di = tap / 3, dj = tap - di * 3;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        if (col_tap[j] != tap || !col_ok[j]) continue;
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            const int h = wrow[i].h0 + di * win.D, w = wrow[i].w0 + dj * win.D;
+                            if (ty * 4 + i < rows && (unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W)
+                                Fp[(col_plane[j] * R + (h & (R - 1))) * W + w] += acc[i][j];
+                        }
+                    }
+                    __syncthreads();
+                }
+            }
+            flush_rows(flushed, H);
+            __syncthreads();       // before the ring is used for the next image
+        }
+    } else {
+        for (int t = u_begin; t < u_end; t++) {
+            const int m0 = t * TR, rows = min(TR, d.M - m0);
+            tile(m0, rows, 0, 0, acc, wrow, xoff);
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (ty * 4 + i < rows && col_ok[j]) grad_input[xoff[i] + (size_t)(k0 + tx * 4 + j) * d.HW] = acc[i][j];
+            __syncthreads();   // the next tile overwrites the panels
+        }
+    }
+    __syncthreads();
+    for (int i = tid; i < NG * TCP; i += 256) {
+        const int n = i / TCP, c = i % TCP;
+        if (c < TC && k0 + c < K) atomicAdd(grad_weight + ((size_t)g * NG + n) * K + k0 + c, Gw[n * WLD + c]);
+    }
+}
+
+namespace {
+
+// Image rows per plane the ring must hold: the most that the windows of one tile of 64 positions cover (tiles start
+// at multiples of 64 inside an image), rounded up to a power of two.
+int ring_rows_for(const ImgWin& win, int HW) {
+    int out_rows = 1;
+    for (int pos0 = 0; pos0 < HW; pos0 += TR) {
+        const int last = std::min(HW, pos0 + TR) - 1;
+        out_rows = std::max(out_rows, last / win.WO - pos0 / win.WO + 1);
+        if (pos0 / TR >= win.WO) break;   // the pattern of starts inside an output row repeats by then
+    }
+    const int rows = (out_rows - 1) * win.S + 2 * win.D + 1;
+    int ring = 1;
+    while (ring < rows) ring *= 2;
+    return ring;
+}
+
+template <bool IMG, int IE>
+hipError_t launch_conv_backward(const float* grad_output, const float* input, const float* weight, const float* output,
+                                float* grad_input, float* grad_weight, float p, const Problem& pr, const ImgWin& win,
+                                hipStream_t stream) {
+    ConvBwd d{pr.B, pr.G, pr.K, pr.NG, pr.HW, pr.B * pr.HW, 0, 0, 0, 0};
+    d.tiles_k = IMG ? (win.CG + kPlanes - 1) / kPlanes : (d.K + TCP - 1) / TCP;
+    d.units = IMG ? pr.B : (d.M + TR - 1) / TR;
+    const long pairs = (long)d.tiles_k * d.G;
+    if constexpr (IMG) d.ring_rows = ring_rows_for(win, pr.HW);
+    const size_t lds = lds_bytes(d.NG, IMG ? (size_t)kPlanes * d.ring_rows * win.W : 0);
+    // Units per workgroup: the choice that needs the fewest rounds of resident workgroups times units (the device
+    // holds `resident` of them at once), among those that keep the number of workgroups, each of which flushes a whole
+    // grad_weight tile at the end, within sixteen rounds; ties go to fewer, longer workgroups.
+    long per_cu = (long)(160 * 1024 / lds);
+    if (per_cu > 8) per_cu = 8;
+    if (per_cu < 1) per_cu = 1;
+    const long resident = per_cu * pr.num_cu;
+    long best = -1, best_cost = 0;
+    const long lo = std::max(1L, ((long)d.units * pairs + 16 * resident - 1) / (16 * resident));
+    for (long upw = lo; upw <= d.units && upw < lo + 4096; upw++) {
+        const long wgs = pairs * ((d.units + upw - 1) / upw);
+        const long cost = ((wgs + resident - 1) / resident) * upw;
+        if (best < 0 || cost <= best_cost) { best = upw; best_cost = cost; }
+    }
+    d.units_per_wg = (int)best;
+    const long slices = (d.units + d.units_per_wg - 1) / d.units_per_wg;
+    auto kern = norm_conv_backward_kernel<IMG, IE>;
+    static LdsRecord lds_allowed = {};
+    // the limit is raised once, to the most any layer may ask for
+    if (hipError_t e = allow_lds(kern, kMaxLds, pr.device, lds_allowed); e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, dim3((unsigned)pairs, (unsigned)slices), dim3(256), lds, stream, grad_output, input, weight,
+                       output, grad_input, grad_weight, p - 1.0f, d, win);
+    return hipGetLastError();
+}
+
+template <bool IMG>
+hipError_t dispatch_conv_backward(const float* grad_output, const float* input, const float* weight, const float* output,
+                                  float* grad_input, float* grad_weight, float p, const Problem& pr, const ImgWin& win,
+                                  hipStream_t stream) {
+    switch (small_int_power(p - 1.0f)) {
+        case 1: return launch_conv_backward<IMG, 1>(grad_output, input, weight, output, grad_input, grad_weight, p, pr, win, stream);
+        case 2: return launch_conv_backward<IMG, 2>(grad_output, input, weight, output, grad_input, grad_weight, p, pr, win, stream);
+        case 3: return launch_conv_backward<IMG, 3>(grad_output, input, weight, output, grad_input, grad_weight, p, pr, win, stream);
+        case 7: return launch_conv_backward<IMG, 7>(grad_output, input, weight, output, grad_input, grad_weight, p, pr, win, stream);
+        default: return launch_conv_backward<IMG, 0>(grad_output, input, weight, output, grad_input, grad_weight, p, pr, win, stream);
+    }
+}
+
+bool forced_on() { return g_tile_override == 0 || g_tile_override == 1; }   // tests and tuning
+
+}  // namespace
+
+// Whether the one-pass kernel takes a layer given as unfolded columns: the conv layout with enough rows to give
+// every CU work, and few enough outputs per group for the four LDS tiles (NG KB).
+bool norm_conv_backward_fused_applicable(const Problem& pr) {
+    if (pr.HW == 1 || g_tile_override >= 2) return false;
+    if (lds_bytes(pr.NG, 0) > kMaxLds) return false;
+    return forced_on() || (long)pr.B * pr.HW >= 64L * pr.num_cu;
+}
+
+// The same for a layer given as an image: also the ring of image rows of seven channel planes must fit LDS.
+bool norm_conv_backward_fused_image_applicable(const ConvGeom& q, int G, int CO, int num_cu) {
+    if (g_tile_override >= 2 || (long)q.HO * q.WO <= 1) return false;
+    const ImgWin win{q.C, q.C / G, q.H, q.W, q.HO, q.WO, q.S, q.P, q.D};
+    if (lds_bytes(CO / G, (size_t)kPlanes * ring_rows_for(win, q.HO * q.WO) * q.W) > kMaxLds) return false;
+    return forced_on() || (long)q.B * q.HO * q.WO >= 64L * num_cu;
+}
+
+// From the unfolded input (B, CI, HW): every element of grad_input is written, grad_weight is added to.
+hipError_t norm_conv_backward_fused_columns(const float* grad_output, const float* input, const float* weight,
+                                            const float* output, float* grad_input, float* grad_weight, float p,
+                                            const Problem& pr, hipStream_t stream) {
+    return dispatch_conv_backward<false>(grad_output, input, weight, output, grad_input, grad_weight, p, pr, ImgWin{}, stream);
+}
+
+// From the image (3x3 window): every element of grad_img is written, grad_weight is added to.
+hipError_t norm_conv_backward_fused_image(const float* grad_output, const float* img, const float* weight,
+                                          const float* output, float* grad_img, float* grad_weight, float p,
+                                          const ConvGeom& q, int G, int CO, int num_cu, int device, hipStream_t stream) {
+    const Problem pr{q.B, G, q.C / G * 9, CO / G, q.HO * q.WO, num_cu, device};
+    const ImgWin win{q.C, q.C / G, q.H, q.W, q.HO, q.WO, q.S, q.P, q.D};
+    return dispatch_conv_backward<true>(grad_output, img, weight, output, grad_img, grad_weight, p, pr, win, stream);
+}
+
+}  // namespace ldist

@@ -22,7 +22,8 @@ import torch.nn.functional as F
 from . import norm_dist_cpp
 
 _INF = float("inf")
-# exponents whose powers are a few multiplications: the two separate gradient kernels are the faster way there
+# exponents whose powers are a few multiplications: in the fc layout the two separate gradient kernels are the
+# faster way there
 _MULTIPLY_ONLY_P = (2.0, 3.0, 4.0, 8.0)
 
 
@@ -69,16 +70,17 @@ class DistF(torch.autograd.Function):
                 norm_dist_cpp.inf_dist_backward_weight_overwrite(g, argmax, gw, ctx.group)
         else:
             x, weight, y = ctx.saved_tensors
-            if want_x and want_w and ctx.p not in _MULTIPLY_ONLY_P:
+            if want_x and want_w and (ctx.p not in _MULTIPLY_ONLY_P or x.size(2) > 1):
                 # every term belongs to both sums: one call, which evaluates it once where one kernel can serve both
                 gx, gw = torch.empty_like(x), torch.zeros_like(weight)
                 norm_dist_cpp.norm_dist_backward(g, x, weight, y, gx, gw, ctx.group, ctx.p)
-            elif want_x:
-                gx = torch.empty_like(x)
-                norm_dist_cpp.norm_dist_backward_input(g, x, weight, y, gx, ctx.group, ctx.p)
-            elif want_w:
-                gw = torch.zeros_like(weight)  # this kernel adds onto the buffer
-                norm_dist_cpp.norm_dist_backward_weight(g, x, weight, y, gw, ctx.group, ctx.p)
+            else:
+                if want_x:
+                    gx = torch.empty_like(x)
+                    norm_dist_cpp.norm_dist_backward_input(g, x, weight, y, gx, ctx.group, ctx.p)
+                if want_w:
+                    gw = torch.zeros_like(weight)  # this kernel adds onto the buffer
+                    norm_dist_cpp.norm_dist_backward_weight(g, x, weight, y, gw, ctx.group, ctx.p)
         return gx, gw, None, None, None
 
 
@@ -164,10 +166,13 @@ class _ConvNormDist(torch.autograd.Function):
         img, weight, y = ctx.saved_tensors
         g = grad_output.contiguous()
         grad_img = grad_w = None
-        if ctx.needs_input_grad[0]:
+        if ctx.needs_input_grad[0] and ctx.needs_input_grad[1]:   # every term belongs to both sums: one call
+            grad_img, grad_w = torch.empty_like(img), torch.zeros_like(weight)
+            norm_dist_cpp.norm_dist_conv_backward(g, img, weight, y, grad_img, grad_w, ctx.group, ctx.p, *ctx.window)
+        elif ctx.needs_input_grad[0]:
             grad_img = torch.empty_like(img)   # the call writes every element
             norm_dist_cpp.norm_dist_conv_backward_input(g, img, weight, y, grad_img, ctx.group, ctx.p, *ctx.window)
-        if ctx.needs_input_grad[1]:
+        elif ctx.needs_input_grad[1]:
             grad_w = torch.zeros_like(weight)  # this kernel adds onto the buffer
             norm_dist_cpp.norm_dist_conv_backward_weight(g, img, weight, y, grad_w, ctx.group, ctx.p, *ctx.window)
         return grad_img, grad_w, None, None, None, None, None, None

@@ -380,6 +380,21 @@ def norm_dist_conv_backward_weight(grad_output, img, weight, output, grad_weight
           _p(grad_weight), float(p))
 
 
+def norm_dist_conv_backward(grad_output, img, weight, output, grad_img, grad_weight, G, p, kernel_size, stride=1,
+                            padding=0, dilation=1):
+    """Both gradients of the p-norm conv-shaped layer from the image in one call (every term evaluated once where
+    one kernel can serve both).  grad_img is written whole, grad_weight is added to."""
+    for t, n in ((grad_output, "grad_output"), (img, "img"), (weight, "weight"), (output, "output"),
+                 (grad_img, "grad_img"), (grad_weight, "grad_weight")):
+        _check_input(t, n)
+    dev = _same_device(grad_output, img, weight, output, grad_img, grad_weight)
+    args = _norm_conv_args(img, weight, output, G, kernel_size, stride, padding, dilation)
+    _expect(grad_output.shape == output.shape and grad_img.shape == img.shape and grad_weight.shape == weight.shape,
+            "grad_output must match output, grad_img the image and grad_weight the weight")
+    _call("ldist_norm_dist_conv_backward", dev, _p(grad_output), _p(img), _p(weight), _p(output), *args, _p(grad_img),
+          _p(grad_weight), float(p))
+
+
 def inf_dist_bound_conv_forward_supported(C, H, W, CO, G, kernel_size, stride=1, padding=0, dilation=1):
     """True when inf_dist_bound_conv_forward covers the geometry (3x3, dilation 1, stride 1 or 2, a layer large
     enough to fill the GPU); otherwise unfold both images and call inf_dist_bound_forward."""

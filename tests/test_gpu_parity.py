@@ -4,6 +4,8 @@ Bars: L_inf forward values and indices and the interval bounds are bit-exact
 (torch.equal); scatter gradients and everything p-norm are within rel 1e-5 /
 abs 1e-6 of the oracle's double-precision result.
 """
+import math
+
 import pytest
 import torch
 
@@ -832,7 +834,7 @@ def test_inf_conv_forward_refuses_what_it_does_not_cover():
 
 @pytest.mark.parametrize("p", [float("inf"), 8.0])
 def test_conv_layer_image_path_matches_column_path(p):
-    """NormDistConv on the GPU (native unfold; for p = inf the fused image-space backward) against the same
+    """NormDistConv on the GPU (the kernels that work on the image, for p = inf and for finite p) against the same
     layer evaluated through F.unfold + norm_dist with autograd folding the gradient."""
     import torch.nn.functional as F
     from gpu_common import DEV, pkg
@@ -850,8 +852,10 @@ def test_conv_layer_image_path_matches_column_path(p):
     yb = layer._shift(yb)
     yb.backward(up)
     torch.cuda.synchronize()
-    torch.testing.assert_close(ya, yb, rtol=1e-6, atol=1e-6)
-    torch.testing.assert_close(ga, xb.grad, rtol=RTOL, atol=ATOL)
+    # p = 8: the layer runs the kernels that read the image, the comparison the column kernels (six outputs per
+    # group: not even the same forward kernel); the outputs are of order 5 before the mean shift, to rel 1e-5 each
+    torch.testing.assert_close(ya, yb, rtol=1e-5, atol=1e-6 if math.isinf(p) else 1e-4)
+    torch.testing.assert_close(ga, xb.grad, rtol=RTOL if math.isinf(p) else 1e-4, atol=ATOL if math.isinf(p) else 1e-5)
     # each weight gradient sums 400 terms of order one, in an order the LDS atomics do not fix
     torch.testing.assert_close(gwa, layer.weight.grad, rtol=1e-4, atol=5e-5)
 
@@ -1284,6 +1288,84 @@ def test_norm_backward_both_gradients_at_every_scale(scale, p):
         x, w = x * scale, w * scale
     x, w = x.contiguous(), w.contiguous()
     go = torch.randn(B, CO, HW, generator=gen(38))
+    out = oracle.norm_dist_forward(x, w, G, p)
+    ex, mx = oracle.norm_dist_backward_input(go, x, w, out, G, p, with_abs_terms=True)
+    ew, mw = oracle.norm_dist_backward_weight(go, x, w, out, G, p, with_abs_terms=True)
+    set_tile(0)
+    gx = torch.full((B, CI, HW), float("nan"), device=DEV)
+    gw = torch.zeros((CO, CI // G), device=DEV)
+    cpp.norm_dist_backward(go.to(DEV), x.to(DEV), w.to(DEV), out.to(DEV), gx, gw, G, p)
+    torch.cuda.synchronize()
+    assert_sum_close(gx.cpu(), ex, mx, p, RTOL, ATOL)
+    assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
+
+
+@pytest.mark.parametrize("p", [8.0, 3.0, 5.5, 100.0])
+@pytest.mark.parametrize("case", NORM_IMAGE_CASES)
+def test_norm_conv_backward_both_gradients_in_one_pass_from_the_image(case, p):
+    """norm_dist_conv_backward on the kernel that evaluates every term once for both gradients (forced with the
+    tile override; by itself it takes layers with enough rows), against the oracle on the unfolded columns, folded
+    back in float64 for grad_img.  grad_img starts as NaN (the call writes every element), grad_weight at 0.125."""
+    import torch.nn.functional as F
+    from gpu_common import DEV, cpp, say, set_tile
+    B, C, H, W, CO, G, s_, p_, d_ = case
+    say("norm_conv_backward fused", case, "p", p)
+    img, w, cols, go = _norm_image_problem(case, 93)
+    out = oracle.norm_dist_forward(cols, w, G, p)
+    ex, mx = oracle.norm_dist_backward_input(go, cols, w, out, G, p, with_abs_terms=True)
+    ew, mw = oracle.norm_dist_backward_weight(go, cols, w, out, G, p, with_abs_terms=True)
+    fold = lambda t: F.fold(t.double(), (H, W), 3, d_, p_, s_)
+    args = (go.to(DEV), img.to(DEV), w.to(DEV), out.to(DEV))
+    for choice in (0, 2):   # one pass; the two separate kernels through the same call
+        set_tile(choice)
+        gi = torch.full((B, C, H, W), float("nan"), device=DEV)
+        gw = torch.full((CO, C // G * 9), 0.125, device=DEV)
+        cpp.norm_dist_conv_backward(*args, gi, gw, G, p, 3, s_, p_, d_)
+        torch.cuda.synchronize()
+        assert_sum_close(gi.cpu(), fold(ex), fold(mx), p, RTOL, ATOL)
+        assert_sum_close(gw.cpu() - 0.125, ew, mw, p, RTOL, ATOL)
+
+
+CONV_COLUMN_SHAPES = [sh for sh in TILED_BACKWARD_SHAPES if sh[4] > 1] + [(2, 20, 27, 1, 1024), (3, 24, 30, 2, 49)]
+
+
+@pytest.mark.parametrize("p", [8.0, 2.0, 4.0, 5.5, 100.0])
+@pytest.mark.parametrize("shape", CONV_COLUMN_SHAPES)
+def test_norm_backward_both_gradients_in_one_pass_conv_columns(shape, p):
+    """norm_dist_backward in the unfolded-conv layout on the one-pass kernel (forced with the tile override) against
+    the oracle: every element of grad_input written, grad_weight added onto the buffer."""
+    from gpu_common import DEV, cpp, say, set_tile
+    B, CO, CI, G, HW = shape
+    say("norm_backward fused conv columns", shape, "p", p)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=46 + sum(shape))
+    go = torch.randn(B, CO, HW, generator=gen(47))
+    out = oracle.norm_dist_forward(x, w, G, p)
+    ex, mx = oracle.norm_dist_backward_input(go, x, w, out, G, p, with_abs_terms=True)
+    ew, mw = oracle.norm_dist_backward_weight(go, x, w, out, G, p, with_abs_terms=True)
+    set_tile(0)
+    gx = torch.full((B, CI, HW), float("nan"), device=DEV)
+    gw = torch.full((CO, CI // G), 0.125, device=DEV)
+    cpp.norm_dist_backward(go.to(DEV), x.to(DEV), w.to(DEV), out.to(DEV), gx, gw, G, p)
+    torch.cuda.synchronize()
+    assert_sum_close(gx.cpu(), ex, mx, p, RTOL, ATOL)
+    assert_sum_close(gw.cpu() - 0.125, ew, mw, p, RTOL, ATOL)
+
+
+@pytest.mark.parametrize("p", [3.0, 8.0, 20.0])
+@pytest.mark.parametrize("scale", [1e-6, 1.0, 1e6, "mixed"])
+def test_norm_backward_both_gradients_conv_at_every_scale(scale, p):
+    """The one-pass conv kernel where the factored form leaves the float range and a tile takes the normalised
+    difference instead (images of very different magnitudes side by side)."""
+    from gpu_common import DEV, cpp, say, set_tile
+    B, CO, CI, G, HW = 5, 40, 36, 1, 100
+    say("norm_backward fused conv scale", scale, "p", p)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=48)
+    if scale == "mixed":
+        x = x * torch.tensor([1e-5, 1.0, 1e4, 3e-3, 1.0]).view(B, 1, 1)
+    else:
+        x, w = x * scale, w * scale
+    x, w = x.contiguous(), w.contiguous()
+    go = torch.randn(B, CO, HW, generator=gen(49))
     out = oracle.norm_dist_forward(x, w, G, p)
     ex, mx = oracle.norm_dist_backward_input(go, x, w, out, G, p, with_abs_terms=True)
     ew, mw = oracle.norm_dist_backward_weight(go, x, w, out, G, p, with_abs_terms=True)
