@@ -53,6 +53,13 @@ def fake_native(monkeypatch):
         assert torch.count_nonzero(gw) == 0  # the wrapper must hand over a zero-filled buffer
         oracle.norm_dist_backward_weight(go, x.contiguous(), w.contiguous(), out.contiguous(), G, p, grad_weight=gw)
 
+    def norm_bwd_both(go, x, w, out, gi, gw, G, p):   # the one call that serves both gradients
+        calls.append("norm_dist_backward (input and weight)")
+        assert torch.count_nonzero(gw) == 0  # the wrapper must hand over a zero-filled buffer
+        gi.copy_(oracle.norm_dist_backward_input(go, x.contiguous(), w.contiguous(), out.contiguous(), G, p))
+        oracle.norm_dist_backward_weight(go, x.contiguous(), w.contiguous(), out.contiguous(), G, p, grad_weight=gw)
+
+    monkeypatch.setattr(cpp, "norm_dist_backward", norm_bwd_both)
     for name, fn in [("inf_dist_forward", inf_dist_forward), ("inf_dist_bound_forward", inf_dist_bound_forward),
                      ("inf_dist_backward_input_overwrite", bwd_in_over),
                      ("inf_dist_backward_weight_overwrite", bwd_w_over), ("norm_dist_forward", norm_dist_forward),
@@ -97,6 +104,19 @@ def test_distf_backward_respects_needs_input_grad(fake_native, p):
         kinds = [c for c in fake_native if "backward" in c]
         assert any("input" in c for c in kinds) == rx and any("weight" in c for c in kinds) == rw
         assert (xx.grad is not None) == rx and (ww.grad is not None) == rw
+        if rx and rw and not math.isinf(p):
+            # both wanted: the conv layout (HW = 2 here) and every exponent that needs the transcendental unit take
+            # the one call; a fully connected layer at p = 8 takes the two separate ones
+            assert kinds == ["norm_dist_backward (input and weight)"]
+            fake_native.clear()
+            x1, w1 = x[:, :, :1].clone().requires_grad_(True), w.clone().requires_grad_(True)
+            pkg.norm_dist(x1, w1, 2, p).backward(go[:, :, :1].contiguous())
+            assert sorted(c for c in fake_native if "backward" in c) == ["norm_dist_backward_input", "norm_dist_backward_weight"]
+            assert x1.grad is not None and w1.grad is not None
+            fake_native.clear()
+            x2, w2 = x[:, :, :1].clone().requires_grad_(True), w.clone().requires_grad_(True)
+            pkg.norm_dist(x2, w2, 2, 5.5).backward(go[:, :, :1].contiguous())
+            assert [c for c in fake_native if "backward" in c] == ["norm_dist_backward (input and weight)"]
 
 
 def test_gradients_agree_with_the_dense_torch_formula(fake_native):
