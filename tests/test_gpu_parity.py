@@ -1376,3 +1376,27 @@ def test_norm_backward_both_gradients_conv_at_every_scale(scale, p):
     torch.cuda.synchronize()
     assert_sum_close(gx.cpu(), ex, mx, p, RTOL, ATOL)
     assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
+
+
+def test_fc_and_1x1_layers_accept_non_contiguous_inputs():
+    """A fully connected layer and a 1x1 conv layer take a strided view as input (the reference's F.unfold always
+    hands its kernels a contiguous tensor, so its layers accept such views): same output and input gradient as
+    for the contiguous copy."""
+    from gpu_common import DEV, pkg, say
+    say("non-contiguous layer inputs")
+    torch.manual_seed(11)
+    fc = pkg.NormDist(24, 40, p=float("inf"), bias=True).to(DEV)
+    conv = pkg.NormDistConv(6, 20, 1, p=8.0, bias=False).to(DEV)
+    base_fc = torch.randn(24, 10, device=DEV)                 # (features, batch): the layer sees its transpose
+    base_cv = torch.randn(5, 7, 7, 6, device=DEV)             # channels last: the layer sees a permuted view
+    for layer, view in ((fc, base_fc.t()), (conv, base_cv.permute(0, 3, 1, 2))):
+        assert not view.is_contiguous()
+        a = view.detach().requires_grad_(True)
+        b = view.detach().contiguous().requires_grad_(True)
+        ya, yb = layer(a)[0], layer(b)[0]
+        up = torch.randn_like(yb)
+        ya.backward(up)
+        yb.backward(up)
+        torch.cuda.synchronize()
+        assert torch.equal(ya, yb)
+        assert torch.equal(a.grad, b.grad)
