@@ -495,8 +495,10 @@ def workload_c4p(pkg, torch, dev):
                           ("ms_per_step_with_torch_unfold_and_fold", step_torch_unfold)],
                 name=f"configs[4]'s layer at p={p:g} from the image: 3x3 p-norm dist conv layer, batch 128, 128->128 "
                      "channels, 32x32, groups 4, forward+backward (3 dist-op passes), no unfolded tensor",
-                kernel=("norm_dist_conv_backward_input", lambda go_, img_, w_, o_, *_: 7 * o_.numel() * w_.size(1),
-                        lambda *a: True, "norm_backward_kernel (grad_input added onto the image)", 7))
+                kernel=("norm_dist_conv_backward", lambda go_, img_, w_, o_, *_: 2 * 7 * o_.numel() * w_.size(1),
+                        lambda *a: True,
+                        "norm_conv_backward_kernel (both gradients from one evaluation of every term, straight from the "
+                        "image; the flops are those of the two sums as the reference computes them)", 7))
 
 
 WORKLOADS = {"c0": workload_c0, "c1": workload_c1, "c1t": workload_c1t, "c2": workload_c2, "c3": workload_c3,
@@ -692,19 +694,22 @@ def main():
 
 
 # workload -> (counter summary under profiles/, the roofline kernel's name in it)
-TRAFFIC_PROFILES = {"c1": ("counters_c1_mlp_inf.md", "inf_forward_kernel"), "c1t": ("counters_c1_mlp_inf.md", "inf_forward_kernel"),
-                    "c0": ("counters_c0_fc_layer.md", "inf_forward_kernel"),
-                    "c2": ("counters_c2_mlp_p8.md", "norm_backward_kernel"),
-                    "c3": ("counters_c3_certification.md", "bound_forward_kernel"),
-                    "c4": ("counters_c4_conv_columns.md", "inf_forward_shortk_kernel"),
-                    "c4i": ("counters_c4_conv_from_image.md", "inf_conv_forward_kernel")}
+def traffic_profiles():
+    c2_fused = C2_P not in (2.0, 3.0, 4.0, 8.0)
+    return {"c1": ("counters_c1_mlp_inf.md", "inf_forward_kernel"), "c1t": ("counters_c1t_training_step.md", "inf_forward_kernel"),
+            "c0": ("counters_c0_fc_layer.md", "inf_forward_kernel"),
+            "c2": (f"counters_c2_mlp_p{C2_P:g}.md", "norm_backward_fused_kernel" if c2_fused else "norm_backward_input_tiled_kernel"),
+            "c3": ("counters_c3_certification.md", "bound_forward_kernel"),
+            "c4": ("counters_c4_conv_columns.md", "inf_forward_shortk_kernel"),
+            "c4i": ("counters_c4_conv_from_image.md", "inf_conv_forward_kernel"),
+            "c4p": (f"counters_c4p_conv_p{C4_P:g}_from_image.md", "norm_conv_backward_kernel")}
 
 
 def profile_traffic(workload):
     """(bytes per launch, source file) from the line 'traffic_bytes_per_launch[<kernel>]: <number>' of the
     workload's counter summary under profiles/, or (None, None)."""
     import re
-    name, kernel = TRAFFIC_PROFILES.get(workload, (None, None))
+    name, kernel = traffic_profiles().get(workload, (None, None))
     path = os.path.join(ROOT, "profiles", name) if name else None
     if not path or not os.path.exists(path):
         return None, None
