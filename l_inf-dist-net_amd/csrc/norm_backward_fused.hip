@@ -147,6 +147,10 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
         wl.store(lds + 2 * XS, tid);
     };
 
+    // every (row, output) pair has its own largest term among its K differences, and a row of the test holds
+    // 16 pairs x 4 TN columns per wave: with a short K most rows hold one and the tests only cost
+    const bool sparse = e >= 63.0f && K >= 1024;
+    const float cut = __builtin_exp2f(-36.0f / e);
     const int nstage = (NG + KK - 1) / KK;
     load(0);
     convert();
@@ -160,20 +164,55 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
         // No operand prefetch: a second fragment in flight does not fit next to the patch, the sums and the weight
         // row's partial sums (it spills, and measured 15 % slower); the LDS latency of a row hides behind the forty
         // logarithms and exponentials of the other wave on the SIMD.
-        sweep_chunk_plain<GEO, 2>(fp, wp, tx, ty, [&](const Frag<GEO, 2, 1>& f, int kk) {
-            float sum[TN];
+        if (sparse) {
+            // Large exponents: |u|^(p-1) <= 2^-36 for |u| <= cut, less than the rounding of one term of unit size, and
+            // nearly every normalised difference is that small, while the logarithm and the exponential are most of
+            // a term's cost.  One row of the lane's patch at a time (TN terms that share g and 1/out): when no lane
+            // of the wave has |x - w| / out above the cut, the wave passes over the row for both sums; a step whose
+            // rows are all passed over adds nothing to grad_weight either.  All tests of a step come before the
+            // first branch, so the branches wait for scalar registers only.
+            sweep_chunk_plain<GEO, 2>(fp, wp, tx, ty, [&](const Frag<GEO, 2, 1>& f, int kk) {
+                unsigned long long hot[TM], any = 0;
 #pragma unroll
-            for (int j = 0; j < TN; j++) sum[j] = 0.f;
+                for (int i = 0; i < TM; i++) {
+                    float top = 0.f;
 #pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++) {
-                    const float sp = spower((q[i][j] - f.w[0][j]) * f.x[1][0][i]);
-                    acc[i][j] = __builtin_fmaf(f.x[0][0][i], sp, acc[i][j]);   // two fused multiply-adds, not a
-                    sum[j] = __builtin_fmaf(f.x[0][0][i], sp, sum[j]);         // shared product and two additions
+                    for (int j = 0; j < TN; j++) top = __builtin_fmaxf(top, __builtin_fabsf(q[i][j] - f.w[0][j]));
+                    hot[i] = __builtin_amdgcn_ballot_w64(top * f.x[1][0][i] > cut);
+                    any |= hot[i];
                 }
-            add_weight_row(n_chunk + kk, sum);
-        });
+                if (any == 0) return;
+                float sum[TN];
+#pragma unroll
+                for (int j = 0; j < TN; j++) sum[j] = 0.f;
+#pragma unroll
+                for (int i = 0; i < TM; i++) {
+                    if (hot[i] == 0) continue;
+#pragma unroll
+                    for (int j = 0; j < TN; j++) {
+                        const float sp = spower((q[i][j] - f.w[0][j]) * f.x[1][0][i]);
+                        acc[i][j] = __builtin_fmaf(f.x[0][0][i], sp, acc[i][j]);
+                        sum[j] = __builtin_fmaf(f.x[0][0][i], sp, sum[j]);
+                    }
+                }
+                add_weight_row(n_chunk + kk, sum);
+            });
+        } else {
+            sweep_chunk_plain<GEO, 2>(fp, wp, tx, ty, [&](const Frag<GEO, 2, 1>& f, int kk) {
+                float sum[TN];
+#pragma unroll
+                for (int j = 0; j < TN; j++) sum[j] = 0.f;
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) {
+                        const float sp = spower((q[i][j] - f.w[0][j]) * f.x[1][0][i]);
+                        acc[i][j] = __builtin_fmaf(f.x[0][0][i], sp, acc[i][j]);   // two fused multiply-adds, not a
+                        sum[j] = __builtin_fmaf(f.x[0][0][i], sp, sum[j]);         // shared product and two additions
+                    }
+                add_weight_row(n_chunk + kk, sum);
+            });
+        }
         __syncthreads();   // everyone is done reading the panels
         if (s + 1 < nstage) {
             convert();

@@ -554,6 +554,17 @@ def test_norm_large_exponents(data, p):
     torch.cuda.synchronize()
     assert_sum_close(gx.cpu(), ex, mx, p, RTOL, ATOL)
     assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
+    # the call for both gradients, on the kernels that evaluate every term once (forced on), which pass over the
+    # same negligible rows for both sums
+    from gpu_common import set_tile
+    set_tile(0)
+    gx2 = torch.full((B, CI, HW), float("nan"), device=DEV)
+    gw2 = torch.zeros((CO, CI // G), device=DEV)
+    cpp.norm_dist_backward(*args, gx2, gw2, G, p)
+    torch.cuda.synchronize()
+    set_tile(-1)
+    assert_sum_close(gx2.cpu(), ex, mx, p, RTOL, ATOL)
+    assert_sum_close(gw2.cpu(), ew, mw, p, RTOL, ATOL)
 
 
 @pytest.mark.parametrize("shape", [(512, 5120, 1), (37, 10, 1), (1030, 50, 1), (600, 36, 1), (6, 5, 12), (4, 3, 7),
