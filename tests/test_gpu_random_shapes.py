@@ -2,7 +2,7 @@
 
 The hand-picked shapes of test_gpu_parity.py cover the cases the kernels were written for; this file draws sizes
 nobody picked -- prime row counts, reductions shorter than a vector, one output per group, ragged conv layouts --
-with a random forward tile, a random exponent and, for the conv layer, a random image geometry.  Same bars as
+with a random forward tile, a random exponent and, for the conv layer (p = inf and finite p), a random image geometry.  Same bars as
 everywhere: L_inf values, indices and bounds bit-exact, everything else rel 1e-5 / abs 1e-6.
 """
 import random
@@ -84,6 +84,14 @@ def test_random_problem(seed):
     torch.cuda.synchronize()
     assert_sum_close(gx.cpu(), ex, mx, p, RTOL, ATOL)
     assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
+    # the call for both gradients: with the drawn tile override it runs the kernels that evaluate every term once
+    # (0, 1: forced on where the layout and the alignment allow them), the two separate ones (2, 3) or its own choice
+    gx = torch.full((B, CI, HW), float("nan"), device=DEV)
+    gw = torch.zeros((CO, CI // G), device=DEV)
+    cpp.norm_dist_backward(*args, gx, gw, G, p)
+    torch.cuda.synchronize()
+    assert_sum_close(gx.cpu(), ex, mx, p, RTOL, ATOL)
+    assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
 
 
 def draw_image(seed):
@@ -142,6 +150,54 @@ def test_random_conv_layer_from_the_image(seed):
     cpp.inf_dist_backward_input_folded(go.to(DEV), ep.to(DEV), gimg, G, 3, stride, padding, 1)
     torch.cuda.synchronize()
     assert_sum_close(gimg.cpu(), expect, terms, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("seed", range(96))
+def test_random_conv_layer_at_finite_p_from_the_image(seed):
+    """The p-norm layer from the image on a random geometry, exponent and dilation: forward and both gradients
+    (separate entry points; the one call with the one-pass kernel forced on, off, or left to the library) against
+    the oracle on the unfolded tensor."""
+    import torch.nn.functional as F
+    from gpu_common import DEV, cpp, say, set_tile
+    B, C, H, W, CO, G, stride, padding = draw_image(seed)
+    r = random.Random(9000 + seed)
+    dilation = r.choice([1, 1, 1, 2])
+    if H + 2 * padding < 2 * dilation + 1 or W + 2 * padding < 2 * dilation + 1:
+        dilation = 1
+    p = r.choice(EXPONENTS)
+    mode = r.choice([-1, 0, 2])
+    say("random conv layer, finite p", seed, (B, C, H, W, CO, G, stride, padding, dilation), "p", p, "mode", mode)
+    img = torch.rand(B, C, H, W, generator=gen(6000 + seed))
+    w = (torch.randn(CO, C // G * 9, generator=gen(6500 + seed)) * 0.5).contiguous()
+    cols = F.unfold(img, 3, dilation, padding, stride).contiguous()
+    if cols.size(2) <= 1:
+        assert not cpp.norm_dist_conv_supported(C, H, W, CO, G, 3, stride, padding, dilation)
+        return
+    assert cpp.norm_dist_conv_supported(C, H, W, CO, G, 3, stride, padding, dilation)
+    want = oracle.norm_dist_forward(cols, w, G, p)
+    out = torch.full(want.shape, float("nan"), device=DEV)
+    cpp.norm_dist_conv_forward(img.to(DEV), w.to(DEV), out, G, p, 3, stride, padding, dilation)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out.cpu(), want, rtol=RTOL, atol=0)
+    go = torch.randn(want.shape, generator=gen(7000 + seed))
+    ex, mx = oracle.norm_dist_backward_input(go, cols, w, want, G, p, with_abs_terms=True)
+    ew, mw = oracle.norm_dist_backward_weight(go, cols, w, want, G, p, with_abs_terms=True)
+    fold = lambda t: F.fold(t.double(), (H, W), 3, dilation, padding, stride)
+    args = (go.to(DEV), img.to(DEV), w.to(DEV), want.to(DEV))
+    gi = torch.full(img.shape, float("nan"), device=DEV)
+    gw = torch.zeros(w.shape, device=DEV)
+    cpp.norm_dist_conv_backward_input(*args, gi, G, p, 3, stride, padding, dilation)
+    cpp.norm_dist_conv_backward_weight(*args, gw, G, p, 3, stride, padding, dilation)
+    torch.cuda.synchronize()
+    assert_sum_close(gi.cpu(), fold(ex), fold(mx), p, RTOL, ATOL)
+    assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
+    set_tile(mode)
+    gi = torch.full(img.shape, float("nan"), device=DEV)
+    gw = torch.zeros(w.shape, device=DEV)
+    cpp.norm_dist_conv_backward(*args, gi, gw, G, p, 3, stride, padding, dilation)
+    torch.cuda.synchronize()
+    assert_sum_close(gi.cpu(), fold(ex), fold(mx), p, RTOL, ATOL)
+    assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
 
 
 @pytest.mark.parametrize("seed", range(40))
