@@ -429,7 +429,6 @@ def workload_c4p(pkg, torch, dev):
     layer = pkg.NormDistConv(128, 128, 3, padding=1, group=4, p=p, bias=False, mean_normalize=False).to(dev)
     with torch.no_grad():
         layer.weight.copy_(w.view_as(layer.weight))
-    cpp = pkg.norm_dist_cpp
 
     def step():
         layer.weight.grad = None
@@ -439,12 +438,11 @@ def workload_c4p(pkg, torch, dev):
 
     def step_columns():
         # the same layer through the native unfold, the column kernels and the native fold
-        keep = cpp.norm_dist_conv_supported
-        cpp.norm_dist_conv_supported = lambda *a, **k: False
+        layer.finite_p_route = "columns"
         try:
             step()
         finally:
-            cpp.norm_dist_conv_supported = keep
+            layer.finite_p_route = "image"
 
     wd = w.to(dev).requires_grad_(True)
 

@@ -1222,9 +1222,7 @@ def test_norm_dist_conv_layer_runs_from_the_image_without_columns(p):
     def run(force_columns):
         layer.zero_grad(set_to_none=True)
         xi = x.clone().requires_grad_(True)
-        keep = cpp.norm_dist_conv_supported
-        if force_columns:
-            cpp.norm_dist_conv_supported = lambda *a, **k: False
+        layer.finite_p_route = "columns" if force_columns else "image"
         try:
             torch.cuda.synchronize()
             torch.cuda.reset_peak_memory_stats()
@@ -1234,7 +1232,7 @@ def test_norm_dist_conv_layer_runs_from_the_image_without_columns(p):
             torch.cuda.synchronize()
             peak = torch.cuda.max_memory_allocated() - base
         finally:
-            cpp.norm_dist_conv_supported = keep
+            layer.finite_p_route = "image"
         return y.detach(), xi.grad, layer.weight.grad.clone(), peak
 
     layer.train()
