@@ -66,7 +66,7 @@ inline size_t lds_bytes(int NG, size_t plane_floats) {
 }  // namespace
 
 template <bool IMG, int IE>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, 4)   // four workgroups per CU is what LDS allows at 32 outputs per group: 128 registers
 norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __restrict__ input,
                           const float* __restrict__ weight, const float* __restrict__ output,
                           float* __restrict__ grad_input, float* __restrict__ grad_weight, float e, ConvBwd d,
@@ -99,13 +99,15 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
     }
     // the lane's four columns: whether they exist, and for the image their channel plane and tap
     bool col_ok[4];
-    int col_plane[4], col_tap[4];
+    int col_plane[4], col_tap[4], col_dh[4], col_dw[4];   // IMG: the column's channel plane inside the tile, its tap and the tap's offsets
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const int c = tx * 4 + j;
         col_ok[j] = c < TC && k0 + c < K;
         col_plane[j] = c / 9;
         col_tap[j] = c - col_plane[j] * 9;
+        col_dh[j] = (col_tap[j] / 3) * win.D;
+        col_dw[j] = (col_tap[j] - (col_tap[j] / 3) * 3) * win.D;
     }
 
     // One tile: rows first_row .. first_row + 63 of the unfolded matrix, of which `rows` exist (IMG: rows of image b
@@ -133,8 +135,13 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
                 acc[i][j] = 0.f;
                 bool ok = ty * 4 + i < rows && col_ok[j];
                 size_t off;
-                if constexpr (IMG) ok = win_tap(win, wrow[i], g, ok ? k : 0, off) && ok;
-                else off = xoff[i] + (size_t)k * d.HW;
+                if constexpr (IMG) {   // the window's tap of column j: channel and offsets are the lane's constants
+                    const int h = wrow[i].h0 + col_dh[j], w = wrow[i].w0 + col_dw[j];
+                    ok = ok && (unsigned)h < (unsigned)win.H && (unsigned)w < (unsigned)win.W;
+                    off = (((size_t)b * win.C + g * win.CG + k0 / 9 + col_plane[j]) * win.H + h) * win.W + w;
+                } else {
+                    off = xoff[i] + (size_t)k * d.HW;
+                }
                 q[i][j] = ok ? input[off] : 0.f;
             }
         // g and out of the tile's rows for every output of the group; rows are contiguous in memory
@@ -227,16 +234,22 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
                 flushed = h_lo;
                 __syncthreads();   // ring rows cleared above may be this tile's; every lane is done with the panels
                 // the tile's sums join the planes: nine rounds, one per tap (see the top of the file)
+#pragma unroll
                 for (int tap = 0; tap < 9; tap++) {
-                    const int di = tap / 3, dj = tap - di * 3;
+                    const int dh = (tap / 3) * win.D, dw = (tap % 3) * win.D;
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
-                        if (col_tap[j] != tap || !col_ok[j]) continue;
+                        const bool mine = col_ok[j] && col_tap[j] == tap;
+                        // a wave holds 16 consecutive columns, so one or two of its four j have this tap: the others
+                        // are skipped by the whole wave (a scalar branch) instead of being walked with no lane active
+                        if (__builtin_amdgcn_ballot_w64(mine) == 0) continue;
+                        if (mine) {
 #pragma unroll
-                        for (int i = 0; i < 4; i++) {
-                            const int h = wrow[i].h0 + di * win.D, w = wrow[i].w0 + dj * win.D;
-                            if (ty * 4 + i < rows && (unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W)
-                                Fp[(col_plane[j] * R + (h & (R - 1))) * W + w] += acc[i][j];
+                            for (int i = 0; i < 4; i++) {
+                                const int h = wrow[i].h0 + dh, w = wrow[i].w0 + dw;
+                                if (ty * 4 + i < rows && (unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W)
+                                    Fp[(col_plane[j] * R + (h & (R - 1))) * W + w] += acc[i][j];
+                            }
                         }
                     }
                     __syncthreads();
