@@ -22,46 +22,6 @@
 
 namespace ldist {
 
-namespace {
-
-// Sum over the 16 lanes of a DPP row; the total arrives in the row's last lane (the others hold prefix sums).
-__device__ __forceinline__ float row_total(float v) {
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x111, 0xf, 0xf, true));  // row_shr:1
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x112, 0xf, 0xf, true));  // row_shr:2
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x114, 0xf, 0xf, true));  // row_shr:4
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x118, 0xf, 0xf, true));  // row_shr:8
-    return v;
-}
-
-template <int COLS, int LD, int NT, int KK>
-struct WeightRows {   // P[rr][col] = weight[n0 + rr][k0 + col], 128-bit loads along k
-    static constexpr int PER_ROW = COLS / 4;
-    static constexpr int TOTAL = KK * PER_ROW;
-    static constexpr int N = (TOTAL + NT - 1) / NT;
-    float4 v[N];
-    __device__ __forceinline__ void load(const float* __restrict__ base, int stride, int n0, int R, int k0, int K, int tid) {
-#pragma unroll
-        for (int i = 0; i < N; i++) {
-            const int id = tid + i * NT;
-            const int rr = id / PER_ROW, cq = id % PER_ROW;
-            const int n = n0 + rr, k = k0 + cq * 4;
-            v[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if ((TOTAL % NT == 0 || id < TOTAL) && n < R && k < K) v[i] = *reinterpret_cast<const float4*>(base + (size_t)n * stride + k);
-        }
-    }
-    __device__ __forceinline__ void store(float* __restrict__ panel, int tid) const {
-#pragma unroll
-        for (int i = 0; i < N; i++) {
-            const int id = tid + i * NT;
-            if (TOTAL % NT != 0 && id >= TOTAL) continue;
-            const int rr = id / PER_ROW, cq = id % PER_ROW;
-            *reinterpret_cast<float4*>(panel + rr * LD + ((cq * 4) ^ swz(rr))) = v[i];
-        }
-    }
-};
-
-}  // namespace
-
 template <class GEO>
 __global__ void __launch_bounds__(GEO::NT, 2)
 norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* __restrict__ input,
@@ -72,7 +32,7 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
     constexpr int STAGE = 2 * XS + WS;     // [F or g][1/out][w]
     static_assert(GEO::TY == 16, "the lanes that share a column fill one DPP row");
     using RowLoad = RowsK<BM, GEO::SM, NT, KK, 4>;   // outputs are contiguous in g and out
-    using ColLoad = WeightRows<BN, GEO::SN, NT, KK>;
+    using ColLoad = RowsT<BN, GEO::SN, NT, KK, 4>;
     static_assert((KS - 1) * TM * TN * NGRP <= STAGE, "merge area fits in the panels");
     extern __shared__ __align__(16) float lds[];
 
@@ -110,7 +70,7 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
     auto add_weight_row = [&](int n, const float (&s)[TN]) {
         float tot[TN];
 #pragma unroll
-        for (int j = 0; j < TN; j++) tot[j] = row_total(s[j]);
+        for (int j = 0; j < TN; j++) tot[j] = dpp_row_total(s[j]);
         if (ty == GEO::TY - 1 && n < NG) {
             float* row = gw_group + (size_t)n * K;
 #pragma unroll

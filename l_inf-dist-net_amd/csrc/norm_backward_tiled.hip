@@ -14,47 +14,6 @@
 
 namespace ldist {
 
-// Panel whose columns are contiguous in memory for a fixed row of the reduction: P[rr][col] = src[n0 + rr][k0 + col]
-// (the weights of a stage of outputs for grad_input, the inputs of a stage of rows for grad_weight).  Lanes run
-// along the columns and nothing is transposed.  VEC == 4 needs K % 4 == 0 and a 16-byte aligned base.
-template <int COLS, int LD, int NT, int KK, int VEC>
-struct RowsT {
-    static constexpr int PER_ROW = COLS / VEC;
-    static constexpr int TOTAL = KK * PER_ROW;
-    static constexpr int N = (TOTAL + NT - 1) / NT;
-    float v[N][VEC];
-    // base: pointer to (first row of the reduction, column 0); rows are `stride` apart, R of them, K columns
-    __device__ __forceinline__ void load(const float* __restrict__ base, int stride, int n0, int R, int k0, int K, int tid) {
-#pragma unroll
-        for (int i = 0; i < N; i++) {
-            const int id = tid + i * NT;
-            const int rr = id / PER_ROW, cq = id % PER_ROW;
-            const int n = n0 + rr, k = k0 + cq * VEC;
-            const bool ok = (TOTAL % NT == 0 || id < TOTAL) && n < R && k < K;
-            const float* p = base + (size_t)n * stride + k;
-            if constexpr (VEC == 4) {
-                float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (ok) t = *reinterpret_cast<const float4*>(p);
-                v[i][0] = t.x; v[i][1] = t.y; v[i][2] = t.z; v[i][3] = t.w;
-            } else {
-                v[i][0] = ok ? *p : 0.f;
-            }
-        }
-    }
-    __device__ __forceinline__ void store(float* __restrict__ panel, int tid) const {
-#pragma unroll
-        for (int i = 0; i < N; i++) {
-            const int id = tid + i * NT;
-            if (TOTAL % NT != 0 && id >= TOTAL) continue;
-            const int rr = id / PER_ROW, cq = id % PER_ROW;
-            if constexpr (VEC == 4)
-                *reinterpret_cast<float4*>(panel + rr * LD + ((cq * 4) ^ swz(rr))) = make_float4(v[i][0], v[i][1], v[i][2], v[i][3]);
-            else
-                panel[rr * LD + (cq ^ swz(rr))] = v[i][0];
-        }
-    }
-};
-
 // IE = p - 1 (1, 2, 3 or 7).  d.K is the number of inputs per group (the tile's columns), d.NG the outputs per
 // group (the reduction), d.tiles_n counts column tiles.
 template <class GEO, bool CONV, int IE>

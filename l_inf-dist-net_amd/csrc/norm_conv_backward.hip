@@ -28,9 +28,9 @@
 // IE = p - 1 for the multiply-only exponents (1, 2, 3, 7): the power is taken of the raw difference and the
 // coefficient g / out^(p-1) is staged instead of g, unless a tile holds an output outside [2^-12, 2^12], which then
 // takes the normalised difference like IE = 0 (any p > 1, through v_log_f32 / v_exp_f32).
-#include "conv_window.hpp"
 #include "kernels.hpp"
 #include "pow.hpp"
+#include "tile.hpp"
 
 #include <algorithm>
 
@@ -43,14 +43,6 @@ constexpr int TCP = 64;             // columns a tile has lanes for
 constexpr int WLD = TCP + 4;        // row length of the weight and grad_weight tiles (rows 16-byte aligned)
 constexpr int kPlanes = 7;          // IMG: channels per tile (63 columns)
 constexpr size_t kMaxLds = 159 * 1024;   // all of LDS less the kernel's own static words
-
-__device__ __forceinline__ float row_total16(float v) {   // sum over a DPP row; the total arrives in its last lane
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x111, 0xf, 0xf, true));
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x112, 0xf, 0xf, true));
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x114, 0xf, 0xf, true));
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x118, 0xf, 0xf, true));
-    return v;
-}
 
 struct ConvBwd {
     int B, G, K, NG, HW, M;          // the unfolded problem: K = 9 channels per group (image) or CI / G
@@ -187,7 +179,7 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
                     }
                 float tot[4];
 #pragma unroll
-                for (int j = 0; j < 4; j++) tot[j] = row_total16(s[j]);
+                for (int j = 0; j < 4; j++) tot[j] = dpp_row_total(s[j]);
                 if (ty == 15) {   // d/dw of |x - w| is minus d/dx
                     float4* gp = reinterpret_cast<float4*>(Gw + n * WLD + tx * 4);
                     float4 v = *gp;
