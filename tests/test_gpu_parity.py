@@ -1309,6 +1309,23 @@ def test_norm_backward_both_gradients_at_every_scale(scale, p):
     assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
 
 
+ONE_PASS_EDGE_CASES = [  # B, C, H, W, CO, G, stride, padding, dilation
+    (1, 4, 12, 12, 130, 1, 1, 1, 1),     # 130 outputs in one group: the LDS tiles leave room for one workgroup per CU
+    (1, 4, 12, 12, 150, 1, 1, 1, 1),     # 150: the tiles do not fit, the call runs the two separate kernels
+    (1, 3, 64, 64, 20, 1, 1, 1, 1),      # a tile of 64 positions is one output row: ring of four image rows, 64 wide
+    (2, 9, 40, 24, 18, 1, 2, 1, 1),      # stride 2 on a 40 x 24 image: 20 x 12 positions, tiles cross output rows unevenly
+    (3, 16, 5, 5, 32, 2, 1, 1, 1),       # 25 positions per image: every tile is a partial one
+    (2, 7, 9, 9, 1, 1, 1, 0, 1),         # a single output
+]
+
+
+@pytest.mark.parametrize("p", [8.0, 5.5])
+@pytest.mark.parametrize("case", ONE_PASS_EDGE_CASES)
+def test_norm_conv_backward_one_pass_edge_geometries(case, p):
+    """The one-pass conv backward from the image at the edges of what it takes (see the list), forced on."""
+    test_norm_conv_backward_both_gradients_in_one_pass_from_the_image(case, p)
+
+
 @pytest.mark.parametrize("p", [8.0, 3.0, 5.5, 100.0])
 @pytest.mark.parametrize("case", NORM_IMAGE_CASES)
 def test_norm_conv_backward_both_gradients_in_one_pass_from_the_image(case, p):
