@@ -402,6 +402,11 @@ def workload_c4i(pkg, torch, dev):
     unfolded tensor and its gradient are never built (forward straight from the image, scatter and fold fused)."""
     wl = workload_c4(pkg, torch, dev)
     from_image = dict(wl["step_alt"])["ms_per_step_from_image"]
+    cpp = pkg.norm_dist_cpp
+    geometry = (128, 32, 32, 128, 4, 3, 1, 1, 1)
+    # which kernels the layer's forward takes (a geometry the image kernel does not cover falls back to unfold + columns)
+    wl["routes"] = {"forward_from_image": bool(cpp.inf_dist_conv_forward_supported(*geometry)),
+                    "backward_input_from_image": True}
     wl.update(step=from_image,
               step_alt=[("ms_per_step_columns_only_unfold_outside", wl["step"]),
                         ("ms_per_step_with_torch_unfold_and_fold", dict(wl["step_alt"])["ms_per_step_with_torch_unfold_and_fold"])],
@@ -489,6 +494,9 @@ def workload_c4p(pkg, torch, dev):
 
     return dict(step=step, ops=3 * 128 * 1024 * 128 * 288, images=128, full_rows=128, cpu=cpu, formula=formula,
                 check=check,
+                # a geometry the image kernels do not cover would fall back to unfold + columns + fold
+                routes={"from_image": bool(pkg.norm_dist_cpp.norm_dist_conv_supported(128, 32, 32, 128, 4, 3, 1, 1, 1)),
+                        "finite_p_route": layer.finite_p_route},
                 step_alt=[("ms_per_step_native_unfold_columns_fold", step_columns),
                           ("ms_per_step_with_torch_unfold_and_fold", step_torch_unfold)],
                 name=f"configs[4]'s layer at p={p:g} from the image: 3x3 p-norm dist conv layer, batch 128, 128->128 "
@@ -652,7 +660,7 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": wl["name"], "dist_ops_per_step": ops},
+        "config": {"workload": wl["name"], "dist_ops_per_step": ops, **wl.get("routes", {})},
         "img_per_s": round(wl["images"] / (ms_per_step * 1e-3), 1),
         "pct_fp32_valu_peak": round(100 * value * 1e9 * flops_per_op / (FP32_PEAK_TFLOPS * 1e12), 2),
         "parity": parity,
