@@ -1426,3 +1426,43 @@ def test_fc_and_1x1_layers_accept_non_contiguous_inputs():
         torch.cuda.synchronize()
         assert torch.equal(ya, yb)
         assert torch.equal(a.grad, b.grad)
+
+
+def test_norm_entry_points_added_to_the_abi_check_their_arguments():
+    """Return codes of the entry points without a reference counterpart: null pointers and exponents that are not
+    above 1 are invalid arguments, a window the image kernels do not take is 'unsupported', and in every such case
+    nothing is enqueued (the outputs keep their sentinel)."""
+    from gpu_common import DEV, pkg
+    lib = pkg._lib.lib()
+    EINVAL, EUNSUPPORTED = -1, -5
+    x = torch.rand(2, 8, 1, device=DEV)
+    w = torch.rand(4, 8, device=DEV)
+    y = torch.rand(2, 4, 1, device=DEV) + 1
+    go = torch.randn(2, 4, 1, device=DEV)
+    gx = torch.full_like(x, 7.0)
+    gw = torch.full_like(w, 7.0)
+    P = lambda t: t.data_ptr()
+    assert lib.ldist_strerror(EINVAL).startswith(b"invalid argument") and b"general path" in lib.ldist_strerror(EUNSUPPORTED)
+    assert lib.ldist_norm_dist_backward(P(go), P(x), P(w), P(y), 2, 4, 8, 1, 1, P(gx), P(gw), 1.0, None) == EINVAL
+    assert lib.ldist_norm_dist_backward(P(go), P(x), P(w), P(y), 2, 4, 8, 1, 1, None, P(gw), 8.0, None) == EINVAL
+    assert lib.ldist_norm_dist_backward(P(go), P(x), P(w), P(y), 2, 4, 8, 3, 1, P(gx), P(gw), 8.0, None) == EINVAL   # 8 % 3
+    img = torch.rand(1, 2, 6, 6, device=DEV)
+    w5 = torch.rand(4, 50, device=DEV)
+    y5 = torch.rand(1, 4, 4, device=DEV) + 1
+    g5 = torch.randn(1, 4, 4, device=DEV)
+    gi = torch.full_like(img, 7.0)
+    g5w = torch.full_like(w5, 7.0)
+    conv = (1, 2, 6, 6, 4, 1, 5, 5, 1, 0, 1)     # a 5x5 window
+    assert lib.ldist_norm_dist_conv_supported(2, 6, 6, 4, 1, 5, 5, 1, 0, 1) == 0
+    assert lib.ldist_norm_dist_conv_forward(P(img), P(w5), *conv, P(y5), 8.0, None) == EUNSUPPORTED
+    assert lib.ldist_norm_dist_conv_backward(P(g5), P(img), P(w5), P(y5), *conv, P(gi), P(g5w), 8.0, None) == EUNSUPPORTED
+    conv3 = (1, 2, 6, 6, 4, 1, 3, 3, 1, 1, 1)
+    w3 = torch.rand(4, 18, device=DEV)
+    y3 = torch.rand(1, 4, 36, device=DEV) + 1
+    g3 = torch.randn(1, 4, 36, device=DEV)
+    g3w = torch.full_like(w3, 7.0)
+    assert lib.ldist_norm_dist_conv_backward(P(g3), P(img), P(w3), P(y3), *conv3, P(gi), P(g3w), 0.5, None) == EINVAL
+    assert lib.ldist_norm_dist_conv_backward(P(g3), P(img), None, P(y3), *conv3, P(gi), P(g3w), 8.0, None) == EINVAL
+    torch.cuda.synchronize()
+    for t in (gx, gw, gi, g5w, g3w):
+        assert bool((t == 7.0).all())
