@@ -47,6 +47,11 @@ struct Stager {
         for (int q = 0; q < NX; q++)
             in[q] = CONV ? input[q] : input[q] + ((size_t)m0 * d.G + g) * K;  // fc: row m is image b
         grp_ = g;
+        if constexpr (CLAMPED) {
+            wl.init_clamped(wbase, K, rows_w, tid);
+#pragma unroll
+            for (int q = 0; q < NX; q++) xlk[q].init_clamped(in[q], ld_x, rows_x, tid);
+        }
         if constexpr (IMG) {
 #pragma unroll
             for (int q = 0; q < NX; q++) xli[q].init(win, m0, d.M, tid);
@@ -54,7 +59,21 @@ struct Stager {
             XLoadM::offsets(off_m, m0, d.M, d.HW, d.G, g, K, tid);
         }
     }
+    static constexpr bool CLAMPED = !CONV && VEC == 4;   // fc layout with 128-bit loads: buffer loads (RowsK::load_clamped)
     __device__ __forceinline__ void load(int k0) {
+        if constexpr (CLAMPED) {
+            if (k0 + GEO::KK <= K) {         // a whole stage: no predicates at all
+                asm volatile("" ::: "memory");   // keeps this branch from being folded into the predicated one
+                wl.template load_clamped<true>(k0, K, tid);
+#pragma unroll
+                for (int q = 0; q < NX; q++) xlk[q].template load_clamped<true>(k0, K, tid);
+            } else {
+                wl.template load_clamped<false>(k0, K, tid);
+#pragma unroll
+                for (int q = 0; q < NX; q++) xlk[q].template load_clamped<false>(k0, K, tid);
+            }
+            return;
+        }
         wl.load(wbase, K, rows_w, k0, K, tid);
 #pragma unroll
         for (int q = 0; q < NX; q++) {
@@ -209,7 +228,10 @@ inline bool can_vec4_out(const Problem& pr, const void* a, const void* b = nullp
 
 inline Dims make_dims(const Problem& pr) { return Dims{pr.B, pr.G, pr.K, pr.NG, pr.HW, pr.B * pr.HW, 0, 0, 0, g_xcd_remap}; }
 
+// 128-bit loads of the inputs and weights.  In the fc layout a lane addresses its vectors by 32-bit byte offsets
+// from its tile's first row that must stay below 2 GB (RowsK::init_clamped): at most 256 rows of G * K elements.
 inline bool can_vec4(const Problem& pr, const void* a, const void* b, const void* c = nullptr) {
+    if (pr.HW == 1 && 4LL * 258 * pr.G * pr.K >= (1LL << 31)) return false;
     return pr.K % 4 == 0 && (pr.HW == 1 || pr.HW % 4 == 0) && aligned16(a) && aligned16(b) && aligned16(c);
 }
 

@@ -79,10 +79,23 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
                     }
             });
         } else {
+            if constexpr (HALF) {
 #pragma unroll
-            for (int i = 0; i < TM; i++)
+                for (int i = 0; i < TM; i++)
 #pragma unroll
-                for (int j = 0; j < TN; j++) cur[i][j] = prev[i][j];
+                    for (int j = 0; j < TN; j++) cur[i][j] = prev[i][j];
+            }
+            // the chunk's first fragment takes the running maximum from prev and leaves it in cur: no copy
+            auto body_first = [&](const Frag<GEO, 1, 2>& f, int) {
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) {
+                        const float d0 = __builtin_fabsf(f.x[0][0][i] - f.w[0][j]);
+                        const float d1 = __builtin_fabsf(f.x[0][1][i] - f.w[1][j]);
+                        cur[i][j] = __builtin_fmaxf(__builtin_fmaxf(prev[i][j], d0), d1);
+                    }
+            };
             auto body = [&](const Frag<GEO, 1, 2>& f, int) {
 #pragma unroll
                 for (int i = 0; i < TM; i++)
@@ -93,24 +106,45 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
                         cur[i][j] = __builtin_fmaxf(__builtin_fmaxf(cur[i][j], d0), d1);
                     }
             };
+            // Records `tag` for the outputs whose maximum this part of the chunk raised.  Two patch rows' compares
+            // first, each into its own pair of scalar registers, then their selects: a select straight after its
+            // compare (what the compiler makes of the plain form) waits two cycles for the lane mask.  The empty asm
+            // statements keep their order: the first kind keeps the compiler from folding a mask back into the plain
+            // form, the second ends a group, so that no more than ten masks are live (all forty would push other
+            // scalars out of their registers).
+            static_assert(TM % 2 == 0, "rows in pairs");
+            auto record = [&](int tag) {
+#pragma unroll
+                for (int i = 0; i < TM; i += 2) {
+                    unsigned long long raised[2][TN];
+#pragma unroll
+                    for (int a = 0; a < 2; a++)
+#pragma unroll
+                        for (int j = 0; j < TN; j++) {
+                            raised[a][j] = __builtin_amdgcn_fcmpf(cur[i + a][j], prev[i + a][j], 2 /* ordered > */);
+                            asm volatile("" : "+s"(raised[a][j]));
+                        }
+#pragma unroll
+                    for (int a = 0; a < 2; a++)
+#pragma unroll
+                        for (int j = 0; j < TN; j++) {
+                            if (__builtin_amdgcn_inverse_ballot_w64(raised[a][j])) cidx[i + a][j] = tag;
+                            asm volatile("" : "+v"(cidx[i + a][j]));
+                        }
+                }
+            };
             if constexpr (HALF) {
                 sweep_chunk<GEO, 1, 2, true>(xp, wp, tx, ty, body, [&]() {   // after the first 16 k: record, move prev up
+                    record(2 * c);
 #pragma unroll
                     for (int i = 0; i < TM; i++)
 #pragma unroll
-                        for (int j = 0; j < TN; j++) {
-                            if (cur[i][j] > prev[i][j]) cidx[i][j] = 2 * c;
-                            prev[i][j] = cur[i][j];
-                        }
+                        for (int j = 0; j < TN; j++) prev[i][j] = cur[i][j];
                 });
             } else {
-                sweep_chunk<GEO, 1, 2, true>(xp, wp, tx, ty, body);
+                sweep_chunk_first<GEO, 1, 2>(xp, wp, tx, ty, body_first, body);
             }
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++)
-                    if (cur[i][j] > prev[i][j]) cidx[i][j] = HALF ? 2 * c + 1 : c;
+            record(HALF ? 2 * c + 1 : c);
         }
         if (NBUF == 1) __syncthreads();  // everyone is done reading the only buffer
         if (s + 1 < nstage) st.store(lds + ((s + 1) % NBUF) * STAGE);

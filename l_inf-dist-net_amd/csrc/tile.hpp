@@ -257,6 +257,46 @@ __device__ __forceinline__ void sweep_chunk(const float* xp, const float* wp, in
     }
 }
 
+// The same walk with the chunk's first fragment taken out of the loop and given to `first`, so that it can read
+// its accumulators from one register array and write them to another (the L_inf forward continues the running
+// maximum of the stage before in a second array and would otherwise copy forty registers per chunk).  Byte-address
+// form only.  Fragments 1..14 run as seven trips of two, fragment 15 after the loop.
+template <class GEO, int NX, int KP, class F0, class F>
+__device__ __forceinline__ void sweep_chunk_first(const float* xp, const float* wp, int tx, int ty, F0&& first, F&& f) {
+    static_assert(KP == 2, "sixteen fragments of two k per chunk");
+    constexpr int FRAG_LDS = NX * KP * (GEO::TM / 4) + KP * (GEO::TN == 8 ? 2 : 1) + (GEO::TN == 5 ? 1 : 0);
+    constexpr int WAIT_PREV = 0xc07f | (FRAG_LDS << 8);
+    static_assert(FRAG_LDS < 16, "lgkmcnt field");
+    Frag<GEO, NX, KP> a, b;
+    LaneAddr<GEO> cur, nxt;
+    const LaneCols<GEO> cols(tx, ty);
+    const unsigned xb = lds_address(xp), wb = lds_address(wp);
+    cur.set(xb, wb, 0, cols);
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    read_frag(a, cur, 0);
+    read_frag(b, cur, KP);
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(WAIT_PREV);
+    __builtin_amdgcn_sched_barrier(0);
+    first(a, 0);
+#pragma unroll 1
+    for (int kk = KP; kk < kChunk - KP; kk += 2 * KP) {   // b holds rows kk, kk + 1 of the chunk
+        nxt.set(xb, wb, kk + KP, cols);
+        read_frag(a, nxt, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(WAIT_PREV);
+        __builtin_amdgcn_sched_barrier(0);
+        f(b, kk);
+        read_frag(b, nxt, KP);
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(WAIT_PREV);
+        __builtin_amdgcn_sched_barrier(0);
+        f(a, kk + KP);
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    f(b, kChunk - KP);
+}
+
 // Same walk without the operand prefetch, one k row per trip: for rarely taken
 // paths that must not add to the register budget of the hot loop.
 template <class GEO, int NX, class F>
@@ -286,7 +326,8 @@ struct RowsK {
     static constexpr int N = (TOTAL + NT - 1) / NT;        // vectors per lane
     float v[N][VEC];
 
-    // base: pointer to (row 0 of the tile, k = 0); ld: elements between rows.
+    // base: pointer to (row 0 of the tile, k = 0); ld: elements between rows.  Rows and k outside the matrix read
+    // as zeros, which every reduction here ignores.
     __device__ __forceinline__ void load(const float* __restrict__ base, int ld, int rows_valid, int k0, int K,
                                          int tid) {
 #pragma unroll
@@ -303,6 +344,36 @@ struct RowsK {
             } else {
                 v[i][0] = (ok && k < K) ? *p : 0.f;
             }
+        }
+    }
+    // For callers that never use the results of rows past the matrix (the forward kernels: they are not stored):
+    // such rows read the matrix's last row instead, so a row needs no predicate, and a lane's byte offsets from the
+    // tile's first row are fixed for the whole reduction.  The loads are buffer loads: a descriptor of the tile's
+    // first row in scalar registers (the same for every lane), the lane's 32-bit offset, and the stage's k0 as the
+    // scalar offset, so a load costs no address arithmetic; an offset of all ones lies outside the descriptor's 2 GB
+    // range and reads as zeros, which takes the place of every predicate (lanes without a vector in a round, k >= K
+    // in the last stage) without zeros in registers or branches.  The host checks that real offsets stay below 2 GB.
+    unsigned off[N];   // bytes
+    __amdgpu_buffer_rsrc_t rsrc;
+    typedef float F4 __attribute__((ext_vector_type(4)));
+    __device__ __forceinline__ void init_clamped(const float* base, int ld, int rows_valid, int tid) {
+        rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, (int)0x80000000u, 0x00020000);
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const int id = tid + i * NT;
+            off[i] = 4u * ((unsigned)min(id / PER_ROW, rows_valid - 1) * (unsigned)ld + (unsigned)(id % PER_ROW) * VEC);
+            if (TOTAL % NT != 0 && id >= TOTAL) off[i] = ~0u;
+        }
+    }
+    // INSIDE: the stage lies inside the reduction axis (k0 + KK <= K; uniform over the workgroup).
+    template <bool INSIDE>
+    __device__ __forceinline__ void load_clamped(int k0, int K, int tid) {
+        static_assert(VEC == 4 && NT % PER_ROW == 0, "128-bit loads; a lane keeps its k offset over the rounds");
+        const bool k_ok = INSIDE || k0 + (tid % PER_ROW) * VEC < K;
+#pragma unroll
+        for (int i = 0; i < N; i++) {
+            const F4 t = __builtin_bit_cast(F4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, k_ok ? off[i] : ~0u, k0 * 4, 0));
+            v[i][0] = t.x; v[i][1] = t.y; v[i][2] = t.z; v[i][3] = t.w;
         }
     }
     __device__ __forceinline__ void store(float* __restrict__ panel, int tid) const {
