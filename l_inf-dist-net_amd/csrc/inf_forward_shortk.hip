@@ -77,29 +77,33 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
     // input panel: a lane keeps its four rows (consecutive positions of one image: HW % 4 == 0) and walks k
     const int lmq = tid % (BM / 4), lkx = tid / (BM / 4);
     float4 park[NP];
-    // Loads never branch per lane: a lane outside the tensor (rows past M, k past K in the last pass) reads a clamped,
-    // valid address and its value is replaced by 0 when the panel is written.
-    auto x_base = [&](int t) {
+    // Buffer loads: the descriptor of the whole input in scalar registers, the lane's byte offset of (its four rows,
+    // k = lkx) of the tile in one register, the pass's k rows as the scalar offset.  An offset of all ones lies outside
+    // the descriptor's 2 GB range and reads as zeros: that is how rows past M, k past K in the last pass and the passes
+    // beyond Kp / 32 come out as zeros, without a branch, a predicate or a select when the panel is written (the host
+    // checks that the input is smaller than 2 GB).
+    typedef float F4 __attribute__((ext_vector_type(4)));
+    const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(input), 0, (int)0x80000000u, 0x00020000);
+    auto x_offset = [&](int t) -> unsigned {
         const int tm = t % d.tiles_m, g = (t / d.tiles_m) / d.tiles_n;
-        const int m = min(tm * BM + lmq * 4, d.M - 4);
+        const int m = tm * BM + lmq * 4;
+        if (m >= d.M) return ~0u;                // HW % 4 == 0: four rows are inside the tensor together
         const int b = m / HW, hw = m % HW;
-        return input + ((size_t)(b * d.G + g) * K) * HW + hw;
+        return (unsigned)((((size_t)(b * d.G + g) * K + lkx) * HW + hw) * sizeof(float));
     };
     auto issue_x = [&](int t) {
-        const float* xin = x_base(t);
+        const unsigned off = x_offset(t), off_last = lkx + (npass - 1) * XROWS < K ? off : ~0u;
 #pragma unroll
-        for (int p = 0; p < NP; p++)   // passes beyond Kp / 32 read row K - 1 again and are dropped
-            park[p] = *reinterpret_cast<const float4*>(xin + (size_t)min(lkx + p * XROWS, K - 1) * HW);
+        for (int p = 0; p < NP; p++) {
+            const unsigned o = p < npass - 1 ? off : (p == npass - 1 ? off_last : ~0u);
+            const F4 v = __builtin_bit_cast(F4, __builtin_amdgcn_raw_buffer_load_b128(xrs, o, p * XROWS * HW * (int)sizeof(float), 0));
+            park[p] = make_float4(v.x, v.y, v.z, v.w);
+        }
     };
-    auto store_x = [&](int t) {
-        const bool row_ok = (t % d.tiles_m) * BM + lmq * 4 < d.M;
+    auto store_x = [&](int) {
 #pragma unroll
         for (int p = 0; p < NP; p++)
-            if (p < npass) {
-                const bool ok = row_ok && lkx + p * XROWS < K;
-                *reinterpret_cast<float4*>(X + (lkx + p * XROWS) * BM + lmq * 4) =
-                    ok ? park[p] : make_float4(0.f, 0.f, 0.f, 0.f);
-            }
+            if (p < npass) *reinterpret_cast<float4*>(X + (lkx + p * XROWS) * BM + lmq * 4) = park[p];
     };
     // weight panel of (group g, output tile tn): lanes run along k, a lane takes four neighbouring outputs
     auto load_w = [&](int g, int tn) {
@@ -226,11 +230,28 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
             fetch(xa, wa, 0);
             __builtin_amdgcn_sched_barrier(0);
             reduce(xb, wb, cur);
+            // Eight compares into their own scalar register pairs, then their selects: a select straight after its
+            // compare (what the compiler makes of the plain form) waits two cycles for the lane mask.  The empty asm
+            // statements keep their order: the first kind keeps a mask from being folded back into the plain form,
+            // the second ends a group of eight.
 #pragma unroll
-            for (int i = 0; i < 4; i++)
+            for (int i = 0; i < 4; i += 2) {
+                unsigned long long raised[2][4];
 #pragma unroll
-                for (int j = 0; j < 4; j++)
-                    if (cur[i][j] > prev[i][j]) widx[i][j] = wid;
+                for (int a = 0; a < 2; a++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        raised[a][j] = __builtin_amdgcn_fcmpf(cur[i + a][j], prev[i + a][j], 2 /* ordered > */);
+                        asm volatile("" : "+s"(raised[a][j]));
+                    }
+#pragma unroll
+                for (int a = 0; a < 2; a++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        if (__builtin_amdgcn_inverse_ballot_w64(raised[a][j])) widx[i + a][j] = wid;
+                        asm volatile("" : "+v"(widx[i + a][j]));
+                    }
+            }
         };
         fetch(xa, wa, 0);
         const int w_issue = (nwin / 2) & ~1;
@@ -339,6 +360,7 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
 bool inf_forward_shortk_applicable(const Problem& pr, const void* input, const void* output, const void* pos) {
     if (pr.HW == 1 || pr.HW % 4 != 0) return false;
     if (!aligned16(input) || !aligned16(output) || !aligned16(pos)) return false;
+    if ((size_t)pr.B * pr.G * pr.K * pr.HW * sizeof(float) >= (size_t)1 << 31) return false;   // 32-bit buffer offsets
     const int Kp = shortk::padded_k(pr.K);
     return Kp / shortk::XROWS <= shortk::MAXPASS && Kp / (shortk::NGROUP * shortk::WIN) <= 255 &&
            shortk::lds_bytes(Kp) <= 160 * 1024;
