@@ -58,7 +58,8 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
     // One stage: a k-group sweeps its chunk of the resident panels.  prev holds the running
     // maximum before the chunk and is left alone; cur continues from it, so the chunk raised the
     // maximum iff cur > prev afterwards.  The two arrays swap roles from stage to stage, which
-    // saves copying cur back (EXACT keeps everything in prev).
+    // saves copying cur back (EXACT keeps everything in prev; with HALF the two halves of a chunk
+    // swap them twice, so the result is in prev again).
     auto run_stage = [&](float (&prev)[TM][TN], float (&cur)[TM][TN], int s) {
         const float* stage = lds + (s % NBUF) * STAGE;
         if (s + 1 < nstage) st.load((s + 1) * KK);
@@ -79,41 +80,39 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
                     }
             });
         } else {
-            if constexpr (HALF) {
+            // Sweeps rows [k_begin, k_begin + LEN) of the chunk: the first fragment takes the running maximum from
+            // `from` and leaves it in `to` (no copy), the others continue in `to`.
+            auto sweep_into = [&](const float (&from)[TM][TN], float (&to)[TM][TN], int k_begin, auto len) {
+                auto body_first = [&](const Frag<GEO, 1, 2>& f, int) {
 #pragma unroll
-                for (int i = 0; i < TM; i++)
+                    for (int i = 0; i < TM; i++)
 #pragma unroll
-                    for (int j = 0; j < TN; j++) cur[i][j] = prev[i][j];
-            }
-            // the chunk's first fragment takes the running maximum from prev and leaves it in cur: no copy
-            auto body_first = [&](const Frag<GEO, 1, 2>& f, int) {
+                        for (int j = 0; j < TN; j++) {
+                            const float d0 = __builtin_fabsf(f.x[0][0][i] - f.w[0][j]);
+                            const float d1 = __builtin_fabsf(f.x[0][1][i] - f.w[1][j]);
+                            to[i][j] = __builtin_fmaxf(__builtin_fmaxf(from[i][j], d0), d1);
+                        }
+                };
+                auto body = [&](const Frag<GEO, 1, 2>& f, int) {
 #pragma unroll
-                for (int i = 0; i < TM; i++)
+                    for (int i = 0; i < TM; i++)
 #pragma unroll
-                    for (int j = 0; j < TN; j++) {
-                        const float d0 = __builtin_fabsf(f.x[0][0][i] - f.w[0][j]);
-                        const float d1 = __builtin_fabsf(f.x[0][1][i] - f.w[1][j]);
-                        cur[i][j] = __builtin_fmaxf(__builtin_fmaxf(prev[i][j], d0), d1);
-                    }
+                        for (int j = 0; j < TN; j++) {
+                            const float d0 = __builtin_fabsf(f.x[0][0][i] - f.w[0][j]);
+                            const float d1 = __builtin_fabsf(f.x[0][1][i] - f.w[1][j]);
+                            to[i][j] = __builtin_fmaxf(__builtin_fmaxf(to[i][j], d0), d1);
+                        }
+                };
+                sweep_chunk_first<GEO, 1, 2, decltype(len)::value>(xp, wp, tx, ty, k_begin, body_first, body);
             };
-            auto body = [&](const Frag<GEO, 1, 2>& f, int) {
-#pragma unroll
-                for (int i = 0; i < TM; i++)
-#pragma unroll
-                    for (int j = 0; j < TN; j++) {
-                        const float d0 = __builtin_fabsf(f.x[0][0][i] - f.w[0][j]);
-                        const float d1 = __builtin_fabsf(f.x[0][1][i] - f.w[1][j]);
-                        cur[i][j] = __builtin_fmaxf(__builtin_fmaxf(cur[i][j], d0), d1);
-                    }
-            };
-            // Records `tag` for the outputs whose maximum this part of the chunk raised.  Two patch rows' compares
+            // Records `tag` for the outputs whose maximum a sweep raised (newer > older).  Two patch rows' compares
             // first, each into its own pair of scalar registers, then their selects: a select straight after its
             // compare (what the compiler makes of the plain form) waits two cycles for the lane mask.  The empty asm
             // statements keep their order: the first kind keeps the compiler from folding a mask back into the plain
             // form, the second ends a group, so that no more than ten masks are live (all forty would push other
             // scalars out of their registers).
             static_assert(TM % 2 == 0, "rows in pairs");
-            auto record = [&](int tag) {
+            auto record = [&](const float (&newer)[TM][TN], const float (&older)[TM][TN], int tag) {
 #pragma unroll
                 for (int i = 0; i < TM; i += 2) {
                     unsigned long long raised[2][TN];
@@ -121,7 +120,7 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
                     for (int a = 0; a < 2; a++)
 #pragma unroll
                         for (int j = 0; j < TN; j++) {
-                            raised[a][j] = __builtin_amdgcn_fcmpf(cur[i + a][j], prev[i + a][j], 2 /* ordered > */);
+                            raised[a][j] = __builtin_amdgcn_fcmpf(newer[i + a][j], older[i + a][j], 2 /* ordered > */);
                             asm volatile("" : "+s"(raised[a][j]));
                         }
 #pragma unroll
@@ -133,18 +132,15 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
                         }
                 }
             };
-            if constexpr (HALF) {
-                sweep_chunk<GEO, 1, 2, true>(xp, wp, tx, ty, body, [&]() {   // after the first 16 k: record, move prev up
-                    record(2 * c);
-#pragma unroll
-                    for (int i = 0; i < TM; i++)
-#pragma unroll
-                        for (int j = 0; j < TN; j++) prev[i][j] = cur[i][j];
-                });
+            if constexpr (HALF) {   // two halves of 16: the second goes back into prev, which ends up holding the result
+                sweep_into(prev, cur, 0, std::integral_constant<int, kChunk / 2>{});
+                record(cur, prev, 2 * c);
+                sweep_into(cur, prev, kChunk / 2, std::integral_constant<int, kChunk / 2>{});
+                record(prev, cur, 2 * c + 1);
             } else {
-                sweep_chunk_first<GEO, 1, 2>(xp, wp, tx, ty, body_first, body);
+                sweep_into(prev, cur, 0, std::integral_constant<int, kChunk>{});
+                record(cur, prev, c);
             }
-            record(HALF ? 2 * c + 1 : c);
         }
         if (NBUF == 1) __syncthreads();  // everyone is done reading the only buffer
         if (s + 1 < nstage) st.store(lds + ((s + 1) % NBUF) * STAGE);
@@ -152,6 +148,8 @@ inf_forward_kernel(const float* __restrict__ input, const float* __restrict__ we
     };
     if constexpr (EXACT) {
         for (int s = 0; s < nstage; s++) run_stage(acc, acc, s);
+    } else if constexpr (HALF) {
+        for (int s = 0; s < nstage; s++) run_stage(acc, cm, s);
     } else {
         for (int s = 0; s < nstage; s += 2) {
             run_stage(acc, cm, s);

@@ -257,13 +257,15 @@ __device__ __forceinline__ void sweep_chunk(const float* xp, const float* wp, in
     }
 }
 
-// The same walk with the chunk's first fragment taken out of the loop and given to `first`, so that it can read
-// its accumulators from one register array and write them to another (the L_inf forward continues the running
-// maximum of the stage before in a second array and would otherwise copy forty registers per chunk).  Byte-address
-// form only.  Fragments 1..14 run as seven trips of two, fragment 15 after the loop.
-template <class GEO, int NX, int KP, class F0, class F>
-__device__ __forceinline__ void sweep_chunk_first(const float* xp, const float* wp, int tx, int ty, F0&& first, F&& f) {
-    static_assert(KP == 2, "sixteen fragments of two k per chunk");
+// The same walk over rows [k_begin, k_begin + LEN) of the chunk (LEN = 32: all of it, 16: one half) with the first
+// fragment taken out of the loop and given to `first`, so that it can read its accumulators from one register array
+// and write them to another (the L_inf forward continues the running maximum of the stage before in a second array
+// and would otherwise copy forty registers per chunk).  Byte-address form only.  The fragments between the first
+// and the last run as trips of two, the last one after the loop.
+template <class GEO, int NX, int KP, int LEN, class F0, class F>
+__device__ __forceinline__ void sweep_chunk_first(const float* xp, const float* wp, int tx, int ty, int k_begin,
+                                                  F0&& first, F&& f) {
+    static_assert(KP == 2 && LEN % 4 == 0 && LEN >= 8, "fragments of two k, trips of two fragments");
     constexpr int FRAG_LDS = NX * KP * (GEO::TM / 4) + KP * (GEO::TN == 8 ? 2 : 1) + (GEO::TN == 5 ? 1 : 0);
     constexpr int WAIT_PREV = 0xc07f | (FRAG_LDS << 8);
     static_assert(FRAG_LDS < 16, "lgkmcnt field");
@@ -271,16 +273,16 @@ __device__ __forceinline__ void sweep_chunk_first(const float* xp, const float* 
     LaneAddr<GEO> cur, nxt;
     const LaneCols<GEO> cols(tx, ty);
     const unsigned xb = lds_address(xp), wb = lds_address(wp);
-    cur.set(xb, wb, 0, cols);
+    cur.set(xb, wb, k_begin, cols);
     __builtin_amdgcn_s_waitcnt(0xc07f);
     read_frag(a, cur, 0);
     read_frag(b, cur, KP);
     __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt(WAIT_PREV);
     __builtin_amdgcn_sched_barrier(0);
-    first(a, 0);
+    first(a, k_begin);
 #pragma unroll 1
-    for (int kk = KP; kk < kChunk - KP; kk += 2 * KP) {   // b holds rows kk, kk + 1 of the chunk
+    for (int kk = k_begin + KP; kk < k_begin + LEN - KP; kk += 2 * KP) {   // b holds rows kk, kk + 1 of the chunk
         nxt.set(xb, wb, kk + KP, cols);
         read_frag(a, nxt, 0);
         __builtin_amdgcn_sched_barrier(0);
@@ -294,7 +296,7 @@ __device__ __forceinline__ void sweep_chunk_first(const float* xp, const float* 
         f(a, kk + KP);
     }
     __builtin_amdgcn_s_waitcnt(0xc07f);
-    f(b, kChunk - KP);
+    f(b, k_begin + LEN - KP);
 }
 
 // Same walk without the operand prefetch, one k row per trip: for rarely taken
