@@ -60,6 +60,31 @@ def test_inf_forward_bit_exact(shape, tile, quant):
     assert torch.equal(pos, ep)
 
 
+@pytest.mark.parametrize("K", [2_000_000, 2_100_000, 2_100_002])
+def test_forward_kernels_with_very_long_rows(K):
+    """The fc panels are read through 32-bit buffer offsets, which cover tile rows of up to 2 GB: 258 rows of
+    K = 2 000 000 floats still fit, K = 2 100 000 does not and takes the path with 64-bit addresses (as does a K
+    that is not a multiple of four).  All three forward kernels, values and indices against the oracle."""
+    from gpu_common import DEV, cpp, gpu_inf_forward, say
+    say("long rows", K)
+    g = torch.Generator().manual_seed(K % 1000)
+    x = torch.rand(3, K, 1, generator=g)
+    w = torch.rand(5, K, generator=g)
+    out, pos = gpu_inf_forward(x, w, 1)
+    eo, ep = oracle.inf_dist_forward(x, w, 1)
+    assert torch.equal(out, eo) and torch.equal(pos, ep)
+    lo, up = x - 0.01, x + 0.02
+    L = torch.empty(3, 5, 1, device=DEV)
+    U = torch.empty(3, 5, 1, device=DEV)
+    cpp.inf_dist_bound_forward(lo.to(DEV), up.to(DEV), w.to(DEV), L, U, 1)
+    eL, eU = oracle.inf_dist_bound_forward(lo, up, w, 1)
+    assert torch.equal(L.cpu(), eL) and torch.equal(U.cpu(), eU)
+    o8 = torch.empty(3, 5, 1, device=DEV)
+    cpp.norm_dist_forward(x.to(DEV), w.to(DEV), o8, 1, 8.0)
+    e8 = oracle.norm_dist_forward(x, w, 1, 8.0)
+    assert torch.allclose(o8.cpu(), e8.float(), rtol=1e-4, atol=ATOL)   # a float32 sum of two million terms
+
+
 # B, CO, CI, G, HW -- unfolded-conv layouts for the kernel that keeps a tile's whole reduction axis in LDS
 SHORTK_SHAPES = [
     (2, 64, 64, 2, 64),       # K = 32: one window per k range
