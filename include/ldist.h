@@ -54,12 +54,14 @@ LDIST_API int ldist_last_hip_error(void);
 
 /* Testing and tuning knob, no counterpart in the reference: forces the workgroup
  * tiling of the three forward kernels.  -1 = choose by shape (default), 0 = 128x80
- * tile with two k-groups, 1 = 128x64, 2 = 256x32, 3 = 32x32 with eight k-groups.
- * 0..3 also keep the L_inf forward of an unfolded-conv layout on the tiled kernels
+ * tile with two k-groups, 1 = 128x64, 2 = 256x32, 3 = 32x32 with eight k-groups,
+ * 4 = 64x80 with two k-groups (two 256-lane workgroups per CU) for the L_inf forward
+ * of a fully connected layer with 128-bit loads, the other kernels choosing by shape.
+ * 0..4 also keep the L_inf forward of an unfolded-conv layout on the tiled kernels
  * where it would otherwise take the kernel that holds a tile's whole reduction axis
  * in LDS (K up to 320), and 0 / 1 force the register-tiled p-norm backward kernels
  * (128x80 / 128x64 tiles), the one-pass kernel of ldist_norm_dist_backward included,
- * 2 / 3 keep them off.  Process-wide; not thread safe. */
+ * 2 / 3 / 4 keep them off.  Process-wide; not thread safe. */
 LDIST_API int ldist_set_tile_override(int choice);
 /* Tuning knob, no counterpart in the reference: 1 (default) orders the tiles of
  * the forward kernels so that each of the 8 XCDs works on one contiguous run of

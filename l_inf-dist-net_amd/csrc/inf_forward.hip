@@ -526,8 +526,22 @@ hipError_t inf_forward(const float* input, const float* weight, float* output, i
     // unfolded-conv layout with a short reduction: the kernel that keeps the whole K of a tile in LDS
     if (g_tile_override < 0 && inf_forward_shortk_applicable(pr, input, output, pos))
         return inf_forward_shortk(input, weight, output, pos, pr, stream);
-    return dispatch_forward<InfForward>(pr, can_vec4(pr, input, weight), can_vec4_out(pr, output, pos), stream, input,
-                                        weight, output, pos);
+    const bool vec4 = can_vec4(pr, input, weight), ovec = can_vec4_out(pr, output, pos);
+    // fc layout: where the 128 x 80 tiles (one 512-lane workgroup per CU) would be chosen, tiles of 64 x 80 with 256
+    // lanes run two workgroups per CU instead.  Same patch per lane, same two waves per SIMD, but the two workgroups
+    // drift apart, so one's epilogue (no arithmetic: merge, argmax search, stores) runs beside the other's k loop.
+    if (pr.HW == 1 && vec4 &&
+        (g_tile_override == 4 ||
+         (g_tile_override < 0 && pr.B > 64 && choose_tile(pr.B, pr.NG, pr.G, pr.num_cu) == TileChoice::M128N80K2))) {
+        using G64 = Geo<64, 80, 8, 5, 2>;
+        Dims d = make_dims(pr);
+        d.ovec = ovec;
+        d.tiles_m = (d.M + G64::BM - 1) / G64::BM;
+        d.tiles_n = (d.NG + G64::BN - 1) / G64::BN;
+        return InfForward<G64, false, 4>::launch((unsigned)d.tiles_m * d.tiles_n * d.G, d, pr.device, stream, input, weight,
+                                                 output, pos);
+    }
+    return dispatch_forward<InfForward>(pr, vec4, ovec, stream, input, weight, output, pos);
 }
 
 }  // namespace ldist

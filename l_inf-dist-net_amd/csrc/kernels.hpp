@@ -26,6 +26,8 @@ enum class TileChoice { M128N80K2, M128N64K1, M256N32K1, M32N32K8 };
 // it makes 80 times more workgroups than the big tiles, at twice their LDS traffic per difference.
 // -1 = choose by shape; 0, 1, 2, 3 force M128N80K2, M128N64K1, M256N32K1, M32N32K8 (tests and tuning), which also
 // keeps the L_inf forward of the unfolded-conv layout on the tiled kernels instead of the short-reduction kernel.
+// 4 forces the 64 x 80 tiles that the L_inf forward of a fully connected layer runs two workgroups per CU with
+// (inf_forward.hip; by itself it takes them where M128N80K2 would be chosen) and leaves every other kernel's choice alone.
 extern int g_tile_override;
 extern int g_xcd_remap;  // 1 (default): XCD-aware tile order; 0: plain order (tuning)
 

@@ -47,7 +47,7 @@ def test_version_and_error_strings(lib):
     assert lib.ldist_version() == 100
     for code in (0, -1, -2, -3, -4, -5, -99):
         assert isinstance(lib.ldist_strerror(code), bytes) and lib.ldist_strerror(code)
-    assert lib.ldist_set_tile_override(7) == -1 and lib.ldist_set_tile_override(3) == 0 and lib.ldist_set_tile_override(-1) == 0
+    assert lib.ldist_set_tile_override(7) == -1 and lib.ldist_set_tile_override(4) == 0 and lib.ldist_set_tile_override(-1) == 0
 
 
 def test_argument_checks_need_no_device(lib):

@@ -33,7 +33,7 @@ SHAPES = [
     (4, 128, 1152, 4, 100),   # the unfolded 3x3 conv layer shape at a small image
     (1, 40, 2000, 1, 36),     # conv layout, long K
 ]
-TILES = [-1, 0, 1, 2, 3]
+TILES = [-1, 0, 1, 2, 3, 4]
 
 
 @pytest.fixture(autouse=True)

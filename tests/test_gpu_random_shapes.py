@@ -28,7 +28,7 @@ def draw(seed):
     HW = r.choice([1, 1, 1, 2, 5, 16, 36, 49])
     budget = 6_000_000 // (NG * K * HW)
     B = max(1, min(r.choice([1, 2, 3, 17, 64, 129, 200]), budget))
-    return B, NG * G, K * G, G, HW, r.choice([-1, 0, 1, 2, 3]), r.choice(EXPONENTS)
+    return B, NG * G, K * G, G, HW, r.choice([-1, 0, 1, 2, 3, 4]), r.choice(EXPONENTS)
 
 
 @pytest.fixture(autouse=True)
