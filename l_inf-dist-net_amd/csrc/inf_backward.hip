@@ -5,10 +5,15 @@
 //   grad_input [b, g*K + idx, hw] += (pos >= 0 ? g : -g)
 //   grad_weight[g*NG + n, idx]    += (pos <  0 ? g : -g)
 // The reference issues one global atomic per (m,n).  Here every workgroup owns a
-// slab of the gradient, gathers its contributions in LDS bins (ds_add_f32) and
-// writes the slab out with coalesced stores, so the pass is bounded by streaming
-// grad_output/pos in and the gradient out.  In "overwrite" mode the slab is
-// stored whole (zeros included), which replaces the caller's zero fill.
+// slab of the gradient, gathers its contributions in LDS bins and writes the slab
+// out with coalesced stores, so the pass is bounded by streaming grad_output/pos
+// in and the gradient out.  In "overwrite" mode the slab is stored whole (zeros
+// included), which replaces the caller's zero fill.
+// The bins of grad_input (and of grad_weight in the conv layout) are doubles: on gfx950 an LDS atomic add of a
+// double (ds_add_f64) retires about nine times as many lanes per clock as one of a float (ds_add_f32: 0.33 lanes
+// per clock and CU, measured on random addresses; 2.9 for doubles, 6 for 32-bit integer adds), and the binning was
+// what those kernels waited for.  A bin's sum is rounded to float once, when the slab is written: exact where an
+// element receives one contribution, otherwise at least as close to the true sum as any order of float additions.
 #include "kernels.hpp"
 
 namespace ldist {
@@ -24,7 +29,7 @@ template <bool OVERWRITE>
 __global__ void __launch_bounds__(1024)
 inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* __restrict__ pos,
                           float* __restrict__ grad_input, BwdDims d, int th_log2, int KC, int hw_tiles, int vec) {
-    extern __shared__ __align__(16) float bins[];
+    extern __shared__ __align__(16) double bins[];
     const int NT = blockDim.x;
     const int TH = 1 << th_log2;
     const int tile = blockIdx.x % hw_tiles;
@@ -40,8 +45,8 @@ inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* 
         // fc layout (TH == 1) with NG, K, kc multiples of 4 and 16-byte aligned tensors: the rows of
         // pos / grad_output and the slab of grad_input are contiguous, so everything moves 128 bits
         // at a time; the loads of a lane's four elements are in flight together.
-        float4* b4 = reinterpret_cast<float4*>(bins);
-        for (int e = threadIdx.x; e < kc / 4; e += NT) b4[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+        double2* b2 = reinterpret_cast<double2*>(bins);
+        for (int e = threadIdx.x; e < kc / 2; e += NT) b2[e] = make_double2(0.0, 0.0);
         __syncthreads();
         const int4* p4 = reinterpret_cast<const int4*>(pos + obase);
         const float4* g4 = reinterpret_cast<const float4*>(grad_output + obase);
@@ -53,13 +58,14 @@ inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* 
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 const int idx = (ps[q] & 0x7fffffff) - k0;
-                if (idx >= 0 && idx < kc) atomicAdd(&bins[idx], ps[q] >= 0 ? gs[q] : -gs[q]);
+                if (idx >= 0 && idx < kc) atomicAdd(&bins[idx], (double)(ps[q] >= 0 ? gs[q] : -gs[q]));
             }
         }
         __syncthreads();
         float4* dst = reinterpret_cast<float4*>(grad_input + xbase);
         for (int e = threadIdx.x; e < kc / 4; e += NT) {
-            const float4 v = b4[e];
+            const double2 lo = b2[2 * e], hi = b2[2 * e + 1];
+            const float4 v = make_float4((float)lo.x, (float)lo.y, (float)hi.x, (float)hi.y);
             if (OVERWRITE) {
                 dst[e] = v;
             } else if (v.x != 0.f || v.y != 0.f || v.z != 0.f || v.w != 0.f) {
@@ -77,8 +83,8 @@ inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* 
                       ((reinterpret_cast<uintptr_t>(grad_output) | reinterpret_cast<uintptr_t>(pos) |
                         reinterpret_cast<uintptr_t>(grad_input)) & 15u) == 0;
     if (quad) {
-        float4* b4 = reinterpret_cast<float4*>(bins);
-        for (int e = threadIdx.x; e < nb / 4; e += NT) b4[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+        double2* b2 = reinterpret_cast<double2*>(bins);
+        for (int e = threadIdx.x; e < nb / 2; e += NT) b2[e] = make_double2(0.0, 0.0);
         __syncthreads();
         const int tq_log2 = th_log2 - 2;                 // quads per tile row
         const int total_q = d.NG << tq_log2;
@@ -94,7 +100,7 @@ inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* 
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
                     const int idx = (ps[q] & 0x7fffffff) - k0;
-                    if (idx >= 0 && idx < kc) atomicAdd(&bins[(idx << th_log2) + j + q], ps[q] >= 0 ? gs[q] : -gs[q]);
+                    if (idx >= 0 && idx < kc) atomicAdd(&bins[(idx << th_log2) + j + q], (double)(ps[q] >= 0 ? gs[q] : -gs[q]));
                 }
             }
         }
@@ -104,7 +110,8 @@ inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* 
             const int hw = hw0 + j;
             if (hw < d.HW) {
                 float4* dst = reinterpret_cast<float4*>(grad_input + xbase + (size_t)k * d.HW + hw);
-                const float4 v = b4[e];
+                const double2 lo = b2[2 * e], hi = b2[2 * e + 1];
+                const float4 v = make_float4((float)lo.x, (float)lo.y, (float)hi.x, (float)hi.y);
                 if (OVERWRITE) {
                     *dst = v;
                 } else if (v.x != 0.f || v.y != 0.f || v.z != 0.f || v.w != 0.f) {
@@ -117,7 +124,7 @@ inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* 
         return;
     }
 
-    for (int e = threadIdx.x; e < nb; e += NT) bins[e] = 0.f;
+    for (int e = threadIdx.x; e < nb; e += NT) bins[e] = 0.0;
     __syncthreads();
 
     const int total = d.NG * TH;
@@ -130,7 +137,7 @@ inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* 
             const int idx = (p & 0x7fffffff) - k0;
             if (idx >= 0 && idx < kc) {
                 const float gv = grad_output[o];
-                atomicAdd(&bins[(idx << th_log2) + j], p >= 0 ? gv : -gv);
+                atomicAdd(&bins[(idx << th_log2) + j], (double)(p >= 0 ? gv : -gv));
             }
         }
     }
@@ -141,7 +148,7 @@ inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* 
         const int hw = hw0 + j;
         if (hw < d.HW) {
             float* dst = grad_input + xbase + (size_t)k * d.HW + hw;
-            const float v = bins[e];
+            const float v = (float)bins[e];
             if (OVERWRITE) *dst = v;
             else if (v != 0.f) *dst += v;
         }
@@ -155,11 +162,17 @@ inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* 
 // When the images are split over several workgroups (SPLIT) the bins are added
 // to grad_weight with global atomics, otherwise the workgroup is the only
 // writer of its slab.
-template <bool OVERWRITE, bool SPLIT>
+// BIN: float bins in the fc layout (a row of bins receives at most one contribution per image, and what the kernel
+// waits for are its strided reads of grad_output / pos columns: twice the rows per workgroup count for more than
+// faster atomics), double bins otherwise (B * HW contributions per row: 131 072 in a 3x3 conv layer of 32 x 32
+// images at batch 128, where the float atomics took three times as long as everything else).
+template <bool OVERWRITE, bool SPLIT, class BIN>
 __global__ void __launch_bounds__(256)
 inf_backward_weight_kernel(const float* __restrict__ grad_output, const int32_t* __restrict__ pos,
                            float* __restrict__ grad_weight, BwdDims d, int NB, int KC, int n_blocks, int b_per_wg) {
-    extern __shared__ float bins[];
+    extern __shared__ __align__(16) unsigned char bin_bytes[];
+    BIN* bins = reinterpret_cast<BIN*>(bin_bytes);
+    constexpr int NT = 256;
     // Neighbouring blocks of outputs read neighbouring few-byte pieces of the same memory lines (in the fc layout a
     // block's grad_output / pos entries of one image are NB * 4 bytes).  Workgroups go to the eight XCDs in turn, each
     // with its own L2, so XCD x takes the x-th eighth of the blocks: neighbours then share the lines in one L2
@@ -177,11 +190,11 @@ inf_backward_weight_kernel(const float* __restrict__ grad_output, const int32_t*
     const int b1 = min(d.B, b0 + b_per_wg);
     // kc is a multiple of 4 whenever vec is set, so rows of bins and of grad_weight stay 16-byte aligned
     const bool vec = (kc & 3) == 0 && (d.K & 3) == 0 && (reinterpret_cast<uintptr_t>(grad_weight) & 15u) == 0;
-    if (vec) {
+    if (vec) {   // 16 bytes of bins per store
         float4* b4 = reinterpret_cast<float4*>(bins);
-        for (int e = threadIdx.x; e < nb * kc / 4; e += 256) b4[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int e = threadIdx.x; e < nb * kc * (int)sizeof(BIN) / 16; e += NT) b4[e] = make_float4(0.f, 0.f, 0.f, 0.f);
     } else {
-        for (int e = threadIdx.x; e < nb * kc; e += 256) bins[e] = 0.f;
+        for (int e = threadIdx.x; e < nb * kc; e += NT) bins[e] = (BIN)0;
     }
     __syncthreads();
 
@@ -193,12 +206,12 @@ inf_backward_weight_kernel(const float* __restrict__ grad_output, const int32_t*
         // index and gradient of four elements are fetched together: one after the other (the gradient only once the
         // index says it is wanted) a wave waited out two memory latencies per element
         const int total = (b1 - b0) * nb;
-        for (int i0 = threadIdx.x; i0 < total; i0 += 1024) {
+        for (int i0 = threadIdx.x; i0 < total; i0 += 4 * NT) {
             int p[4], nn[4];
             float gv[4];
 #pragma unroll
             for (int u = 0; u < 4; u++) {
-                const int i = i0 + 256 * u < total ? i0 + 256 * u : i0;   // past the end: the first one again, not added
+                const int i = i0 + NT * u < total ? i0 + NT * u : i0;   // past the end: the first one again, not added
                 const int bb = i / nb;
                 nn[u] = i - bb * nb;
                 const size_t o = (size_t)(b0 + bb) * img_stride + first + nn[u];
@@ -208,14 +221,14 @@ inf_backward_weight_kernel(const float* __restrict__ grad_output, const int32_t*
 #pragma unroll
             for (int u = 0; u < 4; u++) {
                 const int idx = (p[u] & 0x7fffffff) - k0;
-                if ((u == 0 || i0 + 256 * u < total) && idx >= 0 && idx < kc)
-                    atomicAdd(&bins[nn[u] * kc + idx], p[u] < 0 ? gv[u] : -gv[u]);
+                if ((u == 0 || i0 + NT * u < total) && idx >= 0 && idx < kc)
+                    atomicAdd(&bins[nn[u] * kc + idx], (BIN)(p[u] < 0 ? gv[u] : -gv[u]));
             }
         }
     } else {
         auto add = [&](int p, float gv, int nn) {
             const int idx = (p & 0x7fffffff) - k0;
-            if (idx >= 0 && idx < kc) atomicAdd(&bins[nn * kc + idx], p < 0 ? gv : -gv);
+            if (idx >= 0 && idx < kc) atomicAdd(&bins[nn * kc + idx], (BIN)(p < 0 ? gv : -gv));
         };
         // HW % 4 == 0 and aligned tensors: four positions per lane with 128-bit loads and two such groups in
         // flight (one position per trip, the index first and the gradient after it, left a wave waiting out two
@@ -227,8 +240,8 @@ inf_backward_weight_kernel(const float* __restrict__ grad_output, const int32_t*
                 const int4* pq = reinterpret_cast<const int4*>(pos + base);
                 const float4* gq = reinterpret_cast<const float4*>(grad_output + base);
                 const int quads = run / 4, hwq = d.HW / 4;
-                for (int q0 = threadIdx.x; q0 < quads; q0 += 512) {
-                    const int q1 = q0 + 256 < quads ? q0 + 256 : q0;
+                for (int q0 = threadIdx.x; q0 < quads; q0 += 2 * NT) {
+                    const int q1 = q0 + NT < quads ? q0 + NT : q0;
                     const int4 pa = pq[q0], pb = pq[q1];
                     const float4 ga = gq[q0], gb = gq[q1];
                     const int na = q0 / hwq;
@@ -239,7 +252,7 @@ inf_backward_weight_kernel(const float* __restrict__ grad_output, const int32_t*
                     }
                 }
             } else {
-                for (int e = threadIdx.x; e < run; e += 256) add(pos[base + e], grad_output[base + e], e / d.HW);
+                for (int e = threadIdx.x; e < run; e += NT) add(pos[base + e], grad_output[base + e], e / d.HW);
             }
         }
     }
@@ -247,18 +260,18 @@ inf_backward_weight_kernel(const float* __restrict__ grad_output, const int32_t*
 
     if (vec && OVERWRITE && !SPLIT) {
         const int kc4 = kc / 4;
-        const float4* b4 = reinterpret_cast<const float4*>(bins);
-        for (int e = threadIdx.x; e < nb * kc4; e += 256) {
+        for (int e = threadIdx.x; e < nb * kc4; e += NT) {
             const int nn = e / kc4, k4 = e - nn * kc4;
             float* dst = grad_weight + ((size_t)g * d.NG + n0 + nn) * d.K + k0 + k4 * 4;
-            *reinterpret_cast<float4*>(dst) = b4[e];
+            const BIN* b = bins + 4 * e;   // nn * kc + 4 * k4, kc a multiple of four
+            *reinterpret_cast<float4*>(dst) = make_float4((float)b[0], (float)b[1], (float)b[2], (float)b[3]);
         }
         return;
     }
-    for (int e = threadIdx.x; e < nb * kc; e += 256) {
+    for (int e = threadIdx.x; e < nb * kc; e += NT) {
         const int nn = e / kc, k = e - nn * kc;
         float* dst = grad_weight + ((size_t)g * d.NG + n0 + nn) * d.K + k0 + k;
-        const float v = bins[e];
+        const float v = (float)bins[e];
         if (SPLIT) {
             if (v != 0.f) atomicAdd(dst, v);
         } else if (OVERWRITE) {
@@ -280,19 +293,20 @@ __global__ void __launch_bounds__(256) fill_zero_kernel(float* __restrict__ p, s
     }
 }
 
-static constexpr int kBinFloats = 16384;  // 64 KB of LDS bins per workgroup
+static constexpr int kBinBytes = 64 * 1024;                           // LDS bins per workgroup
+static constexpr int kInputBins = kBinBytes / (int)sizeof(double);
 
 hipError_t inf_backward_input(const float* grad_output, const int32_t* pos, float* grad_input, const Problem& pr,
                               bool overwrite, hipStream_t stream) {
     const BwdDims d{pr.B, pr.G, pr.K, pr.NG, pr.HW};
     // widest hw tile (power of two, at most 64) whose bins still cover all K channels in one pass
     int th_log2 = 0;
-    while ((2 << th_log2) <= pr.HW && (2 << th_log2) <= 64 && (size_t)(2 << th_log2) * pr.K <= kBinFloats) th_log2++;
+    while ((2 << th_log2) <= pr.HW && (2 << th_log2) <= 64 && (size_t)(2 << th_log2) * pr.K <= kInputBins) th_log2++;
     const int TH = 1 << th_log2;
-    const int KC = min(pr.K, kBinFloats / TH);
+    const int KC = min(pr.K, kInputBins / TH);
     const int hw_tiles = (pr.HW + TH - 1) / TH;
     const dim3 grid((unsigned)pr.B * pr.G * hw_tiles, (unsigned)((pr.K + KC - 1) / KC));
-    const size_t lds = (size_t)KC * TH * sizeof(float);
+    const size_t lds = (size_t)KC * TH * sizeof(double);
     // fc layout, everything a multiple of four floats and 16-byte aligned: 128-bit path
     const int vec = pr.HW == 1 && pr.NG % 4 == 0 && pr.K % 4 == 0 && KC % 4 == 0 && aligned16(grad_output) &&
                     aligned16(pos) && aligned16(grad_input);
@@ -311,13 +325,22 @@ hipError_t inf_backward_input(const float* grad_output, const int32_t* pos, floa
     return hipGetLastError();
 }
 
+template <bool OVERWRITE, bool SPLIT, class BIN>
+static void launch_backward_weight(dim3 grid, size_t lds, hipStream_t stream, const float* grad_output, const int32_t* pos,
+                                   float* grad_weight, const BwdDims& d, int NB, int KC, int n_blocks, int b_per_wg) {
+    hipLaunchKernelGGL((inf_backward_weight_kernel<OVERWRITE, SPLIT, BIN>), grid, dim3(256), lds, stream, grad_output, pos,
+                       grad_weight, d, NB, KC, n_blocks, b_per_wg);
+}
+
 hipError_t inf_backward_weight(const float* grad_output, const int32_t* pos, float* grad_weight, const Problem& pr,
                                bool overwrite, hipStream_t stream) {
     const BwdDims d{pr.B, pr.G, pr.K, pr.NG, pr.HW};
+    const bool wide = pr.HW > 1;   // double bins, see the kernel
+    const int slots = kBinBytes / (wide ? (int)sizeof(double) : (int)sizeof(float));
     // One pass over all K channels per workgroup when a row of bins fits: re-reading the strided
     // grad_output/pos columns for every channel range costs more than the smaller row block.
-    const int KC = min(pr.K, kBinFloats);
-    const int NB = max(1, min(min(pr.NG, 8), kBinFloats / KC));
+    const int KC = min(pr.K, slots);
+    const int NB = max(1, min(min(pr.NG, 8), slots / KC));
     const int real_blocks = (pr.NG + NB - 1) / NB;
     // many blocks: a multiple of eight, for the kernel's XCD-aware block order (the extra workgroups leave at once)
     const int n_blocks = real_blocks >= 64 ? (real_blocks + 7) / 8 * 8 : real_blocks;
@@ -334,22 +357,27 @@ hipError_t inf_backward_weight(const float* grad_output, const int32_t* pos, flo
     const int b_per_wg = (pr.B + splits - 1) / splits;
     splits = (pr.B + b_per_wg - 1) / b_per_wg;
     const dim3 grid((unsigned)(pr.G * n_blocks), (unsigned)k_ranges, (unsigned)splits);
-    const size_t lds = (size_t)NB * KC * sizeof(float);
+    const size_t lds = (size_t)NB * KC * (wide ? sizeof(double) : sizeof(float));
+#define LDIST_BWD_W(OVER, SPLIT)                                                                                        \
+    do {                                                                                                                \
+        if (wide) launch_backward_weight<OVER, SPLIT, double>(grid, lds, stream, grad_output, pos, grad_weight, d, NB, KC, \
+                                                              n_blocks, b_per_wg);                                      \
+        else launch_backward_weight<OVER, SPLIT, float>(grid, lds, stream, grad_output, pos, grad_weight, d, NB, KC,     \
+                                                        n_blocks, b_per_wg);                                            \
+    } while (0)
     if (splits > 1) {
         if (overwrite) {
             const size_t n = (size_t)pr.G * pr.NG * pr.K;
             const unsigned blocks = (unsigned)min((size_t)4096, (n + 1023) / 1024);
             hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, stream, grad_weight, n);
         }
-        hipLaunchKernelGGL((inf_backward_weight_kernel<false, true>), grid, dim3(256), lds, stream, grad_output, pos,
-                           grad_weight, d, NB, KC, n_blocks, b_per_wg);
+        LDIST_BWD_W(false, true);
     } else if (overwrite) {
-        hipLaunchKernelGGL((inf_backward_weight_kernel<true, false>), grid, dim3(256), lds, stream, grad_output, pos,
-                           grad_weight, d, NB, KC, n_blocks, b_per_wg);
+        LDIST_BWD_W(true, false);
     } else {
-        hipLaunchKernelGGL((inf_backward_weight_kernel<false, false>), grid, dim3(256), lds, stream, grad_output,
-                           pos, grad_weight, d, NB, KC, n_blocks, b_per_wg);
+        LDIST_BWD_W(false, false);
     }
+#undef LDIST_BWD_W
     return hipGetLastError();
 }
 
