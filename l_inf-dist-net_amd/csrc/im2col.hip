@@ -130,7 +130,7 @@ __global__ void __launch_bounds__(256)
 inf_backward_input_folded_kernel(const float* __restrict__ grad_output, const int32_t* __restrict__ pos,
                                  float* __restrict__ grad_img, ConvGeom q, int G, int NG, int R, int row_tiles, int vec, int vec_img,
                                  SmallDiv by_khw, SmallDiv by_kw, SmallDiv by_wo) {
-    extern __shared__ __align__(16) float bins[];
+    extern __shared__ __align__(16) double bins[];   // doubles: their LDS atomic add retires nine times the lanes of the float one
     const int CG = q.C / G;
     const int tile = blockIdx.x % row_tiles;
     const int bg = blockIdx.x / row_tiles;          // b * G + g
@@ -139,9 +139,9 @@ inf_backward_input_folded_kernel(const float* __restrict__ grad_output, const in
     const int rows = min(R, q.H - y0);
     const int nb = CG * rows * q.W;
     if (vec_img) {                                    // W % 4 == 0: nb is a multiple of four
-        for (int e = threadIdx.x * 4; e < nb; e += 1024) *reinterpret_cast<float4*>(bins + e) = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int e = threadIdx.x * 2; e < nb; e += 512) *reinterpret_cast<double2*>(bins + e) = make_double2(0.0, 0.0);
     } else {
-        for (int e = threadIdx.x; e < nb; e += 256) bins[e] = 0.f;
+        for (int e = threadIdx.x; e < nb; e += 256) bins[e] = 0.0;
     }
     __syncthreads();
 
@@ -162,7 +162,7 @@ inf_backward_input_folded_kernel(const float* __restrict__ grad_output, const in
             const int h = h_lo + th, w = t - th * q.WO;
             const int y = h * q.S + i * q.D - q.P - y0, x = w * q.S + j * q.D - q.P;
             if ((unsigned)y < (unsigned)rows && (unsigned)x < (unsigned)q.W && c < CG)
-                atomicAdd(&bins[(c * rows + y) * q.W + x], p >= 0 ? gv : -gv);
+                atomicAdd(&bins[(c * rows + y) * q.W + x], (double)(p >= 0 ? gv : -gv));
         };
         // lanes run along the positions of one output channel, channels are shared out over the waves
         if (vec) {
@@ -200,13 +200,14 @@ inf_backward_input_folded_kernel(const float* __restrict__ grad_output, const in
     if (vec_img) {
         for (int e = threadIdx.x * 4; e < nb; e += 1024) {
             const int c = e / per_c, rest = e - c * per_c;
+            const double2 lo = *reinterpret_cast<const double2*>(bins + e), hi = *reinterpret_cast<const double2*>(bins + e + 2);
             *reinterpret_cast<float4*>(grad_img + (((size_t)b * q.C + (size_t)g * CG + c) * q.H + y0) * q.W + rest) =
-                *reinterpret_cast<const float4*>(bins + e);
+                make_float4((float)lo.x, (float)lo.y, (float)hi.x, (float)hi.y);
         }
     } else {
         for (int e = threadIdx.x; e < nb; e += 256) {
             const int c = e / per_c, rest = e - c * per_c;
-            grad_img[(((size_t)b * q.C + (size_t)g * CG + c) * q.H + y0) * q.W + rest] = bins[e];
+            grad_img[(((size_t)b * q.C + (size_t)g * CG + c) * q.H + y0) * q.W + rest] = (float)bins[e];
         }
     }
 }
@@ -248,14 +249,18 @@ hipError_t fold(const float* gcols, float* gimg, const ConvGeom& q, hipStream_t 
 hipError_t inf_backward_input_folded(const float* grad_output, const int32_t* pos, float* grad_img, const ConvGeom& q,
                                      int G, int CO, hipStream_t stream) {
     const int CG = q.C / G, NG = CO / G;
-    // as many image rows per workgroup as 32 KB of bins hold (four workgroups per CU: their zeroing, scanning
-    // and write-out phases overlap); a single row may take up to 64 KB
+    // as many image rows per workgroup as 64 KB of bins (doubles) hold (two workgroups per CU: their zeroing,
+    // scanning and write-out phases overlap); a single row may take up to 128 KB
     if ((long long)CG * q.W > 16384) return hipErrorInvalidValue;          // the API layer screens this out
     int R = (int)(8192 / ((long long)CG * q.W));
     if (R < 1) R = 1;
     if (R > q.H) R = q.H;
     const int row_tiles = (q.H + R - 1) / R;
-    const size_t lds = (size_t)CG * R * q.W * sizeof(float);
+    const size_t lds = (size_t)CG * R * q.W * sizeof(double);
+    static LdsRecord lds_allowed = {};
+    int device = 0;
+    if (hipError_t e = hipGetDevice(&device); e != hipSuccess) return e;
+    if (hipError_t e = allow_lds(inf_backward_input_folded_kernel, 128 * 1024, device, lds_allowed); e != hipSuccess) return e;
     // 128-bit loads of four neighbouring positions: every run of output rows starts on a multiple of four
     const int vec = q.WO % 4 == 0 && aligned16(grad_output) && aligned16(pos);
     const int vec_img = q.W % 4 == 0 && aligned16(grad_img);   // the slab of a channel starts and ends on multiples of four
