@@ -65,17 +65,31 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
         }
     }
     float* const gw_group = grad_weight + (size_t)g * NG * K;
-    // Adds the lane's column sums of output n (already summed over its rows) over the 16 lanes of the row and
-    // onto grad_weight; the sign: d/dw of |x - w| is minus d/dx.
-    auto add_weight_row = [&](int n, const float (&s)[TN]) {
+    // The lane's column sums of output n (already summed over its rows) are summed over the 16 lanes of the row and
+    // parked in an LDS tile [stage's outputs][BN columns]; the sign: d/dw of |x - w| is minus d/dx.  The tile goes
+    // onto grad_weight once per stage (flush_weight_tile): straight from here an atomic instruction had four active
+    // lanes (the last lane of each row of sixteen), and the float atomics of a 5120-wide layer, 105 M in 26 M
+    // instructions, took 1.7 ms of the launch's 4.2.
+    float* const Gs = lds + 2 * XS + GEO::WS;   // [KK][BN], all zero between stages
+    auto add_weight_row = [&](int n_local, const float (&s)[TN]) {
         float tot[TN];
 #pragma unroll
         for (int j = 0; j < TN; j++) tot[j] = dpp_row_total(s[j]);
-        if (ty == GEO::TY - 1 && n < NG) {
-            float* row = gw_group + (size_t)n * K;
+        if (ty == GEO::TY - 1) {
 #pragma unroll
-            for (int j = 0; j < TN; j++)
-                if (wcol[j] >= 0) atomicAdd(row + wcol[j], -tot[j]);
+            for (int j = 0; j < TN; j++) Gs[n_local * BN + GEO::col(tx, j)] = -tot[j];
+        }
+    };
+    // All lanes of the workgroup: 64 consecutive columns of one output per wave instruction; a parked zero (nothing
+    // added: padding, or a row the large-exponent path passed over) costs no atomic.  Leaves the tile zero.
+    auto flush_weight_tile = [&](int n_first) {
+        for (int i = tid; i < KK * BN; i += GEO::NT) {
+            const float v = Gs[i];
+            if (v != 0.f) {
+                Gs[i] = 0.f;
+                const int nl = i / BN, c = i - nl * BN;
+                if (n_first + nl < NG && k0 + c < K) atomicAdd(gw_group + (size_t)(n_first + nl) * K + k0 + c, v);
+            }
         }
     };
 
@@ -112,6 +126,7 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
     const bool sparse = e >= 63.0f && K >= 1024;
     const float cut = __builtin_exp2f(-36.0f / e);
     const int nstage = (NG + KK - 1) / KK;
+    for (int i = tid; i < KK * BN; i += GEO::NT) Gs[i] = 0.f;
     load(0);
     convert();
     store();
@@ -120,7 +135,6 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
         if (s + 1 < nstage) load((s + 1) * KK);
         const float* fp = lds + grp * kChunk * GEO::SM;
         const float* wp = lds + 2 * XS + grp * kChunk * GEO::SN;
-        const int n_chunk = s * KK + grp * kChunk;
         // No operand prefetch: a second fragment in flight does not fit next to the patch, the sums and the weight
         // row's partial sums (it spills, and measured 15 % slower); the LDS latency of a row hides behind the forty
         // logarithms and exponentials of the other wave on the SIMD.
@@ -155,7 +169,7 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
                         sum[j] = __builtin_fmaf(f.x[0][0][i], sp, sum[j]);
                     }
                 }
-                add_weight_row(n_chunk + kk, sum);
+                add_weight_row(grp * kChunk + kk, sum);
             });
         } else {
             sweep_chunk_plain<GEO, 2>(fp, wp, tx, ty, [&](const Frag<GEO, 2, 1>& f, int kk) {
@@ -170,10 +184,11 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
                         acc[i][j] = __builtin_fmaf(f.x[0][0][i], sp, acc[i][j]);   // two fused multiply-adds, not a
                         sum[j] = __builtin_fmaf(f.x[0][0][i], sp, sum[j]);         // shared product and two additions
                     }
-                add_weight_row(n_chunk + kk, sum);
+                add_weight_row(grp * kChunk + kk, sum);
             });
         }
-        __syncthreads();   // everyone is done reading the panels
+        __syncthreads();   // everyone is done reading the panels; the stage's grad_weight tile is complete
+        flush_weight_tile(s * KK);
         if (s + 1 < nstage) {
             convert();
             store();
@@ -215,7 +230,7 @@ static hipError_t launch_fused(const Problem& pr, hipStream_t stream, const floa
     d.tiles_m = (d.M + GEO::BM - 1) / GEO::BM;
     d.tiles_n = (d.K + GEO::BN - 1) / GEO::BN;
     const unsigned grid = (unsigned)d.tiles_m * d.tiles_n * d.G;
-    constexpr size_t lds = (size_t)(2 * GEO::XS + GEO::WS) * sizeof(float);
+    constexpr size_t lds = (size_t)(2 * GEO::XS + GEO::WS + GEO::KK * GEO::BN) * sizeof(float);   // panels, grad_weight tile
     auto kern = norm_backward_fused_kernel<GEO>;
     static LdsRecord lds_allowed = {};
     if (hipError_t e = allow_lds(kern, lds, pr.device, lds_allowed); e != hipSuccess) return e;
