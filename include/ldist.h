@@ -78,6 +78,15 @@ LDIST_API int ldist_set_xcd_remap(int on);
 LDIST_API int ldist_inf_dist_forward(const float* input, const float* weight, int B, int CO, int CI, int G, int HW,
                            float* output, int32_t* pos, ldist_stream_t stream);
 
+/* L_inf forward without pos: output as ldist_inf_dist_forward writes it, bit for bit.  No counterpart in the
+ * reference, whose forward always computes pos (model/norm_dist.py:14-15); for forward passes that no gradient
+ * follows (evaluation, the value path of a certification pass), which then skip the index bookkeeping and the
+ * search for the lowest k.  Covers the fc layout (HW == 1) with more than 16 outputs per group, K a multiple of
+ * four and 16-byte aligned tensors; LDIST_EUNSUPPORTED for the rest (nothing is enqueued: call
+ * ldist_inf_dist_forward). */
+LDIST_API int ldist_inf_dist_forward_values(const float* input, const float* weight, int B, int CO, int CI, int G, int HW,
+                                  float* output, ldist_stream_t stream);
+
 /* Interval-bound forward.  Replaces inf_dist_bound_forward_cuda
  * (model/norm_dist.cpp:15-16, model/inf_dist_cuda.cu:181-188).
  *   output_upper = max_k max(|l-w|, |u-w|)

@@ -19,6 +19,7 @@ _d = ctypes.c_double
 # name -> argument types, in the order of include/ldist.h
 SIGNATURES = {
     "ldist_inf_dist_forward": [_F, _F, _i, _i, _i, _i, _i, _F, _I, _S],
+    "ldist_inf_dist_forward_values": [_F, _F, _i, _i, _i, _i, _i, _F, _S],
     "ldist_inf_dist_bound_forward": [_F, _F, _F, _i, _i, _i, _i, _i, _F, _F, _S],
     "ldist_inf_dist_value_bound_forward": [_F, _F, _F, _F, _i, _i, _i, _i, _i, _F, _F, _F, _F, _F, _S],
     "ldist_inf_dist_backward_input": [_F, _I, _i, _i, _i, _i, _i, _F, _S],
@@ -79,6 +80,9 @@ def lib():
         handle.ldist_last_hip_error.restype = ctypes.c_int
         _lib = handle
     return _lib
+
+
+EUNSUPPORTED = -5   # LDIST_EUNSUPPORTED of include/ldist.h: a specialised entry point does not cover the problem
 
 
 def check(rc, name):

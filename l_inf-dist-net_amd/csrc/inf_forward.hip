@@ -411,6 +411,121 @@ struct InfForward {
 };
 
 // ---------------------------------------------------------------------------
+// Values only (no pos): what a forward pass that no gradient will follow needs -- evaluation, and the value path of
+// a certification pass.  The reference always computes pos (model/norm_dist.py:14-15, inf_dist_cuda.cu:36-43); without
+// it the loop is one v_sub_f32 and half a v_max3_f32 per (row, output, input) and nothing else: no second register
+// array, no chunk records, and no search after the loop (which is a twelfth of the full kernel's launch at K = 5120
+// and a third at K = 784).  The k-groups meet in LDS and the first writes the tile.  Same subtractions and maxima
+// of the same numbers: the values are those of inf_forward_kernel bit for bit.  fc layout with 128-bit loads.
+// ---------------------------------------------------------------------------
+template <class GEO>
+__global__ void __launch_bounds__(GEO::NT, 2)
+inf_forward_values_kernel(const float* __restrict__ input, const float* __restrict__ weight, float* __restrict__ output,
+                          Dims d) {
+    constexpr int BM = GEO::BM, BN = GEO::BN, TM = GEO::TM, TN = GEO::TN, KS = GEO::KS, KK = GEO::KK;
+    constexpr int NGRP = GEO::NGRP;
+    using Stage = Stager<GEO, false, 4, 1>;
+    constexpr int STAGE = Stage::STAGE, NBUF = Stage::NBUF;
+    static_assert((KS - 1) * TM * TN * NGRP <= NBUF * STAGE, "merge area fits in the panels");
+    extern __shared__ __align__(16) float lds[];
+
+    int tm, tn, g;
+    tile_of_block(d, tm, tn, g);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int tid = threadIdx.x;
+    const int grp = tid / NGRP, t = tid % NGRP;
+    const int tx = t % GEO::TX, ty = t / GEO::TX;
+
+    Stage st;
+    const float* const ins[1] = {input};
+    st.init(ins, weight, d, m0, n0, g, tid);
+    float acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = 0.f;
+
+    const int nstage = (d.K + KK - 1) / KK;
+    st.load(0);
+    st.store(lds);
+    __syncthreads();
+    for (int s = 0; s < nstage; s++) {
+        const float* stage = lds + (s % NBUF) * STAGE;
+        if (s + 1 < nstage) st.load((s + 1) * KK);
+        sweep_chunk<GEO, 1, 2, true>(stage + grp * kChunk * GEO::SM, stage + GEO::XS + grp * kChunk * GEO::SN, tx, ty,
+                                     [&](const Frag<GEO, 1, 2>& f, int) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    const float d0 = __builtin_fabsf(f.x[0][0][i] - f.w[0][j]);
+                    const float d1 = __builtin_fabsf(f.x[0][1][i] - f.w[1][j]);
+                    acc[i][j] = __builtin_fmaxf(__builtin_fmaxf(acc[i][j], d0), d1);
+                }
+        });
+        if (NBUF == 1) __syncthreads();
+        if (s + 1 < nstage) st.store(lds + ((s + 1) % NBUF) * STAGE);
+        __syncthreads();
+    }
+    if constexpr (KS > 1) {   // the other k-groups hand their maxima to the first
+        float* part = lds;    // [KS-1][TM*TN][NGRP]
+        if (grp > 0) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) part[((grp - 1) * TM * TN + i * TN + j) * NGRP + t] = acc[i][j];
+        }
+        __syncthreads();
+        if (grp > 0) return;
+#pragma unroll
+        for (int q = 0; q < KS - 1; q++)
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_fmaxf(acc[i][j], part[(q * TM * TN + i * TN + j) * NGRP + t]);
+    }
+    store_patch<GEO, false>(output, acc, d, m0, n0, g, tx, ty, d.ovec != 0);
+}
+
+template <class GEO>
+static hipError_t launch_values(const Problem& pr, bool ovec, hipStream_t stream, const float* input, const float* weight,
+                                float* output) {
+    Dims d = make_dims(pr);
+    d.ovec = ovec;
+    d.tiles_m = (d.M + GEO::BM - 1) / GEO::BM;
+    d.tiles_n = (d.NG + GEO::BN - 1) / GEO::BN;
+    const size_t lds = Stager<GEO, false, 4, 1>::LDS_BYTES;
+    auto kern = inf_forward_values_kernel<GEO>;
+    static LdsRecord lds_allowed = {};
+    if (hipError_t e = allow_lds(kern, lds, pr.device, lds_allowed); e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, dim3((unsigned)d.tiles_m * d.tiles_n * d.G), dim3(GEO::NT), lds, stream, input, weight,
+                       output, d);
+    return hipGetLastError();
+}
+
+// The shapes the values-only kernel takes: the fc layout with 128-bit loads and more than a handful of outputs per
+// group (the skinny kernels serve those, and pos costs them nothing).  Everything else computes pos as well.
+bool inf_forward_values_applicable(const Problem& pr, const void* input, const void* weight) {
+    return pr.HW == 1 && pr.NG > kSkinnyMaxNG && can_vec4(pr, input, weight);
+}
+
+hipError_t inf_forward_values(const float* input, const float* weight, float* output, const Problem& pr,
+                              hipStream_t stream) {
+    const bool ovec = can_vec4_out(pr, output);
+    if (g_tile_override == 4) return launch_values<Geo<64, 80, 8, 5, 2>>(pr, ovec, stream, input, weight, output);
+    switch (choose_tile(pr.B, pr.NG, pr.G, pr.num_cu)) {
+        case TileChoice::M128N80K2:
+            // as in inf_forward(): two 256-lane workgroups per CU where one 512-lane workgroup would be chosen
+            if (pr.B > 64 && g_tile_override < 0) return launch_values<Geo<64, 80, 8, 5, 2>>(pr, ovec, stream, input, weight, output);
+            return launch_values<Geo<128, 80, 8, 5, 2>>(pr, ovec, stream, input, weight, output);
+        case TileChoice::M256N32K1: return launch_values<Geo<256, 32, 8, 4, 1>>(pr, ovec, stream, input, weight, output);
+        case TileChoice::M32N32K8: return launch_values<Geo<32, 32, 4, 4, 8>>(pr, ovec, stream, input, weight, output);
+        default: return launch_values<Geo<128, 64, 8, 4, 1>>(pr, ovec, stream, input, weight, output);
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Few outputs per group (the 10-way classification head): a workgroup takes RW
 // rows m of one group, its 256 lanes split k, each lane keeps the exact
 // (value, k) pair per (row, output), and the pairs are reduced with "larger

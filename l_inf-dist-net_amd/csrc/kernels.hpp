@@ -68,6 +68,10 @@ inline hipError_t allow_lds(Kern kern, size_t bytes, int device, LdsRecord& done
 
 hipError_t inf_forward(const float* input, const float* weight, float* output, int32_t* pos, const Problem& pr,
                        hipStream_t stream);
+// Values without pos, for forward passes that no gradient follows (inf_forward.hip); the fc layout with 128-bit loads.
+bool inf_forward_values_applicable(const Problem& pr, const void* input, const void* weight);
+hipError_t inf_forward_values(const float* input, const float* weight, float* output, const Problem& pr,
+                              hipStream_t stream);
 bool inf_forward_shortk_applicable(const Problem& pr, const void* input, const void* output, const void* pos);
 hipError_t inf_forward_shortk(const float* input, const float* weight, float* output, int32_t* pos, const Problem& pr,
                               hipStream_t stream);

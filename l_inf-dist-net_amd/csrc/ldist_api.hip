@@ -112,6 +112,15 @@ int ldist_inf_dist_forward(const float* input, const float* weight, int B, int C
     return finish(ldist::inf_forward(input, weight, output, pos, pr, (hipStream_t)stream));
 }
 
+int ldist_inf_dist_forward_values(const float* input, const float* weight, int B, int CO, int CI, int G, int HW,
+                                  float* output, ldist_stream_t stream) {
+    if (!input || !weight || !output) return LDIST_EINVAL;
+    ldist::Problem pr{};
+    if (int rc = check_dims(B, CO, CI, G, HW, pr)) return rc;
+    if (!ldist::inf_forward_values_applicable(pr, input, weight)) return LDIST_EUNSUPPORTED;
+    return finish(ldist::inf_forward_values(input, weight, output, pr, (hipStream_t)stream));
+}
+
 int ldist_inf_dist_bound_forward(const float* input_lower, const float* input_upper, const float* weight, int B,
                                  int CO, int CI, int G, int HW, float* output_lower, float* output_upper,
                                  ldist_stream_t stream) {

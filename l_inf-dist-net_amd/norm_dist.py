@@ -192,6 +192,14 @@ def norm_dist(input, weight, group, p, use_custom_cuda_func=True, tag=None):
     option of that name does; it is never chosen automatically.
     """
     if use_custom_cuda_func:
+        # No gradient will follow (evaluation, torch.no_grad(), the value path of a certification pass): the argmax
+        # that the reference always computes (model/norm_dist.py:14-15) has no reader, and the kernel without it is
+        # faster.  Where the library has no such kernel for the layout the call says so and the usual path runs.
+        if math.isinf(p) and not (torch.is_grad_enabled() and (input.requires_grad or weight.requires_grad)):
+            assert weight.size(1) * group == input.size(1)
+            y = torch.empty(_out_shape(input, weight), device=input.device, dtype=input.dtype)
+            if norm_dist_cpp.inf_dist_forward_values(input, weight, y, group):
+                return y
         return DistF.apply(input, weight, group, p, tag)
     diff = _pairwise_difference(input, weight, group)
     with torch.no_grad():

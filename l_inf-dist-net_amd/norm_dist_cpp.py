@@ -122,6 +122,27 @@ def inf_dist_forward(input, weight, output, pos, G):
     _call("ldist_inf_dist_forward", dev, _p(input), _p(weight), B, CO, CI, G, HW, _p(output), _p(pos))
 
 
+def inf_dist_forward_values(input, weight, output, G):
+    """inf_dist_forward without pos, for a forward pass that no gradient follows (no counterpart in the reference,
+    whose forward always computes pos).  Returns False, with nothing written, where the library has no kernel for
+    it (anything but a fully connected layer with more than 16 outputs per group and 128-bit loadable rows):
+    call inf_dist_forward then."""
+    for t, n in ((input, "input"), (weight, "weight"), (output, "output")):
+        _check_input(t, n)
+    dev = _same_device(input, weight, output)
+    B, CO, CI, HW = input.size(0), output.size(1), input.size(1), input.size(2)
+    _expect(input.dim() == 3 and weight.dim() == 2, "input must be 3-D, weight 2-D")
+    _expect(weight.size(0) == CO and weight.size(1) * G == CI, "weight must be (CO, CI/G)")
+    _expect(tuple(output.shape) == (B, CO, HW), "output must be (B, CO, HW)")
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        rc = _lib.lib().ldist_inf_dist_forward_values(_p(input), _p(weight), B, CO, CI, G, HW, _p(output), stream)
+    if rc == _lib.EUNSUPPORTED:
+        return False
+    _lib.check(rc, "ldist_inf_dist_forward_values")
+    return True
+
+
 def inf_dist_bound_forward(input_lower, input_upper, weight, output_lower, output_upper, G):
     """model/norm_dist.cpp:64-74."""
     for t, n in ((input_lower, "input_lower"), (input_upper, "input_upper"), (weight, "weight"),

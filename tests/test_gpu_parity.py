@@ -60,6 +60,41 @@ def test_inf_forward_bit_exact(shape, tile, quant):
     assert torch.equal(pos, ep)
 
 
+@pytest.mark.parametrize("tile", TILES)
+@pytest.mark.parametrize("shape", SHAPES + [(130, 170, 300, 1, 1), (70, 96, 1028, 2, 1), (512, 5120, 784, 1, 1)])
+def test_inf_forward_values_only_matches_the_full_forward(shape, tile):
+    """inf_dist_forward_values (no pos; what a forward without a gradient to follow calls) against the oracle's
+    values, bit for bit, on every tiling; where it says it has no kernel (conv layout, 16 outputs per group or
+    fewer, K not a multiple of four) it must leave the output alone."""
+    from gpu_common import DEV, cpp, say, set_tile
+    B, CO, CI, G, HW = shape
+    say("inf_forward values only", shape, "tile", tile)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=sum(shape) + 1)
+    set_tile(tile)
+    out = torch.full((B, CO, HW), -7.0, device=DEV)
+    done = cpp.inf_dist_forward_values(x.to(DEV), w.to(DEV), out, G)
+    assert done == (HW == 1 and CO // G > 16 and (CI // G) % 4 == 0)
+    if done:
+        assert torch.equal(out.cpu(), oracle.inf_dist_forward(x, w, G)[0])
+    else:
+        assert bool((out == -7.0).all())
+
+
+def test_norm_dist_without_a_gradient_takes_the_values_only_forward():
+    """norm_dist at p = inf: the same values with and without a gradient to follow (the second through the kernel
+    without pos), and a gradient where one is asked for."""
+    from gpu_common import DEV, pkg
+    g = torch.Generator().manual_seed(5)
+    x, w = torch.rand(96, 200, 1, generator=g).to(DEV), torch.rand(160, 200, generator=g).to(DEV)
+    with torch.no_grad():
+        y0 = pkg.norm_dist(x, w.clone().requires_grad_(), 1, float("inf"))
+    wr = w.clone().requires_grad_()
+    y1 = pkg.norm_dist(x, wr, 1, float("inf"))
+    assert not y0.requires_grad and y1.requires_grad and torch.equal(y0, y1.detach())
+    y1.sum().backward()
+    assert wr.grad is not None and bool((wr.grad != 0).any())
+
+
 @pytest.mark.parametrize("K", [2_000_000, 2_100_000, 2_100_002])
 def test_forward_kernels_with_very_long_rows(K):
     """The fc panels are read through 32-bit buffer offsets, which cover tile rows of up to 2 GB: 258 rows of

@@ -27,6 +27,13 @@ def fake_native(monkeypatch):
         o, p = oracle.inf_dist_forward(x.contiguous(), w.contiguous(), G)
         out.copy_(o); pos.copy_(p)
 
+    def inf_dist_forward_values(x, w, out, G):   # the fc layout only, like the library
+        if x.size(2) != 1:
+            return False
+        calls.append("inf_dist_forward_values")
+        out.copy_(oracle.inf_dist_forward(x.contiguous(), w.contiguous(), G)[0])
+        return True
+
     def inf_dist_bound_forward(lo, up, w, ol, ou, G):
         calls.append("inf_dist_bound_forward")
         a, b = oracle.inf_dist_bound_forward(lo.contiguous(), up.contiguous(), w.contiguous(), G)
@@ -60,7 +67,8 @@ def fake_native(monkeypatch):
         oracle.norm_dist_backward_weight(go, x.contiguous(), w.contiguous(), out.contiguous(), G, p, grad_weight=gw)
 
     monkeypatch.setattr(cpp, "norm_dist_backward", norm_bwd_both)
-    for name, fn in [("inf_dist_forward", inf_dist_forward), ("inf_dist_bound_forward", inf_dist_bound_forward),
+    for name, fn in [("inf_dist_forward", inf_dist_forward), ("inf_dist_forward_values", inf_dist_forward_values),
+                     ("inf_dist_bound_forward", inf_dist_bound_forward),
                      ("inf_dist_backward_input_overwrite", bwd_in_over),
                      ("inf_dist_backward_weight_overwrite", bwd_w_over), ("norm_dist_forward", norm_dist_forward),
                      ("norm_dist_backward_input", norm_bwd_in), ("norm_dist_backward_weight", norm_bwd_w)]:
@@ -81,7 +89,19 @@ def test_distf_dispatch_and_errors(fake_native):
     x = torch.rand(3, 6, 2, generator=gen(0))
     w = torch.rand(4, 3, generator=gen(1))
     y = pkg.norm_dist(x, w, 2, float("inf"))
-    assert fake_native == ["inf_dist_forward"] and y.shape == (3, 4, 2)
+    assert fake_native == ["inf_dist_forward"] and y.shape == (3, 4, 2)   # no gradient wanted, but not a layout the values-only call takes
+    fake_native.clear()
+    # fc layout: without a gradient to follow the forward skips the argmax; with one it records it
+    xf, wf = torch.rand(3, 6, 1, generator=gen(2)), torch.rand(4, 3, generator=gen(3))
+    y0 = pkg.norm_dist(xf, wf, 2, float("inf"))
+    assert fake_native == ["inf_dist_forward_values"]
+    fake_native.clear()
+    y1 = pkg.norm_dist(xf.clone().requires_grad_(), wf, 2, float("inf"))
+    assert fake_native == ["inf_dist_forward"] and torch.equal(y0, y1.detach())
+    fake_native.clear()
+    with torch.no_grad():
+        pkg.norm_dist(xf.clone().requires_grad_(), wf, 2, float("inf"))
+    assert fake_native == ["inf_dist_forward_values"]
     fake_native.clear()
     pkg.norm_dist(x, w, 2, 8.0)
     assert fake_native == ["norm_dist_forward"]
