@@ -222,6 +222,13 @@ LDIST_API int ldist_inf_dist_conv_forward_supported(int C, int H, int W, int CO,
 LDIST_API int ldist_inf_dist_conv_forward(const float* img, const float* weight, int B, int C, int H, int W, int CO, int G,
                                 int KH, int KW, int stride, int padding, int dilation, float* output, int32_t* pos,
                                 ldist_stream_t stream);
+
+/* The same without pos, for forward passes that no gradient follows: output as ldist_inf_dist_conv_forward
+ * writes it, bit for bit, from a kernel that keeps no per-channel record and searches for no index.  No counterpart
+ * in the reference.  Covers what ldist_inf_dist_conv_forward_supported says; LDIST_EUNSUPPORTED otherwise. */
+LDIST_API int ldist_inf_dist_conv_forward_values(const float* img, const float* weight, int B, int C, int H, int W, int CO,
+                                       int G, int KH, int KW, int stride, int padding, int dilation, float* output,
+                                       ldist_stream_t stream);
 /* Interval-bound forward of the convolution-shaped layer straight from the lower and upper images: what
  * ldist_unfold of both followed by ldist_inf_dist_bound_forward computes (the reference: F.unfold at
  * model/norm_dist.py:144-145, then inf_dist_bound_forward_cuda), bit for bit, irregular boxes included.

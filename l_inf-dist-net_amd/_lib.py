@@ -34,6 +34,7 @@ SIGNATURES = {
     "ldist_unfold": [_F, _i, _i, _i, _i, _i, _i, _i, _i, _i, _F, _S],
     "ldist_inf_dist_conv_forward_supported": [_i, _i, _i, _i, _i, _i, _i, _i, _i, _i],
     "ldist_inf_dist_conv_forward": [_F, _F, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _F, _I, _S],
+    "ldist_inf_dist_conv_forward_values": [_F, _F, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _F, _S],
     "ldist_inf_dist_bound_conv_forward_supported": [_i, _i, _i, _i, _i, _i, _i, _i, _i, _i],
     "ldist_inf_dist_bound_conv_forward": [_F, _F, _F, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _F, _F, _S],
     "ldist_norm_dist_conv_supported": [_i, _i, _i, _i, _i, _i, _i, _i, _i, _i],

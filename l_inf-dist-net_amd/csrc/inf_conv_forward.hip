@@ -28,7 +28,10 @@ namespace {
 
 using namespace convimg;
 
-template <int S, bool RESIDENT>
+// POS = false: values only, for a forward pass that no gradient follows (pos has no reader then): the maximum is kept
+// across channels without the per-channel record, and the search after the loop is left out.  Same subtractions and
+// maxima: the values are those of POS = true bit for bit.
+template <int S, bool RESIDENT, bool POS>
 __global__ void __launch_bounds__(kMaxThreads, 2)
 inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__ weight, float* __restrict__ out,
                         int32_t* __restrict__ pos, ConvFwd a) {
@@ -205,11 +208,11 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
         // arithmetic instructions, and its registers are all the compiler has to keep.
 #pragma unroll 1
         for (int u = 0; u < kCC / kTrack; u++) {
-            float cm[kTM][kTN];
+            float cm[kTM][kTN];   // the unit's maximum; without pos, the running maximum itself
 #pragma unroll
             for (int e = 0; e < kTM; e++)
 #pragma unroll
-                for (int t = 0; t < kTN; t++) cm[e][t] = 0.f;
+                for (int t = 0; t < kTN; t++) cm[e][t] = POS ? 0.f : acc[e][t];
             // The 3*kTrack window rows of the unit, unrolled, with the reads of a row issued before the
             // arithmetic of the row before it.
             struct Row { float x[NXR * 4]; float w[3][kTN]; };
@@ -248,7 +251,11 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
             for (int e = 0; e < kTM; e++)
 #pragma unroll
                 for (int t = 0; t < kTN; t++)
-                    if (cm[e][t] > acc[e][t]) { acc[e][t] = cm[e][t]; unit[e][t] = un; }
+                    if constexpr (POS) {
+                        if (cm[e][t] > acc[e][t]) { acc[e][t] = cm[e][t]; unit[e][t] = un; }
+                    } else {
+                        acc[e][t] = cm[e][t];
+                    }
         }
         xch += kCC * CST;
         if (ch + 1 < nstage) {
@@ -262,10 +269,27 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
         __syncthreads();
     }
 
-    // ---- the lowest k of the recorded unit, from the image rows in LDS and the weight rows in cache ----
     const int h = h0 + hr;
     if (h >= a.HO) return;
     const int L = a.HO * a.WO;
+    if constexpr (!POS) {
+#pragma unroll
+        for (int t = 0; t < kTN; t++) {
+            const int n = n0 + kTN * nl + t;
+            if (n >= a.NG) break;
+            const size_t at = (((size_t)b * a.G + g) * a.NG + n) * L + (size_t)h * a.WO + w0;
+            if (a.vec_out) {
+                *reinterpret_cast<float4*>(out + at) = make_float4(acc[0][t], acc[1][t], acc[2][t], acc[3][t]);
+                *reinterpret_cast<float4*>(out + at + 4) = make_float4(acc[4][t], acc[5][t], acc[6][t], acc[7][t]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < kTM; e++)
+                    if (w0 + e < a.WO) out[at + e] = acc[e][t];
+            }
+        }
+        return;
+    }
+    // ---- the lowest k of the recorded unit, from the image rows in LDS and the weight rows in cache ----
     // Per output the recorded channel's nine weights are contiguous: two 16-byte loads at 4-byte alignment
     // and one word instead of one load per candidate, issued for the lane's eight positions together.
     typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
@@ -346,17 +370,23 @@ bool inf_conv_forward_supported(const ConvGeom& q, int G, int CO) {
     return plan(q, G, CO, a);
 }
 
+// pos == nullptr: values only (the kernel without the argmax).
 hipError_t inf_conv_forward(const float* img, const float* weight, float* out, int32_t* pos, const ConvGeom& q, int G,
                             int CO, int device, hipStream_t stream) {
     ConvFwd a{};
     if (!plan(q, G, CO, a)) return hipErrorInvalidValue;   // the API layer asks inf_conv_forward_supported first
+    const bool with_pos = pos != nullptr;
     a.vec_in = q.W % 4 == 0 && aligned16(img);
     a.vec_out = q.WO % kTM == 0 && aligned16(out) && aligned16(pos);   // every run of 8 positions whole and aligned
     const size_t lds = ((size_t)a.xwords + 2 * (size_t)kKC * kBNP) * sizeof(float);
-    static std::atomic<bool> raised[64][4] = {};   // callers may come from several threads
-    const int ki = (q.S - 1) * 2 + a.resident;
-    auto kern = q.S == 1 ? (a.resident ? inf_conv_forward_kernel<1, true> : inf_conv_forward_kernel<1, false>)
-                         : (a.resident ? inf_conv_forward_kernel<2, true> : inf_conv_forward_kernel<2, false>);
+    static std::atomic<bool> raised[64][8] = {};   // callers may come from several threads
+    const int ki = ((q.S - 1) * 2 + a.resident) * 2 + (with_pos ? 1 : 0);
+    using Kern = void (*)(const float*, const float*, float*, int32_t*, ConvFwd);
+    const Kern table[8] = {inf_conv_forward_kernel<1, false, false>, inf_conv_forward_kernel<1, false, true>,
+                           inf_conv_forward_kernel<1, true, false>,  inf_conv_forward_kernel<1, true, true>,
+                           inf_conv_forward_kernel<2, false, false>, inf_conv_forward_kernel<2, false, true>,
+                           inf_conv_forward_kernel<2, true, false>,  inf_conv_forward_kernel<2, true, true>};
+    const Kern kern = table[ki];
     if (!(device >= 0 && device < 64 && raised[device][ki].load(std::memory_order_acquire))) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                            (int)kLdsLimit);

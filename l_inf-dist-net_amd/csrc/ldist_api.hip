@@ -268,11 +268,12 @@ int ldist_inf_dist_conv_forward_supported(int C, int H, int W, int CO, int G, in
     return ldist::inf_conv_forward_supported(q, G, CO) ? 1 : 0;
 }
 
-int ldist_inf_dist_conv_forward(const float* img, const float* weight, int B, int C, int H, int W, int CO, int G,
-                                int KH, int KW, int stride, int padding, int dilation, float* output, int32_t* pos,
-                                ldist_stream_t stream) {
+// pos == nullptr: values only
+static int inf_conv_forward_entry(const float* img, const float* weight, int B, int C, int H, int W, int CO, int G,
+                                  int KH, int KW, int stride, int padding, int dilation, float* output, int32_t* pos,
+                                  ldist_stream_t stream) {
     ldist::ConvGeom q{};
-    if (!img || !weight || !output || !pos || CO <= 0 || G <= 0) return LDIST_EINVAL;
+    if (!img || !weight || !output || CO <= 0 || G <= 0) return LDIST_EINVAL;
     if (int rc = conv_geometry(B, C, H, W, KH, KW, stride, padding, dilation, q)) return rc;
     if (C % G != 0 || CO % G != 0) return LDIST_EINVAL;
     if ((long long)B * CO * q.HO * q.WO >= (1LL << 31) || (long long)CO * (C / G) * KH * KW >= (1LL << 31))
@@ -281,6 +282,20 @@ int ldist_inf_dist_conv_forward(const float* img, const float* weight, int B, in
     ldist::Problem pr{};
     if (int rc = current_device(pr)) return rc;
     return finish(ldist::inf_conv_forward(img, weight, output, pos, q, G, CO, pr.device, (hipStream_t)stream));
+}
+
+int ldist_inf_dist_conv_forward(const float* img, const float* weight, int B, int C, int H, int W, int CO, int G,
+                                int KH, int KW, int stride, int padding, int dilation, float* output, int32_t* pos,
+                                ldist_stream_t stream) {
+    if (!pos) return LDIST_EINVAL;
+    return inf_conv_forward_entry(img, weight, B, C, H, W, CO, G, KH, KW, stride, padding, dilation, output, pos, stream);
+}
+
+int ldist_inf_dist_conv_forward_values(const float* img, const float* weight, int B, int C, int H, int W, int CO, int G,
+                                       int KH, int KW, int stride, int padding, int dilation, float* output,
+                                       ldist_stream_t stream) {
+    return inf_conv_forward_entry(img, weight, B, C, H, W, CO, G, KH, KW, stride, padding, dilation, output, nullptr,
+                                  stream);
 }
 
 int ldist_inf_dist_bound_conv_forward_supported(int C, int H, int W, int CO, int G, int KH, int KW, int stride,

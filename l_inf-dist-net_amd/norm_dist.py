@@ -400,7 +400,16 @@ class NormDistConv(nn.Module):
             shape = (x.size(0), -1, *out_hw)
             return y.view(shape), lo.view(shape), hi.view(shape)
         if self._fused_inf_conv(x):
-            y = _ConvInfDist.apply(x, w2d, self.group, self.kernel_size, self.dilation, self.padding, self.stride)
+            wants_grad = torch.is_grad_enabled() and (x.requires_grad or w2d.requires_grad)
+            if wants_grad or not norm_dist_cpp.inf_dist_conv_forward_supported(
+                    x.size(1), x.size(2), x.size(3), w2d.size(0), self.group, self.kernel_size, self.stride,
+                    self.padding, self.dilation):
+                y = _ConvInfDist.apply(x, w2d, self.group, self.kernel_size, self.dilation, self.padding, self.stride)
+            else:   # no gradient follows: the argmax has no reader, and the kernel without it is faster
+                ho, wo = out_hw
+                y = torch.empty(x.size(0), w2d.size(0), ho * wo, device=x.device, dtype=x.dtype)
+                norm_dist_cpp.inf_dist_conv_forward_values(x.contiguous(), w2d, y, self.group, self.kernel_size,
+                                                           self.stride, self.padding, self.dilation)
         elif self._norm_from_image(x):
             y = _ConvNormDist.apply(x, w2d, self.group, self.p, self.kernel_size, self.dilation, self.padding,
                                     self.stride)

@@ -344,6 +344,20 @@ def inf_dist_conv_forward(img, weight, output, pos, G, kernel_size, stride=1, pa
           _p(pos))
 
 
+def inf_dist_conv_forward_values(img, weight, output, G, kernel_size, stride=1, padding=0, dilation=1):
+    """inf_dist_conv_forward without pos, for a forward pass that no gradient follows (no counterpart in the
+    reference); the geometries of inf_dist_conv_forward_supported."""
+    for t, n in ((img, "img"), (weight, "weight"), (output, "output")):
+        _check_input(t, n)
+    dev = _same_device(img, weight, output)
+    B, C, H, W, KH, KW, S, P, D = _conv_args(img, kernel_size, stride, padding, dilation)
+    HO, WO = conv_output_size(H, W, KH, S, P, D)
+    _expect(weight.dim() == 2 and C % G == 0 and weight.size(1) == C // G * KH * KW, "weight must be (CO, C/G*k*k)")
+    CO = weight.size(0)
+    _expect(output.shape == (B, CO, HO * WO), "output must be (B, CO, HO*WO)")
+    _call("ldist_inf_dist_conv_forward_values", dev, _p(img), _p(weight), B, C, H, W, CO, G, KH, KW, S, P, D, _p(output))
+
+
 def norm_dist_conv_supported(C, H, W, CO, G, kernel_size, stride=1, padding=0, dilation=1):
     """True when the three norm_dist_conv_* calls cover the geometry (3x3 windows, more than one output position);
     otherwise unfold + the column calls are the way."""

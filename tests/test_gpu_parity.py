@@ -95,6 +95,19 @@ def test_norm_dist_without_a_gradient_takes_the_values_only_forward():
     assert wr.grad is not None and bool((wr.grad != 0).any())
 
 
+def test_conv_layer_without_a_gradient_takes_the_values_only_forward():
+    """NormDistConv at p = inf in evaluation under torch.no_grad(): the same output as with gradients enabled
+    (which records the argmax), from the kernel without pos."""
+    from gpu_common import DEV, pkg
+    torch.manual_seed(3)
+    layer = pkg.NormDistConv(32, 64, 3, stride=1, padding=1, group=2, p=float("inf"), bias=True, mean_normalize=True).to(DEV).eval()
+    x = torch.rand(4, 32, 32, 32, device=DEV)
+    y1 = layer(x)[0]
+    with torch.no_grad():
+        y0 = layer(x)[0]
+    assert y1.requires_grad and not y0.requires_grad and torch.equal(y0, y1.detach())
+
+
 @pytest.mark.parametrize("K", [2_000_000, 2_100_000, 2_100_002])
 def test_forward_kernels_with_very_long_rows(K):
     """The fc panels are read through 32-bit buffer offsets, which cover tile rows of up to 2 GB: 258 rows of
@@ -825,6 +838,10 @@ def test_inf_conv_forward_matches_column_path_bit_exact(case, quant, rows):
     torch.cuda.synchronize()
     assert torch.equal(out.cpu(), eo)
     assert torch.equal(pos.cpu(), ep)
+    # the kernel without pos (for passes that no gradient follows): the same values
+    only = torch.full(eo.shape, float("nan"), device=DEV)
+    cpp.inf_dist_conv_forward_values(img.to(DEV), w.to(DEV), only, G, 3, s_, p_, 1)
+    assert torch.equal(only.cpu(), eo)
 
 
 STAGED_CASES = [  # B, C, H, W, CO, G, stride, padding: channels per group a multiple of four
@@ -858,11 +875,14 @@ def test_inf_conv_forward_staged_channels_bit_exact(case, quant, rows):
         out = torch.full(eo.shape, float("nan"), device=DEV)
         pos = torch.full(eo.shape, -7, device=DEV, dtype=torch.int32)
         cpp.inf_dist_conv_forward(img.to(DEV), w.to(DEV), out, pos, G, 3, s_, p_, 1)
+        only = torch.full(eo.shape, float("nan"), device=DEV)   # the same variant of the kernel without pos
+        cpp.inf_dist_conv_forward_values(img.to(DEV), w.to(DEV), only, G, 3, s_, p_, 1)
         torch.cuda.synchronize()
     finally:
         lib.ldist_set_conv_staging_override(0)
     assert torch.equal(out.cpu(), eo)
     assert torch.equal(pos.cpu(), ep)
+    assert torch.equal(only.cpu(), eo)
 
 
 @pytest.mark.parametrize("rows", [1, 2, 3, 5, 8])
