@@ -50,6 +50,11 @@ def test_random_problem(seed):
     out, pos = gpu_inf_forward(x, w, G)
     eo, ep = oracle.inf_dist_forward(x, w, G)
     assert torch.equal(out, eo) and torch.equal(pos, ep)
+    only = torch.full((B, CO, HW), -7.0, device=DEV)   # the forward without pos: the same values, or left alone
+    if cpp.inf_dist_forward_values(x.to(DEV), w.to(DEV), only, G):
+        assert torch.equal(only.cpu(), eo)
+    else:
+        assert bool((only == -7.0).all())
 
     lo, up = (x - 0.05).contiguous(), (x + 0.05).contiguous()
     ol, ou = gpu_bound_forward(lo, up, w, G)
