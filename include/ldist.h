@@ -171,6 +171,14 @@ LDIST_API int ldist_inf_dist_backward_input_overwrite(const float* grad_output, 
 LDIST_API int ldist_inf_dist_backward_weight_overwrite(const float* grad_output, const int32_t* pos, int B, int CO, int CI,
                                              int G, int HW, float* grad_weight, ldist_stream_t stream);
 
+/* Both of them in one call: what DistF.backward needs when both gradients are wanted (model/norm_dist.py:33-38
+ * calls the two native functions one after the other).  For a fully connected layer (HW == 1) the two scatters run
+ * as one launch whose workgroups do either, so the short, latency-bound grad_input workgroups run beside the
+ * streaming grad_weight ones; other layouts run the two kernels inside the call.  Results are those of the two
+ * overwrite entry points. */
+LDIST_API int ldist_inf_dist_backward_overwrite(const float* grad_output, const int32_t* pos, int B, int CO, int CI, int G,
+                                      int HW, float* grad_input, float* grad_weight, ldist_stream_t stream);
+
 /* Per-channel mean shift of a contiguous (B, C, L) tensor in one kernel:
  *   mean[c] = mean over b and l of x[b,c,l];   y[b,c,l] = x[b,c,l] - mean[c]
  *   running_mean[c] = (1 - momentum) * running_mean[c] + momentum * mean[c]   (when running_mean != NULL)

@@ -26,6 +26,7 @@ SIGNATURES = {
     "ldist_inf_dist_backward_weight": [_F, _I, _i, _i, _i, _i, _i, _F, _S],
     "ldist_inf_dist_backward_input_overwrite": [_F, _I, _i, _i, _i, _i, _i, _F, _S],
     "ldist_inf_dist_backward_weight_overwrite": [_F, _I, _i, _i, _i, _i, _i, _F, _S],
+    "ldist_inf_dist_backward_overwrite": [_F, _I, _i, _i, _i, _i, _i, _F, _F, _S],
     "ldist_norm_dist_forward": [_F, _F, _i, _i, _i, _i, _i, _F, _f, _S],
     "ldist_norm_dist_backward_input": [_F, _F, _F, _F, _i, _i, _i, _i, _i, _F, _f, _S],
     "ldist_norm_dist_backward_weight": [_F, _F, _F, _F, _i, _i, _i, _i, _i, _F, _f, _S],

@@ -16,6 +16,8 @@
 // element receives one contribution, otherwise at least as close to the true sum as any order of float additions.
 #include "kernels.hpp"
 
+#include <algorithm>
+
 namespace ldist {
 
 struct BwdDims {
@@ -25,17 +27,18 @@ struct BwdDims {
 // ---- grad_input ------------------------------------------------------------
 // Workgroup = (image b, group g, TH consecutive hw, KC consecutive k).
 // bins[kc][th]; element (k, hw) of the slab lives at ((b*G+g)*K + k)*HW + hw.
+// bx, by: the workgroup's place in the grid of this scatter (the kernel below passes blockIdx; the kernel that runs
+// both scatters of a layer in one launch passes what it dealt to this workgroup).
 template <bool OVERWRITE>
-__global__ void __launch_bounds__(1024)
-inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* __restrict__ pos,
-                          float* __restrict__ grad_input, BwdDims d, int th_log2, int KC, int hw_tiles, int vec) {
-    extern __shared__ __align__(16) double bins[];
+__device__ __forceinline__ void backward_input_body(double* bins, int bx, int by, const float* __restrict__ grad_output,
+                                                    const int32_t* __restrict__ pos, float* __restrict__ grad_input,
+                                                    const BwdDims& d, int th_log2, int KC, int hw_tiles, int vec) {
     const int NT = blockDim.x;
     const int TH = 1 << th_log2;
-    const int tile = blockIdx.x % hw_tiles;
-    const int bg = blockIdx.x / hw_tiles;  // b*G + g
+    const int tile = bx % hw_tiles;
+    const int bg = bx / hw_tiles;  // b*G + g
     const int hw0 = tile * TH;
-    const int k0 = blockIdx.y * KC;
+    const int k0 = by * KC;
     const int kc = min(KC, d.K - k0);
     const int nb = kc * TH;
     const size_t obase = (size_t)bg * d.NG * d.HW;
@@ -155,6 +158,14 @@ inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* 
     }
 }
 
+template <bool OVERWRITE>
+__global__ void __launch_bounds__(1024)
+inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* __restrict__ pos,
+                          float* __restrict__ grad_input, BwdDims d, int th_log2, int KC, int hw_tiles, int vec) {
+    extern __shared__ __align__(16) double bins[];
+    backward_input_body<OVERWRITE>(bins, blockIdx.x, blockIdx.y, grad_output, pos, grad_input, d, th_log2, KC, hw_tiles, vec);
+}
+
 // ---- grad_weight -----------------------------------------------------------
 // Workgroup = (group g, NB consecutive outputs n, KC consecutive k -- all of K when
 // a row of bins fits in 64 KB -- and a slice of the images b).  For one image the NB rows of grad_output/pos are one
@@ -167,26 +178,24 @@ inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* 
 // faster atomics), double bins otherwise (B * HW contributions per row: 131 072 in a 3x3 conv layer of 32 x 32
 // images at batch 128, where the float atomics took three times as long as everything else).
 template <bool OVERWRITE, bool SPLIT, class BIN>
-__global__ void __launch_bounds__(256)
-inf_backward_weight_kernel(const float* __restrict__ grad_output, const int32_t* __restrict__ pos,
-                           float* __restrict__ grad_weight, BwdDims d, int NB, int KC, int n_blocks, int b_per_wg) {
-    extern __shared__ __align__(16) unsigned char bin_bytes[];
-    BIN* bins = reinterpret_cast<BIN*>(bin_bytes);
+__device__ __forceinline__ void backward_weight_body(BIN* bins, int bx, int by, int bz, const float* __restrict__ grad_output,
+                                                     const int32_t* __restrict__ pos, float* __restrict__ grad_weight,
+                                                     const BwdDims& d, int NB, int KC, int n_blocks, int b_per_wg) {
     constexpr int NT = 256;
     // Neighbouring blocks of outputs read neighbouring few-byte pieces of the same memory lines (in the fc layout a
     // block's grad_output / pos entries of one image are NB * 4 bytes).  Workgroups go to the eight XCDs in turn, each
     // with its own L2, so XCD x takes the x-th eighth of the blocks: neighbours then share the lines in one L2
     // instead of fetching them eight times.  Where that matters (many blocks) the launcher rounds n_blocks up to a
     // multiple of eight; otherwise the blocks keep their order.
-    const int id = blockIdx.x % n_blocks;
-    const int g = blockIdx.x / n_blocks;
+    const int id = bx % n_blocks;
+    const int g = bx / n_blocks;
     const int nblk = (n_blocks & 7) == 0 ? (id % 8) * (n_blocks / 8) + id / 8 : id;
     const int n0 = nblk * NB;
     if (n0 >= d.NG) return;
     const int nb = min(NB, d.NG - n0);
-    const int k0 = blockIdx.y * KC;
+    const int k0 = by * KC;
     const int kc = min(KC, d.K - k0);
-    const int b0 = blockIdx.z * b_per_wg;
+    const int b0 = bz * b_per_wg;
     const int b1 = min(d.B, b0 + b_per_wg);
     // kc is a multiple of 4 whenever vec is set, so rows of bins and of grad_weight stay 16-byte aligned
     const bool vec = (kc & 3) == 0 && (d.K & 3) == 0 && (reinterpret_cast<uintptr_t>(grad_weight) & 15u) == 0;
@@ -280,6 +289,42 @@ inf_backward_weight_kernel(const float* __restrict__ grad_output, const int32_t*
             *dst += v;
         }
     }
+}
+
+template <bool OVERWRITE, bool SPLIT, class BIN>
+__global__ void __launch_bounds__(256)
+inf_backward_weight_kernel(const float* __restrict__ grad_output, const int32_t* __restrict__ pos,
+                           float* __restrict__ grad_weight, BwdDims d, int NB, int KC, int n_blocks, int b_per_wg) {
+    extern __shared__ __align__(16) unsigned char bin_bytes[];
+    backward_weight_body<OVERWRITE, SPLIT, BIN>(reinterpret_cast<BIN*>(bin_bytes), blockIdx.x, blockIdx.y, blockIdx.z,
+                                                grad_output, pos, grad_weight, d, NB, KC, n_blocks, b_per_wg);
+}
+
+// ---- both scatters of a fully connected layer in one launch ------------------
+// grad_input (a workgroup per image and group: few bytes, mostly waiting for memory) and grad_weight (a workgroup per
+// block of output rows: bound by the stores of its slab) are independent.  As two launches one runs after the other;
+// on two streams they overlap but pay for the joins (measured: slower).  Here the workgroups of one grid do either:
+// the grad_weight workgroups come first and the grad_input workgroups last, where they run beside the tail of the
+// stores (512 x 5120 x 5120: 36.5 us against 41.5 us for the two launches; grad_input first: 39.5 us; one grad_input
+// workgroup after every three of grad_weight: 46 us).  Both write their slabs whole ("overwrite"); one k range each.
+struct BothPlan {
+    int wgs_x, wgs_w;                 // workgroups per scatter
+    int th_log2, kc_x, hw_tiles, vec; // grad_input's launch parameters
+    int nb, kc_w, n_blocks;           // grad_weight's
+};
+
+__global__ void __launch_bounds__(256)
+inf_backward_both_kernel(const float* __restrict__ grad_output, const int32_t* __restrict__ pos,
+                         float* __restrict__ grad_input, float* __restrict__ grad_weight, BwdDims d, BothPlan pl) {
+    extern __shared__ __align__(16) unsigned char bin_bytes[];
+    const int i = blockIdx.x;
+    if (i >= pl.wgs_w) {
+        backward_input_body<true>(reinterpret_cast<double*>(bin_bytes), i - pl.wgs_w, 0, grad_output, pos, grad_input, d, pl.th_log2,
+                                  pl.kc_x, pl.hw_tiles, pl.vec);
+        return;
+    }
+    backward_weight_body<true, false, float>(reinterpret_cast<float*>(bin_bytes), i, 0, 0, grad_output, pos, grad_weight, d,
+                                             pl.nb, pl.kc_w, pl.n_blocks, d.B);
 }
 
 __global__ void __launch_bounds__(256) fill_zero_kernel(float* __restrict__ p, size_t n) {
@@ -378,6 +423,40 @@ hipError_t inf_backward_weight(const float* grad_output, const int32_t* pos, flo
         LDIST_BWD_W(false, false);
     }
 #undef LDIST_BWD_W
+    return hipGetLastError();
+}
+
+// Both scatters of a layer, each writing its gradient whole.  One launch (inf_backward_both_kernel) for the fully
+// connected layout when each scatter is a single k range and grad_weight needs no split over the images; otherwise
+// the two launches of the separate entry points.
+hipError_t inf_backward_both(const float* grad_output, const int32_t* pos, float* grad_input, float* grad_weight,
+                             const Problem& pr, hipStream_t stream) {
+    const int slots_w = kBinBytes / (int)sizeof(float);
+    const int nb = max(1, min(min(pr.NG, 8), slots_w / max(pr.K, 1)));
+    const int real_blocks = (pr.NG + nb - 1) / nb;
+    const int n_blocks = real_blocks >= 64 ? (real_blocks + 7) / 8 * 8 : real_blocks;
+    const long wgs_x = (long)pr.B * pr.G, wgs_w = (long)pr.G * n_blocks;
+    const bool one_launch = pr.HW == 1 && pr.K <= kInputBins && pr.K <= slots_w &&
+                            (long)pr.G * real_blocks >= 2L * pr.num_cu &&   // inf_backward_weight would not split the images
+                            wgs_x + wgs_w < (1L << 31);
+    if (!one_launch) {
+        if (hipError_t e = inf_backward_input(grad_output, pos, grad_input, pr, true, stream); e != hipSuccess) return e;
+        return inf_backward_weight(grad_output, pos, grad_weight, pr, true, stream);
+    }
+    const BwdDims d{pr.B, pr.G, pr.K, pr.NG, pr.HW};
+    BothPlan pl{};
+    pl.wgs_x = (int)wgs_x;
+    pl.wgs_w = (int)wgs_w;
+    pl.th_log2 = 0;
+    pl.kc_x = pr.K;
+    pl.hw_tiles = 1;
+    pl.vec = pr.NG % 4 == 0 && pr.K % 4 == 0 && aligned16(grad_output) && aligned16(pos) && aligned16(grad_input);
+    pl.nb = nb;
+    pl.kc_w = pr.K;
+    pl.n_blocks = n_blocks;
+    const size_t lds = std::max((size_t)pr.K * sizeof(double), (size_t)nb * pr.K * sizeof(float));
+    hipLaunchKernelGGL(inf_backward_both_kernel, dim3((unsigned)(wgs_x + wgs_w)), dim3(256), lds, stream, grad_output, pos,
+                       grad_input, grad_weight, d, pl);
     return hipGetLastError();
 }
 

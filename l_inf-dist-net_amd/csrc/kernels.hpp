@@ -80,6 +80,9 @@ hipError_t value_bound_forward(const float* input, const float* lower, const flo
                                const Problem& pr, hipStream_t stream);
 hipError_t bound_forward(const float* lower, const float* upper, const float* weight, float* out_lower,
                          float* out_upper, const Problem& pr, hipStream_t stream);
+// Both L_inf scatters, each gradient written whole; one launch where the layout allows (inf_backward.hip).
+hipError_t inf_backward_both(const float* grad_output, const int32_t* pos, float* grad_input, float* grad_weight,
+                             const Problem& pr, hipStream_t stream);
 hipError_t inf_backward_input(const float* grad_output, const int32_t* pos, float* grad_input, const Problem& pr,
                               bool overwrite, hipStream_t stream);
 hipError_t inf_backward_weight(const float* grad_output, const int32_t* pos, float* grad_weight, const Problem& pr,

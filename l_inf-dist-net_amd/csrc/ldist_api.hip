@@ -179,6 +179,14 @@ int ldist_inf_dist_backward_weight_overwrite(const float* grad_output, const int
     return inf_backward_weight_impl(grad_output, pos, B, CO, CI, G, HW, grad_weight, true, stream);
 }
 
+int ldist_inf_dist_backward_overwrite(const float* grad_output, const int32_t* pos, int B, int CO, int CI, int G, int HW,
+                                      float* grad_input, float* grad_weight, ldist_stream_t stream) {
+    if (!grad_output || !pos || !grad_input || !grad_weight) return LDIST_EINVAL;
+    ldist::Problem pr{};
+    if (int rc = check_dims(B, CO, CI, G, HW, pr)) return rc;
+    return finish(ldist::inf_backward_both(grad_output, pos, grad_input, grad_weight, pr, (hipStream_t)stream));
+}
+
 int ldist_norm_dist_forward(const float* input, const float* weight, int B, int CO, int CI, int G, int HW,
                             float* output, float p, ldist_stream_t stream) {
     if (!input || !weight || !output || !valid_p(p)) return LDIST_EINVAL;

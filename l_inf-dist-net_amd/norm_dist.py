@@ -62,10 +62,13 @@ class DistF(torch.autograd.Function):
         if math.isinf(ctx.p):
             x, weight, _, argmax = ctx.saved_tensors
             # the scatter kernels write every element, zeros included: no fill needed here
-            if want_x:
+            if want_x and want_w:   # one call: a fully connected layer's two scatters share a launch
+                gx, gw = torch.empty_like(x), torch.empty_like(weight)
+                norm_dist_cpp.inf_dist_backward_overwrite(g, argmax, gx, gw, ctx.group)
+            elif want_x:
                 gx = torch.empty_like(x)
                 norm_dist_cpp.inf_dist_backward_input_overwrite(g, argmax, gx, ctx.group)
-            if want_w:
+            elif want_w:
                 gw = torch.empty_like(weight)
                 norm_dist_cpp.inf_dist_backward_weight_overwrite(g, argmax, gw, ctx.group)
         else:

@@ -226,6 +226,22 @@ def inf_dist_backward_weight_overwrite(grad_output, pos, grad_weight, G):
     _inf_backward_weight("ldist_inf_dist_backward_weight_overwrite", grad_output, pos, grad_weight, G)
 
 
+def inf_dist_backward_overwrite(grad_output, pos, grad_input, grad_weight, G):
+    """Both L_inf gradients in one call, each written whole (what inf_dist_backward_input_overwrite followed by
+    inf_dist_backward_weight_overwrite computes): for a fully connected layer the two scatters share one launch."""
+    _check_input(grad_output, "grad_output")
+    _check_input(pos, "pos", torch.int32)
+    _check_input(grad_input, "grad_input")
+    _check_input(grad_weight, "grad_weight")
+    dev = _same_device(grad_output, pos, grad_input, grad_weight)
+    B, CO, CI, HW = grad_output.size(0), grad_output.size(1), grad_input.size(1), grad_input.size(2)
+    _expect(tuple(pos.shape) == tuple(grad_output.shape), "pos must match grad_output")
+    _expect(grad_input.size(0) == B and grad_output.size(2) == HW, "grad_input must be (B, CI, HW)")
+    _expect(grad_weight.size(0) == CO and grad_weight.size(1) * G == CI, "grad_weight must be (CO, CI/G)")
+    _call("ldist_inf_dist_backward_overwrite", dev, _p(grad_output), _p(pos), B, CO, CI, G, HW, _p(grad_input),
+          _p(grad_weight))
+
+
 def mean_shift(x, y, mean_out=None, running_mean=None, momentum=0.0):
     """y = x minus its per-channel mean over dims 0 and 2 of a (B, C, L) tensor, in one kernel.
 

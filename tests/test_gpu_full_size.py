@@ -58,6 +58,13 @@ def test_config1_hidden_layer_forward_and_backward(ci):
     mx, mw = _scatter_magnitudes(go, ep, ci, 1)
     assert_sum_close(gx.cpu(), oracle.inf_dist_backward_input(go, ep, ci, 1), mx)
     assert_sum_close(gw.cpu(), oracle.inf_dist_backward_weight(go, ep, ci, 1), mw)
+    # both gradients in one call: at this size one launch whose workgroups do either scatter
+    gx2 = torch.full((512, ci, 1), float("nan"), device=DEV)
+    gw2 = torch.full((5120, ci), float("nan"), device=DEV)
+    cpp.inf_dist_backward_overwrite(go.to(DEV), pos.to(DEV), gx2, gw2, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(gx2, gx)     # double bins: the rounded sums do not depend on the order of the additions
+    assert_sum_close(gw2.cpu(), oracle.inf_dist_backward_weight(go, ep, ci, 1), mw)
 
 
 def test_config1_head_forward_bit_exact():

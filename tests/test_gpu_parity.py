@@ -95,6 +95,29 @@ def test_norm_dist_without_a_gradient_takes_the_values_only_forward():
     assert wr.grad is not None and bool((wr.grad != 0).any())
 
 
+@pytest.mark.parametrize("shape", [(70, 4104, 36, 1, 1), (300, 4096, 784, 1, 1), (33, 1600, 5120, 1, 1), (16, 2064, 100, 2, 1),
+                                   (40, 96, 64, 1, 1), (3, 24, 18, 3, 4)])
+def test_inf_backward_both_gradients_in_one_call(shape):
+    """inf_dist_backward_overwrite against the oracle.  The first four shapes run as one launch whose workgroups do
+    either scatter (fc layout, enough blocks of output rows to fill the device; ragged blocks, groups, K = 5120 with
+    three rows of bins per workgroup); the last two fall back to the two kernels inside the call."""
+    from gpu_common import DEV, cpp, say
+    B, CO, CI, G, HW = shape
+    say("inf_backward both", shape)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=sum(shape), quantize=8)   # quantised: ties and shared maxima
+    _, ep = oracle.inf_dist_forward(x, w, G)
+    go = torch.randn(B, CO, HW, generator=gen(77))
+    gx = torch.full((B, CI, HW), float("nan"), device=DEV)
+    gw = torch.full((CO, CI // G), float("nan"), device=DEV)
+    cpp.inf_dist_backward_overwrite(go.to(DEV), ep.to(DEV), gx, gw, G)
+    torch.cuda.synchronize()
+    SIGN = -(1 << 31)
+    tx = oracle.inf_dist_backward_input(go.abs(), ep & ~SIGN, CI, G).abs()
+    tw = oracle.inf_dist_backward_weight(go.abs(), ep & ~SIGN, CI, G).abs()
+    assert_sum_close(gx.cpu(), oracle.inf_dist_backward_input(go, ep, CI, G), tx, None, RTOL, ATOL)
+    assert_sum_close(gw.cpu(), oracle.inf_dist_backward_weight(go, ep, CI, G), tw, None, RTOL, ATOL)
+
+
 def test_conv_layer_without_a_gradient_takes_the_values_only_forward():
     """NormDistConv at p = inf in evaluation under torch.no_grad(): the same output as with gradients enabled
     (which records the argmax), from the kernel without pos."""

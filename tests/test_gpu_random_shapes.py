@@ -76,6 +76,11 @@ def test_random_problem(seed):
     tw = oracle.inf_dist_backward_weight(go.abs(), ep & ~SIGN, CI, G).abs()
     assert_sum_close(gx.cpu(), oracle.inf_dist_backward_input(go, ep, CI, G), tx, rtol=RTOL, atol=ATOL)
     assert_sum_close(gw.cpu(), oracle.inf_dist_backward_weight(go, ep, CI, G), tw, rtol=RTOL, atol=ATOL)
+    gx2 = torch.full((B, CI, HW), float("nan"), device=DEV)     # both in one call
+    gw2 = torch.full((CO, CI // G), float("nan"), device=DEV)
+    cpp.inf_dist_backward_overwrite(go.to(DEV), ep.to(DEV), gx2, gw2, G)
+    assert_sum_close(gx2.cpu(), oracle.inf_dist_backward_input(go, ep, CI, G), tx, rtol=RTOL, atol=ATOL)
+    assert_sum_close(gw2.cpu(), oracle.inf_dist_backward_weight(go, ep, CI, G), tw, rtol=RTOL, atol=ATOL)
 
     want = oracle.norm_dist_forward(x, w, G, p)
     torch.testing.assert_close(gpu_norm_forward(x, w, G, p), want, rtol=RTOL, atol=0)

@@ -47,6 +47,11 @@ def fake_native(monkeypatch):
         calls.append("inf_dist_backward_weight_overwrite")
         gw.copy_(oracle.inf_dist_backward_weight(go, pos, gw.size(1) * G, G))
 
+    def bwd_both_over(go, pos, gi, gw, G):
+        calls.append("inf_dist_backward_overwrite (input and weight)")
+        gi.copy_(oracle.inf_dist_backward_input(go, pos, gi.size(1), G))
+        gw.copy_(oracle.inf_dist_backward_weight(go, pos, gw.size(1) * G, G))
+
     def norm_dist_forward(x, w, out, G, p):
         calls.append("norm_dist_forward")
         out.copy_(oracle.norm_dist_forward(x.contiguous(), w.contiguous(), G, p))
@@ -70,7 +75,8 @@ def fake_native(monkeypatch):
     for name, fn in [("inf_dist_forward", inf_dist_forward), ("inf_dist_forward_values", inf_dist_forward_values),
                      ("inf_dist_bound_forward", inf_dist_bound_forward),
                      ("inf_dist_backward_input_overwrite", bwd_in_over),
-                     ("inf_dist_backward_weight_overwrite", bwd_w_over), ("norm_dist_forward", norm_dist_forward),
+                     ("inf_dist_backward_weight_overwrite", bwd_w_over), ("inf_dist_backward_overwrite", bwd_both_over),
+                     ("norm_dist_forward", norm_dist_forward),
                      ("norm_dist_backward_input", norm_bwd_in), ("norm_dist_backward_weight", norm_bwd_w)]:
         monkeypatch.setattr(cpp, name, fn)
     return calls
@@ -450,12 +456,12 @@ def test_stack_checker_passes_on_a_correct_net_and_catches_a_wrong_one(fake_nati
     assert not bad.ok and any("values" in f for f in bad.failures)
 
     # a wrong gradient: grad_weight scaled
-    wname = "inf_dist_backward_weight_overwrite" if math.isinf(p) else "norm_dist_backward_weight"
+    wname = "inf_dist_backward_overwrite" if math.isinf(p) else "norm_dist_backward_weight"   # both gradients are wanted
     good_w = getattr(cpp, wname)
 
     def off_grad(*a):
         good_w(*a)
-        (a[2] if math.isinf(p) else a[4]).mul_(1.001)
+        (a[3] if math.isinf(p) else a[4]).mul_(1.001)   # the grad_weight argument of either call
     setattr(cpp, wname, off_grad)
     try:
         bad = stack_check.check_training_step(model, x, up, p, torch.device("cpu"))
