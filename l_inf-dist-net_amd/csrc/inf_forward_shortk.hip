@@ -17,12 +17,15 @@
 // the lane that finishes an output reads the four pairs in ascending order of k ("strictly larger wins",
 // which keeps the lowest k on ties).
 // LDS: X[k][64 rows] and W[k][32 outputs] (k-major), plus 40 KB of slabs; K = 288 (a 3x3 window over 32
-// channels) takes 148 KB.  The weight panel is loaded once per run of tiles that share it.  The input panel
-// of the next tile is loaded into registers before the current tile's arithmetic and written to LDS after
-// its epilogue, so the loads wait behind a whole tile of arithmetic.  The input is row-contiguous in memory
-// and goes in with 128-bit stores.  The weights are read along k with coalesced 32-bit loads, four
-// neighbouring outputs per lane, and stored as one 128-bit word (the lanes of such a store differ in k and
-// meet in few banks; it happens once per run of tiles, and plain rows let every later read of the panel use
+// channels) takes 148 KB.  The weight panel is loaded once per run of tiles that share it.
+// During the reduction nobody but the wave itself reads its block of the input panel (its 32 rows, its k range),
+// so every wave brings in its own block: a window of the block (8 k x 32 rows) is one 128-bit load per lane.  The
+// loads of the next tile's block stay parked in registers for a whole tile; the wave writes a window to LDS one
+// window ahead of reducing it and at once reuses the registers for the same window of the tile after that.  So
+// the panel is written and the loads are issued a few instructions at a time, in the shadow of the arithmetic,
+// and no barrier stands between them and the reduction.  The weights are read along k with coalesced 32-bit
+// loads, four neighbouring outputs per lane, and stored as one 128-bit word (the lanes of such a store differ in
+// k and meet in few banks; it happens once per run of tiles, and plain rows let every later read of the panel use
 // one address register and constant offsets).
 #include "fwd_engine.hpp"
 
@@ -31,9 +34,7 @@ namespace ldist {
 namespace shortk {
 constexpr int BM = 64, BN = 32, NT = 512, NGROUP = 4, WIN = 8;
 constexpr int KQ = NGROUP * WIN;                  // K is padded to a multiple of this
-constexpr int XROWS = NT / (BM / 4);              // k rows of the input panel that one pass of the workgroup loads
-constexpr int MAXPASS = 10;                       // padded K / 32 the kernel is built for: K <= 320
-static_assert(XROWS == KQ, "one pass loads one padding quantum of k");
+constexpr int MAXWIN = 10;                        // windows per k range the kernel is built for: K <= 320
 inline int padded_k(int K) { return (K + KQ - 1) / KQ * KQ; }
 // panels, four value slabs (float) and four window slabs (one byte per output: at most 40 windows)
 inline size_t lds_bytes(int Kp) { return ((size_t)Kp * (BM + BN) + NGROUP * BM * BN) * sizeof(float) + NGROUP * BM * BN; }
@@ -49,15 +50,14 @@ __device__ __forceinline__ constexpr int cslot(int n, int m) {
 __device__ __forceinline__ constexpr int bslot(int n, int m) { return (((m >> 2) * BN + (n ^ ((m >> 3) & 3))) << 2) | (m & 3); }
 }  // namespace shortk
 
-// Kp = padded K.  Kp / 32 is the number of windows per k range and also the number of passes in which the
-// workgroup loads an input panel; NP >= Kp / 32 is how many of them the kernel is built for (the loads are
-// issued as one straight run: no branch between them, so nothing waits until the panel is written).
-template <int NP>
+// NW = windows per k range = padded K / 32; the window loop is unrolled over it, so that the parked loads are
+// named registers and no branch stands between a load and the write that waits for it.
+template <int NW>
 __global__ void __launch_bounds__(shortk::NT, 2)
 inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restrict__ weight,
-                          float* __restrict__ output, int32_t* __restrict__ pos, Dims d, int Kp, int tiles_total) {
+                          float* __restrict__ output, int32_t* __restrict__ pos, Dims d, int tiles_total) {
     using namespace shortk;
-    const int npass = Kp / KQ, nwin = npass, Kg = Kp / NGROUP;
+    constexpr int Kp = NW * KQ, nwin = NW, Kg = NW * WIN;
     extern __shared__ __align__(16) float lds[];
     float* X = lds;                         // [Kp][BM]
     float* W = lds + (size_t)Kp * BM;       // [Kp][BN]
@@ -74,37 +74,43 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
     const int t_begin = blockIdx.x, t_step = gridDim.x, t_end = tiles_total;
     if (t_begin >= t_end) return;           // the whole workgroup leaves together
 
-    // input panel: a lane keeps its four rows (consecutive positions of one image: HW % 4 == 0) and walks k
-    const int lmq = tid % (BM / 4), lkx = tid / (BM / 4);
-    float4 park[NP];
+    const int lane = tid & 63, wave = tid >> 6;
+    const int half = wave / NGROUP, grp = wave % NGROUP;
+    const int tx = lane % 8, ty = lane / 8;
+
+    // The wave's block of the input panel: rows half*32.. of the tile, k in [grp*Kg, (grp+1)*Kg).  In pass p a lane
+    // takes four rows (consecutive positions of one image: HW % 4 == 0) at k = grp*Kg + 8 p + lane / 8.
+    const int lrow = half * 32 + (lane % 8) * 4, lk = grp * Kg + lane / 8;
+    float4 park[NW];
     // Buffer loads: the descriptor of the whole input in scalar registers, the lane's byte offset of (its four rows,
-    // k = lkx) of the tile in one register, the pass's k rows as the scalar offset.  An offset of all ones lies outside
-    // the descriptor's 2 GB range and reads as zeros: that is how rows past M, k past K in the last pass and the passes
-    // beyond Kp / 32 come out as zeros, without a branch, a predicate or a select when the panel is written (the host
-    // checks that the input is smaller than 2 GB).
+    // k = lk) of the tile in one register, the pass's k rows as the scalar offset.  An offset of all ones lies outside
+    // the descriptor's 2 GB range and reads as zeros: that is how rows past M, k past K and the tile after the last
+    // come out as zeros, without a branch or a predicate (the host checks that the input is smaller than 2 GB).
     typedef float F4 __attribute__((ext_vector_type(4)));
     const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(input), 0, (int)0x80000000u, 0x00020000);
-    auto x_offset = [&](int t) -> unsigned {
-        const int tm = t % d.tiles_m, g = (t / d.tiles_m) / d.tiles_n;
-        const int m = tm * BM + lmq * 4;
-        if (m >= d.M) return ~0u;                // HW % 4 == 0: four rows are inside the tensor together
-        const int b = m / HW, hw = m % HW;
-        return (unsigned)((((size_t)(b * d.G + g) * K + lkx) * HW + hw) * sizeof(float));
-    };
-    auto issue_x = [&](int t) {
-        const unsigned off = x_offset(t), off_last = lkx + (npass - 1) * XROWS < K ? off : ~0u;
-#pragma unroll
-        for (int p = 0; p < NP; p++) {
-            const unsigned o = p < npass - 1 ? off : (p == npass - 1 ? off_last : ~0u);
-            const F4 v = __builtin_bit_cast(F4, __builtin_amdgcn_raw_buffer_load_b128(xrs, o, p * XROWS * HW * (int)sizeof(float), 0));
-            park[p] = make_float4(v.x, v.y, v.z, v.w);
+    // k of this range that exist: whole passes below p_full, lanes with lane / 8 < rem in pass p_full, none above
+    const int k_valid = min(max(K - grp * Kg, 0), Kg), p_full = k_valid / WIN, rem = k_valid % WIN;
+    struct Offsets { unsigned all, edge; };
+    auto x_offsets = [&](int t) -> Offsets {
+        Offsets o = {~0u, ~0u};
+        if (t < t_end) {
+            const int tm = t % d.tiles_m, g = (t / d.tiles_m) / d.tiles_n;
+            const int m = tm * BM + lrow;
+            if (m < d.M) {                       // HW % 4 == 0: four rows are inside the tensor together
+                const int b = m / HW, hw = m % HW;
+                o.all = (unsigned)((((size_t)(b * d.G + g) * K + lk) * HW + hw) * sizeof(float));
+                if (lane / 8 < rem) o.edge = o.all;
+            }
         }
+        return o;
     };
-    auto store_x = [&](int) {
-#pragma unroll
-        for (int p = 0; p < NP; p++)
-            if (p < npass) *reinterpret_cast<float4*>(X + (lkx + p * XROWS) * BM + lmq * 4) = park[p];
+    auto issue_pass = [&](int p, const Offsets& o) {
+        const unsigned off = p < p_full ? o.all : (p == p_full ? o.edge : ~0u);
+        const F4 v = __builtin_bit_cast(F4, __builtin_amdgcn_raw_buffer_load_b128(xrs, off, p * WIN * HW * (int)sizeof(float), 0));
+        park[p] = make_float4(v.x, v.y, v.z, v.w);
     };
+    float* const xblock = X + (size_t)lk * BM + lrow;
+    auto store_pass = [&](int p) { *reinterpret_cast<float4*>(xblock + p * WIN * BM) = park[p]; };
     // weight panel of (group g, output tile tn): lanes run along k, a lane takes four neighbouring outputs
     auto load_w = [&](int g, int tn) {
         const int n0 = tn * BN;
@@ -138,14 +144,8 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
         }
     };
 
-    const int lane = tid & 63, wave = tid >> 6;
-    const int half = wave / NGROUP, grp = wave % NGROUP;
-    const int tx = lane % 8, ty = lane / 8;
-
     // Tile -> global, from slabs 0 and 1: a lane stores four neighbouring rows of one output with 128-bit stores.
-    // A tile's results go out at the start of the next tile, after that tile's input panel has been written to
-    // LDS and the loads of the panel after it are on their way: the wait for parked loads (the counter also covers
-    // stores) then only ever waits for loads that are older than the stores.
+    // A tile's results go out at the start of the next tile.
     auto flush = [&](int t) {
         const int tm = t % d.tiles_m, wkey = t / d.tiles_m;
         const int tn = wkey % d.tiles_n, g = wkey / d.tiles_n;
@@ -161,27 +161,25 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
     };
 
     int w_loaded = -1;
-    issue_x(t_begin);
+    {
+        const Offsets first = x_offsets(t_begin);
+#pragma unroll
+        for (int p = 0; p < NW; p++) issue_pass(p, first);
+    }
 #pragma unroll 1
     for (int t = t_begin; t < t_end; t += t_step) {
         const int wkey = t / d.tiles_m;
         if (wkey != w_loaded) {   // every lane of the previous tile is past its epilogue
             load_w(wkey / d.tiles_n, wkey % d.tiles_n);
             w_loaded = wkey;
+            __syncthreads();
         }
-        store_x(t);
-        __syncthreads();
-        // The next tile's panel, parked in registers until this tile is done.  The loads go out before the stores of
-        // the flush: behind them they would first wait until the stores have read the registers they share.
-        // The load unit takes some thirty clocks per load of a wave, and a wave that issues loads does nothing else: the
-        // upper half's waves issue theirs here, the lower half's waves in the middle of their reduction, so that on
-        // every SIMD one of its two waves computes while the other queues loads.
-        const bool more = t + t_step < t_end;
-        if (more && half == 0) issue_x(t + t_step);
-        if (t > t_begin) {
-            flush(t - t_step);
-            __syncthreads();      // the slabs are read before any wave of this tile parks its patch there
-        }
+        const Offsets next = x_offsets(t + t_step);      // all ones behind the last tile: those loads read zeros
+        // The first window's write waits for this tile's parked loads, all of them a window old or older.  The flush
+        // comes after it: the wait counts stores too, and behind the flush it would wait for those.
+        store_pass(0);
+        issue_pass(0, next);
+        if (t > t_begin) flush(t - t_step);
 
         // ---- the reduction: the wave takes rows half*32.. of the tile and k in [grp*Kg, (grp+1)*Kg) --------
         float accA[4][4], accB[4][4];
@@ -254,20 +252,18 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
             }
         };
         fetch(xa, wa, 0);
-        const int w_issue = (nwin / 2) & ~1;
-#pragma unroll 1
-        for (int w = 0; w < nwin; w += 2) {
-            if (more && half == 1 && w == w_issue) issue_x(t + t_step);
-            window(accA, accB, w);
-            if (w + 1 < nwin) {
-                window(accB, accA, w + 1);
-            } else {
+        // Window w + 1 of the block goes to LDS, and its registers take the same window of the next tile, before
+        // window w is reduced: the reads of window w + 1 start in the last quarter of window w.
 #pragma unroll
-                for (int i = 0; i < 4; i++)
-#pragma unroll
-                    for (int j = 0; j < 4; j++) accA[i][j] = accB[i][j];
+        for (int w = 0; w < NW; w++) {
+            if (w + 1 < NW) {
+                store_pass(w + 1);
+                issue_pass(w + 1, next);
             }
+            if (w % 2 == 0) window(accA, accB, w); else window(accB, accA, w);
         }
+        float (&acc)[4][4] = NW % 2 == 1 ? accB : accA;   // where the last window left the maxima
+        __syncthreads();      // every lane has read the previous tile's results (flush) out of slabs 0 and 1
 
         // ---- every wave parks its patch in the slab of its k range: values as 128-bit words of four rows, windows
         // (counted inside the range: they fit a byte) as one word of four rows
@@ -277,7 +273,7 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const int n = tx * 4 + j, m = half * 32 + ty * 4;
-                *reinterpret_cast<float4*>(sv + cslot(n, m)) = make_float4(accA[0][j], accA[1][j], accA[2][j], accA[3][j]);
+                *reinterpret_cast<float4*>(sv + cslot(n, m)) = make_float4(acc[0][j], acc[1][j], acc[2][j], acc[3][j]);
                 sw[bslot(n, m) >> 2] = (unsigned)widx[0][j] | ((unsigned)widx[1][j] << 8) | ((unsigned)widx[2][j] << 16) |
                                        ((unsigned)widx[3][j] << 24);
             }
@@ -362,17 +358,16 @@ bool inf_forward_shortk_applicable(const Problem& pr, const void* input, const v
     if (!aligned16(input) || !aligned16(output) || !aligned16(pos)) return false;
     if ((size_t)pr.B * pr.G * pr.K * pr.HW * sizeof(float) >= (size_t)1 << 31) return false;   // 32-bit buffer offsets
     const int Kp = shortk::padded_k(pr.K);
-    return Kp / shortk::XROWS <= shortk::MAXPASS && Kp / (shortk::NGROUP * shortk::WIN) <= 255 &&
-           shortk::lds_bytes(Kp) <= 160 * 1024;
+    return Kp / shortk::KQ <= shortk::MAXWIN && shortk::lds_bytes(Kp) <= 160 * 1024;
 }
 
-template <int NP>
+template <int NW>
 static hipError_t launch_shortk(unsigned grid, size_t lds, int device, hipStream_t stream, const float* input,
-                                const float* weight, float* output, int32_t* pos, const Dims& d, int Kp, int tiles) {
+                                const float* weight, float* output, int32_t* pos, const Dims& d, int tiles) {
     static LdsRecord lds_allowed = {};
-    if (hipError_t e = allow_lds(inf_forward_shortk_kernel<NP>, 160 * 1024, device, lds_allowed); e != hipSuccess) return e;
-    hipLaunchKernelGGL(inf_forward_shortk_kernel<NP>, dim3(grid), dim3(shortk::NT), lds, stream, input, weight, output,
-                       pos, d, Kp, tiles);
+    if (hipError_t e = allow_lds(inf_forward_shortk_kernel<NW>, 160 * 1024, device, lds_allowed); e != hipSuccess) return e;
+    hipLaunchKernelGGL(inf_forward_shortk_kernel<NW>, dim3(grid), dim3(shortk::NT), lds, stream, input, weight, output,
+                       pos, d, tiles);
     return hipGetLastError();
 }
 
@@ -386,15 +381,15 @@ hipError_t inf_forward_shortk(const float* input, const float* weight, float* ou
     // one workgroup per CU
     const long tiles = (long)d.tiles_m * d.tiles_n * d.G;
     const unsigned grid = (unsigned)(tiles < pr.num_cu ? tiles : pr.num_cu);
-    const int np = Kp / shortk::KQ;
-#define LDIST_SHORTK(NP) \
-    return launch_shortk<NP>(grid, lds, pr.device, stream, input, weight, output, pos, d, Kp, (int)tiles)
-    if (np <= 2) LDIST_SHORTK(2);
-    if (np <= 4) LDIST_SHORTK(4);
-    if (np <= 6) LDIST_SHORTK(6);
-    if (np <= 9) LDIST_SHORTK(9);
-    LDIST_SHORTK(shortk::MAXPASS);
+#define LDIST_SHORTK(NW) \
+    case NW: return launch_shortk<NW>(grid, lds, pr.device, stream, input, weight, output, pos, d, (int)tiles)
+    switch (Kp / shortk::KQ) {
+        LDIST_SHORTK(1); LDIST_SHORTK(2); LDIST_SHORTK(3); LDIST_SHORTK(4); LDIST_SHORTK(5);
+        LDIST_SHORTK(6); LDIST_SHORTK(7); LDIST_SHORTK(8); LDIST_SHORTK(9); LDIST_SHORTK(10);
+    }
 #undef LDIST_SHORTK
+    static_assert(shortk::MAXWIN == 10, "one case per window count");
+    return hipErrorInvalidValue;   // not reached: inf_forward_shortk_applicable() admits ten windows at most
 }
 
 }  // namespace ldist
