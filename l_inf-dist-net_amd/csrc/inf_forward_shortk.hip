@@ -81,13 +81,23 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
     // The wave's block of the input panel: rows half*32.. of the tile, k in [grp*Kg, (grp+1)*Kg).  In pass p a lane
     // takes four rows (consecutive positions of one image: HW % 4 == 0) at k = grp*Kg + 8 p + lane / 8.
     const int lrow = half * 32 + (lane % 8) * 4, lk = grp * Kg + lane / 8;
-    float4 park[NW];
+    typedef float F4 __attribute__((ext_vector_type(4)));
+    typedef int I4 __attribute__((ext_vector_type(4)));
+    F4 park[NW];
     // Buffer loads: the descriptor of the whole input in scalar registers, the lane's byte offset of (its four rows,
     // k = lk) of the tile in one register, the pass's k rows as the scalar offset.  An offset of all ones lies outside
     // the descriptor's 2 GB range and reads as zeros: that is how rows past M, k past K and the tile after the last
     // come out as zeros, without a branch or a predicate (the host checks that the input is smaller than 2 GB).
-    typedef float F4 __attribute__((ext_vector_type(4)));
-    const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(input), 0, (int)0x80000000u, 0x00020000);
+    // The loads and the waits for them are written out (inline assembly): the compiler's own wait in front of the
+    // first panel write of a tile was for all outstanding loads, the youngest of which is two windows old, and
+    // the tail of the memory latency showed (0.29 ms against 0.27 ms with the same loads served from L2).  Written
+    // out, every panel write waits for its own load only: when pass p of a tile is written, the passes behind it, the
+    // next tile's pass 0 and that tile's passes up to p have been issued since -- NW - 1 loads, at every p and for
+    // the first tile too (its loads go out in one run before the loop), plus at most the two stores of a flush.  So
+    // "at most NW - 1 memory operations outstanding" means the load has returned; the loads of load_w() are issued and
+    // waited for while all of these are older, which keeps the compiler's own counts for them on the safe side.
+    const unsigned long long xbase = reinterpret_cast<unsigned long long>(input);
+    const I4 xrs = {(int)(unsigned)xbase, (int)(unsigned)((xbase >> 32) & 0xffffu), (int)0x80000000u, 0x00020000};
     // k of this range that exist: whole passes below p_full, lanes with lane / 8 < rem in pass p_full, none above
     const int k_valid = min(max(K - grp * Kg, 0), Kg), p_full = k_valid / WIN, rem = k_valid % WIN;
     struct Offsets { unsigned all, edge; };
@@ -106,11 +116,15 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
     };
     auto issue_pass = [&](int p, const Offsets& o) {
         const unsigned off = p < p_full ? o.all : (p == p_full ? o.edge : ~0u);
-        const F4 v = __builtin_bit_cast(F4, __builtin_amdgcn_raw_buffer_load_b128(xrs, off, p * WIN * HW * (int)sizeof(float), 0));
-        park[p] = make_float4(v.x, v.y, v.z, v.w);
+        asm volatile("buffer_load_dwordx4 %0, %1, %2, %3 offen"
+                     : "=v"(park[p])
+                     : "v"(off), "s"(xrs), "s"(p * WIN * HW * (int)sizeof(float)));
     };
     float* const xblock = X + (size_t)lk * BM + lrow;
-    auto store_pass = [&](int p) { *reinterpret_cast<float4*>(xblock + p * WIN * BM) = park[p]; };
+    auto store_pass = [&](int p) {
+        asm volatile("s_waitcnt vmcnt(%1)" : "+v"(park[p]) : "n"(NW - 1));
+        *reinterpret_cast<F4*>(xblock + p * WIN * BM) = park[p];
+    };
     // weight panel of (group g, output tile tn): lanes run along k, a lane takes four neighbouring outputs
     auto load_w = [&](int g, int tn) {
         const int n0 = tn * BN;
@@ -348,6 +362,7 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
         }
         __syncthreads();   // the panels are free for the next tile; its results wait in the merge area
     }
+    asm volatile("s_waitcnt vmcnt(0)");   // the loads issued for the tile after the last (zeros) have landed before the wave ends
     flush(t_begin + (t_end - 1 - t_begin) / t_step * t_step);
 }
 
