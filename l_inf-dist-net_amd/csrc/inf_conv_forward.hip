@@ -187,12 +187,12 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
     const int xlane_off = (hr * S) * WP + w0 * S;              // + (c*NR + i)*WP: 16-byte aligned (WP % 4 == 0)
     const float* xlane = tile + xlane_off;
 
-    float acc[kTM][kTN];
+    float acc[kTM][kTN], cm[kTM][kTN];   // running maxima; the units alternate between them
     int unit[kTM][kTN];
 #pragma unroll
     for (int e = 0; e < kTM; e++)
 #pragma unroll
-        for (int t = 0; t < kTN; t++) { acc[e][t] = 0.f; unit[e][t] = 0; }
+        for (int t = 0; t < kTN; t++) { acc[e][t] = 0.f; cm[e][t] = 0.f; unit[e][t] = 0; }
 
     const int nstage = a.CGP / kCC;
     const float* xch = xlane;
@@ -204,58 +204,134 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
         const float* wrow = wst + (ch & 1) * kKC * BNP + kTN * nl;   // walks down the 9*kCC rows of the stage
         // walks down the window rows of the stage's channels
         const float* xrow = RESIDENT ? xch : tile + (ch & 1) * xhalf + xlane_off;
-        // The loops over units, channels and window rows stay rolled: one trip is 6 LDS reads and 144
-        // arithmetic instructions, and its registers are all the compiler has to keep.
-#pragma unroll 1
-        for (int u = 0; u < kCC / kTrack; u++) {
-            float cm[kTM][kTN];   // the unit's maximum; without pos, the running maximum itself
+        static_assert(kTrack == 1 && kCC % 2 == 0, "a unit is a channel; units in pairs");
+        if constexpr (RESIDENT) {
+            // A unit (one channel: nine differences per position and output) continues the running maximum: cur
+            // starts from prev, which is left alone, so the unit raised the maximum iff cur > prev afterwards, and the
+            // two arrays swap roles from unit to unit (no copy, one compare and one select per unit and output).
+            // The loop over pairs of units stays rolled.
+            auto unit_pass = [&](const float (&prev)[kTM][kTN], float (&cur)[kTM][kTN], int un) {
+                // The three window rows of the unit, unrolled, with the reads of a row issued before the arithmetic
+                // of the row before it.
+                struct Row { float x[NXR * 4]; float w[3][kTN]; };
+                auto fetch = [&](Row& f, int r) {
+                    const float* xp = xrow + r * WP;
 #pragma unroll
-            for (int e = 0; e < kTM; e++)
+                    for (int q = 0; q < NXR; q++) {
+                        const float4 v = *reinterpret_cast<const float4*>(xp + 4 * q);
+                        f.x[4 * q] = v.x; f.x[4 * q + 1] = v.y; f.x[4 * q + 2] = v.z; f.x[4 * q + 3] = v.w;
+                    }
 #pragma unroll
-                for (int t = 0; t < kTN; t++) cm[e][t] = POS ? 0.f : acc[e][t];
-            // The 3*kTrack window rows of the unit, unrolled, with the reads of a row issued before the
-            // arithmetic of the row before it.
-            struct Row { float x[NXR * 4]; float w[3][kTN]; };
-            auto fetch = [&](Row& f, int r) {     // r = cc*3 + i: window row i of the unit's channel cc
-                const float* xp = xrow + ((r / 3) * NR + r % 3) * WP;
+                    for (int j = 0; j < 3; j++) {
+                        const float4 w4 = *reinterpret_cast<const float4*>(wrow + (3 * r + j) * BNP);
+                        f.w[j][0] = w4.x; f.w[j][1] = w4.y; f.w[j][2] = w4.z; f.w[j][3] = w4.w;
+                    }
+                };
+                Row fa, fb;
+                fetch(fa, 0);
 #pragma unroll
-                for (int q = 0; q < NXR; q++) {
-                    const float4 v = *reinterpret_cast<const float4*>(xp + 4 * q);
-                    f.x[4 * q] = v.x; f.x[4 * q + 1] = v.y; f.x[4 * q + 2] = v.z; f.x[4 * q + 3] = v.w;
+                for (int r = 0; r < 3; r++) {
+                    Row& now = (r & 1) ? fb : fa;
+                    Row& nxt = (r & 1) ? fa : fb;
+                    if (r + 1 < 3) fetch(nxt, r + 1);
+#pragma unroll
+                    for (int j = 0; j < 3; j++)
+#pragma unroll
+                        for (int e = 0; e < kTM; e++)
+#pragma unroll
+                            for (int t = 0; t < kTN; t++)
+                                cur[e][t] = __builtin_fmaxf(r == 0 && j == 0 ? prev[e][t] : cur[e][t],
+                                                            __builtin_fabsf(now.x[e * S + j] - now.w[j][t]));
                 }
+                xrow += CST;
+                wrow += 9 * BNP;
+                if constexpr (POS) {
+                    // Eight compares into their own scalar register pairs, then their selects: a select straight
+                    // after its compare waits two cycles for the lane mask.  The empty asm statements keep their
+                    // order: the first kind keeps a mask from being folded back into the plain form, the second
+                    // ends a group.
+                    static_assert(kTM % 2 == 0, "rows in pairs");
 #pragma unroll
-                for (int j = 0; j < 3; j++) {
-                    const float4 w4 = *reinterpret_cast<const float4*>(wrow + (3 * r + j) * BNP);
-                    f.w[j][0] = w4.x; f.w[j][1] = w4.y; f.w[j][2] = w4.z; f.w[j][3] = w4.w;
+                    for (int e = 0; e < kTM; e += 2) {
+                        unsigned long long raised[2][kTN];
+#pragma unroll
+                        for (int a2 = 0; a2 < 2; a2++)
+#pragma unroll
+                            for (int t = 0; t < kTN; t++) {
+                                raised[a2][t] = __builtin_amdgcn_fcmpf(cur[e + a2][t], prev[e + a2][t], 2 /* ordered > */);
+                                asm volatile("" : "+s"(raised[a2][t]));
+                            }
+#pragma unroll
+                        for (int a2 = 0; a2 < 2; a2++)
+#pragma unroll
+                            for (int t = 0; t < kTN; t++) {
+                                if (__builtin_amdgcn_inverse_ballot_w64(raised[a2][t])) unit[e + a2][t] = un;
+                                asm volatile("" : "+v"(unit[e + a2][t]));
+                            }
+                    }
                 }
             };
-            Row fa, fb;
-            fetch(fa, 0);
-#pragma unroll
-            for (int r = 0; r < 3 * kTrack; r++) {
-                Row& cur = (r & 1) ? fb : fa;
-                Row& nxt = (r & 1) ? fa : fb;
-                if (r + 1 < 3 * kTrack) fetch(nxt, r + 1);
-#pragma unroll
-                for (int j = 0; j < 3; j++)
-#pragma unroll
-                    for (int e = 0; e < kTM; e++)
-#pragma unroll
-                        for (int t = 0; t < kTN; t++)
-                            cm[e][t] = __builtin_fmaxf(cm[e][t], __builtin_fabsf(cur.x[e * S + j] - cur.w[j][t]));
+#pragma unroll 1
+            for (int u = 0; u < kCC; u += 2) {
+                const int un = ch * kCC + u;
+                unit_pass(acc, cm, un);
+                unit_pass(cm, acc, un + 1);
             }
-            xrow += kTrack * CST;
-            wrow += 9 * kTrack * BNP;
-            const int un = ch * (kCC / kTrack) + u;
+        } else {
+            // The staged variant has no registers to spare for that (it also carries the parked image words of the
+            // next stage; any other arrangement of this loop that was tried spilled): one unit per trip, its maximum
+            // taken from zero and then compared with the running one (compare and two selects per unit and output).
+#pragma unroll 1
+            for (int u = 0; u < kCC / kTrack; u++) {
+                float cm[kTM][kTN];   // the unit's maximum; without pos, the running maximum itself
 #pragma unroll
-            for (int e = 0; e < kTM; e++)
+                for (int e = 0; e < kTM; e++)
 #pragma unroll
-                for (int t = 0; t < kTN; t++)
-                    if constexpr (POS) {
-                        if (cm[e][t] > acc[e][t]) { acc[e][t] = cm[e][t]; unit[e][t] = un; }
-                    } else {
-                        acc[e][t] = cm[e][t];
+                    for (int t = 0; t < kTN; t++) cm[e][t] = POS ? 0.f : acc[e][t];
+                // The 3*kTrack window rows of the unit, unrolled, with the reads of a row issued before the
+                // arithmetic of the row before it.
+                struct Row { float x[NXR * 4]; float w[3][kTN]; };
+                auto fetch = [&](Row& f, int r) {     // r = cc*3 + i: window row i of the unit's channel cc
+                    const float* xp = xrow + ((r / 3) * NR + r % 3) * WP;
+#pragma unroll
+                    for (int q = 0; q < NXR; q++) {
+                        const float4 v = *reinterpret_cast<const float4*>(xp + 4 * q);
+                        f.x[4 * q] = v.x; f.x[4 * q + 1] = v.y; f.x[4 * q + 2] = v.z; f.x[4 * q + 3] = v.w;
                     }
+#pragma unroll
+                    for (int j = 0; j < 3; j++) {
+                        const float4 w4 = *reinterpret_cast<const float4*>(wrow + (3 * r + j) * BNP);
+                        f.w[j][0] = w4.x; f.w[j][1] = w4.y; f.w[j][2] = w4.z; f.w[j][3] = w4.w;
+                    }
+                };
+                Row fa, fb;
+                fetch(fa, 0);
+#pragma unroll
+                for (int r = 0; r < 3 * kTrack; r++) {
+                    Row& cur = (r & 1) ? fb : fa;
+                    Row& nxt = (r & 1) ? fa : fb;
+                    if (r + 1 < 3 * kTrack) fetch(nxt, r + 1);
+#pragma unroll
+                    for (int j = 0; j < 3; j++)
+#pragma unroll
+                        for (int e = 0; e < kTM; e++)
+#pragma unroll
+                            for (int t = 0; t < kTN; t++)
+                                cm[e][t] = __builtin_fmaxf(cm[e][t], __builtin_fabsf(cur.x[e * S + j] - cur.w[j][t]));
+                }
+                xrow += kTrack * CST;
+                wrow += 9 * kTrack * BNP;
+                const int un = ch * (kCC / kTrack) + u;
+#pragma unroll
+                for (int e = 0; e < kTM; e++)
+#pragma unroll
+                    for (int t = 0; t < kTN; t++)
+                        if constexpr (POS) {
+                            if (cm[e][t] > acc[e][t]) { acc[e][t] = cm[e][t]; unit[e][t] = un; }
+                        } else {
+                            acc[e][t] = cm[e][t];
+                        }
+            }
         }
         xch += kCC * CST;
         if (ch + 1 < nstage) {
