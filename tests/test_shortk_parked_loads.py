@@ -97,10 +97,14 @@ def test_no_read_of_a_parked_register_before_its_wait(tmp_path):
     cmd = ["hipcc", "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
            "-packed-fp32-ops", "-S", "--cuda-device-only", "-I", os.path.join(ROOT, "include"), SRC, "-o", str(out)]
     subprocess.run(cmd, check=True, capture_output=True)
-    found = kernels(out.read_text())
+    asm = out.read_text()
+    found = kernels(asm)
     assert sorted(found) == list(range(1, 11))
     for nw, lines in found.items():
         check_kernel(nw, lines)
+    # the window loop is unrolled over the parked registers: none of them may have gone to scratch memory
+    spills = re.findall(r"\.vgpr_spill_count:\s*(\d+)", asm)
+    assert len(spills) == 10 and all(int(n) == 0 for n in spills), spills
 
 
 def test_the_check_itself_flags_an_early_read():
