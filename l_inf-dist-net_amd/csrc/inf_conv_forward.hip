@@ -13,10 +13,10 @@
 //   staged    CC channels at a time travel through a second double-buffered stage beside the weights.
 // A lane owns 8 neighbouring positions of one output row times 4 outputs.  For a window row (c, i) it reads the
 // 8 + 2 pixels its positions cover for j = 0, 1, 2 with three (stride 2: five) aligned 128-bit reads, so 12 LDS
-// words serve 24 differences.  The loop keeps the maximum per channel and records the channel of the running
-// maximum (subtract + half a v_max3 per difference, three instructions per channel and output); the lowest k
-// inside the recorded channel is found afterwards from nine pixels (LDS when RESIDENT, else the image in
-// global memory) and the channel's nine contiguous weights.
+// words serve 24 differences.  The loop takes the running maximum through a channel and records the channel where
+// that raised it (subtract + half a v_max3 per difference, two instructions per channel and output, three in the
+// staged variant); the lowest k inside the recorded channel is found afterwards from nine pixels (LDS when
+// RESIDENT, else the image in global memory) and the channel's nine contiguous weights.
 #include "conv_image.hpp"
 
 namespace ldist {
