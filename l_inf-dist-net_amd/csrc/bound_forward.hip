@@ -177,6 +177,7 @@ bound_forward_skinny_kernel(const float* __restrict__ lower, const float* __rest
 
 template <class GEO, bool CONV, int VEC>
 struct BoundForward {
+    static constexpr int X_PANELS = 2;   // lower and upper
     static hipError_t launch(unsigned grid, const Dims& d, int device, hipStream_t stream, const float* lower,
                              const float* upper, const float* weight, float* out_lower, float* out_upper) {
         const size_t lds = Stager<GEO, CONV, VEC, 2>::LDS_BYTES;

@@ -226,7 +226,28 @@ inline bool can_vec4_out(const Problem& pr, const void* a, const void* b = nullp
     return aligned16(a) && aligned16(b) && (pr.HW == 1 ? pr.NG % 4 == 0 : pr.HW % 4 == 0);
 }
 
-inline Dims make_dims(const Problem& pr) { return Dims{pr.B, pr.G, pr.K, pr.NG, pr.HW, pr.B * pr.HW, 0, 0, 0, g_xcd_remap}; }
+inline Dims make_dims(const Problem& pr) { return Dims{pr.B, pr.G, pr.K, pr.NG, pr.HW, pr.B * pr.HW, 0, 0, 0, g_xcd_remap, 0}; }
+
+// Dims::m_block for a kernel whose workgroup reads x_rows rows of the input panels (BM times the number of panels)
+// and w_rows rows of weights per stage: `resident` workgroups share an L2 at a time (workgroups per CU times the CUs
+// of an XCD); among the divisors mb of tiles_m, the piece mb x (resident / mb) with the fewest rows to stream wins.
+// 0 (walk all row tiles) when that is the best there is.
+inline int choose_m_block(int tiles_m, int x_rows, int w_rows, int resident) {
+    int best = tiles_m;
+    long best_cost = -1;
+    for (int mb = 1; mb <= tiles_m && mb <= resident; mb++) {
+        if (tiles_m % mb) continue;
+        const long cost = (long)mb * x_rows + (long)((resident + mb - 1) / mb) * w_rows;
+        if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = mb; }
+    }
+    return best >= tiles_m ? 0 : best;
+}
+// workgroups of nt lanes and lds bytes that a CU holds (two waves per SIMD: these kernels use up to 256 registers)
+inline int resident_per_xcd(int nt, size_t lds, int num_cu) {
+    const int by_lds = (int)((size_t)160 * 1024 / (lds ? lds : 1)), by_waves = 512 / nt;
+    const int per_cu = by_lds < by_waves ? by_lds : by_waves;
+    return (per_cu > 0 ? per_cu : 1) * (num_cu / 8 > 0 ? num_cu / 8 : 1);
+}
 
 // 128-bit loads of the inputs and weights.  In the fc layout a lane addresses its vectors by 32-bit byte offsets
 // from its tile's first row that must stay below 2 GB (RowsK::init_clamped): at most 256 rows of G * K elements.
@@ -234,6 +255,10 @@ inline bool can_vec4(const Problem& pr, const void* a, const void* b, const void
     if (pr.HW == 1 && 4LL * 258 * pr.G * pr.K >= (1LL << 31)) return false;
     return pr.K % 4 == 0 && (pr.HW == 1 || pr.HW % 4 == 0) && aligned16(a) && aligned16(b) && aligned16(c);
 }
+
+// Input panels per stage of a kernel wrapper (its X_PANELS member; one when it has none).
+template <class T, class = void> struct XPanels { static constexpr int value = 1; };
+template <class T> struct XPanels<T, std::void_t<decltype(T::X_PANELS)>> { static constexpr int value = T::X_PANELS; };
 
 // Launches KERNEL<GEO, CONV, VEC>::run for the layout and vector width of the
 // problem.  KERNEL is a class template wrapping the __global__ function so that
@@ -245,6 +270,11 @@ hipError_t launch_forward(const Problem& pr, bool vec4, bool ovec, hipStream_t s
     d.tiles_m = (d.M + GEO::BM - 1) / GEO::BM;
     d.tiles_n = (d.NG + GEO::BN - 1) / GEO::BN;
     const unsigned grid = (unsigned)d.tiles_m * d.tiles_n * d.G;
+    if (pr.HW == 1) {
+        constexpr int NX = XPanels<KERNEL<GEO, false, 4>>::value;
+        d.m_block = choose_m_block(d.tiles_m, GEO::BM * NX, GEO::BN,
+                                   resident_per_xcd(GEO::NT, Stager<GEO, false, 4, NX>::LDS_BYTES, pr.num_cu));
+    }
     if (pr.HW == 1)
         return vec4 ? KERNEL<GEO, false, 4>::launch(grid, d, pr.device, stream, args...)
                     : KERNEL<GEO, false, 1>::launch(grid, d, pr.device, stream, args...);

@@ -496,6 +496,7 @@ static hipError_t launch_values(const Problem& pr, bool ovec, hipStream_t stream
     d.tiles_m = (d.M + GEO::BM - 1) / GEO::BM;
     d.tiles_n = (d.NG + GEO::BN - 1) / GEO::BN;
     const size_t lds = Stager<GEO, false, 4, 1>::LDS_BYTES;
+    d.m_block = choose_m_block(d.tiles_m, GEO::BM, GEO::BN, resident_per_xcd(GEO::NT, lds, pr.num_cu));
     auto kern = inf_forward_values_kernel<GEO>;
     static LdsRecord lds_allowed = {};
     if (hipError_t e = allow_lds(kern, lds, pr.device, lds_allowed); e != hipSuccess) return e;
@@ -653,6 +654,8 @@ hipError_t inf_forward(const float* input, const float* weight, float* output, i
         d.ovec = ovec;
         d.tiles_m = (d.M + G64::BM - 1) / G64::BM;
         d.tiles_n = (d.NG + G64::BN - 1) / G64::BN;
+        d.m_block = choose_m_block(d.tiles_m, G64::BM, G64::BN,
+                                   resident_per_xcd(G64::NT, Stager<G64, false, 4, 1>::LDS_BYTES, pr.num_cu));
         return InfForward<G64, false, 4>::launch((unsigned)d.tiles_m * d.tiles_n * d.G, d, pr.device, stream, input, weight,
                                                  output, pos);
     }

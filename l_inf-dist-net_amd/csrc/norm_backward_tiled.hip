@@ -49,7 +49,7 @@ norm_backward_input_tiled_kernel(const float* __restrict__ grad_output, const fl
 #pragma unroll
     for (int i = 0; i < TM; i++) {
         const int m = m0 + GEO::row(ty, i);
-        const RowAddr<CONV> ra(Dims{d.B, d.G, K, K, d.HW, d.M, 0, 0, 0, 0}, m < d.M ? m : 0, g);
+        const RowAddr<CONV> ra(Dims{d.B, d.G, K, K, d.HW, d.M, 0, 0, 0, 0, 0}, m < d.M ? m : 0, g);
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const int k = k0 + GEO::col(tx, j);

@@ -33,6 +33,7 @@ struct Dims {
     int tiles_m, tiles_n;
     int ovec;             // outputs may be written with 128-bit stores
     int xcd_remap;        // 1: hand each XCD a contiguous run of tiles
+    int m_block;          // > 0: row tiles are walked in blocks of this many (tile_of_block); 0: all of them
 };
 
 // XOR applied to the m (or n) coordinate of LDS row kk.  It permutes aligned
@@ -548,15 +549,27 @@ struct RowsImg {
 // to different XCDs (8 per device, each with its own L2); the remap hands every
 // XCD one contiguous run of tiles, m fastest, so the workgroups that share an
 // L2 also share their w strip (and, across runs, their x strips).
+// With many row tiles a run is longer than what an XCD holds at a time, and walking all row tiles before the next
+// column tile would make each round of resident workgroups read every x strip again.  m_block > 0 walks the row
+// tiles in blocks of that many instead (block, then column tile, then row tile inside the block), so that a
+// round covers a near-square piece of the output: few x strips and few w strips (choose_m_block() on the host).
 __device__ __forceinline__ void tile_of_block(const Dims& d, int& tm, int& tn, int& g) {
     const int total = gridDim.x;
     int id = blockIdx.x;
     constexpr int XCD = 8;
     if (d.xcd_remap && total % XCD == 0) id = (id % XCD) * (total / XCD) + id / XCD;
-    tm = id % d.tiles_m;
-    const int r = id / d.tiles_m;
-    tn = r % d.tiles_n;
-    g = r / d.tiles_n;
+    const int per_group = d.tiles_m * d.tiles_n;
+    g = id / per_group;
+    const int j = id - g * per_group;
+    if (d.m_block > 0) {                       // tiles_m is a multiple of m_block
+        const int per_block = d.m_block * d.tiles_n;
+        const int mb = j / per_block, r = j - mb * per_block;
+        tn = r / d.m_block;
+        tm = mb * d.m_block + (r - tn * d.m_block);
+    } else {
+        tn = j / d.tiles_m;
+        tm = j - tn * d.tiles_m;
+    }
 }
 
 }  // namespace ldist

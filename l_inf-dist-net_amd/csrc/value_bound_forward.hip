@@ -223,6 +223,7 @@ value_bound_forward_skinny_kernel(const float* __restrict__ input, const float* 
 
 template <class GEO, bool CONV, int VEC>
 struct ValueBoundForward {
+    static constexpr int X_PANELS = 3;   // the point, lower and upper
     static hipError_t launch(unsigned grid, const Dims& d, int device, hipStream_t stream, const float* input,
                              const float* lower, const float* upper, const float* weight, const float* mean,
                              const float* bias, float* out, float* out_lower, float* out_upper) {
