@@ -156,6 +156,36 @@ def test_forward_kernels_with_very_long_rows(K):
     assert torch.allclose(o8.cpu(), e8.float(), rtol=1e-4, atol=ATOL)   # a float32 sum of two million terms
 
 
+@pytest.mark.parametrize("tile", TILES)
+@pytest.mark.parametrize("B,NG,G", [(1024, 160, 1), (1100, 400, 2), (1536, 96, 1), (2048, 80, 2)])
+def test_forward_kernels_with_many_row_tiles(B, NG, G, tile):
+    """More row tiles than the workgroups that share an L2 cover per column tile: the launchers walk the row tiles
+    in blocks then.  Every tile of the output must still be computed exactly once: the L_inf forward (values and
+    indices), its values-only form and the interval kernel against the oracle, on every tiling."""
+    from gpu_common import DEV, cpp, gpu_inf_forward, say, set_tile
+    say("many row tiles", B, NG, G, tile)
+    K = 48
+    g = torch.Generator().manual_seed(B + NG + G)
+    x = torch.rand(B, G * K, 1, generator=g)
+    w = torch.randn(G * NG, K, generator=g)
+    eo, ep = oracle.inf_dist_forward(x, w, G)
+    set_tile(tile)
+    try:
+        out, pos = gpu_inf_forward(x, w, G)
+        assert torch.equal(out, eo) and torch.equal(pos, ep)
+        v = torch.full((B, G * NG, 1), -1.0, device=DEV)
+        if cpp.inf_dist_forward_values(x.to(DEV), w.to(DEV), v, G):
+            assert torch.equal(v.cpu(), eo)
+        lo, up = x - 0.01, x + 0.02
+        L = torch.empty(B, G * NG, 1, device=DEV)
+        U = torch.empty(B, G * NG, 1, device=DEV)
+        cpp.inf_dist_bound_forward(lo.to(DEV), up.to(DEV), w.to(DEV), L, U, G)
+        eL, eU = oracle.inf_dist_bound_forward(lo, up, w, G)
+        assert torch.equal(L.cpu(), eL) and torch.equal(U.cpu(), eU)
+    finally:
+        set_tile(-1)
+
+
 # B, CO, CI, G, HW -- unfolded-conv layouts for the kernel that keeps a tile's whole reduction axis in LDS
 SHORTK_SHAPES = [
     (2, 64, 64, 2, 64),       # K = 32: one window per k range
