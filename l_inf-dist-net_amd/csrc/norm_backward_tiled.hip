@@ -345,6 +345,7 @@ static hipError_t launch_nbi(const Problem& pr, bool ovec, hipStream_t stream, c
     d.tiles_n = (d.K + GEO::BN - 1) / GEO::BN;
     const unsigned grid = (unsigned)d.tiles_m * d.tiles_n * d.G;
     constexpr size_t lds = (size_t)(2 * GEO::XS + GEO::WS) * sizeof(float);
+    if (!CONV) d.m_block = choose_m_block(d.tiles_m, 2 * GEO::BM, GEO::BN, resident_per_xcd(GEO::NT, lds, pr.num_cu));
     auto kern = norm_backward_input_tiled_kernel<GEO, CONV, IE>;
     static LdsRecord lds_allowed = {};
     if (hipError_t e = allow_lds(kern, lds, pr.device, lds_allowed); e != hipSuccess) return e;
@@ -360,6 +361,10 @@ static hipError_t launch_nbw(const Problem& pr, hipStream_t stream, const float*
     d.tiles_n = (d.K + GEO::BN - 1) / GEO::BN;
     const unsigned grid = (unsigned)d.tiles_m * d.tiles_n * d.G;
     constexpr size_t lds = (size_t)(2 * GEO::XS + GEO::WS) * sizeof(float);
+    // A tile of outputs streams two panels over all rows (grad_output, output), a tile of inputs one: walked with
+    // all output tiles before the next input tile, the workgroups that share an L2 read their own two panels each
+    // (40 output tiles of 0.5 MB on a 5120-wide layer); in blocks they share both kinds of panel.
+    d.m_block = choose_m_block(d.tiles_m, 2 * GEO::BM, GEO::BN, resident_per_xcd(GEO::NT, lds, pr.num_cu));
     auto kern = norm_backward_weight_tiled_kernel<GEO, IE>;
     static LdsRecord lds_allowed = {};
     if (hipError_t e = allow_lds(kern, lds, pr.device, lds_allowed); e != hipSuccess) return e;
