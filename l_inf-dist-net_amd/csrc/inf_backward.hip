@@ -230,8 +230,21 @@ __device__ __forceinline__ void backward_weight_body(BIN* bins, int bx, int by, 
 #pragma unroll
             for (int u = 0; u < 4; u++) {
                 const int idx = (p[u] & 0x7fffffff) - k0;
-                if ((u == 0 || i0 + NT * u < total) && idx >= 0 && idx < kc)
-                    atomicAdd(&bins[nn[u] * kc + idx], (BIN)(p[u] < 0 ? gv[u] : -gv[u]));
+                if ((u == 0 || i0 + NT * u < total) && idx >= 0 && idx < kc) {
+                    // A float add in LDS retires a third of a lane per clock and CU, an exchange some six lanes.  A
+                    // row of bins takes one contribution per image, so most bins take none or one: the value goes in
+                    // by exchange, and what it displaced (another image's contribution to the same bin: some five in
+                    // a hundred) is added back with the slow instruction.  Whatever the interleaving, every
+                    // displaced value is added exactly once.
+                    BIN* bin = &bins[nn[u] * kc + idx];
+                    const BIN v = (BIN)(p[u] < 0 ? gv[u] : -gv[u]);
+                    if constexpr (sizeof(BIN) == sizeof(float)) {
+                        const float displaced = atomicExch(reinterpret_cast<float*>(bin), (float)v);
+                        if (displaced != 0.f) atomicAdd(reinterpret_cast<float*>(bin), displaced);
+                    } else {
+                        atomicAdd(bin, v);
+                    }
+                }
             }
         }
     } else {
