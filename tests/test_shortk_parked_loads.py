@@ -18,6 +18,14 @@ WRITE = re.compile(r"^\s*ds_write_b128 v(\d+), v\[(\d+):(\d+)\]")
 WAIT = re.compile(r"^\s*s_waitcnt vmcnt\((\d+)\)\s*$")
 
 
+def library_flags():
+    """The compiler flags of the library's Makefile (FLAGS := ... with its continuation line), ARCH filled in."""
+    text = open(os.path.join(os.path.dirname(SRC), "Makefile")).read()
+    arch = re.search(r"^ARCH\s*\?=\s*(\S+)", text, re.M).group(1)
+    flags = re.search(r"^FLAGS\s*:=\s*((?:.*\\\n)*.*)$", text, re.M).group(1).replace("\\\n", " ")
+    return flags.replace("$(ARCH)", arch).split()
+
+
 def registers(text):
     """Vector registers named in an operand string."""
     regs = set()
@@ -94,8 +102,7 @@ def check_kernel(nw, lines):
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="hipcc not on PATH")
 def test_no_read_of_a_parked_register_before_its_wait(tmp_path):
     out = tmp_path / "shortk.s"
-    cmd = ["hipcc", "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
-           "-packed-fp32-ops", "-S", "--cuda-device-only", "-I", os.path.join(ROOT, "include"), SRC, "-o", str(out)]
+    cmd = ["hipcc"] + library_flags() + ["-S", "--cuda-device-only", SRC, "-o", str(out)]
     subprocess.run(cmd, check=True, capture_output=True)
     asm = out.read_text()
     found = kernels(asm)
