@@ -313,17 +313,83 @@ inf_backward_weight_kernel(const float* __restrict__ grad_output, const int32_t*
                                                 grad_output, pos, grad_weight, d, NB, KC, n_blocks, b_per_wg);
 }
 
+// ---- grad_weight of a fully connected layer, written whole: bins of one row ----------------
+// The kernel above keeps bins for all rows of its block, 60 KB for three rows of K = 5120, so two workgroups share a
+// CU, and each of them waits in turn for its reads and (before it can leave) for its stores.  Here a workgroup still
+// reads a block of NBR rows at once (NBR * 4 bytes of every image's row), keeps the values in registers and then
+// takes the rows one after the other through bins of a single row: add, store the row and put the zeros back.  The
+// bins are a third of the size, so three times the workgroups wait side by side.
+constexpr int kRowBinsPre = 8;   // values per lane: 2048 per block
+__device__ __forceinline__ void backward_weight_rowbins(float* bins, int bx, const float* __restrict__ grad_output,
+                                                        const int32_t* __restrict__ pos, float* __restrict__ grad_weight,
+                                                        const BwdDims& d, int NBR, int n_blocks) {
+    constexpr int NT = 256;
+    const int K = d.K, tid = threadIdx.x;
+    const int idb = bx % n_blocks, g = bx / n_blocks;
+    const int nblk = (n_blocks & 7) == 0 ? (idb % 8) * (n_blocks / 8) + idb / 8 : idb;   // see backward_weight_body
+    const int n0 = nblk * NBR;
+    if (n0 >= d.NG) return;
+    const int nb = min(NBR, d.NG - n0);
+    const int total = d.B * nb;                    // <= kRowBinsPre * NT: the launcher's condition
+    const size_t img_stride = (size_t)d.G * d.NG, first = (size_t)g * d.NG + n0;
+    int p[kRowBinsPre], nn[kRowBinsPre];
+    float gv[kRowBinsPre];
+#pragma unroll
+    for (int u = 0; u < kRowBinsPre; u++) {
+        const int i = tid + NT * u;
+        const int ii = i < total ? i : 0;          // past the end: element 0 again, never added
+        const int bb = ii / nb;
+        nn[u] = i < total ? ii - bb * nb : -1;
+        const size_t o = (size_t)bb * img_stride + first + (ii - bb * nb);
+        p[u] = pos[o];
+        gv[u] = grad_output[o];
+    }
+    for (int e = tid; e < K; e += NT) bins[e] = 0.f;
+    __syncthreads();
+    const bool vec = (K & 3) == 0 && (reinterpret_cast<uintptr_t>(grad_weight) & 15u) == 0;
+    for (int r = 0; r < nb; r++) {
+#pragma unroll
+        for (int u = 0; u < kRowBinsPre; u++) {
+            const int idx = p[u] & 0x7fffffff;
+            if (nn[u] == r && idx < K) {           // by exchange, displaced values added back: see backward_weight_body
+                const float displaced = atomicExch(&bins[idx], p[u] < 0 ? gv[u] : -gv[u]);
+                if (displaced != 0.f) atomicAdd(&bins[idx], displaced);
+            }
+        }
+        __syncthreads();
+        float* row = grad_weight + (first + r) * K;
+        if (vec) {
+            for (int e = tid; e < K / 4; e += NT) {
+                float4* b4 = reinterpret_cast<float4*>(bins) + e;
+                reinterpret_cast<float4*>(row)[e] = *b4;
+                *b4 = make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        } else {
+            for (int e = tid; e < K; e += NT) { row[e] = bins[e]; bins[e] = 0.f; }
+        }
+        __syncthreads();
+    }
+}
+
+__global__ void __launch_bounds__(256)
+inf_backward_weight_rowbins_kernel(const float* __restrict__ grad_output, const int32_t* __restrict__ pos,
+                                   float* __restrict__ grad_weight, BwdDims d, int NBR, int n_blocks) {
+    extern __shared__ __align__(16) unsigned char bin_bytes[];
+    backward_weight_rowbins(reinterpret_cast<float*>(bin_bytes), blockIdx.x, grad_output, pos, grad_weight, d, NBR, n_blocks);
+}
+
 // ---- both scatters of a fully connected layer in one launch ------------------
 // grad_input (a workgroup per image and group: few bytes, mostly waiting for memory) and grad_weight (a workgroup per
 // block of output rows: bound by the stores of its slab) are independent.  As two launches one runs after the other;
 // on two streams they overlap but pay for the joins (measured: slower).  Here the workgroups of one grid do either:
 // the grad_weight workgroups come first and the grad_input workgroups last, where they run beside the tail of the
-// stores (512 x 5120 x 5120: 36.5 us against 41.5 us for the two launches; grad_input first: 39.5 us; one grad_input
+// stores (512 x 5120 x 5120, bins for whole blocks: 36.5 us against 41.5 us for the two launches; grad_input first: 39.5 us; one grad_input
 // workgroup after every three of grad_weight: 46 us).  Both write their slabs whole ("overwrite"); one k range each.
 struct BothPlan {
     int wgs_x, wgs_w;                 // workgroups per scatter
     int th_log2, kc_x, hw_tiles, vec; // grad_input's launch parameters
     int nb, kc_w, n_blocks;           // grad_weight's
+    int rowbins;                      // grad_weight through bins of one row (backward_weight_rowbins)
 };
 
 __global__ void __launch_bounds__(256)
@@ -336,8 +402,11 @@ inf_backward_both_kernel(const float* __restrict__ grad_output, const int32_t* _
                                   pl.kc_x, pl.hw_tiles, pl.vec);
         return;
     }
-    backward_weight_body<true, false, float>(reinterpret_cast<float*>(bin_bytes), i, 0, 0, grad_output, pos, grad_weight, d,
-                                             pl.nb, pl.kc_w, pl.n_blocks, d.B);
+    if (pl.rowbins)
+        backward_weight_rowbins(reinterpret_cast<float*>(bin_bytes), i, grad_output, pos, grad_weight, d, pl.nb, pl.n_blocks);
+    else
+        backward_weight_body<true, false, float>(reinterpret_cast<float*>(bin_bytes), i, 0, 0, grad_output, pos, grad_weight,
+                                                 d, pl.nb, pl.kc_w, pl.n_blocks, d.B);
 }
 
 __global__ void __launch_bounds__(256) fill_zero_kernel(float* __restrict__ p, size_t n) {
@@ -423,6 +492,16 @@ hipError_t inf_backward_weight(const float* grad_output, const int32_t* pos, flo
         else launch_backward_weight<OVER, SPLIT, float>(grid, lds, stream, grad_output, pos, grad_weight, d, NB, KC,     \
                                                         n_blocks, b_per_wg);                                            \
     } while (0)
+    {   // bins of one row, see inf_backward_weight_rowbins_kernel
+        const int nbr = min(pr.NG, min(4, (kRowBinsPre * 256) / max(pr.B, 1)));
+        const int blocks_r = nbr > 0 ? (pr.NG + nbr - 1) / nbr : 0;
+        if (!wide && overwrite && nbr >= 2 && k_ranges == 1 && (long)pr.G * blocks_r >= 4L * pr.num_cu) {
+            const int nblocks_r = blocks_r >= 64 ? (blocks_r + 7) / 8 * 8 : blocks_r;
+            hipLaunchKernelGGL(inf_backward_weight_rowbins_kernel, dim3((unsigned)(pr.G * nblocks_r)), dim3(256),
+                               (size_t)pr.K * sizeof(float), stream, grad_output, pos, grad_weight, d, nbr, nblocks_r);
+            return hipGetLastError();
+        }
+    }
     if (splits > 1) {
         if (overwrite) {
             const size_t n = (size_t)pr.G * pr.NG * pr.K;
@@ -445,7 +524,9 @@ hipError_t inf_backward_weight(const float* grad_output, const int32_t* pos, flo
 hipError_t inf_backward_both(const float* grad_output, const int32_t* pos, float* grad_input, float* grad_weight,
                              const Problem& pr, hipStream_t stream) {
     const int slots_w = kBinBytes / (int)sizeof(float);
-    const int nb = max(1, min(min(pr.NG, 8), slots_w / max(pr.K, 1)));
+    const int nbr = min(pr.NG, min(4, (kRowBinsPre * 256) / max(pr.B, 1)));
+    const bool rowbins = nbr >= 2 && (long)pr.G * ((pr.NG + nbr - 1) / nbr) >= 4L * pr.num_cu;
+    const int nb = rowbins ? nbr : max(1, min(min(pr.NG, 8), slots_w / max(pr.K, 1)));
     const int real_blocks = (pr.NG + nb - 1) / nb;
     const int n_blocks = real_blocks >= 64 ? (real_blocks + 7) / 8 * 8 : real_blocks;
     const long wgs_x = (long)pr.B * pr.G, wgs_w = (long)pr.G * n_blocks;
@@ -467,7 +548,8 @@ hipError_t inf_backward_both(const float* grad_output, const int32_t* pos, float
     pl.nb = nb;
     pl.kc_w = pr.K;
     pl.n_blocks = n_blocks;
-    const size_t lds = std::max((size_t)pr.K * sizeof(double), (size_t)nb * pr.K * sizeof(float));
+    pl.rowbins = rowbins;
+    const size_t lds = std::max((size_t)pr.K * sizeof(double), (size_t)(rowbins ? 1 : nb) * pr.K * sizeof(float));
     hipLaunchKernelGGL(inf_backward_both_kernel, dim3((unsigned)(wgs_x + wgs_w)), dim3(256), lds, stream, grad_output, pos,
                        grad_input, grad_weight, d, pl);
     return hipGetLastError();
