@@ -192,7 +192,13 @@ def mlp_workload(pkg, torch, dev, p):
         # one training step of the whole stack, every layer repeated by the oracle on what the GPU really fed it:
         # p = inf on the full batch; p-norm (slow on the CPU) on 16 batch rows and 32 weight rows per layer
         if math.isinf(p):
-            return stack_check.check_training_step(model, x, upstream, p, dev)
+            def inf_forward(xs, ws):      # the library's forward entry point on a recorded layer input
+                o = torch.empty(xs.size(0), ws.size(0), 1, device=dev)
+                ps = torch.empty(xs.size(0), ws.size(0), 1, device=dev, dtype=torch.int32)
+                pkg.norm_dist_cpp.inf_dist_forward(xs.to(dev), ws.to(dev), o, ps, 1)
+                torch.cuda.synchronize()
+                return o.cpu(), ps.cpu()
+            return stack_check.check_training_step(model, x, upstream, p, dev, inf_forward=inf_forward)
         return stack_check.check_training_step(model, x, upstream, p, dev, rows=slice(100, 116), weight_rows=slice(64, 96))
 
     return step, cpu, formula, check
@@ -365,25 +371,26 @@ def workload_c4(pkg, torch, dev):
         rep = stack_check.Report()
         xs, gs = cols[:rows].contiguous(), go[:rows].contiguous()
         ev, ep = oracle.inf_dist_forward(xs, w, 4)
-        mag = ep & 0x7FFFFFFF
-        egx, mgx = oracle.inf_dist_backward_input(gs, ep, 1152, 4), oracle.inf_dist_backward_input(gs.abs(), mag, 1152, 4)
-        egw, mgw = oracle.inf_dist_backward_weight(gs, ep, 1152, 4), -oracle.inf_dist_backward_weight(gs.abs(), mag, 1152, 4)
+        egx = oracle.inf_dist_backward_input(gs, ep, 1152, 4)
+        egw = oracle.inf_dist_backward_weight(gs, ep, 1152, 4)
         xs_d = xs.to(dev).requires_grad_(True)
         w_d = w.to(dev).requires_grad_(True)
         y = pkg.norm_dist(xs_d, w_d, 4, INF)
         y.backward(gs.to(dev))
         rep.equal("columns: values", y.detach().cpu(), ev)
-        rep.ratio("columns: grad_input", stack_check.sum_ratio(xs_d.grad.cpu(), egx, mgx), xs_d.grad.cpu(), egx)
-        rep.ratio("columns: grad_weight", stack_check.sum_ratio(w_d.grad.cpu(), egw, mgw), w_d.grad.cpu(), egw)
+        pos_d = torch.empty(rows, 128, 1024, device=dev, dtype=torch.int32)
+        pkg.norm_dist_cpp.inf_dist_forward(xs_d.detach(), w_d.detach(), torch.empty(rows, 128, 1024, device=dev), pos_d, 4)
+        rep.equal("columns: arg-max indices and signs", pos_d.cpu(), ep)
+        rep.ratio("columns: grad_input", stack_check.close_ratio(xs_d.grad.cpu(), egx), xs_d.grad.cpu(), egx)
+        rep.ratio("columns: grad_weight", stack_check.close_ratio(w_d.grad.cpu(), egw), w_d.grad.cpu(), egw)
         layer.weight.grad = None
         xi = imgd[:rows].detach().requires_grad_(True)
         yi, _, _ = layer(xi)
         yi.backward(god4[:rows])
         rep.equal("image: values", yi.detach().cpu().reshape(rows, 128, 1024), ev)
-        egi = F.fold(egx.double(), (32, 32), 3, padding=1)
-        mgi = F.fold(mgx.double(), (32, 32), 3, padding=1)
-        rep.ratio("image: grad_image", stack_check.sum_ratio(xi.grad.cpu(), egi, mgi), xi.grad.cpu(), egi)
-        rep.ratio("image: grad_weight", stack_check.sum_ratio(layer.weight.grad.cpu().reshape(128, 288), egw, mgw),
+        egi = F.fold(oracle.inf_dist_backward_input_f64(gs, ep, 1152, 4), (32, 32), 3, padding=1)
+        rep.ratio("image: grad_image", stack_check.close_ratio(xi.grad.cpu(), egi), xi.grad.cpu(), egi)
+        rep.ratio("image: grad_weight", stack_check.close_ratio(layer.weight.grad.cpu().reshape(128, 288), egw),
                   layer.weight.grad.cpu().reshape(128, 288), egw)
         layer.weight.grad = None
         return rep
@@ -486,9 +493,9 @@ def workload_c4p(pkg, torch, dev):
         rep.ratio("image: values", stack_check.close_ratio(got, ev), got, ev)
         egi = F.fold(egx.double(), (32, 32), 3, padding=1)
         mgi = F.fold(mgx.double(), (32, 32), 3, padding=1)
-        rep.ratio("image: grad_image", stack_check.sum_ratio(xi.grad.cpu(), egi, mgi, p=p), xi.grad.cpu(), egi)
+        rep.ratio("image: grad_image", stack_check.sum_ratio(xi.grad.cpu(), egi, mgi, p), xi.grad.cpu(), egi)
         gw = layer.weight.grad.cpu().reshape(128, 288)
-        rep.ratio("image: grad_weight", stack_check.sum_ratio(gw, egw, mgw, p=p, n_terms=torch.full_like(egw, rows * 1024)), gw, egw)
+        rep.ratio("image: grad_weight", stack_check.sum_ratio(gw, egw, mgw, p), gw, egw)
         layer.weight.grad = None
         return rep
 

@@ -93,7 +93,8 @@ unfold_3x3_kernel(const float* __restrict__ img, float* __restrict__ cols, int p
     }
 }
 
-// One lane = one image pixel: gathers the KH*KW column entries that were copied from it.
+// One lane = one image pixel: gathers the KH*KW column entries that were copied from it, sums them in double and
+// rounds once (the kernel waits for memory; the result is the correctly rounded sum, in a fixed order).
 __global__ void __launch_bounds__(256)
 fold_kernel(const float* __restrict__ gcols, float* __restrict__ gimg, ConvGeom q) {
     const int L = q.HO * q.WO;
@@ -104,7 +105,7 @@ fold_kernel(const float* __restrict__ gcols, float* __restrict__ gimg, ConvGeom 
         const int y = (int)(r1 % q.H);
         const long long bc = r1 / q.H;
         const float* base = gcols + bc * q.KH * q.KW * L;
-        float s = 0.f;
+        double s = 0.0;
         for (int i = 0; i < q.KH; i++) {
             const int hy = y + q.P - i * q.D;
             if (hy < 0 || hy % q.S != 0) continue;
@@ -118,7 +119,7 @@ fold_kernel(const float* __restrict__ gcols, float* __restrict__ gimg, ConvGeom 
                 s += base[(long long)(i * q.KW + j) * L + h * q.WO + w];
             }
         }
-        gimg[id] = s;
+        gimg[id] = (float)s;
     }
 }
 

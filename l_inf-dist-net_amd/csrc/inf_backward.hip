@@ -9,11 +9,13 @@
 // out with coalesced stores, so the pass is bounded by streaming grad_output/pos
 // in and the gradient out.  In "overwrite" mode the slab is stored whole (zeros
 // included), which replaces the caller's zero fill.
-// The bins of grad_input (and of grad_weight in the conv layout) are doubles: on gfx950 an LDS atomic add of a
-// double (ds_add_f64) retires about nine times as many lanes per clock as one of a float (ds_add_f32: 0.33 lanes
-// per clock and CU, measured on random addresses; 2.9 for doubles, 6 for 32-bit integer adds), and the binning was
-// what those kernels waited for.  A bin's sum is rounded to float once, when the slab is written: exact where an
-// element receives one contribution, otherwise at least as close to the true sum as any order of float additions.
+// All bins are doubles: on gfx950 an LDS atomic add of a double (ds_add_f64) retires about nine times as many lanes
+// per clock as one of a float (ds_add_f32: 0.33 lanes per clock and CU, measured on random addresses; 2.9 for
+// doubles, 6 for 32-bit integer adds), and a sum of floats held in a double does not depend on the order of the
+// additions (exactly so while the addends' exponents span fewer than 29 binades, to 2^-53 otherwise).  A bin's sum is
+// rounded to float once, when the slab is written: the gradients are the correctly rounded sums, the same bits in
+// every run, whatever the scheduling.  "Accumulate" entry points add the bin to the caller's value in double and
+// round once as well.
 #include "kernels.hpp"
 
 #include <algorithm>
@@ -72,9 +74,9 @@ __device__ __forceinline__ void backward_input_body(double* bins, int bx, int by
             if (OVERWRITE) {
                 dst[e] = v;
             } else if (v.x != 0.f || v.y != 0.f || v.z != 0.f || v.w != 0.f) {
-                float4 o = dst[e];
-                o.x += v.x; o.y += v.y; o.z += v.z; o.w += v.w;
-                dst[e] = o;
+                const float4 o = dst[e];
+                dst[e] = make_float4((float)((double)o.x + lo.x), (float)((double)o.y + lo.y), (float)((double)o.z + hi.x),
+                                     (float)((double)o.w + hi.y));
             }
         }
         return;
@@ -118,9 +120,9 @@ __device__ __forceinline__ void backward_input_body(double* bins, int bx, int by
                 if (OVERWRITE) {
                     *dst = v;
                 } else if (v.x != 0.f || v.y != 0.f || v.z != 0.f || v.w != 0.f) {
-                    float4 o = *dst;
-                    o.x += v.x; o.y += v.y; o.z += v.z; o.w += v.w;
-                    *dst = o;
+                    const float4 o = *dst;
+                    *dst = make_float4((float)((double)o.x + lo.x), (float)((double)o.y + lo.y), (float)((double)o.z + hi.x),
+                                       (float)((double)o.w + hi.y));
                 }
             }
         }
@@ -151,9 +153,9 @@ __device__ __forceinline__ void backward_input_body(double* bins, int bx, int by
         const int hw = hw0 + j;
         if (hw < d.HW) {
             float* dst = grad_input + xbase + (size_t)k * d.HW + hw;
-            const float v = (float)bins[e];
-            if (OVERWRITE) *dst = v;
-            else if (v != 0.f) *dst += v;
+            const double v = bins[e];
+            if (OVERWRITE) *dst = (float)v;
+            else if (v != 0.0) *dst = (float)((double)*dst + v);
         }
     }
 }
@@ -167,21 +169,17 @@ inf_backward_input_kernel(const float* __restrict__ grad_output, const int32_t* 
 }
 
 // ---- grad_weight -----------------------------------------------------------
-// Workgroup = (group g, NB consecutive outputs n, KC consecutive k -- all of K when
-// a row of bins fits in 64 KB -- and a slice of the images b).  For one image the NB rows of grad_output/pos are one
-// contiguous run of NB*HW elements.  bins[nb][kc].
-// When the images are split over several workgroups (SPLIT) the bins are added
-// to grad_weight with global atomics, otherwise the workgroup is the only
-// writer of its slab.
-// BIN: float bins in the fc layout (a row of bins receives at most one contribution per image, and what the kernel
-// waits for are its strided reads of grad_output / pos columns: twice the rows per workgroup count for more than
-// faster atomics), double bins otherwise (B * HW contributions per row: 131 072 in a 3x3 conv layer of 32 x 32
-// images at batch 128, where the float atomics took three times as long as everything else).
-template <bool OVERWRITE, bool SPLIT, class BIN>
-__device__ __forceinline__ void backward_weight_body(BIN* bins, int bx, int by, int bz, const float* __restrict__ grad_output,
+// Workgroup = (group g, NB consecutive outputs n, KC consecutive k -- all of K when a row of bins fits in 64 KB and
+// the rows alone fill the device).  For one image the NB rows of grad_output/pos are one contiguous run of NB*HW
+// elements.  bins[nb][kc].  A workgroup scans every image and is the only writer of its slab: a layer with few rows
+// (a grouped conv layer: 128 rows of 131 072 contributions each) is spread over the device by giving a row to
+// several workgroups with a k range each (they read the same lines, side by side in one L2), never by splitting the
+// images, whose partial sums could only be joined with float atomics in an order that changes from run to run.
+template <bool OVERWRITE>
+__device__ __forceinline__ void backward_weight_body(double* bins, int bx, int by, const float* __restrict__ grad_output,
                                                      const int32_t* __restrict__ pos, float* __restrict__ grad_weight,
-                                                     const BwdDims& d, int NB, int KC, int n_blocks, int b_per_wg) {
-    constexpr int NT = 256;
+                                                     const BwdDims& d, int NB, int KC, int n_blocks) {
+    const int NT = blockDim.x;
     // Neighbouring blocks of outputs read neighbouring few-byte pieces of the same memory lines (in the fc layout a
     // block's grad_output / pos entries of one image are NB * 4 bytes).  Workgroups go to the eight XCDs in turn, each
     // with its own L2, so XCD x takes the x-th eighth of the blocks: neighbours then share the lines in one L2
@@ -195,15 +193,14 @@ __device__ __forceinline__ void backward_weight_body(BIN* bins, int bx, int by, 
     const int nb = min(NB, d.NG - n0);
     const int k0 = by * KC;
     const int kc = min(KC, d.K - k0);
-    const int b0 = bz * b_per_wg;
-    const int b1 = min(d.B, b0 + b_per_wg);
+    const int b0 = 0, b1 = d.B;
     // kc is a multiple of 4 whenever vec is set, so rows of bins and of grad_weight stay 16-byte aligned
     const bool vec = (kc & 3) == 0 && (d.K & 3) == 0 && (reinterpret_cast<uintptr_t>(grad_weight) & 15u) == 0;
     if (vec) {   // 16 bytes of bins per store
         float4* b4 = reinterpret_cast<float4*>(bins);
-        for (int e = threadIdx.x; e < nb * kc * (int)sizeof(BIN) / 16; e += NT) b4[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int e = threadIdx.x; e < nb * kc / 2; e += NT) b4[e] = make_float4(0.f, 0.f, 0.f, 0.f);
     } else {
-        for (int e = threadIdx.x; e < nb * kc; e += NT) bins[e] = (BIN)0;
+        for (int e = threadIdx.x; e < nb * kc; e += NT) bins[e] = 0.0;
     }
     __syncthreads();
 
@@ -230,97 +227,97 @@ __device__ __forceinline__ void backward_weight_body(BIN* bins, int bx, int by, 
 #pragma unroll
             for (int u = 0; u < 4; u++) {
                 const int idx = (p[u] & 0x7fffffff) - k0;
-                if ((u == 0 || i0 + NT * u < total) && idx >= 0 && idx < kc) {
-                    // A float add in LDS retires a third of a lane per clock and CU, an exchange some six lanes.  A
-                    // row of bins takes one contribution per image, so most bins take none or one: the value goes in
-                    // by exchange, and what it displaced (another image's contribution to the same bin: some five in
-                    // a hundred) is added back with the slow instruction.  Whatever the interleaving, every
-                    // displaced value is added exactly once.
-                    BIN* bin = &bins[nn[u] * kc + idx];
-                    const BIN v = (BIN)(p[u] < 0 ? gv[u] : -gv[u]);
-                    if constexpr (sizeof(BIN) == sizeof(float)) {
-                        const float displaced = atomicExch(reinterpret_cast<float*>(bin), (float)v);
-                        if (displaced != 0.f) atomicAdd(reinterpret_cast<float*>(bin), displaced);
-                    } else {
-                        atomicAdd(bin, v);
-                    }
-                }
+                if ((u == 0 || i0 + NT * u < total) && idx >= 0 && idx < kc)
+                    atomicAdd(&bins[nn[u] * kc + idx], (double)(p[u] < 0 ? gv[u] : -gv[u]));
             }
         }
     } else {
         auto add = [&](int p, float gv, int nn) {
             const int idx = (p & 0x7fffffff) - k0;
-            if (idx >= 0 && idx < kc) atomicAdd(&bins[nn * kc + idx], (BIN)(p < 0 ? gv : -gv));
+            if (idx >= 0 && idx < kc) atomicAdd(&bins[nn * kc + idx], (double)(p < 0 ? gv : -gv));
         };
-        // HW % 4 == 0 and aligned tensors: four positions per lane with 128-bit loads and two such groups in
+        // HW % 4 == 0 and aligned tensors: four positions per lane with 128-bit loads and four such groups in
         // flight (one position per trip, the index first and the gradient after it, left a wave waiting out two
-        // memory latencies per 256 bytes)
+        // memory latencies per 256 bytes).  Images and positions form one index space, so that every lane of a
+        // large workgroup has work even where an image's run is short.
         const bool vec_in = (d.HW & 3) == 0 && ((reinterpret_cast<uintptr_t>(grad_output) | reinterpret_cast<uintptr_t>(pos)) & 15u) == 0;
-        for (int b = b0; b < b1; b++) {
-            const size_t base = (size_t)b * img_stride + first;
-            if (vec_in) {
-                const int4* pq = reinterpret_cast<const int4*>(pos + base);
-                const float4* gq = reinterpret_cast<const float4*>(grad_output + base);
-                const int quads = run / 4, hwq = d.HW / 4;
-                for (int q0 = threadIdx.x; q0 < quads; q0 += 2 * NT) {
-                    const int q1 = q0 + NT < quads ? q0 + NT : q0;
-                    const int4 pa = pq[q0], pb = pq[q1];
-                    const float4 ga = gq[q0], gb = gq[q1];
-                    const int na = q0 / hwq;
-                    add(pa.x, ga.x, na); add(pa.y, ga.y, na); add(pa.z, ga.z, na); add(pa.w, ga.w, na);
-                    if (q1 != q0) {
-                        const int nb_ = q1 / hwq;
-                        add(pb.x, gb.x, nb_); add(pb.y, gb.y, nb_); add(pb.z, gb.z, nb_); add(pb.w, gb.w, nb_);
+        if (vec_in) {
+            const int quads = run / 4, hwq = d.HW / 4;
+            const long total = (long)(b1 - b0) * quads;
+            constexpr int U = 4;
+            for (long i0 = threadIdx.x; i0 < total; i0 += (long)U * NT) {
+                int4 pv[U];
+                float4 gv[U];
+                int nn[U];
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    const long i = i0 + (long)u * NT < total ? i0 + (long)u * NT : i0;   // past the end: the first again, not added
+                    const int bb = (int)(i / quads), q = (int)(i - (long)bb * quads);
+                    const size_t o = (size_t)(b0 + bb) * img_stride + first + (size_t)q * 4;
+                    pv[u] = *reinterpret_cast<const int4*>(pos + o);
+                    gv[u] = *reinterpret_cast<const float4*>(grad_output + o);
+                    nn[u] = q / hwq;
+                }
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    if (u == 0 || i0 + (long)u * NT < total) {
+                        add(pv[u].x, gv[u].x, nn[u]); add(pv[u].y, gv[u].y, nn[u]);
+                        add(pv[u].z, gv[u].z, nn[u]); add(pv[u].w, gv[u].w, nn[u]);
                     }
                 }
-            } else {
-                for (int e = threadIdx.x; e < run; e += NT) add(pos[base + e], grad_output[base + e], e / d.HW);
+            }
+        } else {
+            const long total = (long)(b1 - b0) * run;
+            for (long i = threadIdx.x; i < total; i += NT) {
+                const int bb = (int)(i / run), e = (int)(i - (long)bb * run);
+                const size_t o = (size_t)(b0 + bb) * img_stride + first + e;
+                add(pos[o], grad_output[o], e / d.HW);
             }
         }
     }
     __syncthreads();
 
-    if (vec && OVERWRITE && !SPLIT) {
+    if (vec && OVERWRITE) {
         const int kc4 = kc / 4;
         for (int e = threadIdx.x; e < nb * kc4; e += NT) {
             const int nn = e / kc4, k4 = e - nn * kc4;
             float* dst = grad_weight + ((size_t)g * d.NG + n0 + nn) * d.K + k0 + k4 * 4;
-            const BIN* b = bins + 4 * e;   // nn * kc + 4 * k4, kc a multiple of four
-            *reinterpret_cast<float4*>(dst) = make_float4((float)b[0], (float)b[1], (float)b[2], (float)b[3]);
+            const double2* b = reinterpret_cast<const double2*>(bins) + 2 * e;   // nn * kc + 4 * k4, kc a multiple of four
+            const double2 lo = b[0], hi = b[1];
+            *reinterpret_cast<float4*>(dst) = make_float4((float)lo.x, (float)lo.y, (float)hi.x, (float)hi.y);
         }
         return;
     }
     for (int e = threadIdx.x; e < nb * kc; e += NT) {
         const int nn = e / kc, k = e - nn * kc;
         float* dst = grad_weight + ((size_t)g * d.NG + n0 + nn) * d.K + k0 + k;
-        const float v = (float)bins[e];
-        if (SPLIT) {
-            if (v != 0.f) atomicAdd(dst, v);
-        } else if (OVERWRITE) {
-            *dst = v;
-        } else if (v != 0.f) {
-            *dst += v;
+        const double v = bins[e];
+        if (OVERWRITE) {
+            *dst = (float)v;
+        } else if (v != 0.0) {
+            *dst = (float)((double)*dst + v);
         }
     }
 }
 
-template <bool OVERWRITE, bool SPLIT, class BIN>
-__global__ void __launch_bounds__(256)
+template <bool OVERWRITE>
+__global__ void __launch_bounds__(1024)
 inf_backward_weight_kernel(const float* __restrict__ grad_output, const int32_t* __restrict__ pos,
-                           float* __restrict__ grad_weight, BwdDims d, int NB, int KC, int n_blocks, int b_per_wg) {
+                           float* __restrict__ grad_weight, BwdDims d, int NB, int KC, int n_blocks) {
     extern __shared__ __align__(16) unsigned char bin_bytes[];
-    backward_weight_body<OVERWRITE, SPLIT, BIN>(reinterpret_cast<BIN*>(bin_bytes), blockIdx.x, blockIdx.y, blockIdx.z,
-                                                grad_output, pos, grad_weight, d, NB, KC, n_blocks, b_per_wg);
+    backward_weight_body<OVERWRITE>(reinterpret_cast<double*>(bin_bytes), blockIdx.x, blockIdx.y, grad_output, pos, grad_weight,
+                                    d, NB, KC, n_blocks);
 }
 
-// ---- grad_weight of a fully connected layer, written whole: bins of one row ----------------
-// The kernel above keeps bins for all rows of its block, 60 KB for three rows of K = 5120, so two workgroups share a
-// CU, and each of them waits in turn for its reads and (before it can leave) for its stores.  Here a workgroup still
-// reads a block of NBR rows at once (NBR * 4 bytes of every image's row), keeps the values in registers and then
-// takes the rows one after the other through bins of a single row: add, store the row and put the zeros back.  The
-// bins are a third of the size, so three times the workgroups wait side by side.
+// ---- grad_weight of a fully connected layer: bins of one row ---------------------------------
+// The kernel above keeps bins for all rows of its block; for K = 5120 one row of doubles is 40 KB, so a block of rows
+// would leave a CU with one workgroup, which waits in turn for its reads and (before it can leave) for its stores.
+// Here a workgroup still reads a block of NBR rows at once (NBR * 4 bytes of every image's row), keeps the values in
+// registers and then takes the rows one after the other through bins of a single row: add, write the row and put the
+// zeros back.  Four workgroups then wait side by side on a CU.
 constexpr int kRowBinsPre = 8;   // values per lane: 2048 per block
-__device__ __forceinline__ void backward_weight_rowbins(float* bins, int bx, const float* __restrict__ grad_output,
+template <bool OVERWRITE>
+__device__ __forceinline__ void backward_weight_rowbins(double* bins, int bx, const float* __restrict__ grad_output,
                                                         const int32_t* __restrict__ pos, float* __restrict__ grad_weight,
                                                         const BwdDims& d, int NBR, int n_blocks) {
     constexpr int NT = 256;
@@ -344,38 +341,55 @@ __device__ __forceinline__ void backward_weight_rowbins(float* bins, int bx, con
         p[u] = pos[o];
         gv[u] = grad_output[o];
     }
-    for (int e = tid; e < K; e += NT) bins[e] = 0.f;
-    __syncthreads();
     const bool vec = (K & 3) == 0 && (reinterpret_cast<uintptr_t>(grad_weight) & 15u) == 0;
+    if ((K & 1) == 0) {
+        for (int e = tid; e < K / 2; e += NT) reinterpret_cast<double2*>(bins)[e] = make_double2(0.0, 0.0);
+    } else {
+        for (int e = tid; e < K; e += NT) bins[e] = 0.0;
+    }
+    __syncthreads();
     for (int r = 0; r < nb; r++) {
 #pragma unroll
         for (int u = 0; u < kRowBinsPre; u++) {
             const int idx = p[u] & 0x7fffffff;
-            if (nn[u] == r && idx < K) {           // by exchange, displaced values added back: see backward_weight_body
-                const float displaced = atomicExch(&bins[idx], p[u] < 0 ? gv[u] : -gv[u]);
-                if (displaced != 0.f) atomicAdd(&bins[idx], displaced);
-            }
+            if (nn[u] == r && idx < K) atomicAdd(&bins[idx], (double)(p[u] < 0 ? gv[u] : -gv[u]));
         }
         __syncthreads();
         float* row = grad_weight + (first + r) * K;
         if (vec) {
             for (int e = tid; e < K / 4; e += NT) {
-                float4* b4 = reinterpret_cast<float4*>(bins) + e;
-                reinterpret_cast<float4*>(row)[e] = *b4;
-                *b4 = make_float4(0.f, 0.f, 0.f, 0.f);
+                double2* b2 = reinterpret_cast<double2*>(bins) + 2 * e;
+                const double2 lo = b2[0], hi = b2[1];
+                float4* dst = reinterpret_cast<float4*>(row) + e;
+                if (OVERWRITE) {
+                    *dst = make_float4((float)lo.x, (float)lo.y, (float)hi.x, (float)hi.y);
+                } else if (lo.x != 0.0 || lo.y != 0.0 || hi.x != 0.0 || hi.y != 0.0) {
+                    const float4 o = *dst;
+                    *dst = make_float4((float)((double)o.x + lo.x), (float)((double)o.y + lo.y), (float)((double)o.z + hi.x),
+                                       (float)((double)o.w + hi.y));
+                }
+                b2[0] = make_double2(0.0, 0.0);
+                b2[1] = make_double2(0.0, 0.0);
             }
         } else {
-            for (int e = tid; e < K; e += NT) { row[e] = bins[e]; bins[e] = 0.f; }
+            for (int e = tid; e < K; e += NT) {
+                const double v = bins[e];
+                if (OVERWRITE) row[e] = (float)v;
+                else if (v != 0.0) row[e] = (float)((double)row[e] + v);
+                bins[e] = 0.0;
+            }
         }
         __syncthreads();
     }
 }
 
+template <bool OVERWRITE>
 __global__ void __launch_bounds__(256)
 inf_backward_weight_rowbins_kernel(const float* __restrict__ grad_output, const int32_t* __restrict__ pos,
                                    float* __restrict__ grad_weight, BwdDims d, int NBR, int n_blocks) {
     extern __shared__ __align__(16) unsigned char bin_bytes[];
-    backward_weight_rowbins(reinterpret_cast<float*>(bin_bytes), blockIdx.x, grad_output, pos, grad_weight, d, NBR, n_blocks);
+    backward_weight_rowbins<OVERWRITE>(reinterpret_cast<double*>(bin_bytes), blockIdx.x, grad_output, pos, grad_weight, d, NBR,
+                                       n_blocks);
 }
 
 // ---- both scatters of a fully connected layer in one launch ------------------
@@ -403,21 +417,10 @@ inf_backward_both_kernel(const float* __restrict__ grad_output, const int32_t* _
         return;
     }
     if (pl.rowbins)
-        backward_weight_rowbins(reinterpret_cast<float*>(bin_bytes), i, grad_output, pos, grad_weight, d, pl.nb, pl.n_blocks);
+        backward_weight_rowbins<true>(reinterpret_cast<double*>(bin_bytes), i, grad_output, pos, grad_weight, d, pl.nb, pl.n_blocks);
     else
-        backward_weight_body<true, false, float>(reinterpret_cast<float*>(bin_bytes), i, 0, 0, grad_output, pos, grad_weight,
-                                                 d, pl.nb, pl.kc_w, pl.n_blocks, d.B);
-}
-
-__global__ void __launch_bounds__(256) fill_zero_kernel(float* __restrict__ p, size_t n) {
-    const size_t stride = (size_t)gridDim.x * 256 * 4;
-    for (size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4; i < n; i += stride) {
-        if (i + 4 <= n && (reinterpret_cast<uintptr_t>(p + i) & 15u) == 0) {
-            *reinterpret_cast<float4*>(p + i) = make_float4(0.f, 0.f, 0.f, 0.f);
-        } else {
-            for (size_t j = i; j < n && j < i + 4; j++) p[j] = 0.f;
-        }
-    }
+        backward_weight_body<true>(reinterpret_cast<double*>(bin_bytes), i, 0, grad_output, pos, grad_weight, d, pl.nb, pl.kc_w,
+                                   pl.n_blocks);
 }
 
 static constexpr int kBinBytes = 64 * 1024;                           // LDS bins per workgroup
@@ -452,69 +455,74 @@ hipError_t inf_backward_input(const float* grad_output, const int32_t* pos, floa
     return hipGetLastError();
 }
 
-template <bool OVERWRITE, bool SPLIT, class BIN>
-static void launch_backward_weight(dim3 grid, size_t lds, hipStream_t stream, const float* grad_output, const int32_t* pos,
-                                   float* grad_weight, const BwdDims& d, int NB, int KC, int n_blocks, int b_per_wg) {
-    hipLaunchKernelGGL((inf_backward_weight_kernel<OVERWRITE, SPLIT, BIN>), grid, dim3(256), lds, stream, grad_output, pos,
-                       grad_weight, d, NB, KC, n_blocks, b_per_wg);
+// Launch shape of inf_backward_weight_kernel.
+struct WeightPlan {
+    int NB, KC, n_blocks, real_blocks, k_ranges, threads;
+};
+
+static WeightPlan plan_backward_weight(const Problem& pr) {
+    WeightPlan wp{};
+    const int slots = kInputBins;
+    // One pass over all K channels per workgroup when a row of bins fits and the rows fill the device: every k range
+    // re-reads the row's grad_output / pos.
+    wp.KC = min(pr.K, slots);
+    wp.NB = max(1, min(min(pr.NG, 8), slots / wp.KC));
+    // fewer rows per block while the blocks do not fill the device
+    while (wp.NB > 1 && (long)pr.G * ((pr.NG + wp.NB - 1) / wp.NB) < 2L * pr.num_cu) wp.NB = (wp.NB + 1) / 2;
+    wp.real_blocks = (pr.NG + wp.NB - 1) / wp.NB;
+    const long rows = (long)pr.G * wp.real_blocks;
+    const long scanned = (long)pr.B * pr.HW * wp.NB;               // contributions a workgroup looks at
+    if (rows < pr.num_cu && scanned >= 16384) {
+        // still too few: k ranges of at least 16 channels (multiples of four), up to one workgroup per CU
+        const int want = (int)min((long)((pr.num_cu + rows - 1) / rows), (long)max(1, wp.KC / 16));
+        const int kc = ((wp.KC + want - 1) / want + 3) / 4 * 4;
+        wp.KC = max(4, min(wp.KC, kc));
+    }
+    wp.k_ranges = (pr.K + wp.KC - 1) / wp.KC;
+    // many blocks: a multiple of eight, for the kernel's XCD-aware block order (the extra workgroups leave at once)
+    wp.n_blocks = wp.real_blocks >= 64 ? (wp.real_blocks + 7) / 8 * 8 : wp.real_blocks;
+    // few workgroups with long scans: more lanes each keep more loads in flight
+    const long wgs = rows * wp.k_ranges;
+    wp.threads = 256;
+    if (wgs < 8L * pr.num_cu && scanned >= 8192) wp.threads = 512;
+    if (wgs < 4L * pr.num_cu && scanned >= 32768) wp.threads = 1024;
+    return wp;
+}
+
+// Rows per block for the kernel with bins of one row (0: the layer does not take it): fully connected layout, a
+// block's values fit the lanes' registers, one k range, and enough blocks to keep four workgroups on every CU.
+static int rowbins_rows(const Problem& pr) {
+    if (pr.HW != 1 || pr.K > kInputBins) return 0;
+    const int nbr = min(pr.NG, min(4, (kRowBinsPre * 256) / max(pr.B, 1)));
+    if (nbr < 2 || (long)pr.G * ((pr.NG + nbr - 1) / nbr) < 4L * pr.num_cu) return 0;
+    return nbr;
 }
 
 hipError_t inf_backward_weight(const float* grad_output, const int32_t* pos, float* grad_weight, const Problem& pr,
                                bool overwrite, hipStream_t stream) {
     const BwdDims d{pr.B, pr.G, pr.K, pr.NG, pr.HW};
-    const bool wide = pr.HW > 1;   // double bins, see the kernel
-    const int slots = kBinBytes / (wide ? (int)sizeof(double) : (int)sizeof(float));
-    // One pass over all K channels per workgroup when a row of bins fits: re-reading the strided
-    // grad_output/pos columns for every channel range costs more than the smaller row block.
-    const int KC = min(pr.K, slots);
-    const int NB = max(1, min(min(pr.NG, 8), slots / KC));
-    const int real_blocks = (pr.NG + NB - 1) / NB;
-    // many blocks: a multiple of eight, for the kernel's XCD-aware block order (the extra workgroups leave at once)
-    const int n_blocks = real_blocks >= 64 ? (real_blocks + 7) / 8 * 8 : real_blocks;
-    const int k_ranges = (pr.K + KC - 1) / KC;
-    const long slabs = (long)pr.G * real_blocks * k_ranges;
-    // split the images over workgroups only when the slabs alone cannot fill the device
-    int splits = 1;
-    if (slabs < 2L * pr.num_cu) {
-        const long rows = (long)pr.B * pr.HW;
-        const long by_work = max(1L, rows * NB / 16384);  // keep at least 16K contributions per workgroup
-        splits = (int)min((long)pr.B, min(by_work, (4L * pr.num_cu + slabs - 1) / slabs));
-        if (splits > 65535) splits = 65535;
+    if (const int nbr = rowbins_rows(pr)) {   // bins of one row, see backward_weight_rowbins
+        const int blocks_r = (pr.NG + nbr - 1) / nbr;
+        const int nblocks_r = blocks_r >= 64 ? (blocks_r + 7) / 8 * 8 : blocks_r;
+        const dim3 grid((unsigned)(pr.G * nblocks_r));
+        const size_t lds = (size_t)pr.K * sizeof(double);
+        if (overwrite)
+            hipLaunchKernelGGL(inf_backward_weight_rowbins_kernel<true>, grid, dim3(256), lds, stream, grad_output, pos,
+                               grad_weight, d, nbr, nblocks_r);
+        else
+            hipLaunchKernelGGL(inf_backward_weight_rowbins_kernel<false>, grid, dim3(256), lds, stream, grad_output, pos,
+                               grad_weight, d, nbr, nblocks_r);
+        return hipGetLastError();
     }
-    const int b_per_wg = (pr.B + splits - 1) / splits;
-    splits = (pr.B + b_per_wg - 1) / b_per_wg;
-    const dim3 grid((unsigned)(pr.G * n_blocks), (unsigned)k_ranges, (unsigned)splits);
-    const size_t lds = (size_t)NB * KC * (wide ? sizeof(double) : sizeof(float));
-#define LDIST_BWD_W(OVER, SPLIT)                                                                                        \
-    do {                                                                                                                \
-        if (wide) launch_backward_weight<OVER, SPLIT, double>(grid, lds, stream, grad_output, pos, grad_weight, d, NB, KC, \
-                                                              n_blocks, b_per_wg);                                      \
-        else launch_backward_weight<OVER, SPLIT, float>(grid, lds, stream, grad_output, pos, grad_weight, d, NB, KC,     \
-                                                        n_blocks, b_per_wg);                                            \
-    } while (0)
-    {   // bins of one row, see inf_backward_weight_rowbins_kernel
-        const int nbr = min(pr.NG, min(4, (kRowBinsPre * 256) / max(pr.B, 1)));
-        const int blocks_r = nbr > 0 ? (pr.NG + nbr - 1) / nbr : 0;
-        if (!wide && overwrite && nbr >= 2 && k_ranges == 1 && (long)pr.G * blocks_r >= 4L * pr.num_cu) {
-            const int nblocks_r = blocks_r >= 64 ? (blocks_r + 7) / 8 * 8 : blocks_r;
-            hipLaunchKernelGGL(inf_backward_weight_rowbins_kernel, dim3((unsigned)(pr.G * nblocks_r)), dim3(256),
-                               (size_t)pr.K * sizeof(float), stream, grad_output, pos, grad_weight, d, nbr, nblocks_r);
-            return hipGetLastError();
-        }
-    }
-    if (splits > 1) {
-        if (overwrite) {
-            const size_t n = (size_t)pr.G * pr.NG * pr.K;
-            const unsigned blocks = (unsigned)min((size_t)4096, (n + 1023) / 1024);
-            hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, stream, grad_weight, n);
-        }
-        LDIST_BWD_W(false, true);
-    } else if (overwrite) {
-        LDIST_BWD_W(true, false);
-    } else {
-        LDIST_BWD_W(false, false);
-    }
-#undef LDIST_BWD_W
+    const WeightPlan wp = plan_backward_weight(pr);
+    const dim3 grid((unsigned)(pr.G * wp.n_blocks), (unsigned)wp.k_ranges);
+    const size_t lds = (size_t)wp.NB * wp.KC * sizeof(double);
+    if (overwrite)
+        hipLaunchKernelGGL(inf_backward_weight_kernel<true>, grid, dim3(wp.threads), lds, stream, grad_output, pos, grad_weight, d,
+                           wp.NB, wp.KC, wp.n_blocks);
+    else
+        hipLaunchKernelGGL(inf_backward_weight_kernel<false>, grid, dim3(wp.threads), lds, stream, grad_output, pos, grad_weight, d,
+                           wp.NB, wp.KC, wp.n_blocks);
     return hipGetLastError();
 }
 
@@ -523,16 +531,16 @@ hipError_t inf_backward_weight(const float* grad_output, const int32_t* pos, flo
 // the two launches of the separate entry points.
 hipError_t inf_backward_both(const float* grad_output, const int32_t* pos, float* grad_input, float* grad_weight,
                              const Problem& pr, hipStream_t stream) {
-    const int slots_w = kBinBytes / (int)sizeof(float);
-    const int nbr = min(pr.NG, min(4, (kRowBinsPre * 256) / max(pr.B, 1)));
-    const bool rowbins = nbr >= 2 && (long)pr.G * ((pr.NG + nbr - 1) / nbr) >= 4L * pr.num_cu;
-    const int nb = rowbins ? nbr : max(1, min(min(pr.NG, 8), slots_w / max(pr.K, 1)));
+    const int nbr = rowbins_rows(pr);
+    const bool rowbins = nbr > 0;
+    const WeightPlan wp = plan_backward_weight(pr);
+    const int nb = rowbins ? nbr : wp.NB;
     const int real_blocks = (pr.NG + nb - 1) / nb;
     const int n_blocks = real_blocks >= 64 ? (real_blocks + 7) / 8 * 8 : real_blocks;
     const long wgs_x = (long)pr.B * pr.G, wgs_w = (long)pr.G * n_blocks;
-    const bool one_launch = pr.HW == 1 && pr.K <= kInputBins && pr.K <= slots_w &&
-                            (long)pr.G * real_blocks >= 2L * pr.num_cu &&   // inf_backward_weight would not split the images
-                            wgs_x + wgs_w < (1L << 31);
+    // one launch of 256-lane workgroups: grad_weight as one k range per block of rows, enough blocks to fill the device
+    const bool one_launch = pr.HW == 1 && pr.K <= kInputBins && (rowbins || (wp.k_ranges == 1 && wp.threads == 256)) &&
+                            (long)pr.G * real_blocks >= 2L * pr.num_cu && wgs_x + wgs_w < (1L << 31);
     if (!one_launch) {
         if (hipError_t e = inf_backward_input(grad_output, pos, grad_input, pr, true, stream); e != hipSuccess) return e;
         return inf_backward_weight(grad_output, pos, grad_weight, pr, true, stream);
@@ -549,7 +557,7 @@ hipError_t inf_backward_both(const float* grad_output, const int32_t* pos, float
     pl.kc_w = pr.K;
     pl.n_blocks = n_blocks;
     pl.rowbins = rowbins;
-    const size_t lds = std::max((size_t)pr.K * sizeof(double), (size_t)(rowbins ? 1 : nb) * pr.K * sizeof(float));
+    const size_t lds = (size_t)(rowbins ? 1 : nb) * pr.K * sizeof(double);
     hipLaunchKernelGGL(inf_backward_both_kernel, dim3((unsigned)(wgs_x + wgs_w)), dim3(256), lds, stream, grad_output, pos,
                        grad_input, grad_weight, d, pl);
     return hipGetLastError();

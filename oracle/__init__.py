@@ -108,6 +108,21 @@ def inf_dist_backward_weight(grad_output, pos, CI, group=1, grad_weight=None):
     return grad_weight
 
 
+def inf_dist_backward_input_f64(grad_output, pos, CI, group=1):
+    """The same scatter as inf_dist_backward_input (reference model/inf_dist_cuda.cu:143-156) with the sums left in
+    float64 -- the exact column gradient, for checks that go on summing it (fold) before anything is rounded.
+    torch.scatter_add_ along k; indices past K are dropped like the C loop drops them."""
+    B, CO, HW = grad_output.shape
+    K, NG = CI // group, CO // group
+    idx = (pos & 0x7FFFFFFF).long().reshape(B, group, NG, HW)
+    g = grad_output.double().reshape(B, group, NG, HW)
+    sg = torch.where(pos.reshape(B, group, NG, HW) >= 0, g, -g)
+    keep = idx < K
+    acc = torch.zeros(B, group, K, HW, dtype=torch.float64)
+    acc.scatter_add_(2, torch.where(keep, idx, torch.zeros_like(idx)), torch.where(keep, sg, torch.zeros_like(sg)))
+    return acc.reshape(B, CI, HW)
+
+
 def norm_dist_forward(x, weight, group, p, f32_reference_order=False):
     B, CO, CI, G, HW = _dims(x, weight, group)
     out = torch.empty(B, CO, HW, dtype=torch.float32)

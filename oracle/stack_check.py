@@ -8,7 +8,10 @@ really received and produced on the GPU; the oracle then repeats every layer on 
 ("teacher forced"), so each comparison is as sharp as the operator allows:
 
 * L_inf values: bit-exact (fp32 sub / abs / max are exact and order-independent);
-* argmax routing: checked through both scatter gradients, which move if a single index or sign differs;
+* arg-max indices with their sign bits: bit-exact, from the caller's `inf_forward` (the library's forward entry point
+  run again on the recorded input: the same launch the layer made, whose values must equal the recorded ones bit
+  for bit), and once more through both scatter gradients, which move if a single index or sign differs;
+* L_inf scatter gradients: rel 1e-5 / abs 1e-6 (the library rounds double sums once);
 * p-norm values: rel 1e-5 / abs 1e-6; gradients: the float32-sum tolerance of `sum_ratio` (ratio <= 1 passes);
 * the mean shift: abs 2e-6 against the float64 mean;
 * and, free running from the input (the oracle feeding itself), the last layer's output: every layer is
@@ -25,36 +28,18 @@ from . import (inf_dist_backward_input, inf_dist_backward_weight, inf_dist_bound
                norm_dist_backward_input, norm_dist_backward_weight, norm_dist_forward)
 
 
-U32 = 2.0 ** -24     # unit roundoff of float32
+from .tolerance import plain_ratio, pnorm_grad_ratio
 
 
-def sum_ratio(got, exact, abs_terms, p=None, rtol=1e-5, atol=1e-6, n_terms=None):
-    """Worst |got - exact| / bound over the tensor, bound = s * (rtol*|exact| + a*max(1, sum|terms|)),
-    s = max(1, p/8): the tolerance of a float32 sum of signed terms (see tests/helpers.py:assert_sum_close).
-    a = atol, or, when the number of terms per element is given, max(atol, n_terms * 2^-24): a float32 sum of n
-    terms, in any order, is only guaranteed to n * 2^-24 * sum|terms| (the reference's atomicAdd no better),
-    which passes 1e-6 from 17 terms on -- the scatter of a wide layer puts hundreds on one element."""
-    scale = 1.0 if p is None else max(1.0, p / 8.0)
-    err = (got.double() - exact.double()).abs()
-    a = atol if n_terms is None else (n_terms.double() * U32).clamp_min(atol)
-    bound = scale * (rtol * exact.double().abs() + a * abs_terms.double().clamp_min(1.0))
-    return float((err / bound).max())
-
-
-def worst_element(got, exact, abs_terms, n_terms, rtol=1e-5, atol=1e-6):
-    """The element with the largest error against the plain tolerance: its error, exact value, sum|terms|, term count."""
-    err = (got.double() - exact.double()).abs()
-    r = err / (rtol * exact.double().abs() + atol * abs_terms.double().clamp_min(1.0))
-    i = int(r.reshape(-1).argmax())
-    pick = lambda t: float(t.reshape(-1)[i])
-    return {"err": pick(err), "exact": pick(exact), "sum_abs_terms": pick(abs_terms), "terms": int(pick(n_terms)),
-            "err_over_plain_tolerance": round(pick(r), 3)}
+def sum_ratio(got, exact, abs_terms, p):
+    """A p-norm gradient against the oracle's: worst error / bound with the float32-sum tolerance
+    (oracle/tolerance.py:pnorm_grad_ratio)."""
+    return pnorm_grad_ratio(got, exact, abs_terms, p)
 
 
 def close_ratio(got, exact, rtol=1e-5, atol=1e-6):
-    """Worst |got - exact| / (atol + rtol*|exact|)."""
-    err = (got.double() - exact.double()).abs()
-    return float((err / (atol + rtol * exact.double().abs())).max())
+    """Worst |got - exact| / (atol + rtol*|exact|): the plain tolerance, also for every L_inf scatter gradient."""
+    return plain_ratio(got, exact, rtol, atol)
 
 
 class Report:
@@ -66,12 +51,7 @@ class Report:
         self.toleranced = 0       # tensors compared within a tolerance
         self.worst_ratio = 0.0    # largest err / bound of the toleranced ones
         self.max_rel_err = 0.0    # largest max|got - exact| / max|exact| over all compared tensors
-        self.worst_plain = 0.0    # scatter sums against the tolerance that ignores the number of terms (for the record)
         self.failures = []
-        self.details = {}         # per scatter gradient: the element furthest out against the plain tolerance
-
-    def plain(self, r):
-        self.worst_plain = max(self.worst_plain, r)
 
     def _rel(self, got, exact):
         scale = float(exact.double().abs().max())
@@ -96,7 +76,6 @@ class Report:
 
     def as_json(self):
         return {"checked": self.ok, "max_rel_err": self.max_rel_err, "worst_err_over_tolerance": round(self.worst_ratio, 4),
-                "scatter_err_over_tolerance_without_term_count": round(self.worst_plain, 4),
                 "tensors_bit_exact": self.exact, "tensors_within_tolerance": self.toleranced, "failures": self.failures[:8]}
 
 
@@ -161,10 +140,11 @@ def record_training_step(model, x_dev, upstream_dev):
     return out, (-y).detach().cpu()     # the net negates its output (model/mlp.py:22)
 
 
-def check_training_step(model, x_cpu, upstream_cpu, p, dev, rows=None, weight_rows=None, report=None):
+def check_training_step(model, x_cpu, upstream_cpu, p, dev, rows=None, weight_rows=None, report=None, inf_forward=None):
     """Teacher-forced comparison of one training step of the MLP with the oracle.  `rows` (slice of the batch)
     and `weight_rows` (slice of each layer's outputs) bound the oracle's work for the p-norm operators; None
-    means everything.  Returns the Report."""
+    means everything.  `inf_forward(x_cpu, w_cpu) -> (values, pos)` (CPU tensors) is the library's L_inf forward
+    entry point, for the direct comparison of the indices at p = inf.  Returns the Report."""
     rep = report or Report()
     inf = math.isinf(p)
     layers, y_gpu = record_training_step(model, x_cpu.to(dev), upstream_cpu.to(dev))
@@ -182,6 +162,10 @@ def check_training_step(model, x_cpu, upstream_cpu, p, dev, rows=None, weight_ro
         if inf:
             ev, ep = inf_dist_forward(xin[rs].contiguous(), w, 1)
             rep.equal(name + " values", raw[rs], ev)
+            if inf_forward is not None:
+                gv, gp = inf_forward(xin[rs].contiguous(), w)
+                rep.equal(name + " values of the repeated launch against the layer's own", gv, raw[rs])
+                rep.equal(name + " arg-max indices and signs", gp, ep)
         else:
             ev = norm_dist_forward(xin[rs].contiguous(), w, 1, p)
             rep.ratio(name + " values", close_ratio(raw[rs], ev), raw[rs], ev)
@@ -194,21 +178,11 @@ def check_training_step(model, x_cpu, upstream_cpu, p, dev, rows=None, weight_ro
         g = L["grad_raw"]
         if inf:
             ev_all, ep_all = (ev, ep) if rs == slice(0, B) else inf_dist_forward(xin, w, 1)
-            mag = ep_all & 0x7FFFFFFF
-            ones = torch.ones_like(g)
             egw = inf_dist_backward_weight(g, ep_all, CI, 1)
-            mgw = -inf_dist_backward_weight(g.abs(), mag, CI, 1)
-            ngw = -inf_dist_backward_weight(ones, mag, CI, 1)          # how many gradients land on each element
-            rep.ratio(name + " grad_weight", sum_ratio(L["grad_weight"], egw, mgw, n_terms=ngw), L["grad_weight"], egw)
-            rep.plain(sum_ratio(L["grad_weight"], egw, mgw))
-            rep.details[name + " grad_weight"] = worst_element(L["grad_weight"], egw, mgw, ngw)
+            rep.ratio(name + " grad_weight", close_ratio(L["grad_weight"], egw), L["grad_weight"], egw)
             if L.get("grad_input") is not None:
                 egx = inf_dist_backward_input(g, ep_all, CI, 1)
-                mgx = inf_dist_backward_input(g.abs(), mag, CI, 1)
-                ngx = inf_dist_backward_input(ones, mag, CI, 1)
-                rep.ratio(name + " grad_input", sum_ratio(L["grad_input"], egx, mgx, n_terms=ngx), L["grad_input"], egx)
-                rep.plain(sum_ratio(L["grad_input"], egx, mgx))
-                rep.details[name + " grad_input"] = worst_element(L["grad_input"], egx, mgx, ngx)
+                rep.ratio(name + " grad_input", close_ratio(L["grad_input"], egx), L["grad_input"], egx)
         else:
             gw_s = slice(ws.start, ws.stop)
             egw, mgw = norm_dist_backward_weight(g[:, gw_s].contiguous(), xin, w[gw_s].contiguous(),

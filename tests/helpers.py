@@ -1,7 +1,8 @@
 """Closed forms used to pin the oracle and seeded input makers shared by the tests.
 
-Nothing here calls the oracle or the HIP library: these are independent
-restatements of the mathematics in plain torch broadcasting.
+Nothing here calls the oracle's operators or the HIP library: these are independent
+restatements of the mathematics in plain torch broadcasting.  The two assert_* helpers at
+the end apply the tolerances defined once in oracle/tolerance.py.
 """
 import torch
 
@@ -90,35 +91,36 @@ def dense_inf_backward(grad_out, pos, CI, G):
     return grad_x, grad_w
 
 
-# Worst err / bound seen by assert_sum_close, per exponent (None: the L_inf scatter sums).  The test session
-# prints it at the end (tests/conftest.py), so the margin that the float32-sum tolerance leaves is visible.
+# Worst err / bound seen by the gradient comparisons, per exponent (None: the L_inf scatter sums).  The test session
+# prints it at the end (tests/conftest.py).
 SUM_CLOSE_MARGINS = {}
 
 
-def assert_sum_close(got, exact, abs_terms, p=None, rtol=1e-5, atol=1e-6):
-    """Tolerance for a float32 sum of signed terms checked against its exact value.
-
-    |got - exact| <= tol_scale * (rtol*|exact| + atol*max(1, sum|terms|)).
-    The absolute part scales with the size of what was summed: float32 rounding
-    of the terms alone already leaves an error proportional to sum|terms|, for
-    any implementation.  For the p-norm gradients every term is u^(p-1) with u
-    known to about 2e-7 relative, so the terms themselves are only good to
-    (p-1)*2e-7; tol_scale = max(1, p/8) accounts for that above p = 8.
-    Returns the worst err / bound ratio (<= 1) and records it per exponent.
-    """
-    scale = 1.0 if p is None else max(1.0, p / 8.0)
-    err = (got.double() - exact.double()).abs()
-    bound = scale * (rtol * exact.double().abs() + atol * abs_terms.double().clamp_min(1.0))
-    ratio = err / bound
-    worst = float(ratio.max()) if ratio.numel() else 0.0
-    # the same comparison at the plain tolerance (scale 1, sum|terms| not used), for the record
-    plain = float((err / (rtol * exact.double().abs() + atol)).max()) if ratio.numel() else 0.0
+def _record(p, worst, plain):
     seen = SUM_CLOSE_MARGINS.setdefault(p, {"calls": 0, "worst_err_over_bound": 0.0, "worst_err_over_plain_1e-5_1e-6": 0.0})
     seen["calls"] += 1
     seen["worst_err_over_bound"] = max(seen["worst_err_over_bound"], worst)
     seen["worst_err_over_plain_1e-5_1e-6"] = max(seen["worst_err_over_plain_1e-5_1e-6"], plain)
-    bad = err > bound
-    assert not bool(bad.any()), (
-        f"{int(bad.sum())} of {bad.numel()} elements outside tolerance; worst err/bound {worst:.3f}, worst excess "
-        f"{float((err - bound).max()):.3e} (err {float(err[bad].max()):.3e})")
+
+
+def assert_scatter_close(got, exact, rtol=None, atol=None):
+    """An L_inf scatter gradient against the oracle's: the plain tolerance |got - exact| <= 1e-6 + 1e-5 * |exact|
+    (oracle/tolerance.py:plain_ratio), whatever the number of terms on an element."""
+    from oracle import tolerance
+    worst = tolerance.plain_ratio(got, exact, rtol or tolerance.RTOL, atol or tolerance.ATOL)
+    _record(None, worst, worst)
+    assert worst <= 1.0, f"L_inf scatter: worst error is {worst:.3f} x the tolerance (rel 1e-5 / abs 1e-6)"
+    return worst
+
+
+def assert_sum_close(got, exact, abs_terms, p, rtol=None, atol=None):
+    """A p-norm gradient (a float32 sum of signed terms) against its exact value, with the tolerance of
+    oracle/tolerance.py:pnorm_grad_ratio, which scales with sum|terms| and max(1, p/8).
+    Returns the worst err / bound ratio (<= 1) and records it per exponent."""
+    from oracle import tolerance
+    assert p is not None, "L_inf scatters are compared with assert_scatter_close"
+    rtol, atol = rtol or tolerance.RTOL, atol or tolerance.ATOL
+    worst = tolerance.pnorm_grad_ratio(got, exact, abs_terms, p, rtol, atol)
+    _record(p, worst, tolerance.plain_ratio(got, exact, rtol, atol))
+    assert worst <= 1.0, f"p = {p}: worst error is {worst:.3f} x the float32-sum tolerance"
     return worst

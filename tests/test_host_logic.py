@@ -441,6 +441,21 @@ def test_stack_checker_passes_on_a_correct_net_and_catches_a_wrong_one(fake_nati
     assert rep.ok, rep.failures
     assert rep.toleranced >= 9 and (rep.exact == 3 if math.isinf(p) else rep.exact == 0)
 
+    if math.isinf(p):
+        # the direct comparison of the indices: the entry point run again on every recorded input
+        def inf_forward(xs, ws, flip=False):
+            o = torch.empty(xs.size(0), ws.size(0), 1)
+            ps = torch.empty(xs.size(0), ws.size(0), 1, dtype=torch.int32)
+            cpp.inf_dist_forward(xs, ws, o, ps, 1)
+            if flip:
+                ps[3, 2, 0] ^= 1          # one index off by one, value untouched
+            return o, ps
+        rep = stack_check.check_training_step(model, x, up, p, torch.device("cpu"), inf_forward=inf_forward)
+        assert rep.ok and rep.exact == 9, rep.failures
+        bad = stack_check.check_training_step(model, x, up, p, torch.device("cpu"),
+                                              inf_forward=lambda a, b: inf_forward(a, b, flip=True))
+        assert not bad.ok and all("arg-max indices" in f for f in bad.failures)
+
     # a wrong operator: values off by one ulp-sized factor in one layer
     good = cpp.inf_dist_forward if math.isinf(p) else cpp.norm_dist_forward
 

@@ -200,3 +200,17 @@ def test_forward_backward_finite_difference_tie_free():
             e = torch.zeros_like(wd); e[n, k] = h
             fd = (f(xd, wd + e) - f(xd, wd - e)) / (2 * h)
             assert abs(fd.item() - gw[n, k].item()) < 1e-5
+
+
+@pytest.mark.parametrize("shape", [(3, 12, 10, 1, 1), (2, 8, 12, 2, 5), (4, 6, 9, 3, 7)])
+def test_backward_input_f64_is_the_one_hot_expansion(shape):
+    """oracle.inf_dist_backward_input_f64 (the column gradient left in float64, used where a check goes on summing
+    before anything is rounded) against the dense one-hot expansion, exactly; its float32 rounding is the C oracle's."""
+    B, CO, CI, G, HW = shape
+    x, w = make_inputs(B, CO, CI, G, HW, seed=31, quantize=4)
+    _, pos = oracle.inf_dist_forward(x, w, G)
+    go = torch.randn(B, CO, HW, generator=gen(32))
+    gx64 = oracle.inf_dist_backward_input_f64(go, pos, CI, G)
+    dense_x, _ = dense_inf_backward(go, pos, CI, G)
+    assert gx64.dtype == torch.float64 and torch.equal(gx64, dense_x)
+    assert torch.equal(gx64.float(), oracle.inf_dist_backward_input(go, pos, CI, G))
