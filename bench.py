@@ -396,6 +396,7 @@ def workload_c4(pkg, torch, dev):
         return rep
 
     return dict(step=step, ops=128 * 1024 * 128 * 288, images=128, full_rows=128, cpu=cpu, formula=formula, check=check,
+                layer_routes=lambda: layer.last_route,     # what NormDistConv's last forward took (image / columns)
                 step_alt=[("ms_per_step_from_image", step_from_image),
                           ("ms_per_step_with_torch_unfold_and_fold", step_torch_unfold)],
                 name="configs[4]: unfolded 3x3 L_inf-dist conv layer, batch 128, 128->128 channels, 32x32, groups 4, "
@@ -504,6 +505,7 @@ def workload_c4p(pkg, torch, dev):
                 # a geometry the image kernels do not cover would fall back to unfold + columns + fold
                 routes={"from_image": bool(pkg.norm_dist_cpp.norm_dist_conv_supported(128, 32, 32, 128, 4, 3, 1, 1, 1)),
                         "finite_p_route": layer.finite_p_route},
+                layer_routes=lambda: layer.last_route,
                 step_alt=[("ms_per_step_native_unfold_columns_fold", step_columns),
                           ("ms_per_step_with_torch_unfold_and_fold", step_torch_unfold)],
                 name=f"configs[4]'s layer at p={p:g} from the image: 3x3 p-norm dist conv layer, batch 128, 128->128 "
@@ -667,14 +669,17 @@ def main():
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": wl["name"], "dist_ops_per_step": ops, **wl.get("routes", {})},
+        "config": {"workload": wl["name"], "dist_ops_per_step": ops, **wl.get("routes", {}),
+                   **({"routes": wl["layer_routes"]()} if "layer_routes" in wl else {})},
         "img_per_s": round(wl["images"] / (ms_per_step * 1e-3), 1),
         "pct_fp32_valu_peak": round(100 * value * 1e9 * flops_per_op / (FP32_PEAK_TFLOPS * 1e12), 2),
         "parity": parity,
         "roofline": {
-            "bound": "mfma",
-            "kernel": kdesc + " -- VALU only: a max / power-sum reduction has no multiply-accumulate for MFMA; "
-                              "'mfma' names the compute roof, priced at the fp32 vector peak",
+            "bound": "valu",
+            # the bench contract names "hbm" and "mfma"; this kernel's compute roof is neither: it is the fp32 vector ALU
+            "bound_note": "compute roof, fp32 vector ALU (published dense fp32 peak); a max / power-sum reduction has "
+                          "no multiply-accumulate, so there is no MFMA work on this path",
+            "kernel": kdesc,
             "achieved": round(achieved, 2),
             "peak": FP32_PEAK_TFLOPS,
             "unit": "TFLOP/s",

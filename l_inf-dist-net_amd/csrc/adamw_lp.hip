@@ -13,6 +13,7 @@
 
 #include "kernels.hpp"
 #include "pow.hpp"
+#include "wave_reduce.hpp"
 
 namespace ldist {
 
@@ -38,10 +39,9 @@ __device__ __forceinline__ float adam_update(float w, float g, float& m, float& 
 }
 
 __device__ __forceinline__ float block_max(float v, float* red) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v = __builtin_fmaxf(v, __shfl_xor(v, off, 64));
+    v = wave_max(v);                // lane 63 holds the wave's maximum
     __syncthreads();
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    if ((threadIdx.x & 63) == 63) red[threadIdx.x >> 6] = v;
     __syncthreads();
     float r = red[0];
     for (int q = 1; q < (int)(blockDim.x >> 6); q++) r = __builtin_fmaxf(r, red[q]);
@@ -49,10 +49,9 @@ __device__ __forceinline__ float block_max(float v, float* red) {
 }
 
 __device__ __forceinline__ float block_sum(float v, float* red) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+    v = wave_sum(v);                // lane 63 holds the wave's sum
     __syncthreads();
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    if ((threadIdx.x & 63) == 63) red[threadIdx.x >> 6] = v;
     __syncthreads();
     float r = 0.f;
     for (int q = 0; q < (int)(blockDim.x >> 6); q++) r += red[q];
@@ -118,13 +117,8 @@ adamw_lp_rows_kernel(float* __restrict__ param, const float* __restrict__ grad, 
                 if (m > best) { best = m; where = i * VEC + e; }   // ascending columns per lane: first maximum kept
             }
         }
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) {
-            const float ob = __shfl_xor(best, off, 64);
-            const int ow = __shfl_xor(where, off, 64);
-            if (ob > best || (ob == best && ow < where)) { best = ob; where = ow; }
-        }
-        if ((threadIdx.x & 63) == 0) { red[threadIdx.x >> 6] = best; red_i[threadIdx.x >> 6] = where; }
+        wave_best(best, where);     // larger value, then lower column: lane 63
+        if ((threadIdx.x & 63) == 63) { red[threadIdx.x >> 6] = best; red_i[threadIdx.x >> 6] = where; }
         __syncthreads();
         best = red[0];
         where = red_i[0];

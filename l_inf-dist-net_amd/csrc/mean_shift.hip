@@ -5,6 +5,7 @@
 // (gx = gy - mean(gy)).  HBM-bound: a workgroup owns a slab small enough that its second read
 // comes from cache, so the tensor is fetched once and written once.
 #include "kernels.hpp"
+#include "wave_reduce.hpp"
 
 namespace ldist {
 
@@ -139,9 +140,8 @@ mean_shift_channel_kernel(const float* __restrict__ x, float* __restrict__ y, fl
             for (int u = 0; u < UN; u++) s += v[u];
         }
     }
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) s += __shfl_xor(s, off, 64);
-    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+    s = wave_sum(s);                // lane 63 holds the wave's sum
+    if ((threadIdx.x & 63) == 63) part[threadIdx.x >> 6] = s;
     __syncthreads();
     if (threadIdx.x == 0) {
         float t = 0.f;

@@ -119,7 +119,10 @@ def certified_accuracy(net, inputs, targets, eps, up, down):
     set_p_norm(net, float("inf"))
     net.eval()
     try:
-        worst = net(inputs, lower=_box(inputs - eps, down, up), upper=_box(inputs + eps, down, up), targets=targets)[1]
+        # the lower corner is clipped from below only and the upper corner from above only (reference main.py:178-179)
+        lower = torch.maximum(inputs - eps, torch.as_tensor(down, dtype=inputs.dtype, device=inputs.device))
+        upper = torch.minimum(inputs + eps, torch.as_tensor(up, dtype=inputs.dtype, device=inputs.device))
+        worst = net(inputs, lower=lower, upper=upper, targets=targets)[1]
         return cal_acc(worst, targets).mean().item()
     finally:
         set_p_norm(net, keep[0])

@@ -388,11 +388,17 @@ class NormDistConv(nn.Module):
                 self.kernel_size == 1 and self.stride == 1 and self.padding == 0 and   # windows: the image kernels
                 self.out_channels // self.group <= self.FUSED_VALUE_BOUND_MAX_OUTPUTS)
 
+    # Which kernels the last forward call took, e.g. {"values": "image", "bounds": None}: "image" (straight from
+    # the (B, C, H, W) tensor), "columns" (patches first: the reference's only route, and where every window the image
+    # kernels do not cover ends up), "one_pass" (values and bounds from one kernel).  Not in the reference.
+    last_route = None
+
     def forward(self, x, lower=None, upper=None):
         span = self.kernel_size - 2 * self.padding
         out_hw = ((x.size(2) - span) // self.stride + 1, (x.size(3) - span) // self.stride + 1)
         w2d = self.weight.view(self.weight.size(0), -1)
         if lower is not None and upper is not None and self._value_and_bounds_in_one_pass(x, lower, upper):
+            self.last_route = {"values": "one_pass", "bounds": "one_pass"}
             cx, cl, cu = (self._columns(t).contiguous() for t in (x, lower, upper))
             y = torch.empty(x.size(0), w2d.size(0), out_hw[0] * out_hw[1], device=x.device, dtype=x.dtype)
             lo, hi = torch.empty_like(y), torch.empty_like(y)
@@ -402,11 +408,14 @@ class NormDistConv(nn.Module):
                 None if self.bias is None else self.bias.detach())
             shape = (x.size(0), -1, *out_hw)
             return y.view(shape), lo.view(shape), hi.view(shape)
+        route = {"values": "columns", "bounds": None}
         if self._fused_inf_conv(x):
             wants_grad = torch.is_grad_enabled() and (x.requires_grad or w2d.requires_grad)
-            if wants_grad or not norm_dist_cpp.inf_dist_conv_forward_supported(
-                    x.size(1), x.size(2), x.size(3), w2d.size(0), self.group, self.kernel_size, self.stride,
-                    self.padding, self.dilation):
+            from_image = norm_dist_cpp.inf_dist_conv_forward_supported(
+                x.size(1), x.size(2), x.size(3), w2d.size(0), self.group, self.kernel_size, self.stride, self.padding,
+                self.dilation)
+            route["values"] = "image" if from_image else "columns"   # _ConvInfDist decides by the same call
+            if wants_grad or not from_image:
                 y = _ConvInfDist.apply(x, w2d, self.group, self.kernel_size, self.dilation, self.padding, self.stride)
             else:   # no gradient follows: the argmax has no reader, and the kernel without it is faster
                 ho, wo = out_hw
@@ -414,15 +423,19 @@ class NormDistConv(nn.Module):
                 norm_dist_cpp.inf_dist_conv_forward_values(x.contiguous(), w2d, y, self.group, self.kernel_size,
                                                            self.stride, self.padding, self.dilation)
         elif self._norm_from_image(x):
+            route["values"] = "image"
             y = _ConvNormDist.apply(x, w2d, self.group, self.p, self.kernel_size, self.dilation, self.padding,
                                     self.stride)
         else:
             y = norm_dist(self._columns(x), w2d, self.group, p=self.p, tag=self.tag)
         y = self._shift(y.view(x.size(0), -1, *out_hw))  # in training mode only y moves the running mean
+        self.last_route = route
         if lower is None or upper is None:
             return y, None, None
         assert math.isinf(self.p) and not self.training
+        route["bounds"] = "columns"
         if self._bound_from_images(lower, upper):
+            route["bounds"] = "image"
             lo = torch.empty(x.size(0), w2d.size(0), out_hw[0] * out_hw[1], device=x.device, dtype=x.dtype)
             hi = torch.empty_like(lo)
             with torch.no_grad():

@@ -401,6 +401,24 @@ def test_pgd_stays_in_the_ball_and_the_range_and_raises_the_loss():
     assert torch.allclose(fixed, expect)   # one step without the random start is the signed-gradient step
 
 
+def test_certified_accuracy_clips_each_corner_on_one_side_only():
+    """Reference main.py:178-179: lower = max(inputs - eps, down), upper = min(inputs + eps, up) -- the lower corner is
+    not clipped from above nor the upper corner from below, which shows for inputs outside the data range."""
+    pkg = entry.load_package()
+    seen = {}
+
+    class Net(torch.nn.Module):
+        def forward(self, x, lower=None, upper=None, targets=None):
+            seen["lower"], seen["upper"] = lower, upper
+            return x, x
+
+    x = torch.tensor([[-0.5, 0.2, 1.4], [0.05, 0.95, 0.5]])
+    down, up = torch.zeros(3), torch.ones(3)
+    pkg.certified_accuracy(Net(), x, torch.tensor([0, 1]), 0.1, up, down)
+    assert torch.equal(seen["lower"], torch.max(x - 0.1, down)) and torch.equal(seen["upper"], torch.min(x + 0.1, up))
+    assert float(seen["lower"][0, 2]) == pytest.approx(1.3) and float(seen["upper"][0, 0]) == pytest.approx(-0.4)
+
+
 def test_train_step_and_accuracy_helpers():
     pkg = entry.load_package()
     torch.manual_seed(4)

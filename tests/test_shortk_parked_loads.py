@@ -1,8 +1,8 @@
 """The short-K L_inf forward (csrc/inf_forward_shortk.hip) issues the loads of its input panel and the waits for
-them as inline assembly, so the compiler does not know that a parked register has a load in flight.  That is safe
-only as long as the generated code never reads such a register between the load and the wait that stands in front
-of the panel write.  This test compiles the file to assembly (no GPU needed) and checks exactly that, for every
-instantiation of the kernel."""
+them as inline assembly, so the compiler does not know that a parked register has a load in flight.  The library's
+Makefile checks the generated code with csrc/check_parked_loads.py before it links; this test runs the same check on a
+fresh compile (no GPU needed) and tests the checker itself."""
+import importlib.util
 import os
 import re
 import shutil
@@ -11,92 +11,21 @@ import subprocess
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-SRC = os.path.join(ROOT, "l_inf-dist-net_amd", "csrc", "inf_forward_shortk.hip")
+CSRC = os.path.join(ROOT, "l_inf-dist-net_amd", "csrc")
+SRC = os.path.join(CSRC, "inf_forward_shortk.hip")
 
-LOAD = re.compile(r"^\s*buffer_load_dwordx4 v\[(\d+):(\d+)\], v(\d+), ")
-WRITE = re.compile(r"^\s*ds_write_b128 v(\d+), v\[(\d+):(\d+)\]")
-WAIT = re.compile(r"^\s*s_waitcnt vmcnt\((\d+)\)\s*$")
+_spec = importlib.util.spec_from_file_location("check_parked_loads", os.path.join(CSRC, "check_parked_loads.py"))
+checker = importlib.util.module_from_spec(_spec)
+_spec.loader.exec_module(checker)
+check_kernel = checker.check_kernel
 
 
 def library_flags():
     """The compiler flags of the library's Makefile (FLAGS := ... with its continuation line), ARCH filled in."""
-    text = open(os.path.join(os.path.dirname(SRC), "Makefile")).read()
+    text = open(os.path.join(CSRC, "Makefile")).read()
     arch = re.search(r"^ARCH\s*\?=\s*(\S+)", text, re.M).group(1)
     flags = re.search(r"^FLAGS\s*:=\s*((?:.*\\\n)*.*)$", text, re.M).group(1).replace("\\\n", " ")
     return flags.replace("$(ARCH)", arch).split()
-
-
-def registers(text):
-    """Vector registers named in an operand string."""
-    regs = set()
-    for lo, hi in re.findall(r"\bv\[(\d+):(\d+)\]", text):
-        regs.update(range(int(lo), int(hi) + 1))
-    regs.update(int(r) for r in re.findall(r"\bv(\d+)\b", text))
-    return regs
-
-
-def kernels(asm):
-    """name -> instruction lines (comments and directives dropped) of every shortk kernel in the listing."""
-    out, name = {}, None
-    for line in asm.splitlines():
-        m = re.match(r"^(_ZN5ldist25inf_forward_shortk_kernelILi(\d+)E\S*):", line)
-        if m:
-            name = int(m.group(2))
-            out[name] = []
-            continue
-        if name is None:
-            continue
-        code = line.split(";")[0].rstrip()
-        if re.match(r"^\s+s_endpgm", code):
-            out[name].append(code)
-            name = None
-            continue
-        if re.match(r"^\s+[a-z]", code):
-            out[name].append(code)
-    return out
-
-
-def check_kernel(nw, lines):
-    loads = [i for i, l in enumerate(lines) if LOAD.match(l)]
-    assert loads, "no buffer loads found"
-    parks = set()
-    for i in loads:
-        lo, hi, _ = map(int, LOAD.match(lines[i]).groups())
-        assert hi - lo == 3
-        parks.update(range(lo, hi + 1))
-    assert len(parks) == 4 * nw, (nw, sorted(parks))
-    writes = 0
-    pending = set()      # registers with a load in flight, in listing order (every straight run of the loop is in order)
-    # the region in which the parked registers are live: first load .. last load (the tile loop and its prologue)
-    for i in range(loads[0], loads[-1] + 1):
-        line = lines[i]
-        ld = LOAD.match(line)
-        if ld:
-            lo, hi, addr = map(int, ld.groups())
-            assert addr not in pending, f"address register has a load in flight: {line.strip()}"
-            assert not (set(range(lo, hi + 1)) & pending), f"second load into registers in flight: {line.strip()}"
-            pending.update(range(lo, hi + 1))
-            continue
-        if not (registers(line) & parks):
-            continue
-        w = WRITE.match(line)
-        if w and set(range(int(w.group(2)), int(w.group(3)) + 1)) <= parks:
-            addr, lo, hi = map(int, w.groups())
-            assert addr not in pending, line
-            # the wait stands in front of the write; what the scheduler put between them must leave the data alone
-            j = i - 1
-            while not WAIT.match(lines[j]):
-                assert not (registers(lines[j]) & set(range(lo, hi + 1))), (lines[j], line)
-                j -= 1
-                assert j >= loads[0], f"no wait in front of {line.strip()}"
-            assert int(WAIT.match(lines[j]).group(1)) <= nw - 1, (lines[j], line)
-            pending.difference_update(range(lo, hi + 1))
-            writes += 1
-            continue
-        # anything else may use a parked register only while no load into it is in flight (the offset of the next
-        # load is computed there, between the panel write and the load)
-        assert not (registers(line) & pending), f"touches a register with a load in flight: {line.strip()}"
-    assert writes == nw, (nw, writes)
 
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="hipcc not on PATH")
@@ -104,15 +33,13 @@ def test_no_read_of_a_parked_register_before_its_wait(tmp_path):
     out = tmp_path / "shortk.s"
     cmd = ["hipcc"] + library_flags() + ["-S", "--cuda-device-only", SRC, "-o", str(out)]
     subprocess.run(cmd, check=True, capture_output=True)
-    asm = out.read_text()
-    found = kernels(asm)
-    assert sorted(found) == list(range(1, 11))
-    for nw, lines in found.items():
-        check_kernel(nw, lines)
-    # the window loop is unrolled over the parked registers: none of them may have gone to scratch memory
-    spills = re.findall(r"\.vgpr_spill_count:\s*(\d+)", asm)
-    assert len(spills) == 10 and all(int(n) == 0 for n in spills), spills
+    assert checker.check_listing(out.read_text()) == list(range(1, 11))
 
+
+def test_the_makefile_runs_the_check_before_it_links():
+    text = open(os.path.join(CSRC, "Makefile")).read()
+    assert "check_parked_loads.py" in text
+    assert re.search(r"^\$\(OUT\):.*\$\(SHORTK_OK\)", text, re.M), "the library must depend on the check's stamp"
 
 def test_the_check_itself_flags_an_early_read():
     good = ["\tbuffer_load_dwordx4 v[2:5], v9, s[0:3], s4 offen",
