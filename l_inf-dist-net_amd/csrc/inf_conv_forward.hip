@@ -370,61 +370,68 @@ inf_conv_forward_kernel(const float* __restrict__ img, const float* __restrict__
     // and one word instead of one load per candidate, issued for the lane's eight positions together.
     typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
     static_assert(kTrack == 1, "a unit is one channel: nine candidates");
-#pragma unroll
-    for (int t = 0; t < kTN; t++) {
-        const int n = n0 + kTN * nl + t;
-        if (n >= a.NG) break;
+    // EB positions of one output at a time, in steps (output t, positions e0 .. e0 + EB - 1).  The weight loads of a
+    // step are issued one step ahead (two register sets that take turns), so that the cache latency of a step's
+    // weights passes while the step before it is searched; the pixels come from LDS (RESIDENT) or from the image.
+    constexpr int EB = kTM / 2, STEPS = kTN * (kTM / EB);
+    float wq[2][EB][9];
+    auto issue = [&](int step, float (&wb)[EB][9]) {
+        const int t = step / (kTM / EB), e0 = (step % (kTM / EB)) * EB;
+        const int n = min(n0 + kTN * nl + t, a.NG - 1);     // an output past the layer's last reads that one's weights
         const float* wn = weight + ((size_t)g * a.NG + n) * K;
-        int ps[kTM];
-        // EB positions at a time: their reads are issued together, then searched (the staged variant has less
-        // room in registers: it also carries the image words of the stage)
-        constexpr int EB = RESIDENT ? kTM : kTM / 2;
 #pragma unroll
-        for (int e0 = 0; e0 < kTM; e0 += EB) {
-            float wq[EB][9], xq[EB][9];
+        for (int eb = 0; eb < EB; eb++) {
+            const float* wp = wn + unit[e0 + eb][t] * 9;    // a recorded unit is a real channel: inside the row
+            const f4u q0 = *reinterpret_cast<const f4u*>(wp), q1 = *reinterpret_cast<const f4u*>(wp + 4);
+            wb[eb][0] = q0.x; wb[eb][1] = q0.y; wb[eb][2] = q0.z; wb[eb][3] = q0.w;
+            wb[eb][4] = q1.x; wb[eb][5] = q1.y; wb[eb][6] = q1.z; wb[eb][7] = q1.w;
+            wb[eb][8] = wp[8];
+        }
+    };
+    int ps[kTM];
+    issue(0, wq[0]);
 #pragma unroll
-            for (int eb = 0; eb < EB; eb++) {
-                const int e = e0 + eb;
-                const float* wp = wn + unit[e][t] * 9;       // a recorded unit is a real channel: inside the row
-                const f4u q0 = *reinterpret_cast<const f4u*>(wp), q1 = *reinterpret_cast<const f4u*>(wp + 4);
-                wq[eb][0] = q0.x; wq[eb][1] = q0.y; wq[eb][2] = q0.z; wq[eb][3] = q0.w;
-                wq[eb][4] = q1.x; wq[eb][5] = q1.y; wq[eb][6] = q1.z; wq[eb][7] = q1.w;
-                wq[eb][8] = wp[8];
-            }
+    for (int step = 0; step < STEPS; step++) {
+        const int t = step / (kTM / EB), e0 = (step % (kTM / EB)) * EB;
+        if (step + 1 < STEPS) issue(step + 1, wq[(step + 1) & 1]);
+        float xq[EB][9];
 #pragma unroll
-            for (int eb = 0; eb < EB; eb++) {
-                const int e = e0 + eb;
-                if constexpr (RESIDENT) {
-                    const float* xe = xlane + e * S + unit[e][t] * CST;
+        for (int eb = 0; eb < EB; eb++) {
+            const int e = e0 + eb;
+            if constexpr (RESIDENT) {
+                const float* xe = xlane + e * S + unit[e][t] * CST;
 #pragma unroll
-                    for (int r = 0; r < 9; r++) xq[eb][r] = xe[(r / 3) * WP + r % 3];
-                } else {
-                    // the window of position (h, w0 + e) in the recorded channel; outside the image it reads 0
-                    const unsigned plane = (unsigned)unit[e][t] * (unsigned)(a.H * a.W);
-                    const int yy = h * S - a.P, xx = (w0 + e) * S - a.P;
+                for (int r = 0; r < 9; r++) xq[eb][r] = xe[(r / 3) * WP + r % 3];
+            } else {
+                // the window of position (h, w0 + e) in the recorded channel; outside the image it reads 0
+                const unsigned plane = (unsigned)unit[e][t] * (unsigned)(a.H * a.W);
+                const int yy = h * S - a.P, xx = (w0 + e) * S - a.P;
 #pragma unroll
-                    for (int r = 0; r < 9; r++) {
-                        const int y = yy + r / 3, x = xx + r % 3;
-                        const bool real = (unsigned)y < (unsigned)a.H && (unsigned)x < (unsigned)a.W;
-                        const float v = src[real ? plane + (unsigned)(y * a.W + x) : 0u];
-                        xq[eb][r] = real ? v : 0.f;
-                    }
+                for (int r = 0; r < 9; r++) {
+                    const int y = yy + r / 3, x = xx + r % 3;
+                    const bool real = (unsigned)y < (unsigned)a.H && (unsigned)x < (unsigned)a.W;
+                    const float v = src[real ? plane + (unsigned)(y * a.W + x) : 0u];
+                    xq[eb][r] = real ? v : 0.f;
                 }
-            }
-#pragma unroll
-            for (int eb = 0; eb < EB; eb++) {
-                const int e = e0 + eb;
-                const float target = acc[e][t];
-                int q = 0;
-                float dq = 0.f;
-#pragma unroll
-                for (int r = 8; r >= 0; r--) {                // descending: the lowest match is the one kept
-                    const float df = xq[eb][r] - wq[eb][r];
-                    if (__builtin_fabsf(df) == target) { q = r; dq = df; }
-                }
-                ps[e] = target > 0.f ? ((unit[e][t] * 9 + q) | (__float_as_int(dq) & 0x80000000)) : 0;
             }
         }
+        const float (&wb)[EB][9] = wq[step & 1];
+#pragma unroll
+        for (int eb = 0; eb < EB; eb++) {
+            const int e = e0 + eb;
+            const float target = acc[e][t];
+            int q = 0;
+            float dq = 0.f;
+#pragma unroll
+            for (int r = 8; r >= 0; r--) {                // descending: the lowest match is the one kept
+                const float df = xq[eb][r] - wb[eb][r];
+                if (__builtin_fabsf(df) == target) { q = r; dq = df; }
+            }
+            ps[e] = target > 0.f ? ((unit[e][t] * 9 + q) | (__float_as_int(dq) & 0x80000000)) : 0;
+        }
+        if (e0 + EB < kTM) continue;                      // the output's other positions come with the next step
+        const int n = n0 + kTN * nl + t;
+        if (n >= a.NG) continue;
         const size_t at = (((size_t)b * a.G + g) * a.NG + n) * L + (size_t)h * a.WO + w0;
         if (a.vec_out) {
             *reinterpret_cast<float4*>(out + at) = make_float4(acc[0][t], acc[1][t], acc[2][t], acc[3][t]);

@@ -44,8 +44,9 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
     const int ty = t % GEO::TY, tx = t / GEO::TY;    // m first: the 16 lanes of a column group are neighbours
     const int K = d.K, NG = d.NG;
 
-    // sign(u) * |u|^(p-1); u == 0 gives 0 either way
-    auto spower = [e](float u) { return __builtin_copysignf(pow_pos(__builtin_fabsf(u), e), u); };
+    // sign(u) * |u|^(p-1) as u * |u|^(p-2) (the host sends exponents p <= 2 to the separate kernels); u == 0 gives 0
+    const float em1 = in_vgpr(e - 1.0f);
+    auto spower = [em1](float u) { return spow_by_mul(u, em1); };
 
     // the lane's patch of x, and where its columns' sums go in grad_weight (row n = 0 of group g)
     float q[TM][TN], acc[TM][TN];
@@ -247,6 +248,7 @@ bool norm_backward_fused_applicable(const Problem& pr, float p, const void* grad
                                     const void* grad_weight) {
     const int ie = small_int_power(p - 1.0f);
     if (ie == 1 || ie == 2 || ie == 3 || ie == 7) return false;
+    if (!(p > 2.0f)) return false;   // the kernel takes sign(u) |u|^(p-1) as u |u|^(p-2)
     if (pr.HW != 1 || pr.K % 4 != 0 || pr.NG % 4 != 0) return false;
     if (!(aligned16(grad_output) && aligned16(input) && aligned16(weight) && aligned16(output) && aligned16(grad_input) &&
           aligned16(grad_weight)))

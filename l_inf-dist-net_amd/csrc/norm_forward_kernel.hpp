@@ -51,9 +51,10 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
     const int tid = threadIdx.x;
     const int grp = tid / NGRP, t = tid % NGRP;
     const int tx = t % GEO::TX, ty = t / GEO::TX;
+    const float pv = in_vgpr(p);
     auto power = [&](float v) {   // by reference: the integer-exponent instantiations do not use p
         if constexpr (IP > 0) return pow_int<IP>(v);
-        else return pow_pos(v, p);
+        else return pow_pos(v, pv);
     };
 
     Stage st;
@@ -115,7 +116,7 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
             for (int j = 0; j < TN; j++) {
                 const bool seeded = !(rs[i][j] > 1e-10f);
                 rs[i][j] = seeded ? 1e10f : __builtin_amdgcn_rcpf(rs[i][j]);
-                if (grp == 0) acc[i][j] = 1e-10f * pow_pos(1e-10f * rs[i][j], p);   // the seed, on the final scale
+                if (grp == 0) acc[i][j] = 1e-10f * pow_pos(1e-10f * rs[i][j], pv);   // the seed, on the final scale
                 if (seeded) cut = -1.f;
             }
         // Where most rows do hold a term that counts (moderate p, or differences that crowd below their maximum) the
@@ -130,8 +131,8 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
                     for (int i = 0; i < TM; i++)
 #pragma unroll
                         for (int j = 0; j < TN; j++) {
-                            acc[i][j] += pow_pos(__builtin_fabsf(f.x[0][0][i] - f.w[0][j]) * rs[i][j], p);
-                            acc[i][j] += pow_pos(__builtin_fabsf(f.x[0][1][i] - f.w[1][j]) * rs[i][j], p);
+                            acc[i][j] += pow_pos(__builtin_fabsf(f.x[0][0][i] - f.w[0][j]) * rs[i][j], pv);
+                            acc[i][j] += pow_pos(__builtin_fabsf(f.x[0][1][i] - f.w[1][j]) * rs[i][j], pv);
                         }
                 });
                 return;
@@ -160,8 +161,8 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
                             asm volatile("" : "+v"(x0), "+v"(x1));
 #pragma unroll
                             for (int j = 0; j < TN; j++) {
-                                acc[i][j] += pow_pos(__builtin_fabsf(x0 - f.w[0][j]) * rs[i][j], p);
-                                acc[i][j] += pow_pos(__builtin_fabsf(x1 - f.w[1][j]) * rs[i][j], p);
+                                acc[i][j] += pow_pos(__builtin_fabsf(x0 - f.w[0][j]) * rs[i][j], pv);
+                                acc[i][j] += pow_pos(__builtin_fabsf(x1 - f.w[1][j]) * rs[i][j], pv);
                             }
                         }
                 }
@@ -189,7 +190,7 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
                 for (int j = 0; j < TN; j++) {
                     const float r = cs[i][j] * rs[i][j];
                     if (r > 1.f) {
-                        acc[i][j] *= pow_pos(__builtin_amdgcn_rcpf(r), p);
+                        acc[i][j] *= pow_pos(__builtin_amdgcn_rcpf(r), pv);
                         rs[i][j] = __builtin_amdgcn_rcpf(cs[i][j]);
                     }
                     cs[i][j] = 0.f;
@@ -323,8 +324,8 @@ norm_forward_kernel(const float* __restrict__ input, const float* __restrict__ w
                     const int o = (q * TM * TN + i * TN + j) * NGRP + t;
                     const float a2 = ma[o], r2 = mr[o];
                     const float r = __builtin_fminf(rs[i][j], r2);   // the larger scale
-                    acc[i][j] = acc[i][j] * pow_pos(r * __builtin_amdgcn_rcpf(rs[i][j]), p) +
-                                a2 * pow_pos(r * __builtin_amdgcn_rcpf(r2), p);
+                    acc[i][j] = acc[i][j] * pow_pos(r * __builtin_amdgcn_rcpf(rs[i][j]), pv) +
+                                a2 * pow_pos(r * __builtin_amdgcn_rcpf(r2), pv);
                     rs[i][j] = r;
                 }
     }

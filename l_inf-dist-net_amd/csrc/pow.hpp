@@ -12,6 +12,21 @@ __device__ __forceinline__ float pow_pos(float v, float e) {
     return __builtin_amdgcn_exp2f(e * __builtin_amdgcn_logf(v));
 }
 
+// Keeps a wave-uniform factor in a vector register.  As a scalar-register operand it turns v_mul_f32 into a form that
+// issues at little more than half the rate (measured: 4.2 against 2.4 clocks per wave instruction at two waves per
+// SIMD), and the exponent multiplies every term.
+__device__ __forceinline__ float in_vgpr(float e) {
+    asm volatile("" : "+v"(e));
+    return e;
+}
+
+// sign(u) * |u|^e written as u * |u|^(e-1), em1 = e - 1 > 0: the sign comes with the last multiplication (one plain
+// v_mul_f32) instead of a v_bfi_b32 with a scalar mask (4.4 clocks).  u == 0: exp2(-inf) = 0 and 0 * 0 = 0.  em1 must
+// be positive (p > 2 for a gradient), or u == 0 would multiply 0 by infinity.
+__device__ __forceinline__ float spow_by_mul(float u, float em1) {
+    return u * __builtin_amdgcn_exp2f(em1 * __builtin_amdgcn_logf(__builtin_fabsf(u)));
+}
+
 // v^N by repeated multiplication; N is a compile-time constant.
 template <int N>
 __device__ __forceinline__ float pow_int(float v) {
