@@ -48,6 +48,11 @@ __device__ __forceinline__ constexpr int cslot(int n, int m) {
 // out rows-of-four major with n XORed by two bits of the row group, which spreads a wave's 64 word stores (and
 // the finishing lanes' byte reads) over the banks.
 __device__ __forceinline__ constexpr int bslot(int n, int m) { return (((m >> 2) * BN + (n ^ ((m >> 3) & 3))) << 2) | (m & 3); }
+// The output that lane l (= row l of the tile) of wave v finishes in round r, see the finish phase of the kernel.
+__device__ __forceinline__ constexpr int finish_output(int l, int v, int r) {
+    return ((((l & 3) | ((l >> 5) << 2)) ^ v) << 2) | (((l >> 2) & 3) ^ r);
+}
+static_assert(BN == 32 && NT == 512, "finish_output: eight waves x four rounds cover 32 outputs");
 }  // namespace shortk
 
 // NW = windows per k range = padded K / 32; the window loop is unrolled over it, so that the parked loads are
@@ -297,8 +302,12 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
         // ---- an output is finished by one lane: the four ranges in ascending k (a later range wins only with a
         // strictly larger value), then the lowest k inside the winner's window, from the panels.  Every lane reads a
         // different window, i.e. other rows of the panels, so lanes must differ in the column they read or they meet
-        // in one bank: lane l of a wave takes row l of the tile and, in round r, output (l + r) % 32 -- 64 different
-        // columns of X and 32 of W.
+        // in one bank: lane l of a wave takes row l of the tile (64 different columns of X) and, in round r of wave v,
+        // output finish_output(l, v, r): over the eight waves and four rounds every output of the row once, every
+        // output twice per wave instruction (32 columns of W), and -- what the choice of lane bits is for -- the 64
+        // value words cslot() and the 64 window bytes bslot() of a wave instruction in 64 different banks: the group
+        // of four outputs, which both slots XOR into the row's place, comes from lane bits 0, 1 and 5, which the row's
+        // own bits 2..4 do not cancel (with output (l + r) % 32 the slabs were read through eight banks).
         {
             constexpr int ROUNDS = BN / (NT / 64);
             const int ml = lane;
@@ -310,7 +319,7 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
             int wq[ROUNDS][NGROUP];
 #pragma unroll
             for (int rr = 0; rr < ROUNDS; rr++) {
-                const int nl = (lane + wave * ROUNDS + rr) % BN;
+                const int nl = finish_output(lane, wave, rr);
                 const int ob = bslot(nl, ml);
                 o[rr] = cslot(nl, ml);
 #pragma unroll
@@ -340,7 +349,7 @@ inf_forward_shortk_kernel(const float* __restrict__ input, const float* __restri
             }
 #pragma unroll
             for (int rr = 0; rr < ROUNDS; rr++) {
-                const int nl = (lane + wave * ROUNDS + rr) % BN;
+                const int nl = finish_output(lane, wave, rr);
                 const float* xr = X + kb[rr] * BM + ml;
                 const float* wr = W + kb[rr] * BN + nl;
                 float xv[WIN], wv[WIN];
