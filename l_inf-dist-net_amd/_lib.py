@@ -55,6 +55,7 @@ def build():
     """Compile the library in-tree with hipcc (gfx950).  Needs no GPU."""
     import subprocess
     subprocess.run(["make", "-s", "-j8", "-C", os.path.join(_HERE, "csrc")], check=True)
+    subprocess.run(["make", "-s", "-C", os.path.join(_HERE, "csrc"), "torch_ext"], check=True)
     return LIB_PATH
 
 

@@ -471,3 +471,58 @@ def inf_dist_bound_conv_forward(lower_img, upper_img, weight, output_lower, outp
             "output_lower and output_upper must be (B, CO, HO*WO)")
     _call("ldist_inf_dist_bound_conv_forward", dev, _p(lower_img), _p(upper_img), _p(weight), B, C, H, W, CO, G, KH, KW,
           S, P, D, _p(output_lower), _p(output_upper))
+
+
+# ---- the compiled PyTorch extension -------------------------------------------------------------------------
+# The seven functions of the reference module also exist as a PyTorch-ROCm C++ extension that carries the
+# reference's module name, `norm_dist_cpp` (csrc/torch_ext/norm_dist_cpp.cpp: pybind11 over the same C ABI, built by
+# `make -C csrc torch_ext` or __graft_entry__.build() into torch_ext/).  Where it has been built, this module hands
+# those seven names to it, so the autograd functions of norm_dist.py call a compiled binding as the reference's do;
+# the ctypes functions above stay available as `ctypes_binding[name]` and serve every entry point the reference
+# module does not have.  Either way the work is done by libldist_hip.so: there is no path without it.
+REFERENCE_NAMES = ("norm_dist_forward", "norm_dist_backward_input", "norm_dist_backward_weight", "inf_dist_forward",
+                   "inf_dist_bound_forward", "inf_dist_backward_input", "inf_dist_backward_weight")
+ctypes_binding = {name: globals()[name] for name in REFERENCE_NAMES}
+_extension = None
+BINDING = "ctypes"     # or "torch_extension": what the seven reference names are bound to right now
+
+
+def torch_extension():
+    """The compiled module (torch_ext/norm_dist_cpp*.so), or None when it has not been built."""
+    global _extension
+    if _extension is None:
+        import glob
+        import importlib.util
+        import os
+        hits = glob.glob(os.path.join(os.path.dirname(os.path.abspath(__file__)), "torch_ext", "norm_dist_cpp*.so"))
+        if not hits:
+            return None
+        _lib.lib()     # libldist_hip.so first: a missing library should be reported by its own message
+        spec = importlib.util.spec_from_file_location("norm_dist_cpp", hits[0])
+        _extension = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(_extension)
+    return _extension
+
+
+def use_torch_extension(on=True):
+    """Binds the seven reference names to the compiled extension (on=True; RuntimeError when it has not been built)
+    or back to the ctypes functions (on=False).  Returns the binding now in use."""
+    global BINDING
+    if on:
+        ext = torch_extension()
+        if ext is None:
+            raise RuntimeError("torch_ext/norm_dist_cpp*.so is missing: build it with `make -C csrc torch_ext`")
+        for name in REFERENCE_NAMES:
+            globals()[name] = getattr(ext, name)
+        BINDING = "torch_extension"
+    else:
+        globals().update(ctypes_binding)
+        BINDING = "ctypes"
+    return BINDING
+
+
+try:
+    if torch_extension() is not None:
+        use_torch_extension(True)
+except (RuntimeError, ImportError, OSError):   # no library yet (the first call reports it), or built for another torch
+    pass
