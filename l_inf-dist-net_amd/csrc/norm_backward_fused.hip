@@ -1,28 +1,39 @@
-// Both p-norm gradients of a fully connected layer in one pass over the terms, for exponents that need the
-// transcendental unit (reference model/norm_dist_cuda.cu:294-425 computes the gradients in two kernels that each
-// evaluate every term):
+// Both p-norm gradients of a fully connected layer in one pass over the terms (reference
+// model/norm_dist_cuda.cu:294-425 computes the gradients in two kernels that each evaluate every term):
 //   t[m,n,k]          = g[m,n] * (|x[m,k] - w[n,k]| / out[m,n])^(p-1) * sign(x - w)
 //   grad_input [m,k]  = sum_n t[m,n,k]          grad_weight[n,k] += -sum_m t[m,n,k]
 // For a general p the term is a logarithm and an exponential (v_log_f32, v_exp_f32: a quarter of the rate of
 // the other instructions), and that is what bounds either gradient; sharing the term between the two sums takes
-// 4.2 ms on 512 x 5120 -> 5120 at p = 20.5 where the two separate kernels take 3.7 + 3.1 ms.  (For p = 2, 3, 4, 8
-// a term is a handful of multiplications, the additions below weigh as much as the term itself, and the two
-// register-tiled kernels of norm_backward_tiled.hip stay faster: 3.35 ms against 4.65 ms.)
+// 4.2 ms on 512 x 5120 -> 5120 at p = 20.5 where the two separate kernels take 3.6 + 3.1 ms.
 //
 // The kernel has the shape of the register-tiled grad_input kernel: a workgroup owns 128 rows m x BN inputs k and
 // walks the outputs n; a lane keeps an 8 x TN patch of x and of the grad_input sums.  For grad_weight the lane
 // also adds, per output n, its eight rows' terms of each of its TN columns (one more fused multiply-add per term),
 // the sixteen lanes that share those columns (one DPP row: the lane index runs along m first here) add their
-// partial sums with four row shifts, and the row's last lane adds the total of the tile's 128 rows onto
-// grad_weight[n,k] with a float atomic.  grad_weight therefore collects one addend per tile of 128 rows, in no fixed
-// order, and must be zero-filled (or hold the values to accumulate onto) by the caller, as with the separate call.
-// The power is taken of the normalised difference (x - w) / out, which never leaves the float range.
+// partial sums with four row shifts, the row's last lane parks the total of the tile's 128 rows in an LDS tile
+// [stage's outputs][BN], and once per stage the whole workgroup adds that tile onto grad_weight with float atomics
+// (64 consecutive columns per instruction).  grad_weight therefore collects one addend per tile of 128 rows, in no
+// fixed order, and must be zero-filled (or hold the values to accumulate onto) by the caller, as with the separate
+// call.  IE = 0: any p > 2; the power is taken of the normalised difference (x - w) / out, which never leaves the
+// float range.
+//
+// IE = p - 1 for the multiply-only exponents (1, 2, 3, 7).  There the two register-tiled kernels of
+// norm_backward_tiled.hip each spend a subtraction and the multiplications of the power on every term before their
+// one fused multiply-add; here the term is shared and each sum costs its fused multiply-add only (p = 8: 7.9 vector
+// instructions per term for both sums, counted in the loop, instead of 7.1 + 6.5), and x, w, g and out are staged
+// once.  As in those kernels the power is taken of the raw difference with F = g / out^(p-1) staged in place of g,
+// and a stage that holds an output outside [2^-12, 2^12] is reduced the careful way from g and 1/out.  The loop does
+// not fetch the next row's operands ahead: with a second fragment in flight the kernel spills, and what it spills it
+// reloads behind the stage's global loads, so that every wait for a reloaded value waits for those as well (measured:
+// no faster than this form).  What keeps it from the rate its instruction count promises (1.6 ms at p = 8) is the
+// time its waves do not issue arithmetic: 20 % of it at waits (each row's LDS fetch, the stage's loads), as much again
+// at the stage's barriers, the conversion and the flush, which nothing overlaps with one workgroup per CU.
 #include "fwd_engine.hpp"
 #include "pow.hpp"
 
 namespace ldist {
 
-template <class GEO>
+template <class GEO, int IE>
 __global__ void __launch_bounds__(GEO::NT, 2)
 norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* __restrict__ input,
                            const float* __restrict__ weight, const float* __restrict__ output,
@@ -44,9 +55,15 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
     const int ty = t % GEO::TY, tx = t / GEO::TY;    // m first: the 16 lanes of a column group are neighbours
     const int K = d.K, NG = d.NG;
 
-    // sign(u) * |u|^(p-1) as u * |u|^(p-2) (the host sends exponents p <= 2 to the separate kernels); u == 0 gives 0
+    // sign(u) * |u|^(p-1).  IE == 0: as u * |u|^(p-2) (the host sends exponents p <= 2 to the separate kernels);
+    // u == 0 gives 0
     const float em1 = in_vgpr(e - 1.0f);
-    auto spower = [em1](float u) { return spow_by_mul(u, em1); };
+    auto spower = [&](float u) {   // by reference: the integer-exponent instantiations do not use em1
+        if constexpr (IE == 0) return spow_by_mul(u, em1);
+        else if constexpr (IE == 1) return u;
+        else if constexpr (IE == 2) return u * __builtin_fabsf(u);
+        else return pow_int<IE>(u);
+    };
 
     // the lane's patch of x, and where its columns' sums go in grad_weight (row n = 0 of group g)
     float q[TM][TN], acc[TM][TN];
@@ -100,21 +117,79 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
     const float* gbase = grad_output + ((size_t)m0 * d.G + g) * NG;
     const float* obase = output + ((size_t)m0 * d.G + g) * NG;
     const float* wbase = weight + (size_t)g * NG * K;
+    // Buffer loads whose byte offsets are worked out again from the lane's number at every stage (a handful of
+    // instructions per vector) instead of being kept: kept across the k loop, the eleven offsets (or, before them,
+    // eleven 64-bit addresses) were spilled, and a spilled value that the loop needs is reloaded behind the stage's
+    // loads, so that the loop's wait for it also waits for them -- the whole workgroup then stands still until the
+    // next stage's panels have arrived.  An offset of all ones lies outside the descriptors' 2 GB range and reads as
+    // zeros, which stands for every predicate: rows past the matrix (they must not add to grad_weight), outputs past
+    // NG in the last stage, columns past K, lanes without a vector in a round.
+    const __amdgpu_buffer_rsrc_t g_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(gbase), 0, (int)0x80000000u, 0x00020000);
+    const __amdgpu_buffer_rsrc_t o_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(obase), 0, (int)0x80000000u, 0x00020000);
+    typedef float F4 __attribute__((ext_vector_type(4)));
     auto load = [&](int n_first) {
-        wl.load(wbase, K, n_first, NG, k0, K, tid);
-        gk.load(gbase, d.G * NG, d.M - m0, n_first, NG, tid);
-        ok_.load(obase, d.G * NG, d.M - m0, n_first, NG, tid);
+        int lane = tid;
+        asm volatile("" : "+v"(lane));   // opaque: keeps the offsets below from being computed once and carried along
+        {   // g and out: rows m of the tile, 16 vectors of four outputs per row
+            static_assert(RowLoad::PER_ROW == 16 && NT % RowLoad::PER_ROW == 0, "a lane keeps its outputs over the rounds");
+            const int row0 = lane / RowLoad::PER_ROW, nq = (lane % RowLoad::PER_ROW) * 4;
+            const unsigned ldb = 4u * (unsigned)(d.G * NG);
+            const bool n_ok = n_first + nq < NG;                      // NG % 4 == 0: a vector is inside or outside
+            const int rows_valid = d.M - m0;
+#pragma unroll
+            for (int i = 0; i < RowLoad::N; i++) {
+                const int row = row0 + i * (NT / RowLoad::PER_ROW);
+                const unsigned o = (n_ok && row < rows_valid && row < BM) ? (unsigned)row * ldb + 4u * nq : ~0u;
+                const F4 gv = __builtin_bit_cast(F4, __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, o, n_first * 4, 0));
+                const F4 ov = __builtin_bit_cast(F4, __builtin_amdgcn_raw_buffer_load_b128(o_rsrc, o, n_first * 4, 0));
+                gk.v[i][0] = gv.x; gk.v[i][1] = gv.y; gk.v[i][2] = gv.z; gk.v[i][3] = gv.w;
+                ok_.v[i][0] = ov.x; ok_.v[i][1] = ov.y; ok_.v[i][2] = ov.z; ok_.v[i][3] = ov.w;
+            }
+        }
+        {   // weights: the stage's outputs n_first .. n_first + KK - 1, BN / 4 vectors of four columns per output
+            const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<float*>(wbase + (size_t)n_first * K + k0), 0, (int)0x80000000u, 0x00020000);
+#pragma unroll
+            for (int i = 0; i < ColLoad::N; i++) {
+                const int id = lane + i * NT;
+                const int rr = id / ColLoad::PER_ROW, cq = id - rr * ColLoad::PER_ROW;
+                const bool ok = (ColLoad::TOTAL % NT == 0 || id < ColLoad::TOTAL) && n_first + rr < NG && k0 + cq * 4 < K;
+                const unsigned o = ok ? 4u * ((unsigned)rr * (unsigned)K + (unsigned)cq * 4u) : ~0u;
+                const F4 t = __builtin_bit_cast(F4, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, o, 0, 0));
+                wl.v[i][0] = t.x; wl.v[i][1] = t.y; wl.v[i][2] = t.z; wl.v[i][3] = t.w;
+            }
+        }
     };
     // Turns the parked out values into what the panel holds: 1/out, and 0 where nothing was loaded (padding loads g
     // and out as 0; a real 0 output gives inf like the reference), so that padding multiplies by 0, not by infinity.
-    auto convert = [&]() {
+    // IE > 0, factored: g becomes g / out^IE.
+    auto convert = [&](bool factored) {
 #pragma unroll
         for (int i = 0; i < RowLoad::N; i++)
 #pragma unroll
             for (int c = 0; c < 4; c++) {
                 const bool present = ok_.v[i][c] != 0.f || gk.v[i][c] != 0.f;
-                ok_.v[i][c] = present ? __builtin_amdgcn_rcpf(ok_.v[i][c]) : 0.f;
+                const float ri = present ? __builtin_amdgcn_rcpf(ok_.v[i][c]) : 0.f;
+                ok_.v[i][c] = ri;
+                if constexpr (IE > 0) {
+                    if (factored) gk.v[i][c] *= pow_int<IE>(ri);
+                }
             }
+    };
+    // IE > 0: whether this lane parked an output outside the range in which out^-IE and the raw differences' powers
+    // are safe floats (before the conversion)
+    auto out_of_range = [&]() {
+        bool unsafe = false;
+        if constexpr (IE > 0) {
+#pragma unroll
+            for (int i = 0; i < RowLoad::N; i++)
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    const float ov = ok_.v[i][c];
+                    if (ov != 0.f || gk.v[i][c] != 0.f) unsafe |= !(ov >= 0x1p-12f && ov <= 0x1p12f);
+                }
+        }
+        return unsafe;
     };
     auto store = [&]() {
         gk.store(lds, tid);
@@ -129,7 +204,9 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
     const int nstage = (NG + KK - 1) / KK;
     for (int i = tid; i < KK * BN; i += GEO::NT) Gs[i] = 0.f;
     load(0);
-    convert();
+    bool factored = false;
+    if constexpr (IE > 0) factored = !__syncthreads_or(out_of_range());
+    convert(factored);
     store();
     __syncthreads();
     for (int s = 0; s < nstage; s++) {
@@ -139,7 +216,39 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
         // No operand prefetch: a second fragment in flight does not fit next to the patch, the sums and the weight
         // row's partial sums (it spills, and measured 15 % slower); the LDS latency of a row hides behind the forty
         // logarithms and exponentials of the other wave on the SIMD.
-        if (sparse) {
+        if constexpr (IE > 0) {
+            if (factored) {
+                sweep_chunk_plain<GEO, 1>(fp, wp, tx, ty, [&](const Frag<GEO, 1, 1>& f, int kk) {
+                    float sum[TN];
+#pragma unroll
+                    for (int j = 0; j < TN; j++) sum[j] = 0.f;
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int j = 0; j < TN; j++) {
+                            const float sp = spower(q[i][j] - f.w[0][j]);
+                            acc[i][j] = __builtin_fmaf(f.x[0][0][i], sp, acc[i][j]);
+                            sum[j] = __builtin_fmaf(f.x[0][0][i], sp, sum[j]);
+                        }
+                    add_weight_row(grp * kChunk + kk, sum);
+                });
+            } else {
+                sweep_chunk_plain<GEO, 2>(fp, wp, tx, ty, [&](const Frag<GEO, 2, 1>& f, int kk) {
+                    float sum[TN];
+#pragma unroll
+                    for (int j = 0; j < TN; j++) sum[j] = 0.f;
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int j = 0; j < TN; j++) {
+                            const float sp = spower((q[i][j] - f.w[0][j]) * f.x[1][0][i]);
+                            acc[i][j] = __builtin_fmaf(f.x[0][0][i], sp, acc[i][j]);
+                            sum[j] = __builtin_fmaf(f.x[0][0][i], sp, sum[j]);
+                        }
+                    add_weight_row(grp * kChunk + kk, sum);
+                });
+            }
+        } else if (sparse) {
             // Large exponents: |u|^(p-1) <= 2^-36 for |u| <= cut, less than the rounding of one term of unit size, and
             // nearly every normalised difference is that small, while the logarithm and the exponential are most of
             // a term's cost.  One row of the lane's patch at a time (TN terms that share g and 1/out): when no lane
@@ -188,10 +297,13 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
                 add_weight_row(grp * kChunk + kk, sum);
             });
         }
-        __syncthreads();   // everyone is done reading the panels; the stage's grad_weight tile is complete
+        // everyone is done reading the panels and the stage's grad_weight tile is complete; the vote on the next
+        // stage's outputs rides on the same barrier
+        if constexpr (IE > 0) factored = !__syncthreads_or(s + 1 < nstage ? out_of_range() : false);
+        else __syncthreads();
         flush_weight_tile(s * KK);
         if (s + 1 < nstage) {
-            convert();
+            convert(factored);
             store();
         }
         __syncthreads();
@@ -223,7 +335,7 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
     }
 }
 
-template <class GEO>
+template <class GEO, int IE>
 static hipError_t launch_fused(const Problem& pr, hipStream_t stream, const float* grad_output, const float* input,
                                const float* weight, const float* output, float* grad_input, float* grad_weight, float p) {
     Dims d = make_dims(pr);
@@ -232,7 +344,7 @@ static hipError_t launch_fused(const Problem& pr, hipStream_t stream, const floa
     d.tiles_n = (d.K + GEO::BN - 1) / GEO::BN;
     const unsigned grid = (unsigned)d.tiles_m * d.tiles_n * d.G;
     constexpr size_t lds = (size_t)(2 * GEO::XS + GEO::WS + GEO::KK * GEO::BN) * sizeof(float);   // panels, grad_weight tile
-    auto kern = norm_backward_fused_kernel<GEO>;
+    auto kern = norm_backward_fused_kernel<GEO, IE>;
     static LdsRecord lds_allowed = {};
     if (hipError_t e = allow_lds(kern, lds, pr.device, lds_allowed); e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(GEO::NT), lds, stream, grad_output, input, weight, output, grad_input,
@@ -240,24 +352,47 @@ static hipError_t launch_fused(const Problem& pr, hipStream_t stream, const floa
     return hipGetLastError();
 }
 
-// Whether the one-pass kernel takes the problem: an exponent that is not multiply-only, the fc layout, every panel
-// loadable with 128-bit loads, and a shape that fills the device with 128-row tiles (the rest stays with the two
-// separate kernels).
+// Exponents p - 1 for which the one-pass kernel has a multiply-only instantiation.
+static int fused_int_power(float p) {
+    const int ie = small_int_power(p - 1.0f);
+    return (ie == 1 || ie == 2 || ie == 3 || ie == 7) ? ie : 0;
+}
+
+// Whether the one-pass kernel takes the problem: the fc layout, every panel loadable with 128-bit loads, and a shape
+// that fills the device with 128-row tiles (the rest stays with the two separate kernels).
 bool norm_backward_fused_applicable(const Problem& pr, float p, const void* grad_output, const void* input,
                                     const void* weight, const void* output, const void* grad_input,
                                     const void* grad_weight) {
-    const int ie = small_int_power(p - 1.0f);
-    if (ie == 1 || ie == 2 || ie == 3 || ie == 7) return false;
-    if (!(p > 2.0f)) return false;   // the kernel takes sign(u) |u|^(p-1) as u |u|^(p-2)
+    if (fused_int_power(p) == 0 && !(p > 2.0f)) return false;   // the general kernel takes sign(u) |u|^(p-1) as u |u|^(p-2)
     if (pr.HW != 1 || pr.K % 4 != 0 || pr.NG % 4 != 0) return false;
+    // a lane addresses its vectors by 32-bit byte offsets from its tile's first row: 128 rows of G * NG elements of g
+    // and out, 64 rows of K weights
+    if (4LL * 130 * pr.G * pr.NG >= (1LL << 31) || 4LL * 66 * pr.K >= (1LL << 31)) return false;
     if (!(aligned16(grad_output) && aligned16(input) && aligned16(weight) && aligned16(output) && aligned16(grad_input) &&
           aligned16(grad_weight)))
         return false;
     if (g_tile_override == 0 || g_tile_override == 1) return true;   // tests and tuning: forced on (128 x 80, 128 x 64)
     if (g_tile_override >= 2) return false;                          // forced off
+    // p = 2 and 3: a term is one or two instructions and sharing it saves less than the row sums of grad_weight cost
+    // (512 x 5120 -> 5120: 1.58 against 1.40 ms at p = 2, a tie at p = 3; 2.03 against 2.18 ms at p = 4 and
+    // 2.50 against 2.97 ms at p = 8)
+    if (const int ie = fused_int_power(p); ie == 1 || ie == 2) return false;
     const long M = (long)pr.B * pr.HW;
     const long t80 = ((M + 127) / 128) * ((pr.K + 79) / 80) * pr.G, t64 = ((M + 127) / 128) * ((pr.K + 63) / 64) * pr.G;
     return (t80 > t64 ? t80 : t64) * 10 >= 7L * pr.num_cu && pr.NG >= 256;
+}
+
+template <class GEO>
+static hipError_t launch_fused_for(const Problem& pr, hipStream_t stream, const float* grad_output, const float* input,
+                                   const float* weight, const float* output, float* grad_input, float* grad_weight,
+                                   float p) {
+    switch (fused_int_power(p)) {
+        case 1: return launch_fused<GEO, 1>(pr, stream, grad_output, input, weight, output, grad_input, grad_weight, p);
+        case 2: return launch_fused<GEO, 2>(pr, stream, grad_output, input, weight, output, grad_input, grad_weight, p);
+        case 3: return launch_fused<GEO, 3>(pr, stream, grad_output, input, weight, output, grad_input, grad_weight, p);
+        case 7: return launch_fused<GEO, 7>(pr, stream, grad_output, input, weight, output, grad_input, grad_weight, p);
+        default: return launch_fused<GEO, 0>(pr, stream, grad_output, input, weight, output, grad_input, grad_weight, p);
+    }
 }
 
 hipError_t norm_backward_fused(const float* grad_output, const float* input, const float* weight, const float* output,
@@ -266,8 +401,8 @@ hipError_t norm_backward_fused(const float* grad_output, const float* input, con
     const long t80 = ((rows + 127) / 128) * ((pr.K + 79) / 80) * pr.G, t64 = ((rows + 127) / 128) * ((pr.K + 63) / 64) * pr.G;
     const double c80 = (double)((t80 + pr.num_cu - 1) / pr.num_cu) * 80, c64 = (double)((t64 + pr.num_cu - 1) / pr.num_cu) * 64 * 1.1;
     const bool wide = g_tile_override == 0 || (g_tile_override != 1 && c80 <= c64);
-    return wide ? launch_fused<Geo<128, 80, 8, 5, 2>>(pr, stream, grad_output, input, weight, output, grad_input, grad_weight, p)
-                : launch_fused<Geo<128, 64, 8, 4, 2>>(pr, stream, grad_output, input, weight, output, grad_input, grad_weight, p);
+    return wide ? launch_fused_for<Geo<128, 80, 8, 5, 2>>(pr, stream, grad_output, input, weight, output, grad_input, grad_weight, p)
+                : launch_fused_for<Geo<128, 64, 8, 4, 2>>(pr, stream, grad_output, input, weight, output, grad_input, grad_weight, p);
 }
 
 }  // namespace ldist

@@ -22,11 +22,6 @@ import torch.nn.functional as F
 from . import norm_dist_cpp
 
 _INF = float("inf")
-# exponents whose powers are a few multiplications: in the fc layout the two separate gradient kernels are the
-# faster way there
-_MULTIPLY_ONLY_P = (2.0, 3.0, 4.0, 8.0)
-
-
 def _out_shape(x, weight):
     return x.size(0), weight.size(0), x.size(2)
 
@@ -73,7 +68,7 @@ class DistF(torch.autograd.Function):
                 norm_dist_cpp.inf_dist_backward_weight_overwrite(g, argmax, gw, ctx.group)
         else:
             x, weight, y = ctx.saved_tensors
-            if want_x and want_w and (ctx.p not in _MULTIPLY_ONLY_P or x.size(2) > 1):
+            if want_x and want_w:
                 # every term belongs to both sums: one call, which evaluates it once where one kernel can serve both
                 gx, gw = torch.empty_like(x), torch.zeros_like(weight)
                 norm_dist_cpp.norm_dist_backward(g, x, weight, y, gx, gw, ctx.group, ctx.p)

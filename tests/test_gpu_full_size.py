@@ -93,10 +93,10 @@ def test_config2_pnorm_layer_rows_and_invariants():
 
 @pytest.mark.parametrize("ci", [3072, 5120])
 def test_config2_backward_at_the_full_batch(ci):
-    """Both p-norm gradients on the GPU at batch 512 (the launches the benchmark makes: 64-row tiles for
-    grad_input, the reduction over all 512 rows for grad_weight), compared with the oracle on 16 rows of
-    grad_input (rows are independent) and 32 rows of grad_weight over all 512 images (each weight row is an
-    independent reduction).  Reference: model/norm_dist_cuda.cu:299-425."""
+    """Both p-norm gradients on the GPU at batch 512, from the one call the benchmark's step makes (at p = 8 the
+    kernel that evaluates every term once for both sums) and from the two separate calls (the register-tiled
+    kernels), compared with the oracle on 16 rows of grad_input (rows are independent) and 32 rows of grad_weight
+    over all 512 images (each weight row is an independent reduction).  Reference: model/norm_dist_cuda.cu:299-425."""
     from gpu_common import DEV, cpp, gpu_norm_forward, say
     say("config 2 layer backward at batch 512:", ci, "-> 5120, p = 8")
     p = 8.0
@@ -109,17 +109,22 @@ def test_config2_backward_at_the_full_batch(ci):
     args = (go.to(DEV), x.to(DEV), w.to(DEV), out.to(DEV))
     cpp.norm_dist_backward_input(*args, gx, 1, p)
     cpp.norm_dist_backward_weight(*args, gw, 1, p)
+    gx1 = torch.full((512, ci, 1), float("nan"), device=DEV)
+    gw1 = torch.zeros(5120, ci, device=DEV)
+    cpp.norm_dist_backward(*args, gx1, gw1, 1, p)
     torch.cuda.synchronize()
-    gx, gw = gx.cpu(), gw.cpu()
-    for rows in (slice(100, 116), slice(496, 512)):
-        ex, mx = oracle.norm_dist_backward_input(go[rows].contiguous(), x[rows].contiguous(), w, out[rows].contiguous(), 1, p,
-                                                 with_abs_terms=True)
-        say("  grad_input rows", rows.start, "worst err/bound", round(assert_sum_close(gx[rows], ex, mx, p), 3))
-    for n0 in (0, 2077, 5088):
-        cols = slice(n0, n0 + 32)
-        ew, mw = oracle.norm_dist_backward_weight(go[:, cols].contiguous(), x, w[cols].contiguous(),
-                                                  out[:, cols].contiguous(), 1, p, with_abs_terms=True)
-        say("  grad_weight rows", n0, "worst err/bound", round(assert_sum_close(gw[cols], ew, mw, p), 3))
+    gx, gw, gx1, gw1 = gx.cpu(), gw.cpu(), gx1.cpu(), gw1.cpu()
+    expect_x = [(rows, oracle.norm_dist_backward_input(go[rows].contiguous(), x[rows].contiguous(), w, out[rows].contiguous(),
+                                                       1, p, with_abs_terms=True))
+                for rows in (slice(100, 116), slice(496, 512))]
+    expect_w = [(slice(n0, n0 + 32), oracle.norm_dist_backward_weight(go[:, n0:n0 + 32].contiguous(), x, w[n0:n0 + 32].contiguous(),
+                                                                      out[:, n0:n0 + 32].contiguous(), 1, p, with_abs_terms=True))
+                for n0 in (0, 2077, 5088)]
+    for name, tx, tw in (("separate calls", gx, gw), ("one call", gx1, gw1)):
+        for rows, (ex, mx) in expect_x:
+            say(" ", name, "grad_input rows", rows.start, "worst err/bound", round(assert_sum_close(tx[rows], ex, mx, p), 3))
+        for cols, (ew, mw) in expect_w:
+            say(" ", name, "grad_weight rows", cols.start, "worst err/bound", round(assert_sum_close(tw[cols], ew, mw, p), 3))
     # whole-tensor invariant (Euler: the norm is homogeneous of degree one in (x, w)):
     # sum x*grad_x + sum w*grad_w = sum g*out
     lhs = float((x.double().squeeze(-1) * gx.double().squeeze(-1)).sum() + (w.double() * gw.double()).sum())

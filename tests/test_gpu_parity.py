@@ -1441,11 +1441,11 @@ FUSED_BACKWARD_SHAPES = [sh for sh in TILED_BACKWARD_SHAPES if sh[4] == 1] + [(5
 @pytest.mark.parametrize("p", [5.0, 5.5, 9.0, 20.0, 100.0, 8.0, 2.0, 3.0, 4.0])
 @pytest.mark.parametrize("shape", FUSED_BACKWARD_SHAPES + [(1030, 24, 44, 1, 1), (512, 64, 20, 1, 1)])
 def test_norm_backward_both_gradients_in_one_pass(shape, p, tile):
-    """norm_dist_backward against the oracle.  For exponents that need the transcendental unit it runs the kernel
-    that evaluates every term once for both gradients (forced with the tile override; by itself it only takes
-    large layers); p = 2, 3, 4, 8 are multiply-only and run the two separate kernels through the same call (515 and
-    1030 rows, 20 and 44 columns: partial tiles of those).  grad_weight is added onto the buffer (0.125 here) like
-    the separate call's.  Override 2 switches the one-pass kernel off."""
+    """norm_dist_backward against the oracle: the kernel that evaluates every term once for both gradients, forced
+    with the tile override (by itself it only takes large layers, and p = 2 and 3 never), in its general form
+    (logarithm and exponential) and its multiply-only forms for p = 2, 3, 4, 8; then override 2, which switches it
+    off, so that the same call runs the two separate kernels (515 and 1030 rows, 20 and 44 columns: partial tiles of
+    those).  grad_weight is added onto the buffer (0.125 here) like the separate call's."""
     from gpu_common import DEV, cpp, say, set_tile
     B, CO, CI, G, HW = shape
     say("norm_backward fused", shape, "p", p, "tile", tile)
@@ -1469,8 +1469,8 @@ def test_norm_backward_both_gradients_in_one_pass(shape, p, tile):
 @pytest.mark.parametrize("scale", [1e-6, 3e-4, 1.0, 5e3, 1e6, "mixed", "one tiny row"])
 def test_norm_backward_both_gradients_at_every_scale(scale, p):
     """The one-call backward on inputs of every magnitude: nothing may overflow or vanish with the scale of the data
-    (general p, the one-pass kernel: the power is taken of the normalised difference; p = 3, 8, the two tiled
-    kernels: a stage with an output outside [2^-12, 2^12] leaves the factored form)."""
+    (the one-pass kernel, forced: for a general p the power is taken of the normalised difference; at p = 3 and 8 a
+    stage with an output outside [2^-12, 2^12] leaves the factored form, as in the two tiled kernels)."""
     from gpu_common import DEV, cpp, say, set_tile
     B, CO, CI, G, HW = 200, 72, 132, 1, 1
     say("norm_backward fused scale", scale, "p", p)
