@@ -30,6 +30,7 @@
 // at the stage's barriers, the conversion and the flush, which nothing overlaps with one workgroup per CU.
 #include "fwd_engine.hpp"
 #include "pow.hpp"
+#include "wave_reduce.hpp"
 
 namespace ldist {
 
@@ -58,6 +59,7 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
     // sign(u) * |u|^(p-1).  IE == 0: as u * |u|^(p-2) (the host sends exponents p <= 2 to the separate kernels);
     // u == 0 gives 0
     const float em1 = in_vgpr(e - 1.0f);
+    const float em2 = em1;   // p - 2: the exponent of |x - w| beside the factor (x - w) itself
     auto spower = [&](float u) {   // by reference: the integer-exponent instantiations do not use em1
         if constexpr (IE == 0) return spow_by_mul(u, em1);
         else if constexpr (IE == 1) return u;
@@ -160,6 +162,26 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
             }
         }
     };
+    // every (row, output) pair has its own largest term among its K differences, and a row of the test holds
+    // 16 pairs x 4 TN columns per wave: with a short K most rows hold one and the tests only cost
+    const bool sparse = e >= 63.0f && K >= 1024;
+    const float cut = __builtin_exp2f(-36.0f / e);
+    // General exponent without the tests: the term g * u * |u|^(p-2), u = (x - w) / out, can be taken as
+    //   g * (x - w) * exp2((p - 2) * log2|x - w| + log2(out^-(p-1))),
+    // the second summand staged per (row, output) in place of 1/out: the division of every difference by its output
+    // becomes part of the exponent's fused multiply-add (five plain instructions per term beside the logarithm and
+    // the exponential instead of six; 4.19 -> 3.87 ms on 512 x 5120 -> 5120).  The exponent is then a difference of
+    // two numbers of the size of (p - 1) * |log2 out| for the terms that count (|x - w| near out), and the rounding of
+    // those, 2^-24 each, is a relative error of the term.  So the form is voted per stage, as the factored form of the
+    // multiply-only exponents is: a stage whose outputs all lie in [1/16, 16] takes it (the error is then at most a
+    // quarter of the tolerance the gradients are held to, which grows with p as the error does), any other stage
+    // divides first.
+    // What "near 1" means is settled once per workgroup: `unit` is the power of two at or below the largest output of
+    // the first stage, the lane's patch of x and every stage's weights are taken in that unit (exact: powers of two),
+    // and so are the outputs, so that data of any overall magnitude takes the logarithmic form; rows of very different
+    // magnitudes in one tile do not.
+    const bool logscale = IE == 0 && !sparse;
+    float unit_inv = 1.0f;   // 1 / unit
     // Turns the parked out values into what the panel holds: 1/out, and 0 where nothing was loaded (padding loads g
     // and out as 0; a real 0 output gives inf like the reference), so that padding multiplies by 0, not by infinity.
     // IE > 0, factored: g becomes g / out^IE.
@@ -169,26 +191,38 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
 #pragma unroll
             for (int c = 0; c < 4; c++) {
                 const bool present = ok_.v[i][c] != 0.f || gk.v[i][c] != 0.f;
-                const float ri = present ? __builtin_amdgcn_rcpf(ok_.v[i][c]) : 0.f;
-                ok_.v[i][c] = ri;
+                const float ri = present ? __builtin_amdgcn_rcpf(ok_.v[i][c] * unit_inv) : 0.f;   // unit_inv: 1 unless logscale
                 if constexpr (IE > 0) {
+                    ok_.v[i][c] = ri;
                     if (factored) gk.v[i][c] *= pow_int<IE>(ri);
+                } else {
+                    // general exponent, a stage in the logarithmic form: the panel holds log2 of out^-(p-1), which
+                    // the term's exponent starts from; minus infinity where nothing was loaded, so that the power is 0
+                    ok_.v[i][c] = !factored ? ri : present ? e * __builtin_amdgcn_logf(ri) : -__builtin_inff();
                 }
             }
     };
-    // IE > 0: whether this lane parked an output outside the range in which out^-IE and the raw differences' powers
-    // are safe floats (before the conversion)
+    // logscale: the stage's weights in units of `unit`, like the lane's patch of x
+    auto scale_weights = [&]() {
+        if (logscale) {
+#pragma unroll
+            for (int i = 0; i < ColLoad::N; i++)
+#pragma unroll
+                for (int c = 0; c < 4; c++) wl.v[i][c] *= unit_inv;
+        }
+    };
+    // Whether this lane parked an output outside the range of the short form (before the conversion): IE > 0, the
+    // range in which out^-IE and the raw differences' powers are safe floats; IE == 0, that of the logarithmic form
     auto out_of_range = [&]() {
         bool unsafe = false;
-        if constexpr (IE > 0) {
+        const float lo = IE > 0 ? 0x1p-12f : 0x1p-4f, hi = IE > 0 ? 0x1p12f : 0x1p4f;
 #pragma unroll
-            for (int i = 0; i < RowLoad::N; i++)
+        for (int i = 0; i < RowLoad::N; i++)
 #pragma unroll
-                for (int c = 0; c < 4; c++) {
-                    const float ov = ok_.v[i][c];
-                    if (ov != 0.f || gk.v[i][c] != 0.f) unsafe |= !(ov >= 0x1p-12f && ov <= 0x1p12f);
-                }
-        }
+            for (int c = 0; c < 4; c++) {
+                const float ov = ok_.v[i][c] * unit_inv;
+                if (ok_.v[i][c] != 0.f || gk.v[i][c] != 0.f) unsafe |= !(ov >= lo && ov <= hi);
+            }
         return unsafe;
     };
     auto store = [&]() {
@@ -197,16 +231,39 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
         wl.store(lds + 2 * XS, tid);
     };
 
-    // every (row, output) pair has its own largest term among its K differences, and a row of the test holds
-    // 16 pairs x 4 TN columns per wave: with a short K most rows hold one and the tests only cost
-    const bool sparse = e >= 63.0f && K >= 1024;
-    const float cut = __builtin_exp2f(-36.0f / e);
     const int nstage = (NG + KK - 1) / KK;
     for (int i = tid; i < KK * BN; i += GEO::NT) Gs[i] = 0.f;
     load(0);
-    bool factored = false;
-    if constexpr (IE > 0) factored = !__syncthreads_or(out_of_range());
+    if (logscale) {
+        float top = 0.f;   // the largest finite output this lane loaded
+#pragma unroll
+        for (int i = 0; i < RowLoad::N; i++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const float ov = ok_.v[i][c];
+                top = __builtin_fmaxf(top, ov < __builtin_inff() ? ov : 0.f);   // a NaN is not taken either
+            }
+        top = wave_max(top);
+        float* tops = Gs;   // zero again before the loop below uses it
+        __syncthreads();    // the zero fill above is complete
+        if ((tid & 63) == 63) tops[tid >> 6] = top;
+        __syncthreads();
+#pragma unroll
+        for (int w = 0; w < GEO::NT / 64; w++) top = __builtin_fmaxf(w == 0 ? tops[0] : top, tops[w]);
+        __syncthreads();
+        if ((tid & 63) == 63) tops[tid >> 6] = 0.f;
+        // exponent of the largest output, kept well inside the float range; 2^-exponent by its bits
+        const int ex = min(100, max(-100, (int)((__float_as_uint(top) >> 23) & 0xff) - 127));
+        unit_inv = top > 0.f ? __uint_as_float((unsigned)(127 - ex) << 23) : 1.0f;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) q[i][j] *= unit_inv;
+    }
+    bool factored = false;   // the stage in LDS takes the short form (IE > 0: factored; IE == 0: logarithmic)
+    if (IE > 0 || logscale) factored = !__syncthreads_or(out_of_range());
     convert(factored);
+    scale_weights();
     store();
     __syncthreads();
     for (int s = 0; s < nstage; s++) {
@@ -281,6 +338,22 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
                 }
                 add_weight_row(grp * kChunk + kk, sum);
             });
+        } else if (factored) {
+            sweep_chunk_plain<GEO, 2>(fp, wp, tx, ty, [&](const Frag<GEO, 2, 1>& f, int kk) {
+                float sum[TN];
+#pragma unroll
+                for (int j = 0; j < TN; j++) sum[j] = 0.f;
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) {
+                        const float df = q[i][j] - f.w[0][j];
+                        const float sp = df * __builtin_amdgcn_exp2f(__builtin_fmaf(__builtin_amdgcn_logf(__builtin_fabsf(df)), em2, f.x[1][0][i]));
+                        acc[i][j] = __builtin_fmaf(f.x[0][0][i], sp, acc[i][j]);   // two fused multiply-adds, not a
+                        sum[j] = __builtin_fmaf(f.x[0][0][i], sp, sum[j]);         // shared product and two additions
+                    }
+                add_weight_row(grp * kChunk + kk, sum);
+            });
         } else {
             sweep_chunk_plain<GEO, 2>(fp, wp, tx, ty, [&](const Frag<GEO, 2, 1>& f, int kk) {
                 float sum[TN];
@@ -291,19 +364,20 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
 #pragma unroll
                     for (int j = 0; j < TN; j++) {
                         const float sp = spower((q[i][j] - f.w[0][j]) * f.x[1][0][i]);
-                        acc[i][j] = __builtin_fmaf(f.x[0][0][i], sp, acc[i][j]);   // two fused multiply-adds, not a
-                        sum[j] = __builtin_fmaf(f.x[0][0][i], sp, sum[j]);         // shared product and two additions
+                        acc[i][j] = __builtin_fmaf(f.x[0][0][i], sp, acc[i][j]);
+                        sum[j] = __builtin_fmaf(f.x[0][0][i], sp, sum[j]);
                     }
                 add_weight_row(grp * kChunk + kk, sum);
             });
         }
         // everyone is done reading the panels and the stage's grad_weight tile is complete; the vote on the next
         // stage's outputs rides on the same barrier
-        if constexpr (IE > 0) factored = !__syncthreads_or(s + 1 < nstage ? out_of_range() : false);
+        if (IE > 0 || logscale) factored = !__syncthreads_or(s + 1 < nstage ? out_of_range() : false);
         else __syncthreads();
         flush_weight_tile(s * KK);
         if (s + 1 < nstage) {
             convert(factored);
+            scale_weights();
             store();
         }
         __syncthreads();
