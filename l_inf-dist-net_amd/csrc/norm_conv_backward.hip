@@ -31,6 +31,7 @@
 #include "kernels.hpp"
 #include "pow.hpp"
 #include "tile.hpp"
+#include "wave_reduce.hpp"
 
 #include <algorithm>
 
@@ -89,6 +90,47 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
         Ws[n * WLD + c] = (c < TC && k0 + c < K) ? weight[((size_t)g * NG + n) * K + k0 + c] : 0.f;
         Gw[n * WLD + c] = 0.f;
     }
+    // General exponent (IE == 0): the term g * u * |u|^(p-2), u = (x - w) / out, is taken as
+    //   g * (x - w) * exp2((p - 2) * log2|x - w| + log2(out^-(p-1)))
+    // wherever that is accurate enough (the second summand staged per (row, output) in place of 1/out, so that the
+    // division rides in the exponent's fused multiply-add: one plain instruction less per term, and no copy of the
+    // sign).  The exponent is a difference of two numbers of the size of (p - 1) * |log2 out| for the terms that count,
+    // so everything is taken in units of a power of two read off the outputs of the workgroup's first tile (exact
+    // scalings of x, the weights and the outputs), and a tile takes the form only if all its outputs lie within
+    // [1/16, 16] units (voted on the barrier that follows the staging; the error is then at most a quarter of the
+    // gradients' tolerance); other tiles divide first.
+    float unit_inv = 1.0f;   // 1 / unit
+    const float em1 = e - 1.0f;   // p - 2
+    if constexpr (IE == 0) {
+        float top = 0.f;
+        if (u_begin < u_end) {
+            const int rows = IMG ? min(TR, d.HW) : min(TR, d.M - u_begin * TR);
+            for (int i = tid; i < NG * TR; i += 256) {
+                const int n = i / TR, r = i % TR;
+                if (r < rows) {
+                    size_t o;
+                    if constexpr (IMG) {
+                        o = ((size_t)(u_begin * d.G + g) * NG + n) * d.HW + r;
+                    } else {
+                        const int m = u_begin * TR + r, bi = m / d.HW;
+                        o = ((size_t)(bi * d.G + g) * NG + n) * d.HW + (m - bi * d.HW);
+                    }
+                    const float ov = output[o];
+                    top = __builtin_fmaxf(top, ov < __builtin_inff() ? ov : 0.f);   // a NaN is not taken either
+                }
+            }
+        }
+        top = wave_max(top);
+        __syncthreads();                       // Gw's zero fill above is complete
+        if ((tid & 63) == 63) Gw[tid >> 6] = top;
+        __syncthreads();
+        top = __builtin_fmaxf(__builtin_fmaxf(Gw[0], Gw[1]), __builtin_fmaxf(Gw[2], Gw[3]));
+        __syncthreads();
+        if ((tid & 63) == 63) Gw[tid >> 6] = 0.f;
+        const int ex = min(100, max(-100, (int)((__float_as_uint(top) >> 23) & 0xff) - 127));
+        unit_inv = top > 0.f ? __uint_as_float((unsigned)(127 - ex) << 23) : 1.0f;
+        for (int i = tid; i < NG * TCP; i += 256) Ws[(i / TCP) * WLD + i % TCP] *= unit_inv;   // each lane the words it wrote
+    }
     // the lane's four columns: whether they exist, and for the image their channel plane and tap
     bool col_ok[4];
     int col_plane[4], col_tap[4], col_dh[4], col_dw[4];   // IMG: the column's channel plane inside the tile, its tap and the tap's offsets
@@ -134,10 +176,10 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
                 } else {
                     off = xoff[i] + (size_t)k * d.HW;
                 }
-                q[i][j] = ok ? input[off] : 0.f;
+                q[i][j] = ok ? input[off] * unit_inv : 0.f;   // unit_inv: 1 unless IE == 0
             }
         // g and out of the tile's rows for every output of the group; rows are contiguous in memory
-        bool unsafe = IE == 0;
+        bool unsafe = false;
         for (int i = tid; i < NG * TR; i += 256) {
             const int n = i / TR, r = i % TR;
             float c = 0.f, ri = 0.f;
@@ -150,9 +192,10 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
                     o = ((size_t)(bi * d.G + g) * NG + n) * d.HW + (m - bi * d.HW);
                 }
                 c = grad_output[o];
-                const float out = output[o];
+                const float out = output[o] * unit_inv;
                 ri = __builtin_amdgcn_rcpf(out);
-                unsafe |= !(out >= 0x1p-12f && out <= 0x1p12f);   // the factored form needs out^(p-1) inside the float range
+                // IE > 0: the factored form needs out^(p-1) inside the float range; IE == 0: the logarithmic form's range
+                unsafe |= IE > 0 ? !(out >= 0x1p-12f && out <= 0x1p12f) : !(out >= 0x1p-4f && out <= 0x1p4f);
             }
             Cs[i] = c;
             Rs[i] = ri;
@@ -160,6 +203,10 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
         const bool factored = !__syncthreads_or(unsafe);   // also: the panels are written
         if (IE > 0 && factored) {
             for (int i = tid; i < NG * TR; i += 256) Cs[i] *= pow_int<(IE > 0 ? IE : 1)>(Rs[i]);   // each lane its own elements
+            __syncthreads();
+        }
+        if (IE == 0 && factored) {   // 1/out -> log2 of out^-(p-1); rows that do not exist: minus infinity, a power of 0
+            for (int i = tid; i < NG * TR; i += 256) Rs[i] = i % TR < rows ? e * __builtin_amdgcn_logf(Rs[i]) : -__builtin_inff();
             __syncthreads();
         }
         auto reduce = [&](auto term) {   // term(x - w, 1/out): the power that g (or g / out^IE) multiplies
@@ -189,6 +236,8 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
             }
         };
         if (IE > 0 && factored) reduce([&](float df, float) { return spower(df); });
+        else if (IE == 0 && factored)
+            reduce([&](float df, float c4) { return df * __builtin_amdgcn_exp2f(__builtin_fmaf(__builtin_amdgcn_logf(__builtin_fabsf(df)), em1, c4)); });
         else reduce([&](float df, float ri) { return spower(df * ri); });
     };
 
