@@ -113,6 +113,31 @@ struct Stager {
         }
         return bad;
     }
+    // Visits every value this lane holds of the stage it has loaded (weights and the input panels).
+    template <class F>
+    __device__ __forceinline__ void for_each_parked(F&& f) {
+#pragma unroll
+        for (int i = 0; i < WLoad::N; i++)
+#pragma unroll
+            for (int e = 0; e < VEC; e++) f(wl.v[i][e]);
+#pragma unroll
+        for (int q = 0; q < NX; q++) {
+            if constexpr (IMG) {
+#pragma unroll
+                for (int i = 0; i < XLoadI::N; i++) f(xli[q].v[i]);
+            } else if constexpr (CONV) {
+#pragma unroll
+                for (int i = 0; i < XLoadM::N; i++)
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) f(xlm[q].v[i][e]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < XLoadK::N; i++)
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) f(xlk[q].v[i][e]);
+            }
+        }
+    }
     __device__ __forceinline__ void store(float* stage) const {
 #pragma unroll
         for (int q = 0; q < NX; q++) {
