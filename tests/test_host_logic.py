@@ -131,18 +131,15 @@ def test_distf_backward_respects_needs_input_grad(fake_native, p):
         assert any("input" in c for c in kinds) == rx and any("weight" in c for c in kinds) == rw
         assert (xx.grad is not None) == rx and (ww.grad is not None) == rw
         if rx and rw and not math.isinf(p):
-            # both wanted: the conv layout (HW = 2 here) and every exponent that needs the transcendental unit take
-            # the one call; a fully connected layer at p = 8 takes the two separate ones
+            # both wanted: one call, for either layout and every exponent (the library decides inside it whether
+            # one kernel serves both sums)
             assert kinds == ["norm_dist_backward (input and weight)"]
-            fake_native.clear()
-            x1, w1 = x[:, :, :1].clone().requires_grad_(True), w.clone().requires_grad_(True)
-            pkg.norm_dist(x1, w1, 2, p).backward(go[:, :, :1].contiguous())
-            assert sorted(c for c in fake_native if "backward" in c) == ["norm_dist_backward_input", "norm_dist_backward_weight"]
-            assert x1.grad is not None and w1.grad is not None
-            fake_native.clear()
-            x2, w2 = x[:, :, :1].clone().requires_grad_(True), w.clone().requires_grad_(True)
-            pkg.norm_dist(x2, w2, 2, 5.5).backward(go[:, :, :1].contiguous())
-            assert [c for c in fake_native if "backward" in c] == ["norm_dist_backward (input and weight)"]
+            for q in (p, 5.5, 2.0):
+                fake_native.clear()
+                x1, w1 = x[:, :, :1].clone().requires_grad_(True), w.clone().requires_grad_(True)
+                pkg.norm_dist(x1, w1, 2, q).backward(go[:, :, :1].contiguous())
+                assert [c for c in fake_native if "backward" in c] == ["norm_dist_backward (input and weight)"]
+                assert x1.grad is not None and w1.grad is not None
 
 
 def test_gradients_agree_with_the_dense_torch_formula(fake_native):
@@ -489,12 +486,12 @@ def test_stack_checker_passes_on_a_correct_net_and_catches_a_wrong_one(fake_nati
     assert not bad.ok and any("values" in f for f in bad.failures)
 
     # a wrong gradient: grad_weight scaled
-    wname = "inf_dist_backward_overwrite" if math.isinf(p) else "norm_dist_backward_weight"   # both gradients are wanted
+    wname = "inf_dist_backward_overwrite" if math.isinf(p) else "norm_dist_backward"   # both gradients are wanted: one call
     good_w = getattr(cpp, wname)
 
     def off_grad(*a):
         good_w(*a)
-        (a[3] if math.isinf(p) else a[4]).mul_(1.001)   # the grad_weight argument of either call
+        (a[3] if math.isinf(p) else a[5]).mul_(1.001)   # the grad_weight argument of either call
     setattr(cpp, wname, off_grad)
     try:
         bad = stack_check.check_training_step(model, x, up, p, torch.device("cpu"))
