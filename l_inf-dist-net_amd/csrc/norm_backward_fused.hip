@@ -171,15 +171,17 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
     // the second summand staged per (row, output) in place of 1/out: the division of every difference by its output
     // becomes part of the exponent's fused multiply-add (five plain instructions per term beside the logarithm and
     // the exponential instead of six; 4.19 -> 3.87 ms on 512 x 5120 -> 5120).  The exponent is then a difference of
-    // two numbers of the size of (p - 1) * |log2 out| for the terms that count (|x - w| near out), and the rounding of
-    // those, 2^-24 each, is a relative error of the term.  So the form is voted per stage, as the factored form of the
-    // multiply-only exponents is: a stage whose outputs all lie in [1/16, 16] takes it (the error is then at most a
-    // quarter of the tolerance the gradients are held to, which grows with p as the error does), any other stage
-    // divides first.
-    // What "near 1" means is settled once per workgroup: `unit` is the power of two at or below the largest output of
-    // the first stage, the lane's patch of x and every stage's weights are taken in that unit (exact: powers of two),
-    // and so are the outputs, so that data of any overall magnitude takes the logarithmic form; rows of very different
-    // magnitudes in one tile do not.
+    // two numbers of the size of (p - 1) * |log2 out| for the terms that count (|x - w| near out), and what the
+    // hardware logarithm of either is off by, one unit in the last place of |log2 out|, becomes a relative error of
+    // the term (p - 1) times as large.  A gradient whose terms cancel is held to 1e-6 * p / 8 of the sum of their
+    // magnitudes, which the two errors together stay inside only while |log2 out| < 1 (2 * (p - 1) * 2^-24 * ln 2
+    // = 8e-8 * (p - 1)); outputs in [1/16, 16] measured 1.07 times the tolerance on a 3x3 conv layer of one channel per
+    // group at p = 47.  So the form is voted per stage, as the factored form of the multiply-only exponents is: a
+    // stage whose outputs all lie in [1/2, 2] takes it, any other stage divides first.
+    // What "near 1" means is settled once per workgroup: `unit` is the power of two nearest to the geometric mean of
+    // the largest and the smallest output of the first stage, the lane's patch of x and every stage's weights are taken in that unit
+    // (exact: powers of two), and so are the outputs, so that data of any overall magnitude takes the logarithmic
+    // form; a layer whose outputs differ by more than the window does not.
     const bool logscale = IE == 0 && !sparse;
     float unit_inv = 1.0f;   // 1 / unit
     // Turns the parked out values into what the panel holds: 1/out, and 0 where nothing was loaded (padding loads g
@@ -195,10 +197,17 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
                 if constexpr (IE > 0) {
                     ok_.v[i][c] = ri;
                     if (factored) gk.v[i][c] *= pow_int<IE>(ri);
+                } else if (!factored) {
+                    ok_.v[i][c] = ri;
                 } else {
                     // general exponent, a stage in the logarithmic form: the panel holds log2 of out^-(p-1), which
-                    // the term's exponent starts from; minus infinity where nothing was loaded, so that the power is 0
-                    ok_.v[i][c] = !factored ? ri : present ? e * __builtin_amdgcn_logf(ri) : -__builtin_inff();
+                    // the term's exponent starts from; minus infinity where nothing was loaded, so that the power is 0.
+                    // The logarithm is taken of the output itself (no reciprocal in between), and what the product
+                    // -(p-1) * log2 out loses when it is rounded to a float goes into g as a factor.
+                    const float lo = __builtin_amdgcn_logf(present ? ok_.v[i][c] * unit_inv : 1.0f);   // nothing loaded: g stays 0
+                    const float hi = -e * lo;
+                    gk.v[i][c] *= __builtin_amdgcn_exp2f(__builtin_fmaf(-e, lo, -hi));
+                    ok_.v[i][c] = present ? hi : -__builtin_inff();
                 }
             }
     };
@@ -215,7 +224,7 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
     // range in which out^-IE and the raw differences' powers are safe floats; IE == 0, that of the logarithmic form
     auto out_of_range = [&]() {
         bool unsafe = false;
-        const float lo = IE > 0 ? 0x1p-12f : 0x1p-4f, hi = IE > 0 ? 0x1p12f : 0x1p4f;
+        const float lo = IE > 0 ? 0x1p-12f : 0.5f, hi = IE > 0 ? 0x1p12f : 2.0f;
 #pragma unroll
         for (int i = 0; i < RowLoad::N; i++)
 #pragma unroll
@@ -235,25 +244,36 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
     for (int i = tid; i < KK * BN; i += GEO::NT) Gs[i] = 0.f;
     load(0);
     if (logscale) {
-        float top = 0.f;   // the largest finite output this lane loaded
+        float top = 0.f, nbot = -__builtin_inff();   // the largest and minus the smallest output this lane loaded
 #pragma unroll
         for (int i = 0; i < RowLoad::N; i++)
 #pragma unroll
             for (int c = 0; c < 4; c++) {
                 const float ov = ok_.v[i][c];
-                top = __builtin_fmaxf(top, ov < __builtin_inff() ? ov : 0.f);   // a NaN is not taken either
+                if (ov > 0.f && ov < __builtin_inff()) {   // padding is 0; a NaN is not taken either
+                    top = __builtin_fmaxf(top, ov);
+                    nbot = __builtin_fmaxf(nbot, -ov);
+                }
             }
         top = wave_max(top);
+        nbot = wave_max(nbot);
+        constexpr int NW = GEO::NT / 64;
         float* tops = Gs;   // zero again before the loop below uses it
         __syncthreads();    // the zero fill above is complete
-        if ((tid & 63) == 63) tops[tid >> 6] = top;
+        if ((tid & 63) == 63) { tops[tid >> 6] = top; tops[NW + (tid >> 6)] = nbot; }
         __syncthreads();
 #pragma unroll
-        for (int w = 0; w < GEO::NT / 64; w++) top = __builtin_fmaxf(w == 0 ? tops[0] : top, tops[w]);
+        for (int w = 0; w < NW; w++) {
+            top = __builtin_fmaxf(w == 0 ? tops[0] : top, tops[w]);
+            nbot = __builtin_fmaxf(w == 0 ? tops[NW] : nbot, tops[NW + w]);
+        }
         __syncthreads();
-        if ((tid & 63) == 63) tops[tid >> 6] = 0.f;
-        // exponent of the largest output, kept well inside the float range; 2^-exponent by its bits
-        const int ex = min(100, max(-100, (int)((__float_as_uint(top) >> 23) & 0xff) - 127));
+        if ((tid & 63) == 63) { tops[tid >> 6] = 0.f; tops[NW + (tid >> 6)] = 0.f; }
+        // the power of two nearest (as a ratio) to the geometric mean of the two, so that the window of the vote
+        // reaches as far below the smallest as above the largest; kept well inside the float range; 2^-exponent by
+        // its bits
+        const float mid = __builtin_sqrtf(top) * __builtin_sqrtf(-nbot) * 1.41421356f;
+        const int ex = min(100, max(-100, (int)((__float_as_uint(mid) >> 23) & 0xff) - 127));
         unit_inv = top > 0.f ? __uint_as_float((unsigned)(127 - ex) << 23) : 1.0f;
 #pragma unroll
         for (int i = 0; i < TM; i++)

@@ -95,14 +95,16 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
     // wherever that is accurate enough (the second summand staged per (row, output) in place of 1/out, so that the
     // division rides in the exponent's fused multiply-add: one plain instruction less per term, and no copy of the
     // sign).  The exponent is a difference of two numbers of the size of (p - 1) * |log2 out| for the terms that count,
-    // so everything is taken in units of a power of two read off the outputs of the workgroup's first tile (exact
-    // scalings of x, the weights and the outputs), and a tile takes the form only if all its outputs lie within
-    // [1/16, 16] units (voted on the barrier that follows the staging; the error is then at most a quarter of the
-    // gradients' tolerance); other tiles divide first.
+    // each off by what the hardware logarithm is off by (one unit in the last place of |log2 out|), which the term
+    // carries (p - 1) times as large: inside the tolerance of a gradient whose terms cancel (1e-6 * p / 8 of the sum
+    // of their magnitudes) only while |log2 out| < 1.  So everything is taken in units of a power of two read off the
+    // outputs of the workgroup's first tile (exact scalings of x, the weights and the outputs; the one nearest to the
+    // geometric mean of the largest and the smallest of them), and a tile takes the form only if all its outputs lie within [1/2, 2] units
+    // (voted on the barrier that follows the staging); other tiles divide first.
     float unit_inv = 1.0f;   // 1 / unit
     const float em1 = e - 1.0f;   // p - 2
     if constexpr (IE == 0) {
-        float top = 0.f;
+        float top = 0.f, nbot = -__builtin_inff();   // the largest and minus the smallest output of the first tile
         if (u_begin < u_end) {
             const int rows = IMG ? min(TR, d.HW) : min(TR, d.M - u_begin * TR);
             for (int i = tid; i < NG * TR; i += 256) {
@@ -116,18 +118,25 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
                         o = ((size_t)(bi * d.G + g) * NG + n) * d.HW + (m - bi * d.HW);
                     }
                     const float ov = output[o];
-                    top = __builtin_fmaxf(top, ov < __builtin_inff() ? ov : 0.f);   // a NaN is not taken either
+                    if (ov > 0.f && ov < __builtin_inff()) {   // a NaN is not taken either
+                        top = __builtin_fmaxf(top, ov);
+                        nbot = __builtin_fmaxf(nbot, -ov);
+                    }
                 }
             }
         }
         top = wave_max(top);
+        nbot = wave_max(nbot);
         __syncthreads();                       // Gw's zero fill above is complete
-        if ((tid & 63) == 63) Gw[tid >> 6] = top;
+        if ((tid & 63) == 63) { Gw[tid >> 6] = top; Gw[4 + (tid >> 6)] = nbot; }
         __syncthreads();
         top = __builtin_fmaxf(__builtin_fmaxf(Gw[0], Gw[1]), __builtin_fmaxf(Gw[2], Gw[3]));
+        nbot = __builtin_fmaxf(__builtin_fmaxf(Gw[4], Gw[5]), __builtin_fmaxf(Gw[6], Gw[7]));
         __syncthreads();
-        if ((tid & 63) == 63) Gw[tid >> 6] = 0.f;
-        const int ex = min(100, max(-100, (int)((__float_as_uint(top) >> 23) & 0xff) - 127));
+        if ((tid & 63) == 63) { Gw[tid >> 6] = 0.f; Gw[4 + (tid >> 6)] = 0.f; }
+        // the power of two nearest (as a ratio) to the geometric mean of the two
+        const float mid = __builtin_sqrtf(top) * __builtin_sqrtf(-nbot) * 1.41421356f;
+        const int ex = min(100, max(-100, (int)((__float_as_uint(mid) >> 23) & 0xff) - 127));
         unit_inv = top > 0.f ? __uint_as_float((unsigned)(127 - ex) << 23) : 1.0f;
         for (int i = tid; i < NG * TCP; i += 256) Ws[(i / TCP) * WLD + i % TCP] *= unit_inv;   // each lane the words it wrote
     }
@@ -182,7 +191,7 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
         bool unsafe = false;
         for (int i = tid; i < NG * TR; i += 256) {
             const int n = i / TR, r = i % TR;
-            float c = 0.f, ri = 0.f;
+            float c = 0.f, ri = 0.f;   // IE == 0: ri holds the output itself until the vote is in
             if (r < rows) {
                 size_t o;
                 if constexpr (IMG) {
@@ -193,9 +202,9 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
                 }
                 c = grad_output[o];
                 const float out = output[o] * unit_inv;
-                ri = __builtin_amdgcn_rcpf(out);
+                ri = IE > 0 ? __builtin_amdgcn_rcpf(out) : out;
                 // IE > 0: the factored form needs out^(p-1) inside the float range; IE == 0: the logarithmic form's range
-                unsafe |= IE > 0 ? !(out >= 0x1p-12f && out <= 0x1p12f) : !(out >= 0x1p-4f && out <= 0x1p4f);
+                unsafe |= IE > 0 ? !(out >= 0x1p-12f && out <= 0x1p12f) : !(out >= 0.5f && out <= 2.0f);
             }
             Cs[i] = c;
             Rs[i] = ri;
@@ -205,8 +214,21 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
             for (int i = tid; i < NG * TR; i += 256) Cs[i] *= pow_int<(IE > 0 ? IE : 1)>(Rs[i]);   // each lane its own elements
             __syncthreads();
         }
-        if (IE == 0 && factored) {   // 1/out -> log2 of out^-(p-1); rows that do not exist: minus infinity, a power of 0
-            for (int i = tid; i < NG * TR; i += 256) Rs[i] = i % TR < rows ? e * __builtin_amdgcn_logf(Rs[i]) : -__builtin_inff();
+        if constexpr (IE == 0) {   // each lane its own elements: out -> 1/out, or the logarithmic form's summand
+            for (int i = tid; i < NG * TR; i += 256) {
+                const float out = Rs[i];
+                if (i % TR >= rows) {
+                    Rs[i] = factored ? -__builtin_inff() : 0.f;   // rows that do not exist: a power of 0, a factor 0
+                } else if (factored) {
+                    // log2 of out^-(p-1) from the output itself; what the product loses when it is rounded to a
+                    // float goes into g as a factor
+                    const float lo = __builtin_amdgcn_logf(out), hi = -e * lo;
+                    Cs[i] *= __builtin_amdgcn_exp2f(__builtin_fmaf(-e, lo, -hi));
+                    Rs[i] = hi;
+                } else {
+                    Rs[i] = __builtin_amdgcn_rcpf(out);
+                }
+            }
             __syncthreads();
         }
         auto reduce = [&](auto term) {   // term(x - w, 1/out): the power that g (or g / out^IE) multiplies

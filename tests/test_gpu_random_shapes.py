@@ -159,7 +159,9 @@ def test_random_conv_layer_from_the_image(seed):
     assert_scatter_close(gimg.cpu(), expect)
 
 
-@pytest.mark.parametrize("seed", range(96))
+# 457: one channel per group (K = 9) at p = 47 with the one-pass kernel forced on, outputs between 0.21 and 2.7: the
+# case that set the window of that kernel's logarithmic form (a wider one left grad_weight 7 % outside its bound)
+@pytest.mark.parametrize("seed", list(range(96)) + [457])
 def test_random_conv_layer_at_finite_p_from_the_image(seed):
     """The p-norm layer from the image on a random geometry, exponent and dilation: forward and both gradients
     (separate entry points; the one call with the one-pass kernel forced on, off, or left to the library) against
