@@ -2,7 +2,8 @@
 
 The hand-picked shapes of test_gpu_parity.py cover the cases the kernels were written for; this file draws sizes
 nobody picked -- prime row counts, reductions shorter than a vector, one output per group, ragged conv layouts --
-with a random forward tile, a random exponent and, for the conv layer (p = inf and finite p), a random image geometry.  Same bars as
+with a random forward tile, a random exponent and, for the conv layer (p = inf and finite p), a random image geometry;
+the finite-p kernels also on data whose rows, neurons and overall scale are random powers of two.  Same bars as
 everywhere: L_inf values, indices and bounds bit-exact, everything else rel 1e-5 / abs 1e-6.
 """
 import random
@@ -207,6 +208,94 @@ def test_random_conv_layer_at_finite_p_from_the_image(seed):
     torch.cuda.synchronize()
     assert_sum_close(gi.cpu(), fold(ex), fold(mx), p, RTOL, ATOL)
     assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
+
+
+P_MAGNITUDES = [2.5, 4.0, 5.5, 8.0, 16.5, 20.5, 33.0, 47.0, 63.0, 64.5, 100.0, 300.0, 1000.0]
+
+
+def magnitude_profile(r, n, g):
+    """n positive factors: all one, or powers of two up to 2^+-k drawn per element, per block, or for one element."""
+    k = r.choice([0, 0, 1, 2, 3, 8, 20])
+    if k == 0:
+        return torch.ones(n)
+    kind = r.choice(["iid", "blocks", "one"])
+    if kind == "iid":
+        e = (torch.rand(n, generator=g) * 2 - 1) * k
+    elif kind == "blocks":
+        e = ((torch.arange(n) // r.choice([3, 16, 64, 128])) % 3 - 1).float() * k
+    else:
+        e = torch.zeros(n)
+        e[r.randrange(n)] = r.choice([-1, 1]) * k
+    return torch.pow(2.0, e.round() if r.random() < 0.5 else e)
+
+
+@pytest.mark.parametrize("seed", range(64))
+def test_random_magnitudes_at_finite_p(seed):
+    """The p-norm kernels choose their arithmetic by the data's magnitudes (scales that follow the sweep, factored and
+    logarithmic forms voted per stage, units read off the first outputs): a fully connected layer and a 3x3 conv
+    layer with rows, output neurons and the whole problem scaled by random powers of two (rows up to 2^20 apart, the
+    problem by 10^-8 .. 10^8), forward and both gradients, the one-pass kernels forced on, off and left to the
+    library.  The gradients are invariant under the common scale, so the same bounds apply."""
+    import torch.nn.functional as F
+    from oracle import tolerance
+    from gpu_common import DEV, cpp, gpu_norm_forward, say, set_tile
+    r = random.Random(31000 + seed)
+    g = gen(32000 + seed)
+    p = r.choice(P_MAGNITUDES)
+    gs = 10.0 ** r.uniform(-8, 8) if r.random() < 0.6 else 1.0
+
+    B, NG, K, G = r.choice([3, 64, 129, 200, 256]), r.choice([5, 64, 72, 130, 160]), r.choice([33, 132, 320, 600, 1100]), r.choice([1, 1, 2])
+    if B * NG * K * G > 12_000_000:
+        B = max(3, 12_000_000 // (NG * K * G))
+    say("random magnitudes", seed, "fc", (B, NG, K, G), "p", p, "scale %.3g" % gs)
+    x, w = make_inputs(B, NG * G, K * G, G, 1, seed=33000 + seed)
+    x = (x * magnitude_profile(r, B, g).view(B, 1, 1) * gs).contiguous()
+    w = (w * magnitude_profile(r, NG * G, g).view(-1, 1) * gs).contiguous()
+    go = torch.randn(B, NG * G, 1, generator=g)
+    want = oracle.norm_dist_forward(x, w, G, p)
+    for tile in (-1, r.choice([0, 1, 2, 3, 4])):
+        set_tile(tile)
+        torch.testing.assert_close(gpu_norm_forward(x, w, G, p), want, rtol=RTOL, atol=0)
+    ex, mx = oracle.norm_dist_backward_input(go, x, w, want, G, p, with_abs_terms=True)
+    ew, mw = oracle.norm_dist_backward_weight(go, x, w, want, G, p, with_abs_terms=True)
+    args = (go.to(DEV), x.to(DEV), w.to(DEV), want.to(DEV))
+    for tile in (-1, 0, 2):
+        set_tile(tile)
+        gx = torch.full(x.shape, float("nan"), device=DEV)
+        gw = torch.zeros(w.shape, device=DEV)
+        cpp.norm_dist_backward(*args, gx, gw, G, p)
+        torch.cuda.synchronize()
+        assert_sum_close(gx.cpu(), ex, mx, p, RTOL, ATOL)
+        assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
+    set_tile(-1)
+
+    G, CG, NG = r.choice([1, 2, 4]), r.choice([1, 2, 4, 8, 16]), r.choice([4, 12, 32, 48])
+    H, W, B = r.choice([5, 8, 16, 17]), r.choice([5, 8, 16, 17]), r.choice([1, 2, 5])
+    stride, padding = r.choice([1, 1, 2]), r.choice([0, 1, 1])
+    say("random magnitudes", seed, "conv", (B, CG * G, H, W, NG * G, G, stride, padding))
+    img = (torch.rand(B, CG * G, H, W, generator=g) * magnitude_profile(r, B, g).view(B, 1, 1, 1) * gs).contiguous()
+    w = (torch.randn(NG * G, CG * 9, generator=g) * 0.5 * magnitude_profile(r, NG * G, g).view(-1, 1) * gs).contiguous()
+    cols = F.unfold(img, 3, 1, padding, stride).contiguous()
+    if cols.size(2) <= 1 or not cpp.norm_dist_conv_supported(CG * G, H, W, NG * G, G, 3, stride, padding, 1):
+        return
+    want = oracle.norm_dist_forward(cols, w, G, p)
+    out = torch.full(want.shape, float("nan"), device=DEV)
+    cpp.norm_dist_conv_forward(img.to(DEV), w.to(DEV), out, G, p, 3, stride, padding, 1)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out.cpu(), want, rtol=RTOL, atol=0)
+    go = torch.randn(want.shape, generator=g)
+    ex, mx = oracle.norm_dist_backward_input(go, cols, w, want, G, p, with_abs_terms=True)
+    ew, mw = oracle.norm_dist_backward_weight(go, cols, w, want, G, p, with_abs_terms=True)
+    fold = lambda t: F.fold(t.double(), (H, W), 3, 1, padding, stride)
+    args = (go.to(DEV), img.to(DEV), w.to(DEV), want.to(DEV))
+    for mode in (-1, 0, 2):
+        set_tile(mode)
+        gi = torch.full(img.shape, float("nan"), device=DEV)
+        gw = torch.zeros(w.shape, device=DEV)
+        cpp.norm_dist_conv_backward(*args, gi, gw, G, p, 3, stride, padding, 1)
+        torch.cuda.synchronize()
+        assert_sum_close(gi.cpu(), fold(ex), fold(mx), p, RTOL, ATOL)
+        assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
 
 
 @pytest.mark.parametrize("seed", range(40))
