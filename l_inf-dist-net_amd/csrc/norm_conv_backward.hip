@@ -143,6 +143,7 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
     // the lane's four columns: whether they exist, and for the image their channel plane and tap
     bool col_ok[4];
     int col_plane[4], col_tap[4], col_dh[4], col_dw[4];   // IMG: the column's channel plane inside the tile, its tap and the tap's offsets
+    int col_off[4];                                       // IMG: where the tap lies from the window's corner, in the tile's planes of one image
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const int c = tx * 4 + j;
@@ -151,55 +152,61 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
         col_tap[j] = c - col_plane[j] * 9;
         col_dh[j] = (col_tap[j] / 3) * win.D;
         col_dw[j] = (col_tap[j] - (col_tap[j] / 3) * 3) * win.D;
+        col_off[j] = (col_plane[j] * win.H + col_dh[j]) * win.W + col_dw[j];
     }
+    // IMG: the current image's planes of this tile, and its g and out rows of this group, behind buffer descriptors:
+    // 32-bit offsets from a uniform base, and an offset of all ones (outside the 2 GB range: reads as zero) for
+    // everything that is not there -- padding taps, rows past the image's last position, columns past K.
+    __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(input), 0, (int)0x80000000u, 0x00020000);
+    __amdgpu_buffer_rsrc_t g_rsrc = x_rsrc, o_rsrc = x_rsrc;
 
     // One tile: rows first_row .. first_row + 63 of the unfolded matrix, of which `rows` exist (IMG: rows of image b
     // from position pos0).  Leaves the grad_input sums of the lane's patch in acc.
     auto tile = [&](int first_row, int rows, int b, int pos0, float (&acc)[4][4], WinRow (&wrow)[4], size_t (&xoff)[4]) {
         float q[4][4];
+        if constexpr (!IMG) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int r = min(ty * 4 + i, rows - 1);
-            if constexpr (IMG) {
-                const int pos = pos0 + r, ho = pos / win.WO;
-                wrow[i].b = b;
-                wrow[i].h0 = ho * win.S - win.P;
-                wrow[i].w0 = (pos - ho * win.WO) * win.S - win.P;
-            } else {
+            for (int i = 0; i < 4; i++) {
+                const int r = min(ty * 4 + i, rows - 1);
                 const int m = first_row + r, bi = m / d.HW;
                 xoff[i] = ((size_t)(bi * d.G + g) * K) * d.HW + (m - bi * d.HW);
             }
         }
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+        for (int i = 0; i < 4; i++) {
+            const int corner = IMG ? wrow[i].h0 * win.W + wrow[i].w0 : 0;   // IMG: the window's corner in a plane (may lie in the padding)
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const int k = k0 + tx * 4 + j;
                 acc[i][j] = 0.f;
-                bool ok = ty * 4 + i < rows && col_ok[j];
-                size_t off;
+                const bool ok = ty * 4 + i < rows && col_ok[j];
                 if constexpr (IMG) {   // the window's tap of column j: channel and offsets are the lane's constants
                     const int h = wrow[i].h0 + col_dh[j], w = wrow[i].w0 + col_dw[j];
-                    ok = ok && (unsigned)h < (unsigned)win.H && (unsigned)w < (unsigned)win.W;
-                    off = (((size_t)b * win.C + g * win.CG + k0 / 9 + col_plane[j]) * win.H + h) * win.W + w;
+                    // one select, no branches: the tests are combined bitwise
+                    const bool in = ok & ((unsigned)h < (unsigned)win.H) & ((unsigned)w < (unsigned)win.W);
+                    const unsigned o = in ? 4u * (unsigned)(corner + col_off[j]) : ~0u;
+                    q[i][j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(x_rsrc, o, 0, 0)) * unit_inv;
                 } else {
-                    off = xoff[i] + (size_t)k * d.HW;
+                    q[i][j] = ok ? input[xoff[i] + (size_t)(k0 + tx * 4 + j) * d.HW] * unit_inv : 0.f;   // unit_inv: 1 unless IE == 0
                 }
-                q[i][j] = ok ? input[off] * unit_inv : 0.f;   // unit_inv: 1 unless IE == 0
             }
+        }
         // g and out of the tile's rows for every output of the group; rows are contiguous in memory
         bool unsafe = false;
         for (int i = tid; i < NG * TR; i += 256) {
             const int n = i / TR, r = i % TR;
             float c = 0.f, ri = 0.f;   // IE == 0: ri holds the output itself until the vote is in
-            if (r < rows) {
-                size_t o;
-                if constexpr (IMG) {
-                    o = ((size_t)(b * d.G + g) * NG + n) * d.HW + pos0 + r;
-                } else {
-                    const int m = first_row + r, bi = m / d.HW;
-                    o = ((size_t)(bi * d.G + g) * NG + n) * d.HW + (m - bi * d.HW);
+            if constexpr (IMG) {   // every lane loads (nothing for rows that do not exist); only real rows count
+                const unsigned o = r < rows ? 4u * (unsigned)(n * d.HW + pos0 + r) : ~0u;
+                const float gv = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(g_rsrc, o, 0, 0));
+                const float out = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(o_rsrc, o, 0, 0)) * unit_inv;
+                if (r < rows) {
+                    c = gv;
+                    ri = IE > 0 ? __builtin_amdgcn_rcpf(out) : out;
+                    unsafe |= IE > 0 ? !(out >= 0x1p-12f && out <= 0x1p12f) : !(out >= 0.5f && out <= 2.0f);
                 }
+            } else if (r < rows) {
+                const int m = first_row + r, bi = m / d.HW;
+                const size_t o = ((size_t)(bi * d.G + g) * NG + n) * d.HW + (m - bi * d.HW);
                 c = grad_output[o];
                 const float out = output[o] * unit_inv;
                 ri = IE > 0 ? __builtin_amdgcn_rcpf(out) : out;
@@ -287,9 +294,32 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
                 }
             };
             for (int i = tid; i < kPlanes * R * W; i += 256) Fp[i] = 0.f;   // the first tile's barriers come before its use
+            x_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<float*>(input + ((size_t)b * win.C + g * win.CG + first_ch) * H * W), 0, (int)0x80000000u, 0x00020000);
+            g_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<float*>(grad_output + (size_t)(b * d.G + g) * NG * d.HW), 0, (int)0x80000000u, 0x00020000);
+            o_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<float*>(output + (size_t)(b * d.G + g) * NG * d.HW), 0, (int)0x80000000u, 0x00020000);
+            // the lane's four positions, kept as (output row, output column) and moved on by 64 positions per tile
+            int ho[4], wo[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                ho[i] = (ty * 4 + i) / win.WO;
+                wo[i] = (ty * 4 + i) - ho[i] * win.WO;
+            }
+            const int step_h = TR / win.WO, step_w = TR - step_h * win.WO;
             int flushed = 0;   // image rows below this one are in memory
             for (int pos0 = 0; pos0 < d.HW; pos0 += TR) {
                 const int rows = min(TR, d.HW - pos0);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {   // positions past the image's last one are never used (every use asks for i < rows)
+                    wrow[i].b = b;
+                    wrow[i].h0 = ho[i] * win.S - win.P;
+                    wrow[i].w0 = wo[i] * win.S - win.P;
+                    wo[i] += step_w;
+                    ho[i] += step_h;
+                    if (wo[i] >= win.WO) { wo[i] -= win.WO; ho[i]++; }
+                }
                 tile(0, rows, b, pos0, acc, wrow, xoff);
                 // rows above this tile's first window are final (the last tile's rounds ended with a barrier)
                 const int h_lo = min(H, max(flushed, (pos0 / win.WO) * win.S - win.P));
@@ -422,6 +452,8 @@ bool norm_conv_backward_fused_image_applicable(const ConvGeom& q, int G, int CO,
     if (g_tile_override >= 2 || (long)q.HO * q.WO <= 1) return false;
     const ImgWin win{q.C, q.C / G, q.H, q.W, q.HO, q.WO, q.S, q.P, q.D};
     if (lds_bytes(CO / G, (size_t)kPlanes * ring_rows_for(win, q.HO * q.WO) * q.W) > kMaxLds) return false;
+    // the kernel's 32-bit byte offsets: a tile's planes of one image, one image's outputs of a group
+    if (4L * kPlanes * q.H * q.W >= (1L << 31) || 4L * (CO / G) * q.HO * q.WO >= (1L << 31)) return false;
     return forced_on() || (long)q.B * q.HO * q.WO >= 64L * num_cu;
 }
 
