@@ -192,29 +192,53 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
         }
         // g and out of the tile's rows for every output of the group; rows are contiguous in memory
         bool unsafe = false;
-        for (int i = tid; i < NG * TR; i += 256) {
-            const int n = i / TR, r = i % TR;
-            float c = 0.f, ri = 0.f;   // IE == 0: ri holds the output itself until the vote is in
-            if constexpr (IMG) {   // every lane loads (nothing for rows that do not exist); only real rows count
-                const unsigned o = r < rows ? 4u * (unsigned)(n * d.HW + pos0 + r) : ~0u;
-                const float gv = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(g_rsrc, o, 0, 0));
-                const float out = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(o_rsrc, o, 0, 0)) * unit_inv;
+        if constexpr (IMG) {
+            // A lane takes row r = tid % 64 of outputs tid / 64, + 4, + 8, ...: four outputs per pass, their eight
+            // loads in flight together (one output at a time, every load is waited for on its own).  Rows and outputs
+            // that do not exist load nothing (all-ones offset) and stage 0.
+            const int r = tid & (TR - 1);
+            const unsigned row_off = 4u * (unsigned)(pos0 + r), out_stride = 4u * (unsigned)d.HW;
+#pragma unroll 1
+            for (int n0 = tid / TR; n0 < NG; n0 += 16) {
+                float gv[4], ov[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int n = n0 + 4 * u;
+                    const unsigned o = (r < rows) & (n < NG) ? row_off + (unsigned)n * out_stride : ~0u;
+                    gv[u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(g_rsrc, o, 0, 0));
+                    ov[u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(o_rsrc, o, 0, 0));
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int n = n0 + 4 * u;
+                    if (n < NG) {
+                        const float out = ov[u] * unit_inv;
+                        float ri = 0.f;   // IE == 0: ri holds the output itself until the vote is in
+                        if (r < rows) {
+                            ri = IE > 0 ? __builtin_amdgcn_rcpf(out) : out;
+                            // IE > 0: the factored form needs out^(p-1) inside the float range; IE == 0: the logarithmic form's range
+                            unsafe |= IE > 0 ? !(out >= 0x1p-12f && out <= 0x1p12f) : !(out >= 0.5f && out <= 2.0f);
+                        }
+                        Cs[n * TR + r] = gv[u];
+                        Rs[n * TR + r] = ri;
+                    }
+                }
+            }
+        } else {
+            for (int i = tid; i < NG * TR; i += 256) {
+                const int n = i / TR, r = i % TR;
+                float c = 0.f, ri = 0.f;   // IE == 0: ri holds the output itself until the vote is in
                 if (r < rows) {
-                    c = gv;
+                    const int m = first_row + r, bi = m / d.HW;
+                    const size_t o = ((size_t)(bi * d.G + g) * NG + n) * d.HW + (m - bi * d.HW);
+                    c = grad_output[o];
+                    const float out = output[o] * unit_inv;
                     ri = IE > 0 ? __builtin_amdgcn_rcpf(out) : out;
                     unsafe |= IE > 0 ? !(out >= 0x1p-12f && out <= 0x1p12f) : !(out >= 0.5f && out <= 2.0f);
                 }
-            } else if (r < rows) {
-                const int m = first_row + r, bi = m / d.HW;
-                const size_t o = ((size_t)(bi * d.G + g) * NG + n) * d.HW + (m - bi * d.HW);
-                c = grad_output[o];
-                const float out = output[o] * unit_inv;
-                ri = IE > 0 ? __builtin_amdgcn_rcpf(out) : out;
-                // IE > 0: the factored form needs out^(p-1) inside the float range; IE == 0: the logarithmic form's range
-                unsafe |= IE > 0 ? !(out >= 0x1p-12f && out <= 0x1p12f) : !(out >= 0.5f && out <= 2.0f);
+                Cs[i] = c;
+                Rs[i] = ri;
             }
-            Cs[i] = c;
-            Rs[i] = ri;
         }
         const bool factored = !__syncthreads_or(unsafe);   // also: the panels are written
         if (IE > 0 && factored) {
@@ -275,6 +299,7 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
     size_t xoff[4];
     if constexpr (IMG) {
         const int H = win.H, W = win.W, R = d.ring_rows, first_ch = tk * kPlanes;
+        const int spare = kPlanes * R * W;   // a word behind the planes that collects what has no pixel; never read for its value
         const int planes = min(kPlanes, win.CG - first_ch);
         for (int b = u_begin; b < u_end; b++) {
             float* dst = grad_input + ((size_t)b * win.C + g * win.CG + first_ch) * H * W;
@@ -327,23 +352,36 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
                 flushed = h_lo;
                 __syncthreads();   // ring rows cleared above may be this tile's; every lane is done with the panels
                 // the tile's sums join the planes: nine rounds, one per tap (see the top of the file)
-#pragma unroll
+#pragma unroll 1   // unrolled, the nine rounds' pixel indices are all worked out ahead and spill
                 for (int tap = 0; tap < 9; tap++) {
-                    const int dh = (tap / 3) * win.D, dw = (tap % 3) * win.D;
+                    const int th = (tap * 11) >> 5;   // tap / 3 for 0 .. 8
+                    const int dh = th * win.D, dw = (tap - 3 * th) * win.D;
+                    // the pixels of this tap in a plane's ring, one per position of the lane; a position that has
+                    // none (padding, past the image's last position) gets the spare word behind the planes, so that
+                    // what follows needs no branches: four reads in flight, four additions, four writes
+                    int cell[4];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        const int h = wrow[i].h0 + dh, w = wrow[i].w0 + dw;
+                        const bool in = (ty * 4 + i < rows) & ((unsigned)h < (unsigned)H) & ((unsigned)w < (unsigned)W);
+                        cell[i] = in ? __mul24(h & (R - 1), W) + w : -1;
+                    }
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
                         const bool mine = col_ok[j] && col_tap[j] == tap;
                         // a wave holds 16 consecutive columns, so one or two of its four j have this tap: the others
                         // are skipped by the whole wave (a scalar branch) instead of being walked with no lane active
                         if (__builtin_amdgcn_ballot_w64(mine) == 0) continue;
-                        if (mine) {
+                        const int plane = mine ? col_plane[j] * R * W : -spare - 1;   // not mine: every index below is negative
+                        int at[4];
+                        float v[4];
 #pragma unroll
-                            for (int i = 0; i < 4; i++) {
-                                const int h = wrow[i].h0 + dh, w = wrow[i].w0 + dw;
-                                if (ty * 4 + i < rows && (unsigned)h < (unsigned)H && (unsigned)w < (unsigned)W)
-                                    Fp[(col_plane[j] * R + (h & (R - 1))) * W + w] += acc[i][j];
-                            }
+                        for (int i = 0; i < 4; i++) {
+                            at[i] = (plane | cell[i]) >= 0 ? plane + cell[i] : spare;   // both non-negative: a pixel
+                            v[i] = Fp[at[i]];
                         }
+#pragma unroll
+                        for (int i = 0; i < 4; i++) Fp[at[i]] = v[i] + acc[i][j];
                     }
                     __syncthreads();
                 }
@@ -396,7 +434,7 @@ hipError_t launch_conv_backward(const float* grad_output, const float* input, co
     d.units = IMG ? pr.B : (d.M + TR - 1) / TR;
     const long pairs = (long)d.tiles_k * d.G;
     if constexpr (IMG) d.ring_rows = ring_rows_for(win, pr.HW);
-    const size_t lds = lds_bytes(d.NG, IMG ? (size_t)kPlanes * d.ring_rows * win.W : 0);
+    const size_t lds = lds_bytes(d.NG, IMG ? (size_t)kPlanes * d.ring_rows * win.W + 4 : 0);   // + the spare word
     // Units per workgroup: the choice that needs the fewest rounds of resident workgroups times units (the device
     // holds `resident` of them at once), among those that keep the number of workgroups, each of which flushes a whole
     // grad_weight tile at the end, within sixteen rounds; ties go to fewer, longer workgroups.
@@ -451,7 +489,7 @@ bool norm_conv_backward_fused_applicable(const Problem& pr) {
 bool norm_conv_backward_fused_image_applicable(const ConvGeom& q, int G, int CO, int num_cu) {
     if (g_tile_override >= 2 || (long)q.HO * q.WO <= 1) return false;
     const ImgWin win{q.C, q.C / G, q.H, q.W, q.HO, q.WO, q.S, q.P, q.D};
-    if (lds_bytes(CO / G, (size_t)kPlanes * ring_rows_for(win, q.HO * q.WO) * q.W) > kMaxLds) return false;
+    if (lds_bytes(CO / G, (size_t)kPlanes * ring_rows_for(win, q.HO * q.WO) * q.W + 4) > kMaxLds) return false;
     // the kernel's 32-bit byte offsets: a tile's planes of one image, one image's outputs of a group
     if (4L * kPlanes * q.H * q.W >= (1L << 31) || 4L * (CO / G) * q.HO * q.WO >= (1L << 31)) return false;
     return forced_on() || (long)q.B * q.HO * q.WO >= 64L * num_cu;
