@@ -204,7 +204,7 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
 #pragma unroll
                 for (int u = 0; u < 4; u++) {
                     const int n = n0 + 4 * u;
-                    const unsigned o = (r < rows) & (n < NG) ? row_off + (unsigned)n * out_stride : ~0u;
+                    const unsigned o = ((r < rows) & (n < NG)) ? row_off + (unsigned)n * out_stride : ~0u;
                     gv[u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(g_rsrc, o, 0, 0));
                     ov[u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(o_rsrc, o, 0, 0));
                 }
