@@ -50,10 +50,21 @@ struct ConvBwd {
     int tiles_k;                     // column tiles per group
     int units, units_per_wg;         // what a workgroup walks: tiles of 64 rows (columns), whole images (image)
     int ring_rows;                   // IMG: image rows per channel plane held in LDS, a power of two
+    int park_extra;                  // IMG: floats between the 1/out panel and the ring that the parked tile runs into
 };
 
 inline size_t lds_bytes(int NG, size_t plane_floats) {
     return ((size_t)2 * NG * WLD + (size_t)2 * NG * TR + plane_floats) * sizeof(float);
+}
+
+// IMG: a tile's grad_input sums are parked as [64 columns][64 positions] over the g and 1/out panels; what that
+// takes beyond the panels' 2 * NG * 64 floats
+inline int park_extra(int NG) { return std::max(0, TCP * TR - 2 * NG * TR); }
+
+// IMG: the floats behind the panels: the parked tile's overhang, the ring of image rows, a word that stays zero,
+// and the two tables (image row, tap row) -> output row and (image column, tap column) -> output column
+inline size_t image_floats(int NG, int ring_rows, int H, int W) {
+    return (size_t)park_extra(NG) + (size_t)kPlanes * ring_rows * W + 4 + 3 * (size_t)(H + W);
 }
 
 }  // namespace
@@ -71,7 +82,7 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
     float* Gw = Ws + NG * WLD;           // [NG][WLD]  sums for grad_weight[n][k0 + c]
     float* Cs = Gw + NG * WLD;           // [NG][TR]   g, or g / out^IE
     float* Rs = Cs + NG * TR;            // [NG][TR]   1 / out
-    float* Fp = Rs + NG * TR;            // IMG: [kPlanes][ring_rows][W] gradient of the image rows still being added to
+    float* Fp = Rs + NG * TR + (IMG ? d.park_extra : 0);   // IMG: [kPlanes][ring_rows][W] gradient of the image rows still being added to
     const int tid = threadIdx.x;
     const int ty = tid & 15, tx = tid >> 4;   // rows first: the 16 lanes of a column group form a DPP row
     const int tk = blockIdx.x % d.tiles_k, g = blockIdx.x / d.tiles_k;
@@ -299,8 +310,25 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
     size_t xoff[4];
     if constexpr (IMG) {
         const int H = win.H, W = win.W, R = d.ring_rows, first_ch = tk * kPlanes;
-        const int spare = kPlanes * R * W;   // a word behind the planes that collects what has no pixel; never read for its value
         const int planes = min(kPlanes, win.CG - first_ch);
+        // behind the ring: a word that stays zero (what a pixel reads for a tap that has no position in the tile), and
+        // the tables that turn (image row, tap row) and (image column, tap column) into the output row (times WO) and
+        // the output column whose window has that tap there; a large negative number where there is none
+        float* const zero_word = Fp + kPlanes * R * W;
+        int* const HT = reinterpret_cast<int*>(zero_word + 4);
+        int* const WT = HT + 3 * H;
+        float* const Pk = Cs;   // [64][64]: the tile's grad_input sums by (column, position), over the two panels
+        constexpr int kNone = -(1 << 20);
+        if (tid < 4) zero_word[tid] = 0.f;
+        for (int i = tid; i < 3 * (H + W); i += 256) {
+            const bool row = i < 3 * H;
+            const int e = row ? i : i - 3 * H, at = e / 3, t = e - at * 3;
+            const int lim = row ? win.HO : win.WO;
+            const int hh = at + win.P - t * win.D, o = hh / win.S;
+            const bool ok = hh >= 0 && o * win.S == hh && o < lim;
+            HT[i] = ok ? (row ? o * win.WO : o) : kNone;   // WT follows HT
+        }
+        const float inv_w = 1.0f / (float)W;
         for (int b = u_begin; b < u_end; b++) {
             float* dst = grad_input + ((size_t)b * win.C + g * win.CG + first_ch) * H * W;
             // Writes image rows h_from .. h_to - 1 of the planes to memory and clears their ring rows.  Rows more than
@@ -351,40 +379,41 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
                 if (h_lo > flushed) flush_rows(flushed, h_lo);
                 flushed = h_lo;
                 __syncthreads();   // ring rows cleared above may be this tile's; every lane is done with the panels
-                // the tile's sums join the planes: nine rounds, one per tap (see the top of the file)
-#pragma unroll 1   // unrolled, the nine rounds' pixel indices are all worked out ahead and spill
-                for (int tap = 0; tap < 9; tap++) {
-                    const int th = (tap * 11) >> 5;   // tap / 3 for 0 .. 8
-                    const int dh = th * win.D, dw = (tap - 3 * th) * win.D;
-                    // the pixels of this tap in a plane's ring, one per position of the lane; a position that has
-                    // none (padding, past the image's last position) gets the spare word behind the planes, so that
-                    // what follows needs no branches: four reads in flight, four additions, four writes
-                    int cell[4];
+                // The tile's sums join the planes.  They are parked by (column, position) over the two panels, and
+                // every pixel that a window of this tile can reach fetches its up to nine (position, tap) entries
+                // and adds them to its ring word: one owner per pixel, a fixed order of the nine, no rounds.
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        const int h = wrow[i].h0 + dh, w = wrow[i].w0 + dw;
-                        const bool in = (ty * 4 + i < rows) & ((unsigned)h < (unsigned)H) & ((unsigned)w < (unsigned)W);
-                        cell[i] = in ? __mul24(h & (R - 1), W) + w : -1;
+                for (int j = 0; j < 4; j++)
+                    *reinterpret_cast<float4*>(Pk + (tx * 4 + j) * TR + ty * 4) = make_float4(acc[0][j], acc[1][j], acc[2][j], acc[3][j]);
+                __syncthreads();
+                const int last = pos0 + rows - 1;
+                const int h_first = max(0, (pos0 / win.WO) * win.S - win.P);
+                const int h_last = min(H - 1, (last / win.WO) * win.S - win.P + 2 * win.D);
+                const int nrow = h_last - h_first + 1;
+                const float inv_nrow = 1.0f / (float)nrow;
+                for (int i = tid; i < planes * nrow * W; i += 256) {
+                    // i = (c * nrow + hr) * W + w; quotients of small numbers through the reciprocal
+                    const int rest = (int)(((float)i + 0.5f) * inv_w), w = i - rest * W;
+                    const int c = (int)(((float)rest + 0.5f) * inv_nrow), h = h_first + (rest - c * nrow);
+                    const float* col = Pk + c * 9 * TR - pos0;
+                    int hb[3], wb[3];
+#pragma unroll
+                    for (int t = 0; t < 3; t++) {
+                        hb[t] = HT[h * 3 + t];
+                        wb[t] = WT[w * 3 + t];
                     }
+                    float sum = 0.f;
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        const bool mine = col_ok[j] && col_tap[j] == tap;
-                        // a wave holds 16 consecutive columns, so one or two of its four j have this tap: the others
-                        // are skipped by the whole wave (a scalar branch) instead of being walked with no lane active
-                        if (__builtin_amdgcn_ballot_w64(mine) == 0) continue;
-                        const int plane = mine ? col_plane[j] * R * W : -spare - 1;   // not mine: every index below is negative
-                        int at[4];
-                        float v[4];
+                    for (int th = 0; th < 3; th++)
 #pragma unroll
-                        for (int i = 0; i < 4; i++) {
-                            at[i] = (plane | cell[i]) >= 0 ? plane + cell[i] : spare;   // both non-negative: a pixel
-                            v[i] = Fp[at[i]];
+                        for (int tw = 0; tw < 3; tw++) {
+                            const int pos = hb[th] + wb[tw];   // negative when either has no window
+                            const bool in = (unsigned)(pos - pos0) < (unsigned)rows;
+                            sum += *(in ? col + (th * 3 + tw) * TR + pos : zero_word);
                         }
-#pragma unroll
-                        for (int i = 0; i < 4; i++) Fp[at[i]] = v[i] + acc[i][j];
-                    }
-                    __syncthreads();
+                    Fp[(c * R + (h & (R - 1))) * W + w] += sum;
                 }
+                __syncthreads();   // the next tile stages over the parked sums; its flush reads the ring
             }
             flush_rows(flushed, H);
             __syncthreads();       // before the ring is used for the next image
@@ -429,12 +458,15 @@ template <bool IMG, int IE>
 hipError_t launch_conv_backward(const float* grad_output, const float* input, const float* weight, const float* output,
                                 float* grad_input, float* grad_weight, float p, const Problem& pr, const ImgWin& win,
                                 hipStream_t stream) {
-    ConvBwd d{pr.B, pr.G, pr.K, pr.NG, pr.HW, pr.B * pr.HW, 0, 0, 0, 0};
+    ConvBwd d{pr.B, pr.G, pr.K, pr.NG, pr.HW, pr.B * pr.HW, 0, 0, 0, 0, 0};
     d.tiles_k = IMG ? (win.CG + kPlanes - 1) / kPlanes : (d.K + TCP - 1) / TCP;
     d.units = IMG ? pr.B : (d.M + TR - 1) / TR;
     const long pairs = (long)d.tiles_k * d.G;
-    if constexpr (IMG) d.ring_rows = ring_rows_for(win, pr.HW);
-    const size_t lds = lds_bytes(d.NG, IMG ? (size_t)kPlanes * d.ring_rows * win.W + 4 : 0);   // + the spare word
+    if constexpr (IMG) {
+        d.ring_rows = ring_rows_for(win, pr.HW);
+        d.park_extra = park_extra(d.NG);
+    }
+    const size_t lds = lds_bytes(d.NG, IMG ? image_floats(d.NG, d.ring_rows, win.H, win.W) : 0);
     // Units per workgroup: the choice that needs the fewest rounds of resident workgroups times units (the device
     // holds `resident` of them at once), among those that keep the number of workgroups, each of which flushes a whole
     // grad_weight tile at the end, within sixteen rounds; ties go to fewer, longer workgroups.
@@ -489,7 +521,7 @@ bool norm_conv_backward_fused_applicable(const Problem& pr) {
 bool norm_conv_backward_fused_image_applicable(const ConvGeom& q, int G, int CO, int num_cu) {
     if (g_tile_override >= 2 || (long)q.HO * q.WO <= 1) return false;
     const ImgWin win{q.C, q.C / G, q.H, q.W, q.HO, q.WO, q.S, q.P, q.D};
-    if (lds_bytes(CO / G, (size_t)kPlanes * ring_rows_for(win, q.HO * q.WO) * q.W + 4) > kMaxLds) return false;
+    if (lds_bytes(CO / G, image_floats(CO / G, ring_rows_for(win, q.HO * q.WO), q.H, q.W)) > kMaxLds) return false;
     // the kernel's 32-bit byte offsets: a tile's planes of one image, one image's outputs of a group
     if (4L * kPlanes * q.H * q.W >= (1L << 31) || 4L * (CO / G) * q.HO * q.WO >= (1L << 31)) return false;
     return forced_on() || (long)q.B * q.HO * q.WO >= 64L * num_cu;
