@@ -42,6 +42,7 @@ namespace {
 constexpr int TR = 64;              // rows of a tile
 constexpr int TCP = 64;             // columns a tile has lanes for
 constexpr int WLD = TCP + 4;        // row length of the weight and grad_weight tiles (rows 16-byte aligned)
+constexpr int TI = 8, TJ = 2;       // a lane's patch: rows x columns; 64 / TI lanes share a column pair, inside one DPP row
 constexpr int kPlanes = 7;          // IMG: channels per tile (63 columns)
 constexpr size_t kMaxLds = 159 * 1024;   // all of LDS less the kernel's own static words
 
@@ -84,7 +85,8 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
     float* Rs = Cs + NG * TR;            // [NG][TR]   1 / out
     float* Fp = Rs + NG * TR + (IMG ? d.park_extra : 0);   // IMG: [kPlanes][ring_rows][W] gradient of the image rows still being added to
     const int tid = threadIdx.x;
-    const int ty = tid & 15, tx = tid >> 4;   // rows first: the 16 lanes of a column group form a DPP row
+    constexpr int TYN = TR / TI;             // lanes along the rows
+    const int ty = tid % TYN, tx = tid / TYN;   // rows first: the lanes of a column group are neighbours in a DPP row
     const int tk = blockIdx.x % d.tiles_k, g = blockIdx.x / d.tiles_k;
     const int k0 = tk * TC;
     const int u_begin = blockIdx.y * d.units_per_wg, u_end = min(d.units, u_begin + d.units_per_wg);
@@ -152,12 +154,12 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
         for (int i = tid; i < NG * TCP; i += 256) Ws[(i / TCP) * WLD + i % TCP] *= unit_inv;   // each lane the words it wrote
     }
     // the lane's four columns: whether they exist, and for the image their channel plane and tap
-    bool col_ok[4];
-    int col_plane[4], col_tap[4], col_dh[4], col_dw[4];   // IMG: the column's channel plane inside the tile, its tap and the tap's offsets
-    int col_off[4];                                       // IMG: where the tap lies from the window's corner, in the tile's planes of one image
+    bool col_ok[TJ];
+    int col_plane[TJ], col_tap[TJ], col_dh[TJ], col_dw[TJ];   // IMG: the column's channel plane inside the tile, its tap and the tap's offsets
+    int col_off[TJ];                                      // IMG: where the tap lies from the window's corner, in the tile's planes of one image
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int c = tx * 4 + j;
+    for (int j = 0; j < TJ; j++) {
+        const int c = tx * TJ + j;
         col_ok[j] = c < TC && k0 + c < K;
         col_plane[j] = c / 9;
         col_tap[j] = c - col_plane[j] * 9;
@@ -173,23 +175,23 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
 
     // One tile: rows first_row .. first_row + 63 of the unfolded matrix, of which `rows` exist (IMG: rows of image b
     // from position pos0).  Leaves the grad_input sums of the lane's patch in acc.
-    auto tile = [&](int first_row, int rows, int b, int pos0, float (&acc)[4][4], WinRow (&wrow)[4], size_t (&xoff)[4]) {
-        float q[4][4];
+    auto tile = [&](int first_row, int rows, int b, int pos0, float (&acc)[TI][TJ], WinRow (&wrow)[TI], size_t (&xoff)[TI]) {
+        float q[TI][TJ];
         if constexpr (!IMG) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int r = min(ty * 4 + i, rows - 1);
+            for (int i = 0; i < TI; i++) {
+                const int r = min(ty * TI + i, rows - 1);
                 const int m = first_row + r, bi = m / d.HW;
                 xoff[i] = ((size_t)(bi * d.G + g) * K) * d.HW + (m - bi * d.HW);
             }
         }
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < TI; i++) {
             const int corner = IMG ? wrow[i].h0 * win.W + wrow[i].w0 : 0;   // IMG: the window's corner in a plane (may lie in the padding)
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
+            for (int j = 0; j < TJ; j++) {
                 acc[i][j] = 0.f;
-                const bool ok = ty * 4 + i < rows && col_ok[j];
+                const bool ok = ty * TI + i < rows && col_ok[j];
                 if constexpr (IMG) {   // the window's tap of column j: channel and offsets are the lane's constants
                     const int h = wrow[i].h0 + col_dh[j], w = wrow[i].w0 + col_dw[j];
                     // one select, no branches: the tests are combined bitwise
@@ -197,7 +199,7 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
                     const unsigned o = in ? 4u * (unsigned)(corner + col_off[j]) : ~0u;
                     q[i][j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(x_rsrc, o, 0, 0)) * unit_inv;
                 } else {
-                    q[i][j] = ok ? input[xoff[i] + (size_t)(k0 + tx * 4 + j) * d.HW] * unit_inv : 0.f;   // unit_inv: 1 unless IE == 0
+                    q[i][j] = ok ? input[xoff[i] + (size_t)(k0 + tx * TJ + j) * d.HW] * unit_inv : 0.f;   // unit_inv: 1 unless IE == 0
                 }
             }
         }
@@ -275,27 +277,46 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
         }
         auto reduce = [&](auto term) {   // term(x - w, 1/out): the power that g (or g / out^IE) multiplies
             for (int n = 0; n < NG; n++) {
-                const float4 c4 = *reinterpret_cast<const float4*>(Cs + n * TR + ty * 4);
-                const float4 r4 = *reinterpret_cast<const float4*>(Rs + n * TR + ty * 4);
-                const float4 w4 = *reinterpret_cast<const float4*>(Ws + n * WLD + tx * 4);
-                const float cv[4] = {c4.x, c4.y, c4.z, c4.w}, rv[4] = {r4.x, r4.y, r4.z, r4.w}, wv[4] = {w4.x, w4.y, w4.z, w4.w};
-                float s[4] = {0.f, 0.f, 0.f, 0.f};
+                float cv[TI], rv[TI], wv[TJ];
 #pragma unroll
-                for (int i = 0; i < 4; i++)
+                for (int i = 0; i < TI; i += 4) {
+                    const float4 c4 = *reinterpret_cast<const float4*>(Cs + n * TR + ty * TI + i);
+                    const float4 r4 = *reinterpret_cast<const float4*>(Rs + n * TR + ty * TI + i);
+                    cv[i] = c4.x; cv[i + 1] = c4.y; cv[i + 2] = c4.z; cv[i + 3] = c4.w;
+                    rv[i] = r4.x; rv[i + 1] = r4.y; rv[i + 2] = r4.z; rv[i + 3] = r4.w;
+                }
+                if constexpr (TJ == 4) {
+                    const float4 w4 = *reinterpret_cast<const float4*>(Ws + n * WLD + tx * 4);
+                    wv[0] = w4.x; wv[1] = w4.y; wv[2] = w4.z; wv[3] = w4.w;
+                } else {
+                    const float2 w2 = *reinterpret_cast<const float2*>(Ws + n * WLD + tx * 2);
+                    wv[0] = w2.x; wv[1] = w2.y;
+                }
+                float s[TJ];
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
+                for (int j = 0; j < TJ; j++) s[j] = 0.f;
+#pragma unroll
+                for (int i = 0; i < TI; i++)
+#pragma unroll
+                    for (int j = 0; j < TJ; j++) {
                         const float sp = term(q[i][j] - wv[j], rv[i]);
                         acc[i][j] = __builtin_fmaf(cv[i], sp, acc[i][j]);   // two fused multiply-adds, not a shared
                         s[j] = __builtin_fmaf(cv[i], sp, s[j]);             // product and two additions
                     }
-                float tot[4];
+                float tot[TJ];
 #pragma unroll
-                for (int j = 0; j < 4; j++) tot[j] = dpp_row_total(s[j]);
-                if (ty == 15) {   // d/dw of |x - w| is minus d/dx
-                    float4* gp = reinterpret_cast<float4*>(Gw + n * WLD + tx * 4);
-                    float4 v = *gp;
-                    v.x -= tot[0]; v.y -= tot[1]; v.z -= tot[2]; v.w -= tot[3];
-                    *gp = v;
+                for (int j = 0; j < TJ; j++) tot[j] = dpp_lanes_total<TYN>(s[j]);
+                if (ty == TYN - 1) {   // d/dw of |x - w| is minus d/dx
+                    float* gp = Gw + n * WLD + tx * TJ;
+                    if constexpr (TJ == 4) {
+                        float4 v = *reinterpret_cast<float4*>(gp);
+                        v.x -= tot[0]; v.y -= tot[1]; v.z -= tot[2]; v.w -= tot[3];
+                        *reinterpret_cast<float4*>(gp) = v;
+                    } else {
+                        float2 v = *reinterpret_cast<float2*>(gp);
+                        v.x -= tot[0]; v.y -= tot[1];
+                        *reinterpret_cast<float2*>(gp) = v;
+                    }
                 }
             }
         };
@@ -305,9 +326,9 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
         else reduce([&](float df, float ri) { return spower(df * ri); });
     };
 
-    float acc[4][4];
-    WinRow wrow[4];
-    size_t xoff[4];
+    float acc[TI][TJ];
+    WinRow wrow[TI];
+    size_t xoff[TI];
     if constexpr (IMG) {
         const int H = win.H, W = win.W, R = d.ring_rows, first_ch = tk * kPlanes;
         const int planes = min(kPlanes, win.CG - first_ch);
@@ -353,25 +374,28 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
                 const_cast<float*>(grad_output + (size_t)(b * d.G + g) * NG * d.HW), 0, (int)0x80000000u, 0x00020000);
             o_rsrc = __builtin_amdgcn_make_buffer_rsrc(
                 const_cast<float*>(output + (size_t)(b * d.G + g) * NG * d.HW), 0, (int)0x80000000u, 0x00020000);
-            // the lane's four positions, kept as (output row, output column) and moved on by 64 positions per tile
-            int ho[4], wo[4];
+            // the corners of the windows of the lane's positions, moved on by 64 positions per tile (positions past
+            // the image's last one are never used: every use asks for i < rows)
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                ho[i] = (ty * 4 + i) / win.WO;
-                wo[i] = (ty * 4 + i) - ho[i] * win.WO;
+            for (int i = 0; i < TI; i++) {
+                const int ho = (ty * TI + i) / win.WO, wo = (ty * TI + i) - ho * win.WO;
+                wrow[i].b = b;
+                wrow[i].h0 = ho * win.S - win.P;
+                wrow[i].w0 = wo * win.S - win.P;
             }
-            const int step_h = TR / win.WO, step_w = TR - step_h * win.WO;
+            const int step_rows = TR / win.WO;
+            const int step_h = step_rows * win.S, step_w = (TR - step_rows * win.WO) * win.S;
+            const int wrap_w = win.WO * win.S, end_w = wrap_w - win.P;   // a corner's column stays below end_w
             int flushed = 0;   // image rows below this one are in memory
             for (int pos0 = 0; pos0 < d.HW; pos0 += TR) {
                 const int rows = min(TR, d.HW - pos0);
+                if (pos0 > 0) {
 #pragma unroll
-                for (int i = 0; i < 4; i++) {   // positions past the image's last one are never used (every use asks for i < rows)
-                    wrow[i].b = b;
-                    wrow[i].h0 = ho[i] * win.S - win.P;
-                    wrow[i].w0 = wo[i] * win.S - win.P;
-                    wo[i] += step_w;
-                    ho[i] += step_h;
-                    if (wo[i] >= win.WO) { wo[i] -= win.WO; ho[i]++; }
+                    for (int i = 0; i < TI; i++) {
+                        wrow[i].h0 += step_h;
+                        wrow[i].w0 += step_w;
+                        if (wrow[i].w0 >= end_w) { wrow[i].w0 -= wrap_w; wrow[i].h0 += win.S; }
+                    }
                 }
                 tile(0, rows, b, pos0, acc, wrow, xoff);
                 // rows above this tile's first window are final (the last tile's rounds ended with a barrier)
@@ -383,8 +407,11 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
                 // every pixel that a window of this tile can reach fetches its up to nine (position, tap) entries
                 // and adds them to its ring word: one owner per pixel, a fixed order of the nine, no rounds.
 #pragma unroll
-                for (int j = 0; j < 4; j++)
-                    *reinterpret_cast<float4*>(Pk + (tx * 4 + j) * TR + ty * 4) = make_float4(acc[0][j], acc[1][j], acc[2][j], acc[3][j]);
+                for (int j = 0; j < TJ; j++)
+#pragma unroll
+                    for (int i = 0; i < TI; i += 4)
+                        *reinterpret_cast<float4*>(Pk + (tx * TJ + j) * TR + ty * TI + i) =
+                            make_float4(acc[i][j], acc[i + 1][j], acc[i + 2][j], acc[i + 3][j]);
                 __syncthreads();
                 const int last = pos0 + rows - 1;
                 const int h_first = max(0, (pos0 / win.WO) * win.S - win.P);
@@ -423,10 +450,10 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
             const int m0 = t * TR, rows = min(TR, d.M - m0);
             tile(m0, rows, 0, 0, acc, wrow, xoff);
 #pragma unroll
-            for (int i = 0; i < 4; i++)
+            for (int i = 0; i < TI; i++)
 #pragma unroll
-                for (int j = 0; j < 4; j++)
-                    if (ty * 4 + i < rows && col_ok[j]) grad_input[xoff[i] + (size_t)(k0 + tx * 4 + j) * d.HW] = acc[i][j];
+                for (int j = 0; j < TJ; j++)
+                    if (ty * TI + i < rows && col_ok[j]) grad_input[xoff[i] + (size_t)(k0 + tx * TJ + j) * d.HW] = acc[i][j];
             __syncthreads();   // the next tile overwrites the panels
         }
     }
