@@ -7,12 +7,13 @@
 //
 // A layer of this shape has few outputs per group and very many rows, so a workgroup keeps the weights of its
 // columns k for ALL outputs of the group in LDS, next to a tile of grad_weight sums of the same shape, and walks
-// tiles of 64 rows.  Per tile it stages g and 1/out (NG x 64 each), and every lane reduces a 4 x 4 patch of
+// tiles of 64 rows.  Per tile it stages g and 1/out (NG x 64 each), and every lane reduces an 8 x 2 patch of
 // (row, column) over n: a term is evaluated once, added to the lane's grad_input sum and to the column's partial sum
-// over the lane's four rows; the sixteen lanes that share the columns (one DPP row) add those with four row shifts
-// and the row's last lane, the only one that ever touches these four words, adds the total onto the LDS tile of
-// grad_weight.  After its last tile the workgroup adds the LDS tile onto grad_weight with float atomics (one
-// addend per workgroup and element).
+// over the lane's eight rows; the eight lanes that share the columns (half a DPP row) add those with three row
+// shifts and the last of them, the only lane that ever touches these two words, adds the total onto the LDS tile of
+// grad_weight.  (A DPP addition costs 4.4 clocks against 2.5 for a plain one: with a 4 x 4 patch the sixteen of them
+// per output were 10 % of the loop's instructions and 15 % of its time.)  After its last tile the workgroup adds the
+// LDS tile onto grad_weight with float atomics (one addend per workgroup and element).
 //
 // grad_input.  From the unfolded tensor (IMG = false) a tile is 64 columns wide and every element is written once.
 // From the image (IMG = true, 3x3 windows) a pixel collects up to nine columns.  Float atomics for that, in memory
@@ -20,10 +21,13 @@
 // work is cut such that every pixel has one owner: a tile is 63 columns wide, i.e. seven whole channels, a
 // workgroup takes whole images, and it keeps the image rows of its seven channel planes that its windows are
 // still adding to in LDS (a ring of rows: a tile of 64 positions covers a few output rows, and everything above
-// the next tile's first window is final).  A tile's sums go there in nine rounds, one per tap, with a barrier
-// between them: inside a round the (position, channel) pairs, and therefore the pixels, are all different, so
-// plain read-add-write is safe.  Final rows are written to memory with plain stores and their ring rows cleared:
-// grad_img needs no zero fill, and the result does not depend on the order in which workgroups run.
+// the next tile's first window is final).  A tile's sums are parked in LDS by (column, position), over the g and
+// 1/out panels, which are free by then; then every pixel of the ring rows that the tile's windows reach fetches
+// its up to nine (position, tap) entries -- two small tables give, per image row and tap row, the output row whose
+// window has that tap there, and the same per column -- and adds them to its ring word in a fixed order.  Final
+// rows are written to memory with plain stores and their ring rows cleared: grad_img needs no zero fill, and the
+// result does not depend on the order in which workgroups run.  (Before the parked tile the sums joined the ring in
+// nine rounds, one per tap, with a barrier between them: 1.57 against 1.38 ms on 128 x 128 x 32 x 32, p = 8.)
 //
 // IE = p - 1 for the multiply-only exponents (1, 2, 3, 7): the power is taken of the raw difference and the
 // coefficient g / out^(p-1) is staged instead of g, unless a tile holds an output outside [2^-12, 2^12], which then

@@ -339,8 +339,9 @@ class NormDistConv(nn.Module):
                 (self.in_channels // self.group) * x.size(3) <= norm_dist_cpp.FOLDED_MAX_ROW_FLOATS)
 
     # Finite p: "image" runs the layer from the image (nothing of the unfolded size is allocated); "columns" runs native
-    # unfold + the column kernels + native fold, which is about a fifth faster on 32 x 32 images with 32 to 64 channels
-    # and holds two tensors of nine times the image's size while it runs.  Not in the reference, which always unfolds.
+    # unfold + the column kernels + native fold, which takes about as long (within 5 % either way on the reference's
+    # conv nets) and holds two tensors of nine times the image's size while it runs.  Not in the reference, which
+    # always unfolds.
     finite_p_route = "image"
 
     def _norm_from_image(self, x):
