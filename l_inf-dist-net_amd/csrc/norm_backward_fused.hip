@@ -10,8 +10,9 @@
 // walks the outputs n; a lane keeps an 8 x TN patch of x and of the grad_input sums.  For grad_weight the lane
 // also adds, per output n, its eight rows' terms of each of its TN columns (one more fused multiply-add per term),
 // the sixteen lanes that share those columns (one DPP row: the lane index runs along m first here) add their
-// partial sums with four row shifts, the row's last lane parks the total of the tile's 128 rows in an LDS tile
-// [stage's outputs][BN], and once per stage the whole workgroup adds that tile onto grad_weight with float atomics
+// partial sums over each half of the row with three row shifts, the halves' last lanes park the two totals of the
+// tile's 128 rows in two LDS tiles [stage's outputs][BN], and once per stage the whole workgroup adds the tiles'
+// sum onto grad_weight with float atomics
 // (64 consecutive columns per instruction).  grad_weight therefore collects one addend per tile of 128 rows, in no
 // fixed order, and must be zero-filled (or hold the values to accumulate onto) by the caller, as with the separate
 // call.  IE = 0: any p > 2; the power is taken of the normalised difference (x - w) / out, which never leaves the
@@ -85,30 +86,36 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
         }
     }
     float* const gw_group = grad_weight + (size_t)g * NG * K;
-    // The lane's column sums of output n (already summed over its rows) are summed over the 16 lanes of the row and
-    // parked in an LDS tile [stage's outputs][BN columns]; the sign: d/dw of |x - w| is minus d/dx.  The tile goes
+    // The lane's column sums of output n (already summed over its rows) are summed over each half of the 16 lanes
+    // that share the columns (three DPP row shifts; lanes 7 and 15 of the row hold the halves' totals) and parked in
+    // two LDS tiles [stage's outputs][BN columns], one per half; the sign: d/dw of |x - w| is minus d/dx.  The fourth
+    // shift, which would join the halves, costs more than the second tile: a DPP instruction takes 4.4 clocks, the
+    // twenty-five of a step (five sums) were a quarter of the p = 8 launch, and without the last level 2.51 -> 2.28 ms
+    // on 512 x 5120 -> 5120.  (LDS float atomics from the four quarter totals instead: 3.13 ms.)  The tiles go
     // onto grad_weight once per stage (flush_weight_tile): straight from here an atomic instruction had four active
     // lanes (the last lane of each row of sixteen), and the float atomics of a 5120-wide layer, 105 M in 26 M
     // instructions, took 1.7 ms of the launch's 4.2.
-    float* const Gs = lds + 2 * XS + GEO::WS;   // [KK][BN], all zero between stages
+    float* const Gs = lds + 2 * XS + GEO::WS;   // 2 x [KK][BN], all zero between stages
     auto add_weight_row = [&](int n_local, const float (&s)[TN]) {
         float tot[TN];
 #pragma unroll
-        for (int j = 0; j < TN; j++) tot[j] = dpp_row_total(s[j]);
-        if (ty == GEO::TY - 1) {
+        for (int j = 0; j < TN; j++) tot[j] = dpp_lanes_total<8>(s[j]);
+        if ((ty & 7) == 7) {
+            float* half = Gs + (ty >> 3) * (KK * BN);
 #pragma unroll
-            for (int j = 0; j < TN; j++) Gs[n_local * BN + GEO::col(tx, j)] = -tot[j];
+            for (int j = 0; j < TN; j++) half[n_local * BN + GEO::col(tx, j)] = -tot[j];
         }
     };
-    // All lanes of the workgroup: 64 consecutive columns of one output per wave instruction; a parked zero (nothing
-    // added: padding, or a row the large-exponent path passed over) costs no atomic.  Leaves the tile zero.
+    // All lanes of the workgroup: 64 consecutive columns of one output per wave instruction; two parked zeros (nothing
+    // added: padding, or a row the large-exponent path passed over) cost no atomic.  Leaves the tiles zero.
     auto flush_weight_tile = [&](int n_first) {
         for (int i = tid; i < KK * BN; i += GEO::NT) {
-            const float v = Gs[i];
-            if (v != 0.f) {
+            const float a = Gs[i], b = Gs[i + KK * BN];
+            if (a != 0.f || b != 0.f) {
                 Gs[i] = 0.f;
+                Gs[i + KK * BN] = 0.f;
                 const int nl = i / BN, c = i - nl * BN;
-                if (n_first + nl < NG && k0 + c < K) atomicAdd(gw_group + (size_t)(n_first + nl) * K + k0 + c, v);
+                if (n_first + nl < NG && k0 + c < K) atomicAdd(gw_group + (size_t)(n_first + nl) * K + k0 + c, a + b);
             }
         }
     };
@@ -241,7 +248,7 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
     };
 
     const int nstage = (NG + KK - 1) / KK;
-    for (int i = tid; i < KK * BN; i += GEO::NT) Gs[i] = 0.f;
+    for (int i = tid; i < 2 * KK * BN; i += GEO::NT) Gs[i] = 0.f;
     load(0);
     if (logscale) {
         float top = 0.f, nbot = -__builtin_inff();   // the largest and minus the smallest output this lane loaded
@@ -437,7 +444,7 @@ static hipError_t launch_fused(const Problem& pr, hipStream_t stream, const floa
     d.tiles_m = (d.M + GEO::BM - 1) / GEO::BM;
     d.tiles_n = (d.K + GEO::BN - 1) / GEO::BN;
     const unsigned grid = (unsigned)d.tiles_m * d.tiles_n * d.G;
-    constexpr size_t lds = (size_t)(2 * GEO::XS + GEO::WS + GEO::KK * GEO::BN) * sizeof(float);   // panels, grad_weight tile
+    constexpr size_t lds = (size_t)(2 * GEO::XS + GEO::WS + 2 * GEO::KK * GEO::BN) * sizeof(float);   // panels, the two grad_weight tiles
     auto kern = norm_backward_fused_kernel<GEO, IE>;
     static LdsRecord lds_allowed = {};
     if (hipError_t e = allow_lds(kern, lds, pr.device, lds_allowed); e != hipSuccess) return e;
