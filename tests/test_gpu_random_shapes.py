@@ -210,6 +210,58 @@ def test_random_conv_layer_at_finite_p_from_the_image(seed):
     assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
 
 
+def draw_wide_image(seed):
+    """A 3x3 layer with strides and paddings up to 3, dilations up to 3, images up to 70 x 70, 1 to 139 outputs per
+    group; None where the draw is degenerate, too large for the oracle, or a geometry the image kernels do not take."""
+    r = random.Random(51000 + seed)
+    G, CG = r.choice([1, 1, 2, 4]), r.choice([1, 2, 3, 5, 7, 8, 9, 15, 16, 33])
+    NG = r.choice([1, 2, 7, 16, 31, 32, 33, 64, 100, 130, 139])
+    H, W = r.randint(3, 70), r.randint(3, 70)
+    stride, padding, dilation = r.choice([1, 1, 2, 3]), r.choice([0, 1, 1, 2, 3]), r.choice([1, 1, 2, 3])
+    if H + 2 * padding < 2 * dilation + 1 or W + 2 * padding < 2 * dilation + 1:
+        return None
+    HO, WO = (H + 2 * padding - 2 * dilation - 1) // stride + 1, (W + 2 * padding - 2 * dilation - 1) // stride + 1
+    work = HO * WO * NG * CG * 9 * G
+    if work > 40_000_000 or HO * WO <= 1:
+        return None
+    B = max(1, min(r.choice([1, 2, 3, 8]), 20_000_000 // work))
+    return B, CG * G, H, W, NG * G, G, stride, padding, dilation, r.choice([8.0, 5.5, 20.5, 3.0, 4.0, 70.0])
+
+
+@pytest.mark.parametrize("seed", range(64))
+def test_random_conv_one_pass_backward_on_wide_geometries(seed):
+    """The one-pass conv backward from the image sizes its LDS by the layer (ring of image rows, tables per image row
+    and column, the parked tile's overhang when a group has fewer than 32 outputs) and finds a pixel's windows through
+    those tables: strides, paddings and dilations up to 3 on images up to 70 x 70, forced on and left to the library."""
+    import torch.nn.functional as F
+    from gpu_common import DEV, cpp, say, set_tile
+    drawn = draw_wide_image(seed)
+    if drawn is None:
+        pytest.skip("degenerate draw")
+    B, C, H, W, CO, G, stride, padding, dilation, p = drawn
+    if not cpp.norm_dist_conv_supported(C, H, W, CO, G, 3, stride, padding, dilation):
+        pytest.skip("not a geometry of the image kernels")
+    say("wide conv geometry", seed, (B, C, H, W, CO, G, stride, padding, dilation), "p", p)
+    g = gen(52000 + seed)
+    img = torch.rand(B, C, H, W, generator=g)
+    w = (torch.randn(CO, C // G * 9, generator=g) * 0.5).contiguous()
+    cols = F.unfold(img, 3, dilation, padding, stride).contiguous()
+    want = oracle.norm_dist_forward(cols, w, G, p)
+    go = torch.randn(want.shape, generator=g)
+    ex, mx = oracle.norm_dist_backward_input(go, cols, w, want, G, p, with_abs_terms=True)
+    ew, mw = oracle.norm_dist_backward_weight(go, cols, w, want, G, p, with_abs_terms=True)
+    fold = lambda t: F.fold(t.double(), (H, W), 3, dilation, padding, stride)
+    args = (go.to(DEV), img.to(DEV), w.to(DEV), want.to(DEV))
+    for mode in (0, -1):
+        set_tile(mode)
+        gi = torch.full(img.shape, float("nan"), device=DEV)
+        gw = torch.zeros(w.shape, device=DEV)
+        cpp.norm_dist_conv_backward(*args, gi, gw, G, p, 3, stride, padding, dilation)
+        torch.cuda.synchronize()
+        assert_sum_close(gi.cpu(), fold(ex), fold(mx), p, RTOL, ATOL)
+        assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
+
+
 P_MAGNITUDES = [2.5, 4.0, 5.5, 8.0, 16.5, 20.5, 33.0, 47.0, 63.0, 64.5, 100.0, 300.0, 1000.0]
 
 
