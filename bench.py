@@ -248,7 +248,7 @@ def workload_c2(pkg, torch, dev):
                 kernel=("norm_dist_backward_input", lambda go, x_, w_, *_: 7 * mnk(x_, w_),
                         lambda go, x_, w_, *_: w_.size(0) > 16,
                         "norm_backward_input_tiled_kernel (grad_input, register-tiled)", 7)
-                if C2_P in (2.0, 3.0) else   # the exponents whose two register-tiled kernels beat the one-pass kernel
+                if C2_P == 2.0 else   # the exponent whose two register-tiled kernels beat the one-pass kernel
                        ("norm_dist_backward", lambda go, x_, w_, *_: 2 * 7 * mnk(x_, w_),
                         lambda go, x_, w_, *_: w_.size(0) > 16,
                         "norm_backward_fused_kernel (both gradients from one evaluation of every term; the flops are "
@@ -713,7 +713,7 @@ def main():
 
 # workload -> (counter summary under profiles/, the roofline kernel's name in it)
 def traffic_profiles():
-    c2_fused = C2_P not in (2.0, 3.0)
+    c2_fused = C2_P != 2.0
     return {"c1": ("counters_c1_mlp_inf.md", "inf_forward_kernel"), "c1t": ("counters_c1t_training_step.md", "inf_forward_kernel"),
             "c0": ("counters_c0_fc_layer.md", "inf_forward_kernel"),
             "c2": (f"counters_c2_mlp_p{C2_P:g}.md", "norm_backward_fused_kernel" if c2_fused else "norm_backward_input_tiled_kernel"),

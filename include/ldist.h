@@ -153,7 +153,8 @@ LDIST_API int ldist_norm_dist_backward_weight(const float* grad_output, const fl
  * model/norm_dist.py:41-46).  No single counterpart in the reference.  Every term
  *   g[m,n] * (|x-w| / output[m,n])^(p-1) * sign(x-w)
  * belongs to both sums.  One kernel evaluates it once and adds it to both for fully connected layers large enough to
- * fill the device at every exponent p > 2 other than 3 (p = 2 and 3 are cheaper as two kernels; grad_weight then
+ * fill the device at every exponent p > 2 (p = 2 is cheaper as two kernels, p = 3 too unless the tiles fill nine
+ * tenths of the device; grad_weight then
  * collects one addend per tile of 128 rows with float atomics, in no fixed order), and for the unfolded-conv layout (HW > 1) with up to
  * about 140 outputs per group (one addend per workgroup); other shapes run the two separate kernels.  grad_input is written whole and may be uninitialised;
  * grad_weight is added to and must hold zeros (or the values to accumulate onto) on entry. */

@@ -474,13 +474,15 @@ bool norm_backward_fused_applicable(const Problem& pr, float p, const void* grad
         return false;
     if (g_tile_override == 0 || g_tile_override == 1) return true;   // tests and tuning: forced on (128 x 80, 128 x 64)
     if (g_tile_override >= 2) return false;                          // forced off
-    // p = 2 and 3: a term is one or two instructions and sharing it saves less than the row sums of grad_weight cost
-    // (512 x 5120 -> 5120: 1.58 against 1.40 ms at p = 2, a tie at p = 3; 2.03 against 2.18 ms at p = 4 and
-    // 2.50 against 2.97 ms at p = 8)
-    if (const int ie = fused_int_power(p); ie == 1 || ie == 2) return false;
+    // p = 2: a term is one instruction and sharing it saves less than the row sums of grad_weight cost (512 x 5120 ->
+    // 5120: 1.44 against 1.42 ms).  p = 3: 1.65 against 1.83 ms where the tiles fill the device (10240 inputs: 3.30
+    // against 3.71 ms), a tie at 192 tiles of 256 (3072 inputs), a loss at 128.  p = 4: 1.88 against 2.22 ms, p = 8:
+    // 2.27 against 3.06 ms.
+    const int ie = fused_int_power(p);
+    if (ie == 1) return false;
     const long M = (long)pr.B * pr.HW;
     const long t80 = ((M + 127) / 128) * ((pr.K + 79) / 80) * pr.G, t64 = ((M + 127) / 128) * ((pr.K + 63) / 64) * pr.G;
-    return (t80 > t64 ? t80 : t64) * 10 >= 7L * pr.num_cu && pr.NG >= 256;
+    return (t80 > t64 ? t80 : t64) * 10 >= (ie == 2 ? 9L : 7L) * pr.num_cu && pr.NG >= 256;
 }
 
 template <class GEO>
