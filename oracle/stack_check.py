@@ -13,7 +13,9 @@ really received and produced on the GPU; the oracle then repeats every layer on 
   for bit), and once more through both scatter gradients, which move if a single index or sign differs;
 * L_inf scatter gradients: rel 1e-5 / abs 1e-6 (the library rounds double sums once);
 * p-norm values: rel 1e-5 / abs 1e-6; gradients: the float32-sum tolerance of `sum_ratio` (ratio <= 1 passes);
-* the mean shift: abs 2e-6 against the float64 mean;
+* the mean shift: abs 2e-6 against the float64 mean, or four units in the last place of the largest input where that
+  is more (a float32 difference of numbers of size X cannot be closer than ulp(X); outputs grow past 16 only at
+  exponents below the reference's schedule, p < 8 on 5120 inputs);
 * and, free running from the input (the oracle feeding itself), the last layer's output: every layer is
   1-Lipschitz in the L_inf norm, so rounding of the shifts cannot grow on the way.
 
@@ -173,7 +175,8 @@ def check_training_step(model, x_cpu, upstream_cpu, p, dev, rows=None, weight_ro
         es, _ = mean_shift(raw)
         if L["bias"] is not None:
             es = es + L["bias"].view(1, -1, 1)
-        rep.ratio(name + " mean shift", close_ratio(L["shifted"], es, rtol=1e-6, atol=2e-6), L["shifted"], es)
+        ms_atol = max(2e-6, 4 * 2.0 ** -23 * float(raw.abs().max()))
+        rep.ratio(name + " mean shift", close_ratio(L["shifted"], es, rtol=1e-6, atol=ms_atol), L["shifted"], es)
         # backward: the gradient that reached the operator output on the GPU goes through the oracle
         g = L["grad_raw"]
         if inf:
