@@ -499,19 +499,10 @@ struct RowsT {
     }
 };
 
-// Sum over the 16 lanes of a DPP row (four row shifts); the total arrives in the row's last lane, the others
-// hold prefix sums.  Every lane of the row must be active.
-__device__ __forceinline__ float dpp_row_total(float v) {
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x111, 0xf, 0xf, true));  // row_shr:1
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x112, 0xf, 0xf, true));  // row_shr:2
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x114, 0xf, 0xf, true));  // row_shr:4
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x118, 0xf, 0xf, true));  // row_shr:8
-    return v;
-}
-
-// The same over groups of N = 8 or 16 neighbouring lanes of a DPP row (log2 N row shifts): the total arrives in each
-// group's last lane.  With N = 8 a shift pulls values across the border between a row's two groups, but only into
-// lanes whose result is not used: lane 7 sums lanes 0 .. 7 and lane 15 lanes 8 .. 15.
+// Sum over groups of N = 8 or 16 neighbouring lanes of a DPP row (log2 N row shifts): the total arrives in each
+// group's last lane, the others hold prefix sums.  Every lane of the row must be active.  With N = 8 a shift pulls
+// values across the border between a row's two groups, but only into lanes whose result is not used: lane 7 sums
+// lanes 0 .. 7 and lane 15 lanes 8 .. 15.
 template <int N>
 __device__ __forceinline__ float dpp_lanes_total(float v) {
     static_assert(N == 8 || N == 16, "groups of 8 or 16 lanes");
