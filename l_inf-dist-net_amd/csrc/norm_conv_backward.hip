@@ -56,6 +56,7 @@ struct ConvBwd {
     int units, units_per_wg;         // what a workgroup walks: tiles of 64 rows (columns), whole images (image)
     int ring_rows;                   // IMG: image rows per channel plane held in LDS, a power of two
     int park_extra;                  // IMG: floats between the 1/out panel and the ring that the parked tile runs into
+    int slices;                      // workgroups per (group, column tile): units / units_per_wg, rounded up
 };
 
 inline size_t lds_bytes(int NG, size_t plane_floats) {
@@ -91,9 +92,17 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
     const int tid = threadIdx.x;
     constexpr int TYN = TR / TI;             // lanes along the rows
     const int ty = tid % TYN, tx = tid / TYN;   // rows first: the lanes of a column group are neighbours in a DPP row
-    const int tk = blockIdx.x % d.tiles_k, g = blockIdx.x / d.tiles_k;
+    // Consecutive workgroup ids go to different XCDs (8 per device, each with its own L2).  The grid is padded to a
+    // multiple of 8 and remapped so that every XCD gets one contiguous run of (slice, group, column tile) with the
+    // column tile fastest: the workgroups of one (slice, group) stage the same g and out, walk their units in step,
+    // and now find each other's fetches in their L2 (config 4: five column tiles; 771 MB fetched per launch before).
+    const int remapped = (int)(blockIdx.x % 8u) * (int)(gridDim.x / 8u) + (int)(blockIdx.x / 8u);
+    const int pairs = d.tiles_k * d.G;
+    if (remapped >= pairs * d.slices) return;   // padding
+    const int slice = remapped / pairs, pair = remapped - slice * pairs;
+    const int tk = pair % d.tiles_k, g = pair / d.tiles_k;
     const int k0 = tk * TC;
-    const int u_begin = blockIdx.y * d.units_per_wg, u_end = min(d.units, u_begin + d.units_per_wg);
+    const int u_begin = slice * d.units_per_wg, u_end = min(d.units, u_begin + d.units_per_wg);
 
     auto spower = [&](float u) {   // sign(u) * |u|^(p-1); by reference: the integer-exponent instantiations do not use e
         if constexpr (IE == 0) return __builtin_copysignf(pow_pos(__builtin_fabsf(u), e), u);   // u == 0: 0 either way
@@ -489,7 +498,7 @@ template <bool IMG, int IE>
 hipError_t launch_conv_backward(const float* grad_output, const float* input, const float* weight, const float* output,
                                 float* grad_input, float* grad_weight, float p, const Problem& pr, const ImgWin& win,
                                 hipStream_t stream) {
-    ConvBwd d{pr.B, pr.G, pr.K, pr.NG, pr.HW, pr.B * pr.HW, 0, 0, 0, 0, 0};
+    ConvBwd d{pr.B, pr.G, pr.K, pr.NG, pr.HW, pr.B * pr.HW, 0, 0, 0, 0, 0, 0};
     d.tiles_k = IMG ? (win.CG + kPlanes - 1) / kPlanes : (d.K + TCP - 1) / TCP;
     d.units = IMG ? pr.B : (d.M + TR - 1) / TR;
     const long pairs = (long)d.tiles_k * d.G;
@@ -514,11 +523,13 @@ hipError_t launch_conv_backward(const float* grad_output, const float* input, co
     }
     d.units_per_wg = (int)best;
     const long slices = (d.units + d.units_per_wg - 1) / d.units_per_wg;
+    d.slices = (int)slices;
+    const long grid = (pairs * slices + 7) / 8 * 8;   // whole rounds of the eight XCDs; the padding exits at once
     auto kern = norm_conv_backward_kernel<IMG, IE>;
     static LdsRecord lds_allowed = {};
     // the limit is raised once, to the most any layer may ask for
     if (hipError_t e = allow_lds(kern, kMaxLds, pr.device, lds_allowed); e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3((unsigned)pairs, (unsigned)slices), dim3(256), lds, stream, grad_output, input, weight,
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, stream, grad_output, input, weight,
                        output, grad_input, grad_weight, p - 1.0f, d, win);
     return hipGetLastError();
 }
