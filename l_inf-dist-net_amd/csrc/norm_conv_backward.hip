@@ -251,19 +251,35 @@ norm_conv_backward_kernel(const float* __restrict__ grad_output, const float* __
                 }
             }
         } else {
-            for (int i = tid; i < NG * TR; i += 256) {
-                const int n = i / TR, r = i % TR;
-                float c = 0.f, ri = 0.f;   // IE == 0: ri holds the output itself until the vote is in
-                if (r < rows) {
-                    const int m = first_row + r, bi = m / d.HW;
-                    const size_t o = ((size_t)(bi * d.G + g) * NG + n) * d.HW + (m - bi * d.HW);
-                    c = grad_output[o];
-                    const float out = output[o] * unit_inv;
-                    ri = IE > 0 ? __builtin_amdgcn_rcpf(out) : out;
-                    unsafe |= IE > 0 ? !(out >= 0x1p-12f && out <= 0x1p12f) : !(out >= 0.5f && out <= 2.0f);
+            // the same walk from the unfolded layout: a tile's rows may belong to two images, so a lane keeps the
+            // element offset of its row in output 0 and steps by HW per output
+            const int r = tid & (TR - 1);
+            const int m = first_row + min(r, rows - 1), bi = m / d.HW;
+            const size_t row0 = ((size_t)(bi * d.G + g) * NG) * d.HW + (m - bi * d.HW);
+#pragma unroll 1
+            for (int n0 = tid / TR; n0 < NG; n0 += 16) {
+                float gv[4], ov[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int n = min(n0 + 4 * u, NG - 1);   // past the last output: a valid address, the value is not used
+                    gv[u] = grad_output[row0 + (size_t)n * d.HW];
+                    ov[u] = output[row0 + (size_t)n * d.HW];
                 }
-                Cs[i] = c;
-                Rs[i] = ri;
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const int n = n0 + 4 * u;
+                    if (n < NG) {
+                        const float out = ov[u] * unit_inv;
+                        float c = 0.f, ri = 0.f;   // IE == 0: ri holds the output itself until the vote is in
+                        if (r < rows) {
+                            c = gv[u];
+                            ri = IE > 0 ? __builtin_amdgcn_rcpf(out) : out;
+                            unsafe |= IE > 0 ? !(out >= 0x1p-12f && out <= 0x1p12f) : !(out >= 0.5f && out <= 2.0f);
+                        }
+                        Cs[n * TR + r] = c;
+                        Rs[n * TR + r] = ri;
+                    }
+                }
             }
         }
         const bool factored = !__syncthreads_or(unsafe);   // also: the panels are written
