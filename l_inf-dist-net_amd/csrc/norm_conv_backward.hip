@@ -523,19 +523,25 @@ hipError_t launch_conv_backward(const float* grad_output, const float* input, co
         d.park_extra = park_extra(d.NG);
     }
     const size_t lds = lds_bytes(d.NG, IMG ? image_floats(d.NG, d.ring_rows, win.H, win.W) : 0);
-    // Units per workgroup: the choice that needs the fewest rounds of resident workgroups times units (the device
-    // holds `resident` of them at once), among those that keep the number of workgroups, each of which flushes a whole
-    // grad_weight tile at the end, within sixteen rounds; ties go to fewer, longer workgroups.
+    // Units per workgroup.  A CU issues at the same rate whether two, three or four workgroups share it, so what a
+    // launch takes is what the busiest CU has to work through: workgroups per CU (dealt round robin) times units per
+    // workgroup.  With few long workgroups that is uneven -- 860 workgroups of three images on 256 CUs leave twelve
+    // images on some CUs and nine on the others, a fifth above the mean -- so the choice minimises it, charging every
+    // workgroup a fixed cost (its weight tile and the flush of its grad_weight tile at the end: about a third of a
+    // 64-row tile) and the last one on a CU half its length (it runs partly alone, at half the CU's rate).  The number
+    // of workgroups stays within sixteen times what the device holds at once.
     long per_cu = (long)(160 * 1024 / lds);
     if (per_cu > 8) per_cu = 8;
     if (per_cu < 1) per_cu = 1;
     const long resident = per_cu * pr.num_cu;
-    long best = -1, best_cost = 0;
+    long best = -1;
+    double best_cost = 0;
+    const double fixed = IMG ? 0.3 / std::max(1, (pr.HW + TR - 1) / TR) : 0.3;   // in units: an image is HW / 64 tiles
     const long lo = std::max(1L, ((long)d.units * pairs + 16 * resident - 1) / (16 * resident));
     for (long upw = lo; upw <= d.units && upw < lo + 4096; upw++) {
         const long wgs = pairs * ((d.units + upw - 1) / upw);
-        const long cost = ((wgs + resident - 1) / resident) * upw;
-        if (best < 0 || cost <= best_cost) { best = upw; best_cost = cost; }
+        const double cost = (double)((wgs + pr.num_cu - 1) / pr.num_cu) * ((double)upw + fixed) + 0.5 * (double)upw;
+        if (best < 0 || cost < best_cost) { best = upw; best_cost = cost; }
     }
     d.units_per_wg = (int)best;
     const long slices = (d.units + d.units_per_wg - 1) / d.units_per_wg;
