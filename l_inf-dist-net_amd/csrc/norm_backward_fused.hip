@@ -7,7 +7,8 @@
 // 4.2 ms on 512 x 5120 -> 5120 at p = 20.5 where the two separate kernels take 3.6 + 3.1 ms.
 //
 // The kernel has the shape of the register-tiled grad_input kernel: a workgroup owns 128 rows m x BN inputs k and
-// walks the outputs n; a lane keeps an 8 x TN patch of x and of the grad_input sums.  For grad_weight the lane
+// walks the outputs n; a lane keeps an 8 x TN patch of x and of the grad_input sums (BN x TN = 80 x 5, 64 x 4 or
+// 48 x 3: the host takes the width whose tiles fill the device best).  For grad_weight the lane
 // also adds, per output n, its eight rows' terms of each of its TN columns (one more fused multiply-add per term),
 // the sixteen lanes that share those columns (one DPP row: the lane index runs along m first here) add their
 // partial sums over each half of the row with three row shifts, the halves' last lanes park the two totals of the
@@ -244,7 +245,24 @@ norm_backward_fused_kernel(const float* __restrict__ grad_output, const float* _
     auto store = [&]() {
         gk.store(lds, tid);
         ok_.store(lds + XS, tid);
-        wl.store(lds + 2 * XS, tid);
+        if constexpr (TN == 3) {
+            // three columns per lane at a pitch of four in the panel, so that the sweep's 128-bit reads stay as they
+            // are: column c of the tile lives at word (c / 3) * 4 + c % 3 of its panel row
+            float* panel = lds + 2 * XS;
+#pragma unroll
+            for (int i = 0; i < ColLoad::N; i++) {
+                const int id = tid + i * NT;
+                if (ColLoad::TOTAL % NT != 0 && id >= ColLoad::TOTAL) continue;
+                const int rr = id / ColLoad::PER_ROW, cq = id - rr * ColLoad::PER_ROW;
+#pragma unroll
+                for (int c4 = 0; c4 < 4; c4++) {
+                    const int c = cq * 4 + c4, third = c / 3;
+                    panel[rr * GEO::SN + ((third * 4 + (c - third * 3)) ^ swz(rr))] = wl.v[i][c4];
+                }
+            }
+        } else {
+            wl.store(lds + 2 * XS, tid);
+        }
     };
 
     const int nstage = (NG + KK - 1) / KK;
@@ -481,8 +499,8 @@ bool norm_backward_fused_applicable(const Problem& pr, float p, const void* grad
     const int ie = fused_int_power(p);
     if (ie == 1) return false;
     const long M = (long)pr.B * pr.HW;
-    const long t80 = ((M + 127) / 128) * ((pr.K + 79) / 80) * pr.G, t64 = ((M + 127) / 128) * ((pr.K + 63) / 64) * pr.G;
-    return (t80 > t64 ? t80 : t64) * 10 >= (ie == 2 ? 9L : 7L) * pr.num_cu && pr.NG >= 256;
+    const long t48 = ((M + 127) / 128) * ((pr.K + 47) / 48) * pr.G;   // the narrowest tiles: the most workgroups
+    return t48 * 10 >= (ie == 2 ? 9L : 7L) * pr.num_cu && pr.NG >= 256;
 }
 
 template <class GEO>
@@ -501,11 +519,18 @@ static hipError_t launch_fused_for(const Problem& pr, hipStream_t stream, const 
 hipError_t norm_backward_fused(const float* grad_output, const float* input, const float* weight, const float* output,
                                float* grad_input, float* grad_weight, float p, const Problem& pr, hipStream_t stream) {
     const long rows = (long)pr.B * pr.HW;
-    const long t80 = ((rows + 127) / 128) * ((pr.K + 79) / 80) * pr.G, t64 = ((rows + 127) / 128) * ((pr.K + 63) / 64) * pr.G;
-    const double c80 = (double)((t80 + pr.num_cu - 1) / pr.num_cu) * 80, c64 = (double)((t64 + pr.num_cu - 1) / pr.num_cu) * 64 * 1.1;
-    const bool wide = g_tile_override == 0 || (g_tile_override != 1 && c80 <= c64);
-    return wide ? launch_fused_for<Geo<128, 80, 8, 5, 2>>(pr, stream, grad_output, input, weight, output, grad_input, grad_weight, p)
-                : launch_fused_for<Geo<128, 64, 8, 4, 2>>(pr, stream, grad_output, input, weight, output, grad_input, grad_weight, p);
+    // Rounds of workgroups (one per CU) times columns per tile, the narrower tiles charged for what a term costs more
+    // in them (more LDS words and cross-lane steps per term).  3072 inputs at batch 512: 156 tiles of 80 columns, 192
+    // of 64 or 256 of 48 -- only the last fill the 256 CUs.
+    const long rt = (rows + 127) / 128;
+    const long t80 = rt * ((pr.K + 79) / 80) * pr.G, t64 = rt * ((pr.K + 63) / 64) * pr.G, t48 = rt * ((pr.K + 47) / 48) * pr.G;
+    const double c80 = (double)((t80 + pr.num_cu - 1) / pr.num_cu) * 80, c64 = (double)((t64 + pr.num_cu - 1) / pr.num_cu) * 64 * 1.1,
+                 c48 = (double)((t48 + pr.num_cu - 1) / pr.num_cu) * 48 * 1.2;
+    if (g_tile_override == 0 || (g_tile_override != 1 && c80 <= c64 && c80 <= c48))
+        return launch_fused_for<Geo<128, 80, 8, 5, 2>>(pr, stream, grad_output, input, weight, output, grad_input, grad_weight, p);
+    if (g_tile_override == 1 || c64 <= c48)
+        return launch_fused_for<Geo<128, 64, 8, 4, 2>>(pr, stream, grad_output, input, weight, output, grad_input, grad_weight, p);
+    return launch_fused_for<Geo<128, 48, 8, 3, 2>>(pr, stream, grad_output, input, weight, output, grad_input, grad_weight, p);
 }
 
 }  // namespace ldist

@@ -55,7 +55,7 @@ struct Geo {
     static constexpr int XS = KK * SM;           // floats of one x panel
     static constexpr int WS = KK * SN;
     static_assert(TM == 4 || TM == 8, "TM");
-    static_assert(TN == 4 || TN == 5 || TN == 8, "TN");
+    static_assert(TN == 3 || TN == 4 || TN == 5 || TN == 8, "TN");   // 3: columns tx*3 + j of the tile, kept at a pitch of four in the w panel
     static_assert(BM % TM == 0 && BN % TN == 0, "tile");
     static_assert(NT % 64 == 0, "whole waves");
 
@@ -67,6 +67,7 @@ struct Geo {
     __device__ static constexpr int col(int tx, int j) {
         return TN == 8 ? (j < 4 ? tx * 4 + j : BN / 2 + tx * 4 + (j - 4))
              : TN == 5 ? (j < 4 ? tx * 4 + j : TX * 4 + tx)
+             : TN == 3 ? tx * 3 + j
                        : tx * 4 + j;
     }
 };
@@ -101,7 +102,8 @@ __device__ __forceinline__ void read_x(const float* __restrict__ p, int r, float
 template <class GEO>
 __device__ __forceinline__ void read_w(const LanePtr<GEO>& lp, int r, float (&wf)[GEO::TN]) {
     float4 a = *reinterpret_cast<const float4*>(lp.w + r * GEO::SN);
-    wf[0] = a.x; wf[1] = a.y; wf[2] = a.z; wf[3] = a.w;
+    wf[0] = a.x; wf[1] = a.y; wf[2] = a.z;
+    if constexpr (GEO::TN > 3) wf[3] = a.w;   // TN == 3: the fourth word of the lane's pitch is not a column
     if constexpr (GEO::TN == 8) {
         float4 b = *reinterpret_cast<const float4*>(lp.w + r * GEO::SN + GEO::BN / 2);
         wf[4] = b.x; wf[5] = b.y; wf[6] = b.z; wf[7] = b.w;
@@ -174,7 +176,8 @@ __device__ __forceinline__ void read_frag(Frag<GEO, NX, KP>& f, const LaneAddr<G
     for (int e = 0; e < KP; e++) {
         const unsigned at = lp.w + (r + e) * (GEO::SN * 4u);
         const vec4f a = *(lds_vec4f*)(uintptr_t)at;
-        f.w[e][0] = a.x; f.w[e][1] = a.y; f.w[e][2] = a.z; f.w[e][3] = a.w;
+        f.w[e][0] = a.x; f.w[e][1] = a.y; f.w[e][2] = a.z;
+        if constexpr (GEO::TN > 3) f.w[e][3] = a.w;
         if constexpr (GEO::TN == 8) {
             const vec4f b = *(lds_vec4f*)(uintptr_t)(at + GEO::BN / 2 * 4u);
             f.w[e][4] = b.x; f.w[e][5] = b.y; f.w[e][6] = b.z; f.w[e][7] = b.w;

@@ -1465,6 +1465,28 @@ def test_norm_backward_both_gradients_in_one_pass(shape, p, tile):
         assert_sum_close(gw.cpu() - 0.125, ew, mw, p, RTOL, ATOL)
 
 
+@pytest.mark.parametrize("p", [8.0, 4.0, 20.5, 100.0])
+def test_norm_backward_one_pass_on_48_column_tiles(p):
+    """A layer of about 3072 inputs at batch 500: 128 x 80 and 128 x 64 tiles would leave CUs idle, so the one-call
+    backward takes its 128 x 48 geometry (three columns per lane, the weight panel at a pitch of four) of its own
+    accord; ragged in rows (500), outputs (260 = 4 stages of 64 + 4) and columns (3068 = 63 tiles of 48 + 44)."""
+    from gpu_common import DEV, cpp, say, set_tile
+    B, CO, CI, G, HW = 500, 260, 3068, 1, 1
+    say("norm_backward one pass, 48-column tiles", "p", p)
+    set_tile(-1)
+    x, w = make_inputs(B, CO, CI, G, HW, seed=61)
+    go = torch.randn(B, CO, HW, generator=gen(62))
+    out = oracle.norm_dist_forward(x, w, G, p)
+    ex, mx = oracle.norm_dist_backward_input(go, x, w, out, G, p, with_abs_terms=True)
+    ew, mw = oracle.norm_dist_backward_weight(go, x, w, out, G, p, with_abs_terms=True)
+    gx = torch.full((B, CI, HW), float("nan"), device=DEV)
+    gw = torch.zeros((CO, CI // G), device=DEV)
+    cpp.norm_dist_backward(go.to(DEV), x.to(DEV), w.to(DEV), out.to(DEV), gx, gw, G, p)
+    torch.cuda.synchronize()
+    assert_sum_close(gx.cpu(), ex, mx, p, RTOL, ATOL)
+    assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
+
+
 @pytest.mark.parametrize("p", [2.5, 20.0, 300.0, 8.0, 3.0])
 @pytest.mark.parametrize("scale", [1e-6, 3e-4, 1.0, 5e3, 1e6, "mixed", "one tiny row"])
 def test_norm_backward_both_gradients_at_every_scale(scale, p):
