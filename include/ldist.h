@@ -61,7 +61,9 @@ LDIST_API int ldist_last_hip_error(void);
  * where it would otherwise take the kernel that holds a tile's whole reduction axis
  * in LDS (K up to 320), and 0 / 1 force the register-tiled p-norm backward kernels
  * (128x80 / 128x64 tiles), the one-pass kernel of ldist_norm_dist_backward included,
- * 2 / 3 / 4 keep them off.  Process-wide; not thread safe. */
+ * 2 / 3 / 4 keep them off; 5 forces that one-pass kernel on with 128x48 tiles (its third
+ * width, which it otherwise takes where the wider ones leave CUs idle) and is like 2
+ * for every other kernel.  Process-wide; not thread safe. */
 LDIST_API int ldist_set_tile_override(int choice);
 /* Tuning knob, no counterpart in the reference: 1 (default) orders the tiles of
  * the forward kernels so that each of the 8 XCDs works on one contiguous run of

@@ -99,7 +99,7 @@ int ldist_set_xcd_remap(int on) {
 }
 
 int ldist_set_tile_override(int choice) {
-    if (choice < -1 || choice > 4) return LDIST_EINVAL;
+    if (choice < -1 || choice > 5) return LDIST_EINVAL;
     ldist::g_tile_override = choice;
     return LDIST_OK;
 }

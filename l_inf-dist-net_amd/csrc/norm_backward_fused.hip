@@ -490,7 +490,7 @@ bool norm_backward_fused_applicable(const Problem& pr, float p, const void* grad
     if (!(aligned16(grad_output) && aligned16(input) && aligned16(weight) && aligned16(output) && aligned16(grad_input) &&
           aligned16(grad_weight)))
         return false;
-    if (g_tile_override == 0 || g_tile_override == 1) return true;   // tests and tuning: forced on (128 x 80, 128 x 64)
+    if (g_tile_override == 0 || g_tile_override == 1 || g_tile_override == 5) return true;   // tests and tuning: forced on (128 x 80, 128 x 64, 128 x 48)
     if (g_tile_override >= 2) return false;                          // forced off
     // p = 2: a term is one instruction and sharing it saves less than the row sums of grad_weight cost (512 x 5120 ->
     // 5120: 1.44 against 1.42 ms).  p = 3: 1.65 against 1.83 ms where the tiles fill the device (10240 inputs: 3.30
@@ -526,9 +526,9 @@ hipError_t norm_backward_fused(const float* grad_output, const float* input, con
     const long t80 = rt * ((pr.K + 79) / 80) * pr.G, t64 = rt * ((pr.K + 63) / 64) * pr.G, t48 = rt * ((pr.K + 47) / 48) * pr.G;
     const double c80 = (double)((t80 + pr.num_cu - 1) / pr.num_cu) * 80, c64 = (double)((t64 + pr.num_cu - 1) / pr.num_cu) * 64 * 1.1,
                  c48 = (double)((t48 + pr.num_cu - 1) / pr.num_cu) * 48 * 1.2;
-    if (g_tile_override == 0 || (g_tile_override != 1 && c80 <= c64 && c80 <= c48))
+    if (g_tile_override == 0 || (g_tile_override != 1 && g_tile_override != 5 && c80 <= c64 && c80 <= c48))
         return launch_fused_for<Geo<128, 80, 8, 5, 2>>(pr, stream, grad_output, input, weight, output, grad_input, grad_weight, p);
-    if (g_tile_override == 1 || c64 <= c48)
+    if (g_tile_override == 1 || (g_tile_override != 5 && c64 <= c48))
         return launch_fused_for<Geo<128, 64, 8, 4, 2>>(pr, stream, grad_output, input, weight, output, grad_input, grad_weight, p);
     return launch_fused_for<Geo<128, 48, 8, 3, 2>>(pr, stream, grad_output, input, weight, output, grad_input, grad_weight, p);
 }

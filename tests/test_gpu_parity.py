@@ -1437,7 +1437,7 @@ def test_norm_dist_conv_layer_runs_from_the_image_without_columns(p):
 FUSED_BACKWARD_SHAPES = [sh for sh in TILED_BACKWARD_SHAPES if sh[4] == 1] + [(515, 140, 100, 1, 1), (70, 200, 132, 1, 1)]
 
 
-@pytest.mark.parametrize("tile", [0, 1])
+@pytest.mark.parametrize("tile", [0, 1, 5])
 @pytest.mark.parametrize("p", [5.0, 5.5, 9.0, 20.0, 100.0, 8.0, 2.0, 3.0, 4.0])
 @pytest.mark.parametrize("shape", FUSED_BACKWARD_SHAPES + [(1030, 24, 44, 1, 1), (512, 64, 20, 1, 1)])
 def test_norm_backward_both_gradients_in_one_pass(shape, p, tile):

@@ -103,6 +103,14 @@ def test_random_problem(seed):
     torch.cuda.synchronize()
     assert_sum_close(gx.cpu(), ex, mx, p, RTOL, ATOL)
     assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
+    if seed % 2:   # and the one-pass kernel's third width, 128 x 48 tiles (three columns per lane), forced on
+        set_tile(5)
+        gx = torch.full((B, CI, HW), float("nan"), device=DEV)
+        gw = torch.zeros((CO, CI // G), device=DEV)
+        cpp.norm_dist_backward(*args, gx, gw, G, p)
+        torch.cuda.synchronize()
+        assert_sum_close(gx.cpu(), ex, mx, p, RTOL, ATOL)
+        assert_sum_close(gw.cpu(), ew, mw, p, RTOL, ATOL)
 
 
 def draw_image(seed):
